@@ -1,0 +1,171 @@
+"""Architecture description and synthetic tensors for the FLUX.2-klein denoising transformer.
+
+The tensor names and shapes are the safetensors keys the reference loader reads
+(flux_transformer.c:4452-4602); the default sizes are flux.h:33-41.
+"""
+import ctypes
+import os
+from collections import OrderedDict
+from dataclasses import dataclass, asdict
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+@dataclass(frozen=True)
+class FluxConfig:
+    hidden: int = 3072
+    heads: int = 24
+    head_dim: int = 128
+    mlp: int = 9216
+    n_double: int = 5
+    n_single: int = 20
+    text_dim: int = 7680
+    channels: int = 128
+    axis_dim: int = 32
+    sincos_dim: int = 256
+    rope_theta: float = 2000.0
+
+    def as_dict(self):
+        return asdict(self)
+
+
+KLEIN_4B = FluxConfig()
+# A structurally identical model small enough for the CPU oracle to run in well under a second.
+TINY = FluxConfig(hidden=256, heads=2, mlp=768, n_double=2, n_single=3, text_dim=384)
+# One size up: 4 heads, used to exercise multi-tile GEMM/attention shapes.
+SMALL = FluxConfig(hidden=512, heads=4, mlp=1536, n_double=2, n_single=4, text_dim=768)
+
+
+def tensor_shapes(cfg: FluxConfig) -> "OrderedDict[str, tuple]":
+    H, M, hd = cfg.hidden, cfg.mlp, cfg.head_dim
+    t = OrderedDict()
+    t["x_embedder.weight"] = (H, cfg.channels)
+    t["context_embedder.weight"] = (H, cfg.text_dim)
+    t["time_guidance_embed.timestep_embedder.linear_1.weight"] = (H, cfg.sincos_dim)
+    t["time_guidance_embed.timestep_embedder.linear_2.weight"] = (H, H)
+    t["double_stream_modulation_img.linear.weight"] = (6 * H, H)
+    t["double_stream_modulation_txt.linear.weight"] = (6 * H, H)
+    t["single_stream_modulation.linear.weight"] = (3 * H, H)
+    for i in range(cfg.n_double):
+        p = f"transformer_blocks.{i}."
+        for n in ("norm_q", "norm_k", "norm_added_q", "norm_added_k"):
+            t[p + f"attn.{n}.weight"] = (hd,)
+        for n in ("to_q", "to_k", "to_v", "add_q_proj", "add_k_proj", "add_v_proj"):
+            t[p + f"attn.{n}.weight"] = (H, H)
+        t[p + "attn.to_out.0.weight"] = (H, H)
+        t[p + "attn.to_add_out.weight"] = (H, H)
+        t[p + "ff.linear_in.weight"] = (2 * M, H)
+        t[p + "ff_context.linear_in.weight"] = (2 * M, H)
+        t[p + "ff.linear_out.weight"] = (H, M)
+        t[p + "ff_context.linear_out.weight"] = (H, M)
+    for i in range(cfg.n_single):
+        p = f"single_transformer_blocks.{i}."
+        t[p + "attn.norm_q.weight"] = (hd,)
+        t[p + "attn.norm_k.weight"] = (hd,)
+        t[p + "attn.to_qkv_mlp_proj.weight"] = (3 * H + 2 * M, H)
+        t[p + "attn.to_out.weight"] = (H, H + M)
+    t["norm_out.linear.weight"] = (2 * H, H)
+    t["proj_out.weight"] = (cfg.channels, H)
+    return t
+
+
+def is_qk_norm(name: str) -> bool:
+    return ".attn.norm_" in name
+
+
+_synth = None
+
+
+def synth_lib():
+    global _synth
+    if _synth is None:
+        path = os.path.join(_HERE, "libflux_synth.so")
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is not built; run `python -c 'import __graft_entry__ as g; g.build()'`")
+        lib = ctypes.CDLL(path)
+        vp, i64, u64, f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_uint64, ctypes.c_float
+        lib.flux_synth_normal_f32.argtypes = [vp, i64, u64, u64, f32, f32]
+        lib.flux_synth_normal_bf16.argtypes = [vp, i64, u64, u64, f32, f32]
+        lib.flux_synth_fill_bf16.argtypes = [vp, i64, f32]
+        lib.flux_synth_f32_to_bf16.argtypes = [vp, vp, i64]
+        lib.flux_synth_bf16_to_f32.argtypes = [vp, vp, i64]
+        for f in (lib.flux_synth_normal_f32, lib.flux_synth_normal_bf16, lib.flux_synth_fill_bf16,
+                  lib.flux_synth_f32_to_bf16, lib.flux_synth_bf16_to_f32):
+            f.restype = None
+        _synth = lib
+    return _synth
+
+
+def normal_f32(shape, seed, stream, mean=0.0, std=1.0):
+    out = np.empty(shape, dtype=np.float32)
+    synth_lib().flux_synth_normal_f32(out.ctypes.data, out.size, seed, stream, mean, std)
+    return out
+
+
+def normal_bf16(shape, seed, stream, mean=0.0, std=1.0):
+    out = np.empty(shape, dtype=np.uint16)
+    synth_lib().flux_synth_normal_bf16(out.ctypes.data, out.size, seed, stream, mean, std)
+    return out
+
+
+def f32_to_bf16(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint16)
+    synth_lib().flux_synth_f32_to_bf16(out.ctypes.data, x.ctypes.data, x.size)
+    return out
+
+
+def bf16_to_f32(x):
+    x = np.ascontiguousarray(x, dtype=np.uint16)
+    out = np.empty(x.shape, dtype=np.float32)
+    synth_lib().flux_synth_bf16_to_f32(out.ctypes.data, x.ctypes.data, x.size)
+    return out
+
+
+def make_weights(cfg: FluxConfig, seed=42, std=0.02, qk_norm="literal", only=None):
+    """bf16 weights (uint16 arrays) keyed by tensor name.
+
+    qk_norm="literal": the [head_dim] QK-norm weights are N(0, std) like every other tensor.
+    qk_norm="sharp":   they are 1.0 (the usual RMSNorm initialisation), which gives attention
+                       logits of order one so that RoPE/QK-norm/softmax errors become visible.
+    """
+    out = OrderedDict()
+    for idx, (name, shape) in enumerate(tensor_shapes(cfg).items()):
+        if only is not None and name not in only:
+            continue
+        if is_qk_norm(name) and qk_norm == "sharp":
+            a = np.empty(shape, dtype=np.uint16)
+            synth_lib().flux_synth_fill_bf16(a.ctypes.data, a.size, 1.0)
+        else:
+            a = normal_bf16(shape, seed, idx, 0.0, std)
+        out[name] = a
+    return out
+
+
+def write_safetensors(path, tensors):
+    """Minimal safetensors writer for bf16 tensors (format: flux_safetensors.h:4-8)."""
+    import json
+    header = {}
+    off = 0
+    for name, a in tensors.items():
+        nb = a.size * 2
+        header[name] = {"dtype": "BF16", "shape": list(a.shape), "data_offsets": [off, off + nb]}
+        off += nb
+    hj = json.dumps(header, separators=(",", ":")).encode()
+    hj += b" " * ((8 - len(hj) % 8) % 8)
+    with open(path, "wb") as f:
+        f.write(len(hj).to_bytes(8, "little"))
+        f.write(hj)
+        for a in tensors.values():
+            f.write(np.ascontiguousarray(a).tobytes())
+
+
+def flops_per_forward(cfg: FluxConfig, n_img, n_txt, n_img_out=None):
+    """Algorithmic FLOPs of one forward (1 MAC = 2 FLOP)."""
+    H, C, T = cfg.hidden, cfg.channels, cfg.text_dim
+    n = n_img + n_txt
+    n_out = n_img if n_img_out is None else n_img_out
+    per_block = (2 * n * H * (3 * H + 2 * cfg.mlp) + 2 * n * (H + cfg.mlp) * H) + 4 * n * n * H
+    return (cfg.n_double + cfg.n_single) * per_block + 2 * n_img * C * H + 2 * n_txt * T * H + 2 * n_out * H * C

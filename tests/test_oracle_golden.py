@@ -1,0 +1,204 @@
+"""Pins the CPU oracle against vectors produced by the reference's own C code.
+
+tests/golden/*.npz were written by tests/golden/make_golden.py, which executes the reference
+sources compiled in place (oracle/_ref). The inputs are regenerated here from the same seeds.
+Tolerances: both sides are fp32; the only differences are summation order (BLAS vs naive loops,
+materialised vs online softmax) and -ffast-math, so 2e-5 relative is ample and a dropped term,
+wrong sign, wrong chunk order or transposed operand is orders of magnitude larger.
+"""
+import os
+
+import numpy as np
+import pytest
+
+from metrics import rel_l2
+from model_spec import TINY, KLEIN_4B, make_weights, normal_f32, bf16_to_f32
+
+SEED = 7
+TOL = 2e-5
+
+
+@pytest.fixture(scope="module")
+def ops(golden_dir):
+    return np.load(os.path.join(golden_dir, "ops.npz"))
+
+
+def close(a, b, tol=TOL):
+    assert a.shape == b.shape
+    r = rel_l2(a, b)
+    assert r <= tol, r
+
+
+def test_timestep_embedding(oracle_mod, ops):
+    for t in (0.0, 250.0, 967.384, 1000.0):
+        got = oracle_mod.timestep_embedding(t)
+        np.testing.assert_allclose(got, ops[f"temb_{t}"], atol=2e-6)
+
+
+def test_rope_tables(oracle_mod, ops):
+    for (ph, pw, toff) in ((4, 3, 0), (3, 5, 10), (2, 2, 20)):
+        c, s = oracle_mod.rope_image(ph, pw, 32, 2000.0, toff)
+        np.testing.assert_allclose(c, ops[f"rope_img_{ph}_{pw}_{toff}_cos"], atol=1e-6)
+        np.testing.assert_allclose(s, ops[f"rope_img_{ph}_{pw}_{toff}_sin"], atol=1e-6)
+    c, s = oracle_mod.rope_text(9)
+    np.testing.assert_allclose(c, ops["rope_txt_9_cos"], atol=1e-6)
+    np.testing.assert_allclose(s, ops["rope_txt_9_sin"], atol=1e-6)
+
+
+def test_apply_rope(oracle_mod, ops):
+    x = normal_f32((12, 3 * 128), SEED, 1)
+    c, s = oracle_mod.rope_image(4, 3)
+    close(oracle_mod.apply_rope(x, c, s, 3, 128), ops["apply_rope"], 1e-6)
+
+
+def test_adaln(oracle_mod, ops):
+    x = normal_f32((6, 256), SEED, 2, 0.3, 2.0)
+    sh = normal_f32((256,), SEED, 3)
+    sc = normal_f32((256,), SEED, 4)
+    close(oracle_mod.adaln(x, sh, sc), ops["adaln"], 2e-6)
+
+
+def test_qk_norm(oracle_mod, ops):
+    q = normal_f32((5, 256), SEED, 5)
+    k = normal_f32((5, 256), SEED, 6, 0.0, 3.0)
+    qw = normal_f32((128,), SEED, 7)
+    kw = normal_f32((128,), SEED, 8)
+    gq, gk = oracle_mod.qk_norm(q, k, qw, kw, 2, 128)
+    close(gq, ops["qknorm_q"], 2e-6)
+    close(gk, ops["qknorm_k"], 2e-6)
+
+
+def test_gated_add_linear_softmax_silu(oracle_mod, ops):
+    o = normal_f32((4, 256), SEED, 9)
+    gt = normal_f32((256,), SEED, 10)
+    pr = normal_f32((4, 256), SEED, 11)
+    close(oracle_mod.gated_add(o, gt, pr), ops["gated_add"], 1e-6)
+    x = normal_f32((7, 96), SEED, 12)
+    W = normal_f32((40, 96), SEED, 13)
+    close(oracle_mod.linear(x, W), ops["linear"], 2e-6)
+    close(oracle_mod.softmax(normal_f32((5, 33), SEED, 14, 0.0, 4.0)), ops["softmax"], 2e-6)
+    close(oracle_mod.silu(normal_f32((300,), SEED, 15, 0.0, 3.0)), ops["silu"], 2e-6)
+
+
+def test_attention_vs_reference_flash_and_naive(oracle_mod, ops):
+    for tag, sq, sk in (("small", 12, 19), ("tiled", 70, 141)):
+        q = normal_f32((sq, 256), SEED, 20)
+        k = normal_f32((sk, 256), SEED, 21)
+        v = normal_f32((sk, 256), SEED, 22)
+        close(oracle_mod.attention(q, k, v, 2, 128), ops[f"flash_{tag}"], 5e-6)
+    # the reference's third implementation works on [heads, seq, hd]
+    q = normal_f32((2, 12, 128), SEED, 23)
+    k = normal_f32((2, 19, 128), SEED, 24)
+    v = normal_f32((2, 19, 128), SEED, 25)
+    got = oracle_mod.attention(q.transpose(1, 0, 2).reshape(12, 256), k.transpose(1, 0, 2).reshape(19, 256),
+                               v.transpose(1, 0, 2).reshape(19, 256), 2, 128)
+    close(got.reshape(12, 2, 128).transpose(1, 0, 2), ops["naive_attn"], 5e-6)
+
+
+def test_schedules(oracle_mod, ops):
+    for n in (1, 4, 7):
+        np.testing.assert_allclose(oracle_mod.linear_schedule(n), ops[f"sched_linear_{n}"], atol=1e-7)
+    np.testing.assert_allclose(oracle_mod.power_schedule(5, 2.0), ops["sched_power_5_2"], atol=1e-7)
+    for n, sl in ((4, 256), (4, 1024), (4, 4096), (50, 1024), (4, 5000), (1, 16), (28, 4300)):
+        np.testing.assert_allclose(oracle_mod.official_schedule(n, sl), ops[f"sched_official_{n}_{sl}"], atol=2e-7)
+
+
+def test_rng_and_noise(oracle_mod, ops):
+    np.testing.assert_allclose(oracle_mod.randn(64, 42), ops["randn_42"], atol=1e-6)
+    np.testing.assert_allclose(oracle_mod.init_noise(128, 4, 4, 42), ops["noise_42_4x4"], atol=1e-6)
+    np.testing.assert_allclose(oracle_mod.init_noise(128, 3, 5, 123), ops["noise_123_3x5"], atol=1e-6)
+
+
+def _inputs(cfg):
+    return dict(lat=normal_f32((cfg.channels, 4, 4), SEED, 100), txt=normal_f32((16, cfg.text_dim), SEED, 101),
+                txt_u=normal_f32((12, cfg.text_dim), SEED, 102), ref1=normal_f32((cfg.channels, 2, 3), SEED, 103),
+                ref2=normal_f32((cfg.channels, 3, 2), SEED, 104))
+
+
+@pytest.mark.parametrize("qk", ["literal", "sharp"])
+def test_tiny_model(oracle_mod, golden_dir, qk):
+    O = oracle_mod
+    cfg = TINY
+    g = np.load(os.path.join(golden_dir, f"tiny_{qk}.npz"))
+    W = make_weights(cfg, 42, 0.02, qk)
+    m = O.Oracle(cfg, W)
+    H = cfg.hidden
+    d = _inputs(cfg)
+
+    e = O.timestep_embedding(500.0)
+    fc1 = bf16_to_f32(W["time_guidance_embed.timestep_embedder.linear_1.weight"])
+    fc2 = bf16_to_f32(W["time_guidance_embed.timestep_embedder.linear_2.weight"])
+    close(O.time_mlp(e, fc1, fc2), g["time_mlp"])
+
+    # joint attention: the oracle works on one [text ; image] buffer, the reference on two streams
+    iq, ik, iv = (normal_f32((12, H), SEED, s) for s in (30, 31, 32))
+    tq, tk, tv = (normal_f32((7, H), SEED, s) for s in (33, 34, 35))
+    out = O.attention(np.concatenate([tq, iq]), np.concatenate([tk, ik]), np.concatenate([tv, iv]), cfg.heads, 128)
+    close(out[7:], g["joint_img"], 5e-6)
+    close(out[:7], g["joint_txt"], 5e-6)
+    close(O.attention(iq, ik, iv, cfg.heads, 128), g["mha"], 5e-6)
+
+    ic, isn = O.rope_image(3, 4)
+    tc, ts = O.rope_text(7)
+    ih = normal_f32((12, H), SEED, 40)
+    th = normal_f32((7, H), SEED, 41)
+    im = normal_f32((6 * H,), SEED, 42, 0.0, 0.5)
+    tm = normal_f32((6 * H,), SEED, 43, 0.0, 0.5)
+    gi, gt = m.double_block(1, ih, th, im, tm, ic, isn, tc, ts)
+    close(gi, g["dbl_img"])
+    close(gt, g["dbl_txt"])
+
+    # the reference derives the single-block modulation from t_emb inside the block
+    x = normal_f32((19, H), SEED, 44)
+    temb = normal_f32((H,), SEED, 45, 0.0, 3.0)
+    mod = O.linear(O.silu(temb)[None, :], bf16_to_f32(W["single_stream_modulation.linear.weight"]))[0]
+    close(m.single_block(2, x, mod, ic, isn, tc, ts, 7), g["sgl"])
+
+    close(m.forward(d["lat"], 4, 4, d["txt"], 1.0), g["fwd_t1.0"])
+    close(m.forward(d["lat"], 4, 4, d["txt"], 0.37), g["fwd_t0.37"])
+    r1 = (d["ref1"], 2, 3, 10)
+    r2 = (d["ref2"], 3, 2, 20)
+    close(m.forward(d["lat"], 4, 4, d["txt"], 0.6, refs=[r1]), g["fwd_ref1"])
+    close(m.forward(d["lat"], 4, 4, d["txt"], 0.6, refs=[r1, r2]), g["fwd_ref2"])
+
+    s3 = O.official_schedule(3, 16)
+    close(m.sample_euler(d["lat"], 4, 4, d["txt"], s3), g["euler3"])
+    close(m.sample_euler(d["lat"], 4, 4, d["txt"], s3, refs=[r1]), g["euler3_ref1"])
+    close(m.sample_euler(d["lat"], 4, 4, d["txt"], s3, refs=[r1, r2]), g["euler3_ref2"])
+    close(m.sample_euler_cfg(d["lat"], 4, 4, d["txt"], d["txt_u"], 4.0, s3[:3]), g["cfg2"])
+    close(m.sample_euler_cfg(d["lat"], 4, 4, d["txt"], d["txt_u"], 4.0, s3[:3], refs=[r1]), g["cfg2_ref1"])
+    close(m.sample_euler_cfg(d["lat"], 4, 4, d["txt"], d["txt_u"], 4.0, s3[:3], refs=[r1, r2]), g["cfg2_ref2"])
+    m.close()
+
+
+def test_golden_is_sensitive_to_rope(oracle_mod, golden_dir):
+    """The sharp fixture must notice a wrong rotation; otherwise it would pin nothing about RoPE."""
+    O = oracle_mod
+    cfg = TINY
+    g = np.load(os.path.join(golden_dir, "tiny_sharp.npz"))
+    W = make_weights(cfg, 42, 0.02, "sharp")
+    m = O.Oracle(cfg, W)
+    H = cfg.hidden
+    ic, isn = O.rope_image(3, 4)
+    tc, ts = O.rope_text(7)
+    ih = normal_f32((12, H), SEED, 40)
+    th = normal_f32((7, H), SEED, 41)
+    im = normal_f32((6 * H,), SEED, 42, 0.0, 0.5)
+    tm = normal_f32((6 * H,), SEED, 43, 0.0, 0.5)
+    gi, _ = m.double_block(1, ih, th, im, tm, ic, -isn, tc, ts)  # rotate the wrong way
+    assert rel_l2(gi, g["dbl_img"]) > 1e-3
+    m.close()
+
+
+@pytest.mark.slow
+@pytest.mark.skipif(not os.environ.get("FLUX_SLOW"), reason="full 4B oracle forward: set FLUX_SLOW=1 (needs ~25 GB RAM)")
+@pytest.mark.parametrize("qk", ["literal", "sharp"])
+def test_klein4b_c1(oracle_mod, golden_dir, qk):
+    path = os.path.join(golden_dir, f"klein4b_c1_{qk}.npz")
+    g = np.load(path)
+    cfg = KLEIN_4B
+    m = oracle_mod.Oracle(cfg, make_weights(cfg, 42, 0.02, qk))
+    lat = normal_f32((cfg.channels, 4, 4), 42, 1000)
+    txt = normal_f32((64, cfg.text_dim), 42, 1001)
+    close(m.forward(lat, 4, 4, txt, 1.0), g["velocity"], 5e-5)
+    m.close()

@@ -1,0 +1,122 @@
+"""Pins the oracle's operators against what the mathematics fixes, independently of any fixture."""
+import numpy as np
+
+from metrics import rel_l2
+from model_spec import normal_f32
+
+
+def np_softmax(x):
+    x = x.astype(np.float64)
+    e = np.exp(x - x.max(axis=-1, keepdims=True))
+    return e / e.sum(axis=-1, keepdims=True)
+
+
+def test_linear_matches_numpy(oracle_mod):
+    x = normal_f32((13, 70), 1, 1)
+    W = normal_f32((29, 70), 1, 2)
+    assert rel_l2(oracle_mod.linear(x, W), x.astype(np.float64) @ W.astype(np.float64).T) < 1e-6
+
+
+def test_adaln_zero_modulation_is_layernorm(oracle_mod):
+    x = normal_f32((9, 384), 1, 3, 2.0, 5.0)
+    z = np.zeros(384, np.float32)
+    y = oracle_mod.adaln(x, z, z)
+    assert np.abs(y.mean(axis=1)).max() < 1e-5
+    assert np.abs(y.var(axis=1) - 1.0).max() < 1e-4          # biased variance, eps 1e-6
+    sh = normal_f32((384,), 1, 4)
+    sc = normal_f32((384,), 1, 5)
+    assert rel_l2(oracle_mod.adaln(x, sh, sc), (1.0 + sc) * y + sh) < 1e-6
+
+
+def test_qk_norm_unit_rms(oracle_mod):
+    q = normal_f32((6, 3 * 128), 1, 6, 0.0, 7.0)
+    one = np.ones(128, np.float32)
+    gq, gk = oracle_mod.qk_norm(q, q * 0.01, one, 2 * one, 3, 128)
+    rms = np.sqrt((gq.reshape(6, 3, 128) ** 2).mean(-1))
+    assert np.abs(rms - 1).max() < 1e-4
+    rms_k = np.sqrt((gk.reshape(6, 3, 128) ** 2).mean(-1))
+    assert np.abs(rms_k - 2).max() < 1e-2      # eps matters a little at small magnitude
+
+
+def test_rope_is_pairwise_rotation(oracle_mod):
+    c, s = oracle_mod.rope_image(5, 7, 32, 2000.0, 0)
+    # duplicated on (2d, 2d+1), unit modulus, identity on the T and L axes of image tokens
+    assert np.array_equal(c[:, 0::2], c[:, 1::2]) and np.array_equal(s[:, 0::2], s[:, 1::2])
+    assert np.abs(c * c + s * s - 1).max() < 1e-6
+    assert np.all(c[:, :32] == 1) and np.all(s[:, :32] == 0) and np.all(c[:, 96:] == 1)
+    # closed form: angle = pos * theta^(-2d/32); rows -> axis 1, cols -> axis 2
+    d = np.arange(16)
+    f = 2000.0 ** (-2.0 * d / 32.0)
+    tok = 3 * 7 + 4                                      # row 3, col 4
+    np.testing.assert_allclose(c[tok, 32:64:2], np.cos(3 * f), atol=1e-5)
+    np.testing.assert_allclose(s[tok, 64:96:2], np.sin(4 * f), atol=1e-5)
+    ct, st = oracle_mod.rope_text(11)
+    assert np.all(ct[:, :96] == 1) and np.all(st[:, :96] == 0)
+    np.testing.assert_allclose(st[10, 96::2], np.sin(10 * f), atol=1e-5)
+    cr, sr = oracle_mod.rope_image(2, 2, 32, 2000.0, 10)
+    np.testing.assert_allclose(cr[3, 0:32:2], np.cos(10 * f), atol=1e-5)
+    # application: complex multiplication per pair, norm preserving
+    x = normal_f32((35, 2 * 128), 1, 7)
+    y = oracle_mod.apply_rope(x, c, s, 2, 128)
+    xc = x.reshape(35, 2, 64, 2)
+    z = (xc[..., 0] + 1j * xc[..., 1]) * (c[:, None, 0::2] + 1j * s[:, None, 0::2])
+    want = np.stack([z.real, z.imag], -1).reshape(35, 256)
+    assert rel_l2(y, want) < 1e-6
+    np.testing.assert_allclose(np.linalg.norm(y, axis=1), np.linalg.norm(x, axis=1), rtol=1e-5)
+
+
+def test_attention_closed_forms(oracle_mod):
+    heads, hd = 3, 128
+    q = normal_f32((10, heads * hd), 1, 8)
+    v1 = normal_f32((1, heads * hd), 1, 9)
+    # one key: output is that value row regardless of scores
+    out = oracle_mod.attention(q, v1 * 3, v1, heads, hd)
+    assert rel_l2(out, np.repeat(v1, 10, 0)) < 1e-6
+    # identical keys: uniform weights -> mean of V
+    k = np.repeat(normal_f32((1, heads * hd), 1, 10), 17, 0)
+    v = normal_f32((17, heads * hd), 1, 11)
+    out = oracle_mod.attention(q, k, v, heads, hd)
+    assert rel_l2(out, np.repeat(v.mean(0, keepdims=True), 10, 0)) < 1e-5
+    # brute force in float64, seq_q != seq_k
+    k = normal_f32((23, heads * hd), 1, 12)
+    v = normal_f32((23, heads * hd), 1, 13)
+    want = np.empty((10, heads * hd))
+    for h in range(heads):
+        sl = slice(h * hd, (h + 1) * hd)
+        p = np_softmax(q[:, sl].astype(np.float64) @ k[:, sl].astype(np.float64).T / np.sqrt(hd))
+        want[:, sl] = p @ v[:, sl]
+    assert rel_l2(oracle_mod.attention(q, k, v, heads, hd), want) < 1e-6
+
+
+def test_timestep_embedding_closed_form(oracle_mod):
+    t = 437.5
+    e = oracle_mod.timestep_embedding(t)
+    i = np.arange(128)
+    f = np.exp(-np.log(10000.0) * i / 128.0)
+    np.testing.assert_allclose(e[:128], np.cos(t * f), atol=2e-4)    # cos half first
+    np.testing.assert_allclose(e[128:], np.sin(t * f), atol=2e-4)
+
+
+def test_official_schedule_closed_form(oracle_mod):
+    s = oracle_mod.official_schedule(4, 4096)
+    assert s[0] == 1.0 and s[-1] == 0.0 and np.all(np.diff(s) < 0)
+    a1, b1, a2, b2 = 8.73809524e-05, 1.89833333, 0.00016927, 0.45666666
+    m200, m10 = a2 * 4096 + b2, a1 * 4096 + b1
+    a = (m200 - m10) / 190.0
+    mu = a * 4 + (m200 - 200 * a)
+    assert abs(mu - 2.2912) < 1e-3
+    t = np.array([0.75, 0.5, 0.25])
+    np.testing.assert_allclose(s[1:4], np.exp(mu) / (np.exp(mu) + (1 / t - 1)), rtol=1e-5)
+    # beyond 4300 image tokens mu is the single line a2*n+b2
+    s5 = oracle_mod.official_schedule(2, 5000)
+    mu5 = a2 * 5000 + b2
+    np.testing.assert_allclose(s5[1], np.exp(mu5) / (np.exp(mu5) + 1.0), rtol=1e-5)
+
+
+def test_silu_softmax(oracle_mod):
+    x = normal_f32((64,), 1, 14, 0.0, 4.0)
+    np.testing.assert_allclose(oracle_mod.silu(x), x / (1 + np.exp(-x.astype(np.float64))), rtol=1e-5, atol=1e-6)
+    m = normal_f32((4, 50), 1, 15, 0.0, 5.0)
+    p = oracle_mod.softmax(m)
+    np.testing.assert_allclose(p.sum(1), 1, atol=1e-5)
+    np.testing.assert_allclose(p, np_softmax(m), atol=1e-6)
