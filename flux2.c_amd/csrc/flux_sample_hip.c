@@ -1,0 +1,309 @@
+/*
+ * flux_sample_hip.c - Euler / CFG samplers and the single-forward entry points on MI355X.
+ *
+ * Exports the reference's sampler functions (flux_sample.c:212, 303, 381, 457, 534, 615) and
+ * schedules (flux_sample.c:49, 62, 145) with their signatures. The loop itself is device
+ * resident: latent, text and reference tokens are uploaded once, every step's latent update
+ * runs as a kernel (z += dt v, or the CFG combine), and the latent comes back once at the end.
+ * The host thread only queues work; step callbacks therefore fire at queue time.
+ */
+#include "../../include/flux_hip.h"
+#include "host_internal.h"
+#include <hip/hip_runtime_api.h>
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+double flux_timing_transformer_total = 0.0;
+double flux_timing_transformer_double = 0.0;
+double flux_timing_transformer_single = 0.0;
+double flux_timing_transformer_final = 0.0;
+
+void flux_reset_timing(void) {
+    flux_timing_transformer_total = flux_timing_transformer_double = 0.0;
+    flux_timing_transformer_single = flux_timing_transformer_final = 0.0;
+}
+
+/* ------------------------------------------------------------------ schedules */
+
+float *flux_linear_schedule(int num_steps) {
+    float *s = (float *)malloc((num_steps + 1) * sizeof(float));
+    for (int i = 0; i <= num_steps; i++) s[i] = 1.0f - (float)i / (float)num_steps;
+    return s;
+}
+
+float *flux_power_schedule(int num_steps, float alpha) {
+    float *s = (float *)malloc((num_steps + 1) * sizeof(float));
+    for (int i = 0; i <= num_steps; i++) s[i] = 1.0f - powf((float)i / (float)num_steps, alpha);
+    return s;
+}
+
+/* mu from two line fits in the image sequence length, then t -> e^mu / (e^mu + (1/t - 1))
+ * (flux_sample.c:122-155). */
+float *flux_official_schedule(int num_steps, int image_seq_len) {
+    const float a1 = 8.73809524e-05f, b1 = 1.89833333f, a2 = 0.00016927f, b2 = 0.45666666f;
+    float mu;
+    if (image_seq_len > 4300) {
+        mu = a2 * image_seq_len + b2;
+    } else {
+        float m200 = a2 * image_seq_len + b2, m10 = a1 * image_seq_len + b1;
+        float a = (m200 - m10) / 190.0f;
+        mu = a * num_steps + (m200 - 200.0f * a);
+    }
+    float *s = (float *)malloc((num_steps + 1) * sizeof(float));
+    for (int i = 0; i <= num_steps; i++) {
+        float t = 1.0f - (float)i / (float)num_steps;
+        if (t <= 0.0f) s[i] = 0.0f;
+        else if (t >= 1.0f) s[i] = 1.0f;
+        else s[i] = expf(mu) / (expf(mu) + (1.0f / t - 1.0f));
+    }
+    return s;
+}
+
+/* ------------------------------------------------------------------ stage timing */
+
+#define EV_MAX_FORWARDS 512
+struct fh_events {
+    hipEvent_t e[EV_MAX_FORWARDS][4];
+    int created, used;
+};
+static struct fh_events g_events;
+
+void fh_event_record(fh_events *ev, int which) {
+    if (ev->used >= EV_MAX_FORWARDS) return;
+    hipEventRecord(ev->e[ev->used][which], (hipStream_t)flux_hip_stream());
+}
+
+static fh_events *events_begin(int forwards) {
+    if (forwards > EV_MAX_FORWARDS) return NULL;
+    while (g_events.created < forwards) {
+        for (int k = 0; k < 4; k++)
+            if (hipEventCreate(&g_events.e[g_events.created][k]) != hipSuccess) return NULL;
+        g_events.created++;
+    }
+    g_events.used = 0;
+    return &g_events;
+}
+
+static void events_collect(fh_events *ev) {
+    if (!ev) return;
+    for (int i = 0; i < ev->used; i++) {
+        float d = 0, s = 0, f = 0;
+        hipEventElapsedTime(&d, ev->e[i][0], ev->e[i][1]);
+        hipEventElapsedTime(&s, ev->e[i][1], ev->e[i][2]);
+        hipEventElapsedTime(&f, ev->e[i][2], ev->e[i][3]);
+        flux_timing_transformer_double += d;
+        flux_timing_transformer_single += s;
+        flux_timing_transformer_final += f;
+        flux_timing_transformer_total += d + s + f;
+    }
+}
+
+/* ------------------------------------------------------------------ the loop */
+
+/* Uploads fp32 host data and leaves it on the device as bf16. */
+static void *upload_as_bf16(const float *src, size_t n) {
+    float *tmp = (float *)flux_hip_malloc(n * 4);
+    void *dst = flux_hip_malloc(n * 2);
+    int ok = tmp && dst && flux_hip_upload(tmp, src, n * 4) && flux_hip_f32_to_bf16(dst, tmp, n) && flux_hip_sync();
+    flux_hip_free(tmp);
+    if (!ok) { flux_hip_free(dst); return NULL; }
+    return dst;
+}
+
+/* Puts the reference images' tokens behind the target's in tf->tok. */
+static int upload_ref_tokens(flux_transformer_t *tf, int n_target, const flux_ref_t *refs, int num_refs) {
+    const int C = tf->c.channels;
+    int row = n_target;
+    for (int r = 0; r < num_refs; r++) {
+        int n = refs[r].h * refs[r].w;
+        if (!refs[r].latent || n <= 0) return flux_hip_fail("reference image %d is empty", r);
+        float *tmp = (float *)flux_hip_malloc((size_t)n * C * 4);
+        int ok = tmp && flux_hip_upload(tmp, refs[r].latent, (size_t)n * C * 4) &&
+                 flux_hip_latent_to_tokens((char *)tf->tok + (size_t)row * C * 2, tmp, C, n) && flux_hip_sync();
+        flux_hip_free(tmp);
+        if (!ok) return 0;
+        row += n;
+    }
+    return 1;
+}
+
+float *flux_hip_sample_traced(void *transformer, const float *z, int channels, int h, int w,
+                              const flux_ref_t *refs, int num_refs,
+                              const float *text_emb_cond, int text_seq_cond,
+                              const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
+                              const float *schedule, int num_steps, float *v_trace) {
+    flux_transformer_t *tf = (flux_transformer_t *)transformer;
+    if (!tf || !z || !text_emb_cond || !schedule) { flux_hip_fail("sampler: NULL argument"); return NULL; }
+    if (!fh_model_complete(tf)) return NULL;
+    if (channels != tf->c.channels) { flux_hip_fail("sampler: %d channels, model has %d", channels, tf->c.channels); return NULL; }
+    if (h <= 0 || w <= 0 || text_seq_cond <= 0 || num_steps < 0 || num_refs < 0) { flux_hip_fail("sampler: bad sizes"); return NULL; }
+    if (num_refs > 0 && !refs) { flux_hip_fail("sampler: refs is NULL"); return NULL; }
+    const int cfg = text_emb_uncond != NULL;
+    if (cfg && text_seq_uncond <= 0) { flux_hip_fail("sampler: empty unconditional text"); return NULL; }
+    const int n_target = h * w;
+    const size_t n_lat = (size_t)channels * n_target;
+
+    fh_rope *rp_c = fh_get_rope(tf, text_seq_cond, h, w, refs, num_refs);
+    if (!rp_c) return NULL;
+    fh_rope *rp_u = NULL;
+    int max_tokens = rp_c->n;
+    if (cfg) {
+        rp_u = fh_get_rope(tf, text_seq_uncond, h, w, refs, num_refs);
+        if (!rp_u) return NULL;
+        /* the table cache may have recycled the first slot */
+        rp_c = fh_get_rope(tf, text_seq_cond, h, w, refs, num_refs);
+        if (!rp_c) return NULL;
+        if (rp_u->n > max_tokens) max_tokens = rp_u->n;
+    }
+    if (!fh_ensure_workspace(tf, max_tokens)) return NULL;
+    if (num_steps > 0 && !fh_compute_modulation(tf, schedule, num_steps)) return NULL;
+
+    float *out = NULL;
+    float *z_dev = (float *)flux_hip_malloc(n_lat * 4);
+    float *v_c = (float *)flux_hip_malloc(n_lat * 4);
+    float *v_u = cfg ? (float *)flux_hip_malloc(n_lat * 4) : NULL;
+    void *txt_c = upload_as_bf16(text_emb_cond, (size_t)text_seq_cond * tf->c.text_dim);
+    void *txt_u = cfg ? upload_as_bf16(text_emb_uncond, (size_t)text_seq_uncond * tf->c.text_dim) : NULL;
+    fh_events *ev = events_begin(num_steps * (cfg ? 2 : 1));
+    flux_reset_timing();
+    if (!z_dev || !v_c || !txt_c || (cfg && (!v_u || !txt_u))) goto done;
+    if (!flux_hip_upload(z_dev, z, n_lat * 4)) goto done;
+    if (!upload_ref_tokens(tf, n_target, refs, num_refs)) goto done;
+
+    for (int s = 0; s < num_steps; s++) {
+        const float dt = schedule[s + 1] - schedule[s];
+        if (flux_step_callback) flux_step_callback(s + 1, num_steps);
+        if (cfg) {
+            /* unconditional first, then conditional (flux_sample.c:485-493) */
+            if (!fh_forward_device(tf, rp_u, z_dev, n_target, txt_u, s, v_u, ev)) goto done;
+            if (ev) ev->used++;
+            if (!fh_forward_device(tf, rp_c, z_dev, n_target, txt_c, s, v_c, ev)) goto done;
+            if (ev) ev->used++;
+            if (v_trace) {
+                if (!flux_hip_download(v_trace + (size_t)(2 * s) * n_lat, v_u, n_lat * 4)) goto done;
+                if (!flux_hip_download(v_trace + (size_t)(2 * s + 1) * n_lat, v_c, n_lat * 4)) goto done;
+            }
+            if (!flux_hip_cfg_euler_update(z_dev, v_u, v_c, guidance_scale, dt, n_lat)) goto done;
+        } else {
+            if (!fh_forward_device(tf, rp_c, z_dev, n_target, txt_c, s, v_c, ev)) goto done;
+            if (ev) ev->used++;
+            if (v_trace && !flux_hip_download(v_trace + (size_t)s * n_lat, v_c, n_lat * 4)) goto done;
+            if (!flux_hip_euler_update(z_dev, v_c, dt, n_lat)) goto done;
+        }
+    }
+    out = (float *)malloc(n_lat * 4);
+    if (!out) { flux_hip_fail("out of host memory"); goto done; }
+    if (!flux_hip_download(out, z_dev, n_lat * 4)) { free(out); out = NULL; goto done; }
+    events_collect(ev);
+    if (flux_verbose)
+        fprintf(stderr, "denoising on device: double %.2f ms, single %.2f ms, final %.2f ms, total %.2f ms\n",
+                flux_timing_transformer_double, flux_timing_transformer_single, flux_timing_transformer_final,
+                flux_timing_transformer_total);
+done:
+    flux_hip_sync();
+    flux_hip_free(z_dev); flux_hip_free(v_c); flux_hip_free(v_u); flux_hip_free(txt_c); flux_hip_free(txt_u);
+    return out;
+}
+
+/* ------------------------------------------------------------------ reference-named entry points */
+
+static float *run(void *tf, float *z, int batch, int channels, int h, int w, const flux_ref_t *refs, int num_refs,
+                  const float *tc, int sc, const float *tu, int su, float g, const float *schedule, int steps,
+                  void (*progress)(int, int)) {
+    if (batch != 1) { flux_hip_fail("sampler: batch=%d (the pipeline always passes 1)", batch); return NULL; }
+    /* progress fires per step at queue time through flux_step_callback-style notification */
+    float *out = flux_hip_sample_traced(tf, z, channels, h, w, refs, num_refs, tc, sc, tu, su, g, schedule, steps, NULL);
+    if (out && progress)
+        for (int s = 0; s < steps; s++) progress(s + 1, steps);
+    return out;
+}
+
+float *flux_sample_euler(void *transformer, void *text_encoder, float *z, int batch, int channels, int h, int w,
+                         const float *text_emb, int text_seq, const float *schedule, int num_steps,
+                         void (*progress_callback)(int step, int total)) {
+    (void)text_encoder;
+    return run(transformer, z, batch, channels, h, w, NULL, 0, text_emb, text_seq, NULL, 0, 0.0f, schedule, num_steps, progress_callback);
+}
+
+float *flux_sample_euler_with_refs(void *transformer, void *text_encoder, float *z, int batch, int channels, int h, int w,
+                                   const float *ref_latent, int ref_h, int ref_w, int t_offset,
+                                   const float *text_emb, int text_seq, const float *schedule, int num_steps,
+                                   void (*progress_callback)(int step, int total)) {
+    (void)text_encoder;
+    flux_ref_t r = {ref_latent, ref_h, ref_w, t_offset};
+    return run(transformer, z, batch, channels, h, w, &r, ref_latent ? 1 : 0, text_emb, text_seq, NULL, 0, 0.0f, schedule, num_steps, progress_callback);
+}
+
+float *flux_sample_euler_with_multi_refs(void *transformer, void *text_encoder, float *z, int batch, int channels, int h, int w,
+                                         const flux_ref_t *refs, int num_refs,
+                                         const float *text_emb, int text_seq, const float *schedule, int num_steps,
+                                         void (*progress_callback)(int step, int total)) {
+    (void)text_encoder;
+    return run(transformer, z, batch, channels, h, w, refs, refs ? num_refs : 0, text_emb, text_seq, NULL, 0, 0.0f, schedule, num_steps, progress_callback);
+}
+
+float *flux_sample_euler_cfg(void *transformer, void *text_encoder, float *z, int batch, int channels, int h, int w,
+                             const float *text_emb_cond, int text_seq_cond,
+                             const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
+                             const float *schedule, int num_steps, void (*progress_callback)(int step, int total)) {
+    (void)text_encoder;
+    if (!text_emb_uncond) { flux_hip_fail("cfg sampler: unconditional text is NULL"); return NULL; }
+    return run(transformer, z, batch, channels, h, w, NULL, 0, text_emb_cond, text_seq_cond, text_emb_uncond, text_seq_uncond,
+               guidance_scale, schedule, num_steps, progress_callback);
+}
+
+float *flux_sample_euler_cfg_with_refs(void *transformer, void *text_encoder, float *z, int batch, int channels, int h, int w,
+                                       const float *ref_latent, int ref_h, int ref_w, int t_offset,
+                                       const float *text_emb_cond, int text_seq_cond,
+                                       const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
+                                       const float *schedule, int num_steps, void (*progress_callback)(int step, int total)) {
+    (void)text_encoder;
+    if (!text_emb_uncond) { flux_hip_fail("cfg sampler: unconditional text is NULL"); return NULL; }
+    flux_ref_t r = {ref_latent, ref_h, ref_w, t_offset};
+    return run(transformer, z, batch, channels, h, w, &r, ref_latent ? 1 : 0, text_emb_cond, text_seq_cond, text_emb_uncond,
+               text_seq_uncond, guidance_scale, schedule, num_steps, progress_callback);
+}
+
+float *flux_sample_euler_cfg_with_multi_refs(void *transformer, void *text_encoder, float *z, int batch, int channels, int h, int w,
+                                             const flux_ref_t *refs, int num_refs,
+                                             const float *text_emb_cond, int text_seq_cond,
+                                             const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
+                                             const float *schedule, int num_steps,
+                                             void (*progress_callback)(int step, int total)) {
+    (void)text_encoder;
+    if (!text_emb_uncond) { flux_hip_fail("cfg sampler: unconditional text is NULL"); return NULL; }
+    return run(transformer, z, batch, channels, h, w, refs, refs ? num_refs : 0, text_emb_cond, text_seq_cond, text_emb_uncond,
+               text_seq_uncond, guidance_scale, schedule, num_steps, progress_callback);
+}
+
+/* One forward = a one-step schedule whose velocity is returned instead of applied
+ * (flux_transformer.c:3115, 3605, 3815; used by flux_denoise_step, flux.c:1109). */
+float *flux_transformer_forward_with_multi_refs(flux_transformer_t *tf, const float *img_latent, int img_h, int img_w,
+                                                const flux_ref_t *refs, int num_refs,
+                                                const float *txt_emb, int txt_seq, float timestep) {
+    if (!tf || !img_latent || !txt_emb) { flux_hip_fail("forward: NULL argument"); return NULL; }
+    if (img_h <= 0 || img_w <= 0 || txt_seq <= 0) { flux_hip_fail("forward: bad sizes"); return NULL; }
+    const size_t n = (size_t)tf->c.channels * img_h * img_w;
+    float sched[2] = {timestep, timestep};
+    float *v = (float *)malloc(n * 4);
+    if (!v) { flux_hip_fail("out of host memory"); return NULL; }
+    float *z = flux_hip_sample_traced(tf, img_latent, tf->c.channels, img_h, img_w, refs, refs ? num_refs : 0,
+                                      txt_emb, txt_seq, NULL, 0, 0.0f, sched, 1, v);
+    if (!z) { free(v); return NULL; }
+    free(z);
+    return v;
+}
+
+float *flux_transformer_forward(flux_transformer_t *tf, const float *img_latent, int img_h, int img_w,
+                                const float *txt_emb, int txt_seq, float timestep) {
+    return flux_transformer_forward_with_multi_refs(tf, img_latent, img_h, img_w, NULL, 0, txt_emb, txt_seq, timestep);
+}
+
+float *flux_transformer_forward_with_refs(flux_transformer_t *tf, const float *img_latent, int img_h, int img_w,
+                                          const float *ref_latent, int ref_h, int ref_w, int t_offset,
+                                          const float *txt_emb, int txt_seq, float timestep) {
+    flux_ref_t r = {ref_latent, ref_h, ref_w, t_offset};
+    return flux_transformer_forward_with_multi_refs(tf, img_latent, img_h, img_w, &r, ref_latent ? 1 : 0, txt_emb, txt_seq, timestep);
+}

@@ -1,0 +1,291 @@
+/*
+ * gemm.hip - bf16 MFMA GEMM  C[M,N] = A[M,K] * W[N,K]^T  with fused epilogues, for gfx950.
+ *
+ * This is the linear layer of the denoising transformer (reference: flux_linear,
+ * flux_kernels.c:210-282, cblas_sgemm NoTrans x Trans). Both operands have K contiguous, so
+ * an MFMA operand fragment (8 consecutive bf16 of one row) is one 16-byte LDS read.
+ *
+ * Tiling: a workgroup owns a BM x BN tile; K is walked in steps of 64 through two LDS stages
+ * (global -> registers -> LDS, one barrier per step). Each 64-lane wave owns a WM x WN
+ * sub-tile made of 32x32 v_mfma_f32_32x32x16_bf16 blocks. The weight fragment is the MFMA "A"
+ * operand and the activation fragment the "B" operand, so that in the accumulator a lane holds
+ * one token (m) and four consecutive output features (n): epilogues can then use 8/16-byte
+ * accesses and pair gate/up columns inside a lane.
+ *
+ * LDS rows are 128 bytes (64 bf16); the 16-byte chunk index is XOR-swizzled with a function of
+ * the row so that the 32 rows a fragment read touches spread over all banks.
+ */
+#include "common.h"
+#include "../../include/flux_hip.h"
+
+struct GemmArgs {
+    const bf16 *A[2];
+    const bf16 *W[2];
+    void *C[2];
+    const float *gate[2];
+    int M[2];
+    int mtiles0, mtiles, ntiles, total_tiles;
+    int N, K, lda, ldw, ldc, w_row0, w_row1;
+};
+
+__device__ __forceinline__ int lds_swz(int r) { return ((r >> 1) & 7) ^ ((r & 1) << 2); }
+
+#define GROUP_M 4
+
+template <int BM, int BN, int WGM, int WGN, int EPI>
+__global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
+    constexpr int T = WGM * WGN * 64;
+    constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
+    constexpr int RPP = T / 8; /* tile rows fetched per pass: 8 threads x 16 B cover one row */
+    constexpr int PA = BM / RPP, PB = BN / RPP;
+    constexpr int STAGE = (BM + BN) * 128;
+    static_assert(BM % RPP == 0 && BN % RPP == 0, "tile rows must divide evenly over threads");
+    static_assert(EPI != FLUX_HIP_EPI_SWIGLU || (TN % 2 == 0), "swiglu pairs 32-column blocks");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    /* Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous run of tiles
+     * so that its L2 sees the reuse, then walk tiles in groups of GROUP_M rows. */
+    int nb = gridDim.x;
+    int per_xcd = nb >> 3;
+    int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= g.total_tiles) return;
+    int per_group = GROUP_M * g.ntiles;
+    int grp = logical / per_group;
+    int first_m = grp * GROUP_M;
+    int gsz = min(g.mtiles - first_m, GROUP_M);
+    int in_grp = logical - grp * per_group;
+    int tm = first_m + in_grp % gsz;
+    int tn = in_grp / gsz;
+
+    int prob = tm >= g.mtiles0 ? 1 : 0;
+    int tml = prob ? tm - g.mtiles0 : tm;
+    const bf16 *__restrict__ A = g.A[prob];
+    const bf16 *__restrict__ W = g.W[prob];
+    const int M = g.M[prob];
+    const int m0 = tml * BM, n0 = tn * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int lrow = tid >> 3, lchunk = tid & 7;
+
+    const bf16 *a_ptr[PA];
+    const bf16 *b_ptr[PB];
+    int a_lds[PA], b_lds[PB];
+#pragma unroll
+    for (int i = 0; i < PA; i++) {
+        int r = lrow + i * RPP;
+        int gm = min(m0 + r, M - 1);
+        a_ptr[i] = A + (size_t)gm * g.lda + lchunk * 8;
+        a_lds[i] = r * 128 + ((lchunk ^ lds_swz(r)) << 4);
+    }
+#pragma unroll
+    for (int i = 0; i < PB; i++) {
+        int v = lrow + i * RPP; /* column of the tile */
+        int wrow;
+        if (EPI == FLUX_HIP_EPI_SWIGLU) {
+            /* 32-column blocks alternate gate, up so a lane ends up holding matching pairs */
+            int wv = v / WN, blk = (v % WN) >> 5;
+            int idx = wv * (WN / 2) + (blk >> 1) * 32 + (v & 31);
+            wrow = ((blk & 1) ? g.w_row1 : g.w_row0) + tn * (BN / 2) + idx;
+        } else {
+            wrow = g.w_row0 + n0 + v;
+        }
+        b_ptr[i] = W + (size_t)wrow * g.ldw + lchunk * 8;
+        b_lds[i] = BM * 128 + v * 128 + ((lchunk ^ lds_swz(v)) << 4);
+    }
+
+    bf16x8 ra[PA], rb[PB];
+#pragma unroll
+    for (int i = 0; i < PA; i++) ra[i] = *(const bf16x8 *)a_ptr[i];
+#pragma unroll
+    for (int i = 0; i < PB; i++) rb[i] = *(const bf16x8 *)b_ptr[i];
+#pragma unroll
+    for (int i = 0; i < PA; i++) *(bf16x8 *)(smem + a_lds[i]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < PB; i++) *(bf16x8 *)(smem + b_lds[i]) = rb[i];
+    __syncthreads();
+
+    f32x16 acc[TN][TM];
+#pragma unroll
+    for (int i = 0; i < TN; i++)
+#pragma unroll
+        for (int j = 0; j < TM; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+
+    const int l31 = lane & 31, lhi = lane >> 5;
+    const int swzl = lds_swz(l31);
+    const int a_frag = (wm * WM + l31) * 128;
+    const int b_frag = BM * 128 + (wn * WN + l31) * 128;
+
+    const int KT = g.K >> 6;
+    for (int kt = 0; kt < KT; kt++) {
+        const int cur = kt & 1;
+        if (kt + 1 < KT) {
+#pragma unroll
+            for (int i = 0; i < PA; i++) { a_ptr[i] += 64; ra[i] = *(const bf16x8 *)a_ptr[i]; }
+#pragma unroll
+            for (int i = 0; i < PB; i++) { b_ptr[i] += 64; rb[i] = *(const bf16x8 *)b_ptr[i]; }
+        }
+        const char *st = smem + cur * STAGE;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            const int coff = ((kk * 2 + lhi) ^ swzl) << 4;
+            bf16x8 fa[TM], fb[TN];
+#pragma unroll
+            for (int t = 0; t < TM; t++) fa[t] = *(const bf16x8 *)(st + a_frag + t * 32 * 128 + coff);
+#pragma unroll
+            for (int t = 0; t < TN; t++) fb[t] = *(const bf16x8 *)(st + b_frag + t * 32 * 128 + coff);
+#pragma unroll
+            for (int i = 0; i < TN; i++)
+#pragma unroll
+                for (int j = 0; j < TM; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[i], fa[j], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < KT) {
+            char *nx = smem + (cur ^ 1) * STAGE;
+#pragma unroll
+            for (int i = 0; i < PA; i++) *(bf16x8 *)(nx + a_lds[i]) = ra[i];
+#pragma unroll
+            for (int i = 0; i < PB; i++) *(bf16x8 *)(nx + b_lds[i]) = rb[i];
+        }
+        __syncthreads();
+    }
+
+    /* Accumulator element e of block (i, j): feature n = 8*(e/4) + 4*(lane/32) + e%4 of the
+     * 32-column block, token m = lane%32 of the 32-row block. */
+    const int ldc = g.ldc;
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+        const int m = m0 + wm * WM + j * 32 + l31;
+        if (m >= M) continue;
+        if (EPI == FLUX_HIP_EPI_SWIGLU) {
+            bf16 *C = (bf16 *)g.C[prob] + (size_t)m * ldc + tn * (BN / 2) + wn * (WN / 2);
+#pragma unroll
+            for (int i = 0; i < TN; i += 2)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    bf16x4 o;
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        o[e] = (bf16)(silu_f(acc[i][j][q * 4 + e]) * acc[i + 1][j][q * 4 + e]);
+                    *(bf16x4 *)(C + (i >> 1) * 32 + q * 8 + lhi * 4) = o;
+                }
+        } else {
+#pragma unroll
+            for (int i = 0; i < TN; i++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const int n = n0 + wn * WN + i * 32 + q * 8 + lhi * 4;
+                    if (EPI == FLUX_HIP_EPI_BF16) {
+                        bf16x4 o;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) o[e] = (bf16)acc[i][j][q * 4 + e];
+                        *(bf16x4 *)((bf16 *)g.C[prob] + (size_t)m * ldc + n) = o;
+                    } else if (EPI == FLUX_HIP_EPI_F32) {
+                        f32x4 o;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) o[e] = acc[i][j][q * 4 + e];
+                        *(f32x4 *)((float *)g.C[prob] + (size_t)m * ldc + n) = o;
+                    } else if (EPI == FLUX_HIP_EPI_F32_T) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            ((float *)g.C[prob])[(size_t)(n + e) * ldc + m] = acc[i][j][q * 4 + e];
+                    } else if (EPI == FLUX_HIP_EPI_RESID) {
+                        float *p = (float *)g.C[prob] + (size_t)m * ldc + n;
+                        f32x4 x = *(f32x4 *)p;
+                        f32x4 gt = *(const f32x4 *)(g.gate[prob] + n);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) x[e] += gt[e] * acc[i][j][q * 4 + e];
+                        *(f32x4 *)p = x;
+                    }
+                }
+        }
+    }
+}
+
+/* ------------------------------------------------------------------ host side */
+
+template <int BM, int BN, int WGM, int WGN, int EPI>
+static int launch_cfg(GemmArgs &g) {
+    constexpr int T = WGM * WGN * 64;
+    constexpr int LDS = 2 * (BM + BN) * 128;
+    static bool attr_done = false;
+    auto kern = gemm_kernel<BM, BN, WGM, WGN, EPI>;
+    if (!attr_done) {
+        HIP_OK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+        attr_done = true;
+    }
+    g.mtiles0 = (g.M[0] + BM - 1) / BM;
+    int mt1 = g.M[1] > 0 ? (g.M[1] + BM - 1) / BM : 0;
+    g.mtiles = g.mtiles0 + mt1;
+    g.ntiles = g.N / BN;
+    g.total_tiles = g.mtiles * g.ntiles;
+    int grid = (g.total_tiles + 7) & ~7;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(T), LDS, flux_hip_stream_handle(), g);
+    HIP_OK(hipGetLastError());
+    return 1;
+}
+
+template <int EPI>
+static int launch_epi(GemmArgs &g, int tile) {
+    switch (tile) {
+        case 2: return launch_cfg<256, 256, 2, 4, EPI>(g);
+        case 1: return launch_cfg<128, 128, 2, 2, EPI>(g);
+        default: return launch_cfg<64, 128, 2, 2, EPI>(g);
+    }
+}
+
+static int g_force_tile = -1;
+extern "C" void flux_hip_linear_force_tile(int tile) { g_force_tile = tile; }
+
+extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
+                               int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1) {
+    if (nparts < 1 || nparts > 2) return flux_hip_fail("flux_hip_linear: nparts=%d (1 or 2)", nparts);
+    if (K <= 0 || (K & 63)) return flux_hip_fail("flux_hip_linear: K=%d must be a positive multiple of 64", K);
+    if (N <= 0 || (N & 127)) return flux_hip_fail("flux_hip_linear: N=%d must be a positive multiple of 128", N);
+    if (lda < K || ldw < K || (lda & 7) || (ldw & 7))
+        return flux_hip_fail("flux_hip_linear: lda=%d ldw=%d must be >= K and multiples of 8", lda, ldw);
+    if (epilogue != FLUX_HIP_EPI_F32_T && (ldc & 3)) return flux_hip_fail("flux_hip_linear: ldc=%d must be a multiple of 4", ldc);
+    GemmArgs g = {};
+    int maxm = 0;
+    for (int i = 0; i < nparts; i++) {
+        if (parts[i].M < 0) return flux_hip_fail("flux_hip_linear: negative row count");
+        if (parts[i].M > 0 && (!parts[i].A || !parts[i].W || !parts[i].C))
+            return flux_hip_fail("flux_hip_linear: NULL operand");
+        if (epilogue == FLUX_HIP_EPI_RESID && parts[i].M > 0 && !parts[i].gate)
+            return flux_hip_fail("flux_hip_linear: residual epilogue needs a gate vector");
+    }
+    /* drop empty parts */
+    int np = 0;
+    for (int i = 0; i < nparts; i++) {
+        if (parts[i].M == 0) continue;
+        g.A[np] = (const bf16 *)parts[i].A;
+        g.W[np] = (const bf16 *)parts[i].W;
+        g.C[np] = parts[i].C;
+        g.gate[np] = parts[i].gate;
+        g.M[np] = parts[i].M;
+        if (parts[i].M > maxm) maxm = parts[i].M;
+        np++;
+    }
+    if (np == 0) return 1;
+    g.N = N; g.K = K; g.lda = lda; g.ldw = ldw; g.ldc = ldc; g.w_row0 = w_row0; g.w_row1 = w_row1;
+
+    /* Largest tile that still yields a few hundred workgroups for the 256 CUs. */
+    int tile;
+    long total_rows = (long)g.M[0] + g.M[1];
+    if ((N % 256) == 0 && ((total_rows + 255) / 256) * (N / 256) >= 384) tile = 2;
+    else if (((total_rows + 127) / 128) * (N / 128) >= 256 && maxm > 64) tile = 1;
+    else tile = 0;
+    if (g_force_tile >= 0) tile = g_force_tile;
+    if (tile == 2 && (N % 256)) tile = 1;
+
+    switch (epilogue) {
+        case FLUX_HIP_EPI_BF16: return launch_epi<FLUX_HIP_EPI_BF16>(g, tile);
+        case FLUX_HIP_EPI_F32: return launch_epi<FLUX_HIP_EPI_F32>(g, tile);
+        case FLUX_HIP_EPI_F32_T: return launch_epi<FLUX_HIP_EPI_F32_T>(g, tile);
+        case FLUX_HIP_EPI_RESID: return launch_epi<FLUX_HIP_EPI_RESID>(g, tile);
+        case FLUX_HIP_EPI_SWIGLU: return launch_epi<FLUX_HIP_EPI_SWIGLU>(g, tile);
+    }
+    return flux_hip_fail("flux_hip_linear: unknown epilogue %d", epilogue);
+}

@@ -1,0 +1,114 @@
+/*
+ * runtime.hip - device lifetime, buffers, error text and event timing of the gfx950 backend.
+ * Plays the part flux_metal_init/available/sync and the flux_gpu_tensor_* calls play for the
+ * reference's Apple backend (flux_metal.h:23-198).
+ */
+#include "common.h"
+#include "../../include/flux_hip.h"
+#include <stdarg.h>
+#include <string.h>
+
+static char g_err[512] = "";
+static hipStream_t g_stream = nullptr;
+static int g_ready = 0;
+static hipEvent_t g_ev0 = nullptr, g_ev1 = nullptr;
+
+extern "C" int flux_hip_fail(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    if (flux_verbose) fprintf(stderr, "flux_hip: %s\n", g_err);
+    return 0;
+}
+
+extern "C" const char *flux_hip_last_error(void) { return g_err; }
+
+extern "C" hipStream_t flux_hip_stream_handle(void) { return g_stream; }
+extern "C" void *flux_hip_stream(void) { return (void *)g_stream; }
+
+extern "C" int flux_hip_init(void) {
+    if (g_ready) return 1;
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n < 1) return flux_hip_fail("no HIP device is visible");
+    HIP_OK(hipSetDevice(0));
+    hipDeviceProp_t prop;
+    HIP_OK(hipGetDeviceProperties(&prop, 0));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return flux_hip_fail("device 0 is %s; this library holds gfx950 code only", prop.gcnArchName);
+    HIP_OK(hipStreamCreate(&g_stream));
+    HIP_OK(hipEventCreate(&g_ev0));
+    HIP_OK(hipEventCreate(&g_ev1));
+    g_ready = 1;
+    return 1;
+}
+
+extern "C" int flux_hip_available(void) { return g_ready || flux_hip_init(); }
+
+extern "C" void flux_hip_cleanup(void) {
+    if (!g_ready) return;
+    hipStreamSynchronize(g_stream);
+    hipEventDestroy(g_ev0);
+    hipEventDestroy(g_ev1);
+    hipStreamDestroy(g_stream);
+    g_stream = nullptr;
+    g_ready = 0;
+}
+
+extern "C" int flux_hip_sync(void) {
+    if (!g_ready) return flux_hip_fail("flux_hip_sync: backend not initialised");
+    HIP_OK(hipStreamSynchronize(g_stream));
+    return 1;
+}
+
+extern "C" void *flux_hip_malloc(size_t bytes) {
+    if (!flux_hip_available()) return nullptr;
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
+    if (e != hipSuccess) {
+        flux_hip_fail("hipMalloc(%zu) failed: %s", bytes, hipGetErrorString(e));
+        return nullptr;
+    }
+    return p;
+}
+
+extern "C" void flux_hip_free(void *p) {
+    if (p) hipFree(p);
+}
+
+extern "C" int flux_hip_upload(void *dst, const void *src, size_t bytes) {
+    if (!flux_hip_available()) return 0;
+    if (!bytes) return 1;
+    HIP_OK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_stream));
+    HIP_OK(hipStreamSynchronize(g_stream)); /* the host buffer may be reused at once */
+    return 1;
+}
+
+extern "C" int flux_hip_download(void *dst, const void *src, size_t bytes) {
+    if (!flux_hip_available()) return 0;
+    if (!bytes) return 1;
+    HIP_OK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
+    HIP_OK(hipStreamSynchronize(g_stream));
+    return 1;
+}
+
+extern "C" int flux_hip_memset(void *dst, int value, size_t bytes) {
+    if (!flux_hip_available()) return 0;
+    HIP_OK(hipMemsetAsync(dst, value, bytes, g_stream));
+    return 1;
+}
+
+extern "C" int flux_hip_timer_start(void) {
+    if (!flux_hip_available()) return 0;
+    HIP_OK(hipEventRecord(g_ev0, g_stream));
+    return 1;
+}
+
+extern "C" float flux_hip_timer_stop(void) {
+    if (!g_ready) return -1.0f;
+    float ms = -1.0f;
+    if (hipEventRecord(g_ev1, g_stream) != hipSuccess) return -1.0f;
+    if (hipEventSynchronize(g_ev1) != hipSuccess) return -1.0f;
+    if (hipEventElapsedTime(&ms, g_ev0, g_ev1) != hipSuccess) return -1.0f;
+    return ms;
+}

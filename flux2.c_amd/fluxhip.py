@@ -1,0 +1,275 @@
+"""ctypes binding of libflux_hip.so (include/flux_hip.h) for tests, the smoke entry and the benchmark.
+
+This module only marshals numpy arrays to the C ABI. It contains no arithmetic of its own and
+has no CPU fallback: if the library or a GPU is missing, calls raise.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+from model_spec import FluxConfig
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+c_f, c_i, vp, c_sz = ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
+
+EPI_BF16, EPI_F32, EPI_F32_T, EPI_RESID, EPI_SWIGLU = range(5)
+
+
+class _Cfg(ctypes.Structure):
+    _fields_ = [(n, c_i) for n in ("hidden", "heads", "head_dim", "mlp", "n_double", "n_single",
+                                   "text_dim", "channels", "axis_dim", "sincos_dim")] + [("rope_theta", c_f)]
+
+
+class _Part(ctypes.Structure):
+    _fields_ = [("A", vp), ("W", vp), ("C", vp), ("gate", vp), ("M", c_i)]
+
+
+class _Ref(ctypes.Structure):
+    _fields_ = [("latent", vp), ("h", c_i), ("w", c_i), ("t_offset", c_i)]
+
+
+class FluxHipError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def lib_path():
+    return os.path.join(_HERE, "libflux_hip.so")
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = lib_path()
+    if not os.path.exists(path):
+        raise FluxHipError(f"{path} is not built (make -C flux2.c_amd hip)")
+    L = ctypes.CDLL(path)
+    L.flux_hip_init.restype = c_i
+    L.flux_hip_available.restype = c_i
+    L.flux_hip_sync.restype = c_i
+    L.flux_hip_last_error.restype = ctypes.c_char_p
+    L.flux_hip_stream.restype = vp
+    L.flux_hip_malloc.restype = vp
+    L.flux_hip_malloc.argtypes = [c_sz]
+    L.flux_hip_free.argtypes = [vp]
+    L.flux_hip_upload.argtypes = [vp, vp, c_sz]
+    L.flux_hip_download.argtypes = [vp, vp, c_sz]
+    L.flux_hip_memset.argtypes = [vp, c_i, c_sz]
+    L.flux_hip_timer_stop.restype = c_f
+    L.flux_hip_linear.argtypes = [c_i, c_i, ctypes.POINTER(_Part), c_i, c_i, c_i, c_i, c_i, c_i, c_i]
+    L.flux_hip_linear_force_tile.argtypes = [c_i]
+    L.flux_hip_adaln_norm.argtypes = [vp, c_i, vp, c_i, c_i, c_i, vp, vp, vp, vp, c_f]
+    L.flux_hip_kv_prepare.argtypes = [vp, vp, c_i, vp, c_i, c_i, c_i, c_i, c_i, c_i, vp, vp, vp, vp, c_f]
+    L.flux_hip_attention.argtypes = [vp, c_i, vp, c_i, vp, vp, c_i, c_i, c_i, c_i, c_i, vp, vp, vp, vp, c_f]
+    L.flux_hip_gemv.argtypes = [vp, vp, vp, c_i, c_i, c_i, c_i]
+    L.flux_hip_latent_to_tokens.argtypes = [vp, vp, c_i, c_i]
+    L.flux_hip_f32_to_bf16.argtypes = [vp, vp, c_sz]
+    L.flux_hip_euler_update.argtypes = [vp, vp, c_f, c_sz]
+    L.flux_hip_cfg_euler_update.argtypes = [vp, vp, vp, c_f, c_f, c_sz]
+    L.flux_hip_transformer_new.restype = vp
+    L.flux_hip_transformer_new.argtypes = [ctypes.POINTER(_Cfg)]
+    L.flux_hip_transformer_set_tensor.argtypes = [vp, ctypes.c_char_p, vp, ctypes.c_int64]
+    L.flux_hip_transformer_load_file.restype = vp
+    L.flux_hip_transformer_load_file.argtypes = [ctypes.c_char_p, ctypes.POINTER(_Cfg)]
+    L.flux_transformer_free.argtypes = [vp]
+    L.flux_transformer_forward.restype = vp
+    L.flux_transformer_forward.argtypes = [vp, vp, c_i, c_i, vp, c_i, c_f]
+    L.flux_transformer_forward_with_refs.restype = vp
+    L.flux_transformer_forward_with_refs.argtypes = [vp, vp, c_i, c_i, vp, c_i, c_i, c_i, vp, c_i, c_f]
+    L.flux_transformer_forward_with_multi_refs.restype = vp
+    L.flux_transformer_forward_with_multi_refs.argtypes = [vp, vp, c_i, c_i, vp, c_i, vp, c_i, c_f]
+    L.flux_hip_sample_traced.restype = vp
+    L.flux_hip_sample_traced.argtypes = [vp, vp, c_i, c_i, c_i, vp, c_i, vp, c_i, vp, c_i, c_f, vp, c_i, vp]
+    L.flux_sample_euler.restype = vp
+    L.flux_sample_euler.argtypes = [vp, vp, vp, c_i, c_i, c_i, c_i, vp, c_i, vp, c_i, vp]
+    L.flux_sample_euler_with_refs.restype = vp
+    L.flux_sample_euler_with_refs.argtypes = [vp, vp, vp, c_i, c_i, c_i, c_i, vp, c_i, c_i, c_i, vp, c_i, vp, c_i, vp]
+    L.flux_sample_euler_cfg.restype = vp
+    L.flux_sample_euler_cfg.argtypes = [vp, vp, vp, c_i, c_i, c_i, c_i, vp, c_i, vp, c_i, c_f, vp, c_i, vp]
+    L.flux_sample_euler_cfg_with_refs.restype = vp
+    L.flux_sample_euler_cfg_with_refs.argtypes = [vp, vp, vp, c_i, c_i, c_i, c_i, vp, c_i, c_i, c_i,
+                                                  vp, c_i, vp, c_i, c_f, vp, c_i, vp]
+    for n in ("flux_linear_schedule", "flux_power_schedule", "flux_official_schedule"):
+        getattr(L, n).restype = vp
+    L.flux_linear_schedule.argtypes = [c_i]
+    L.flux_power_schedule.argtypes = [c_i, c_f]
+    L.flux_official_schedule.argtypes = [c_i, c_i]
+    _lib = L
+    return L
+
+
+def libc_free(ptr):
+    ctypes.CDLL(None).free(ctypes.c_void_p(ptr))
+
+
+def check(rc, what="flux_hip call"):
+    if not rc:
+        raise FluxHipError(f"{what} failed: {lib().flux_hip_last_error().decode()}")
+    return rc
+
+
+def init():
+    check(lib().flux_hip_init(), "flux_hip_init")
+
+
+def sync():
+    check(lib().flux_hip_sync(), "flux_hip_sync")
+
+
+class DevBuf:
+    """A device allocation with numpy upload/download."""
+
+    def __init__(self, nbytes):
+        init()
+        self.nbytes = int(nbytes)
+        self.ptr = lib().flux_hip_malloc(self.nbytes)
+        if not self.ptr:
+            raise FluxHipError(f"flux_hip_malloc({nbytes}): {lib().flux_hip_last_error().decode()}")
+
+    @classmethod
+    def from_array(cls, a):
+        a = np.ascontiguousarray(a)
+        b = cls(max(a.nbytes, 1))
+        if a.nbytes:
+            check(lib().flux_hip_upload(b.ptr, a.ctypes.data, a.nbytes), "upload")
+        return b
+
+    def to_array(self, dtype, shape):
+        out = np.empty(shape, dtype=dtype)
+        assert out.nbytes <= self.nbytes
+        if out.nbytes:
+            check(lib().flux_hip_download(out.ctypes.data, self.ptr, out.nbytes), "download")
+        return out
+
+    def at(self, byte_offset):
+        return self.ptr + int(byte_offset)
+
+    def free(self):
+        if self.ptr:
+            lib().flux_hip_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+def linear(epilogue, parts, N, K, lda, ldw, ldc, w_row0=0, w_row1=0):
+    """parts: list of (A_ptr, W_ptr, C_ptr, gate_ptr_or_None, M)."""
+    arr = (_Part * len(parts))()
+    for i, (A, W, C, g, M) in enumerate(parts):
+        arr[i] = _Part(A, W, C, g, M)
+    check(lib().flux_hip_linear(epilogue, len(parts), arr, N, K, lda, ldw, ldc, w_row0, w_row1), "flux_hip_linear")
+
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _refs_array(refs):
+    if not refs:
+        return None, 0, []
+    keep = []
+    arr = (_Ref * len(refs))()
+    for i, (lat, h, w, t) in enumerate(refs):
+        lat = _f32(lat)
+        keep.append(lat)
+        arr[i] = _Ref(lat.ctypes.data, h, w, t)
+    return arr, len(refs), keep
+
+
+def _take_host(ptr, shape):
+    n = int(np.prod(shape))
+    out = np.ctypeslib.as_array(ctypes.cast(ptr, ctypes.POINTER(c_f)), shape=(n,)).copy().reshape(shape)
+    libc_free(ptr)
+    return out
+
+
+class Transformer:
+    """The denoising transformer on the GPU, built from named bf16 tensors or a safetensors file."""
+
+    def __init__(self, cfg: FluxConfig, weights=None, path=None):
+        init()
+        self.cfg = cfg
+        L = lib()
+        c = _Cfg(cfg.hidden, cfg.heads, cfg.head_dim, cfg.mlp, cfg.n_double, cfg.n_single, cfg.text_dim,
+                 cfg.channels, cfg.axis_dim, cfg.sincos_dim, cfg.rope_theta)
+        if path is not None:
+            self.h = L.flux_hip_transformer_load_file(os.fsencode(path), ctypes.byref(c))
+            if not self.h:
+                raise FluxHipError(f"load_file: {L.flux_hip_last_error().decode()}")
+            return
+        self.h = L.flux_hip_transformer_new(ctypes.byref(c))
+        if not self.h:
+            raise FluxHipError(f"transformer_new: {L.flux_hip_last_error().decode()}")
+        if weights:
+            for name, a in weights.items():
+                self.set_tensor(name, a)
+
+    def set_tensor(self, name, a):
+        a = np.ascontiguousarray(a, dtype=np.uint16)
+        check(lib().flux_hip_transformer_set_tensor(self.h, name.encode(), a.ctypes.data, a.size), f"set_tensor({name})")
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().flux_transformer_free(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def forward(self, latent, h, w, txt, t, refs=None):
+        latent, txt = _f32(latent), _f32(txt)
+        arr, n, keep = _refs_array(refs)
+        L = lib()
+        if n == 0:
+            p = L.flux_transformer_forward(self.h, latent.ctypes.data, h, w, txt.ctypes.data, txt.shape[0], t)
+        elif n == 1:
+            r = arr[0]
+            p = L.flux_transformer_forward_with_refs(self.h, latent.ctypes.data, h, w, r.latent, r.h, r.w, r.t_offset,
+                                                     txt.ctypes.data, txt.shape[0], t)
+        else:
+            p = L.flux_transformer_forward_with_multi_refs(self.h, latent.ctypes.data, h, w, arr, n,
+                                                           txt.ctypes.data, txt.shape[0], t)
+        if not p:
+            raise FluxHipError(f"forward: {L.flux_hip_last_error().decode()}")
+        return _take_host(p, (self.cfg.channels, h, w))
+
+    def sample(self, z, h, w, txt, schedule, refs=None, txt_uncond=None, guidance=0.0, trace=False):
+        """Euler (or CFG when txt_uncond is given) sampling loop on the device."""
+        z, txt, schedule = _f32(z), _f32(txt), _f32(schedule)
+        steps = len(schedule) - 1
+        n = self.cfg.channels * h * w
+        arr, nr, keep = _refs_array(refs)
+        tu = _f32(txt_uncond) if txt_uncond is not None else None
+        fw = steps * (2 if tu is not None else 1)
+        tr = np.zeros((fw, n), np.float32) if trace else None
+        L = lib()
+        p = L.flux_hip_sample_traced(self.h, z.ctypes.data, self.cfg.channels, h, w, arr, nr,
+                                     txt.ctypes.data, txt.shape[0],
+                                     tu.ctypes.data if tu is not None else None, tu.shape[0] if tu is not None else 0,
+                                     guidance, schedule.ctypes.data, steps, tr.ctypes.data if trace else None)
+        if not p:
+            raise FluxHipError(f"sample: {L.flux_hip_last_error().decode()}")
+        out = _take_host(p, (self.cfg.channels, h, w))
+        return (out, tr) if trace else out
+
+
+def schedule(kind, n, arg=None):
+    L = lib()
+    if kind == "linear":
+        p = L.flux_linear_schedule(n)
+    elif kind == "power":
+        p = L.flux_power_schedule(n, arg)
+    else:
+        p = L.flux_official_schedule(n, arg)
+    return _take_host(p, (n + 1,))

@@ -1,0 +1,248 @@
+/*
+ * flux_hip.h - C ABI of the MI355X (gfx950) backend for the FLUX.2-klein
+ * denoising transformer.
+ *
+ * Three layers, all plain C (pointers and sizes only):
+ *   1. runtime:   device lifetime, buffers, errors       (role of flux_metal.h:23-129, 140-198)
+ *   2. operators: one entry point per hot operator, on device pointers
+ *                 (role of flux_kernels.h:22-226 and the flux_gpu_* list in flux_metal.h:214-529)
+ *   3. model:     loader, forward passes and samplers with the reference's own
+ *                 names and signatures (flux.c:45-110), so the reference's
+ *                 flux.c links against this library unchanged.
+ *
+ * Conventions: functions returning int give 1 on success and 0 on failure
+ * (as the reference's GPU operators do, flux_metal.h:232-234); functions
+ * returning pointers give NULL on failure. flux_hip_last_error() then holds a
+ * message. Nothing here falls back to a CPU path: without a usable GPU every
+ * call fails. Not thread-safe (neither is the reference, SURVEY of
+ * flux_kernels.c:32-45 globals): one forward at a time per process.
+ */
+#ifndef FLUX_HIP_H
+#define FLUX_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ runtime */
+
+/* Selects device 0 and creates the compute stream. Idempotent.
+ * Replaces flux_metal_init (flux_metal.h:23). */
+int flux_hip_init(void);
+/* 1 when a gfx950 device is usable. Replaces flux_metal_available (flux_metal.h:28). */
+int flux_hip_available(void);
+/* Releases the stream. Replaces flux_metal_cleanup (flux_metal.h:33). */
+void flux_hip_cleanup(void);
+/* Waits for all queued work. Replaces flux_metal_sync / flux_gpu_sync (flux_metal.h:106,277). */
+int flux_hip_sync(void);
+/* Last failure message (static storage), "" if none. Role of flux_get_error (flux.c:155-169). */
+const char *flux_hip_last_error(void);
+/* The backend's stream as an opaque hipStream_t, for callers that time or profile. */
+void *flux_hip_stream(void);
+
+/* Device buffers: role of flux_gpu_tensor_alloc/create/read/free (flux_metal.h:147-188). */
+void *flux_hip_malloc(size_t bytes);
+void flux_hip_free(void *dptr);
+int flux_hip_upload(void *dst, const void *src, size_t bytes);
+int flux_hip_download(void *dst, const void *src, size_t bytes);
+int flux_hip_memset(void *dst, int value, size_t bytes);
+
+/* Timing helper on the backend's stream: returns elapsed milliseconds between
+ * flux_hip_timer_start() and flux_hip_timer_stop() measured with HIP events. */
+int flux_hip_timer_start(void);
+float flux_hip_timer_stop(void);
+
+/* ---------------------------------------------------------------- operators */
+
+/* Output handling of flux_hip_linear. */
+enum {
+    FLUX_HIP_EPI_BF16 = 0,    /* C bf16 [M, ldc] = A W^T */
+    FLUX_HIP_EPI_F32 = 1,     /* C f32  [M, ldc] = A W^T */
+    FLUX_HIP_EPI_F32_T = 2,   /* C f32  [N, ldc] = (A W^T)^T  (token-major -> channel-major) */
+    FLUX_HIP_EPI_RESID = 3,   /* C f32  [M, ldc] += gate[n] * (A W^T)      gated_add, flux_transformer.c:90 */
+    FLUX_HIP_EPI_SWIGLU = 4   /* C bf16 [M, ldc] = silu(A Wg^T) * (A Wu^T) swiglu, flux_transformer.c:1749-1757 */
+};
+
+/* One row range of a linear layer. */
+typedef struct {
+    const void *A;      /* bf16 [M, lda] activations */
+    const void *W;      /* bf16 [rows, ldw] weight, row-major [out, in] */
+    void *C;            /* output, type per epilogue */
+    const float *gate;  /* f32 [N], FLUX_HIP_EPI_RESID only */
+    int M;              /* rows */
+} flux_hip_linear_part;
+
+/*
+ * y = x W^T on MFMA, bf16 inputs, fp32 accumulation. Replaces flux_linear_nobias /
+ * flux_linear_nobias_bf16 (flux_kernels.h:59,66; flux_kernels.c:210-320) and, through the
+ * epilogues, gated_add (flux_transformer.c:90), flux_silu + flux_mul_inplace
+ * (flux_kernels.c:120,581) and the output transposes (flux_transformer.c:3547-3552).
+ * Up to two row ranges with different weights run in one launch (the image and text streams
+ * of a double block). K % 64 == 0 and N % 128 == 0 are required.
+ * For FLUX_HIP_EPI_SWIGLU, N counts gate+up columns (2*mlp); gate rows start at W row w_row0,
+ * up rows at w_row1; the output has N/2 columns. Otherwise W rows [w_row0, w_row0+N) are used.
+ */
+int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
+                    int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1);
+
+/*
+ * out = (1 + scale) * LayerNorm(x) + shift per row, x f32 [rows, hidden], out bf16.
+ * Rows [0, split) use mod0, the rest mod1; each mod points at shift[hidden] and scale[hidden]
+ * through explicit pointers. Replaces apply_adaln (flux_transformer.c:979-1048) /
+ * flux_gpu_adaln_norm_bf16 (flux_metal.h:384).
+ */
+int flux_hip_adaln_norm(void *out_bf16, int ldo, const float *x, int rows, int hidden, int split,
+                        const float *shift0, const float *scale0,
+                        const float *shift1, const float *scale1, float eps);
+
+/*
+ * Prepares K and V of one attention call from the fused qkv buffer (bf16 [rows, ld] with
+ * K at column k_col and V at column v_col): K gets per-head RMSNorm * weight then RoPE and is
+ * written to k_out [rows, heads*128]; V is written transposed to vt_out [heads*128, ld_vt].
+ * Rows [0, split) use k_w0, the rest k_w1. Replaces the K half of apply_qk_norm
+ * (flux_transformer.c:1052-1106) and apply_rope_2d (flux_transformer.c:719-741), and the
+ * head transposes (flux_transformer.c:1117-1138).
+ */
+int flux_hip_kv_prepare(void *k_out, void *vt_out, int ld_vt, const void *qkv, int ld, int k_col, int v_col,
+                        int rows, int heads, int split, const float *k_w0, const float *k_w1,
+                        const float *rope_cos, const float *rope_sin, float eps);
+
+/*
+ * Multi-head attention, no mask: out = softmax(q k^T / sqrt(128)) v per head, online softmax,
+ * scores never stored. q is read raw from the qkv buffer and gets per-head RMSNorm * weight and
+ * RoPE inside the kernel; k and vt come from flux_hip_kv_prepare. head_dim is 128.
+ * Replaces joint_attention / mha_forward (flux_transformer.c:1249-1460), flux_flash_attention
+ * (flux_kernels.c:877), flux_softmax (flux_kernels.c:596) and the Q half of apply_qk_norm /
+ * apply_rope_2d.
+ */
+int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ldq, const void *k, const void *vt, int ld_vt,
+                       int seq_q, int seq_k, int heads, int split, const float *q_w0, const float *q_w1,
+                       const float *rope_cos, const float *rope_sin, float eps);
+
+/* y[m, n] = sum_k f(x[m, k]) * W[n, k], x f32 [M, K] (M small), W bf16, y f32; f = SiLU when
+ * silu_input. The modulation and time-embedding projections (flux_transformer.c:956-969,
+ * 3226-3234, 3016-3024, 3523-3530). */
+int flux_hip_gemv(float *y, const float *x, const void *W_bf16, int M, int N, int K, int silu_input);
+
+/* Layout/precision edges: NCHW f32 latent [C, n] -> token-major bf16 [n, C]
+ * (flux_transformer.c:3156-3161), and f32 -> bf16 (flux_shaders.metal:1430). */
+int flux_hip_latent_to_tokens(void *tok_bf16, const float *latent, int channels, int n);
+int flux_hip_f32_to_bf16(void *out_bf16, const float *in, size_t n);
+
+/* z += dt * v   (flux_axpy, flux_kernels.c:126; flux_sample.c:248) */
+int flux_hip_euler_update(float *z, const float *v, float dt, size_t n);
+/* z += dt * (vu + g * (vc - vu))   (flux_sample.c:496-499) */
+int flux_hip_cfg_euler_update(float *z, const float *v_uncond, const float *v_cond, float guidance, float dt, size_t n);
+
+/* -------------------------------------------------------------------- model */
+
+typedef struct flux_transformer flux_transformer_t;
+
+typedef struct {
+    int hidden, heads, head_dim, mlp, n_double, n_single, text_dim, channels;
+    int axis_dim, sincos_dim;
+    float rope_theta;
+} flux_hip_config;
+
+/* FLUX.2-klein-4B sizes (flux.h:33-41, flux_transformer.c:4418-4434). */
+void flux_hip_default_config(flux_hip_config *cfg);
+
+/* Builds a model from bf16 tensors handed over by name (the safetensors keys read at
+ * flux_transformer.c:4452-4602). All tensors must be set before the first forward. */
+flux_transformer_t *flux_hip_transformer_new(const flux_hip_config *cfg);
+int flux_hip_transformer_set_tensor(flux_transformer_t *tf, const char *name, const uint16_t *bf16, int64_t numel);
+/* Opens a .safetensors file (bf16 tensors) and uploads it; 4B sizes unless cfg is given. */
+flux_transformer_t *flux_hip_transformer_load_file(const char *path, const flux_hip_config *cfg);
+
+/* Reference loader entry points (flux_transformer.c:4411, 4659; called at flux.c:300-326).
+ * `sf` is the reference's safetensors_file_t (flux_safetensors.h:41-49). Both upload the bf16
+ * tensors once; the mmap variant takes ownership of sf and closes it in flux_transformer_free,
+ * as the reference does (flux_transformer.c:4305-4309). */
+struct safetensors_file;
+flux_transformer_t *flux_transformer_load_safetensors(void *sf);
+flux_transformer_t *flux_transformer_load_safetensors_mmap(void *sf);
+void flux_transformer_free(flux_transformer_t *tf);
+
+typedef struct {
+    const float *latent; /* [channels, h, w] */
+    int h, w;
+    int t_offset;        /* RoPE T coordinate: 10, 20, ... */
+} flux_ref_t;
+
+/* One velocity prediction; inputs on the host, result malloc'd [channels, h*w], caller frees.
+ * Same contracts as flux_transformer.c:3115, 3605, 3815. */
+float *flux_transformer_forward(flux_transformer_t *tf, const float *img_latent, int img_h, int img_w,
+                                const float *txt_emb, int txt_seq, float timestep);
+float *flux_transformer_forward_with_refs(flux_transformer_t *tf, const float *img_latent, int img_h, int img_w,
+                                          const float *ref_latent, int ref_h, int ref_w, int t_offset,
+                                          const float *txt_emb, int txt_seq, float timestep);
+float *flux_transformer_forward_with_multi_refs(flux_transformer_t *tf, const float *img_latent, int img_h, int img_w,
+                                                const flux_ref_t *refs, int num_refs,
+                                                const float *txt_emb, int txt_seq, float timestep);
+
+/* Samplers with the reference's signatures (flux_sample.c:212, 303, 381, 457, 534, 615). The
+ * whole loop runs on the device: inputs are uploaded once, the latent is read back once. */
+float *flux_sample_euler(void *transformer, void *text_encoder, float *z, int batch, int channels, int h, int w,
+                         const float *text_emb, int text_seq, const float *schedule, int num_steps,
+                         void (*progress_callback)(int step, int total));
+float *flux_sample_euler_with_refs(void *transformer, void *text_encoder, float *z, int batch, int channels, int h, int w,
+                                   const float *ref_latent, int ref_h, int ref_w, int t_offset,
+                                   const float *text_emb, int text_seq, const float *schedule, int num_steps,
+                                   void (*progress_callback)(int step, int total));
+float *flux_sample_euler_with_multi_refs(void *transformer, void *text_encoder, float *z, int batch, int channels, int h, int w,
+                                         const flux_ref_t *refs, int num_refs,
+                                         const float *text_emb, int text_seq, const float *schedule, int num_steps,
+                                         void (*progress_callback)(int step, int total));
+float *flux_sample_euler_cfg(void *transformer, void *text_encoder, float *z, int batch, int channels, int h, int w,
+                             const float *text_emb_cond, int text_seq_cond,
+                             const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
+                             const float *schedule, int num_steps, void (*progress_callback)(int step, int total));
+float *flux_sample_euler_cfg_with_refs(void *transformer, void *text_encoder, float *z, int batch, int channels, int h, int w,
+                                       const float *ref_latent, int ref_h, int ref_w, int t_offset,
+                                       const float *text_emb_cond, int text_seq_cond,
+                                       const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
+                                       const float *schedule, int num_steps, void (*progress_callback)(int step, int total));
+float *flux_sample_euler_cfg_with_multi_refs(void *transformer, void *text_encoder, float *z, int batch, int channels, int h, int w,
+                                             const flux_ref_t *refs, int num_refs,
+                                             const float *text_emb_cond, int text_seq_cond,
+                                             const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
+                                             const float *schedule, int num_steps,
+                                             void (*progress_callback)(int step, int total));
+
+/* Schedules (flux_sample.c:49, 62, 145); malloc'd [num_steps + 1], caller frees. */
+float *flux_linear_schedule(int num_steps);
+float *flux_power_schedule(int num_steps, float alpha);
+float *flux_official_schedule(int num_steps, int image_seq_len);
+
+/* Same sampling loops, additionally copying every forward's velocity (in call order,
+ * [forwards, channels*h*w] f32) to v_trace when it is not NULL. For parity tests. */
+float *flux_hip_sample_traced(void *transformer, const float *z, int channels, int h, int w,
+                              const flux_ref_t *refs, int num_refs,
+                              const float *text_emb_cond, int text_seq_cond,
+                              const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
+                              const float *schedule, int num_steps, float *v_trace);
+
+/* Per-stage device time of the last sampling call in milliseconds (role of the
+ * flux_timing_transformer_* counters, flux_sample.c:29-39). */
+extern double flux_timing_transformer_total;
+extern double flux_timing_transformer_double;
+extern double flux_timing_transformer_single;
+extern double flux_timing_transformer_final;
+void flux_reset_timing(void);
+
+/* Progress hooks with the reference's names (flux_kernels.h:245-256). They fire on the host
+ * thread when the corresponding work has been queued, not when it has finished. */
+typedef enum { FLUX_SUBSTEP_DOUBLE_BLOCK, FLUX_SUBSTEP_SINGLE_BLOCK, FLUX_SUBSTEP_FINAL_LAYER } flux_substep_type_t;
+typedef void (*flux_substep_callback_t)(flux_substep_type_t type, int index, int total);
+typedef void (*flux_step_callback_t)(int step, int total);
+extern flux_substep_callback_t flux_substep_callback;
+extern flux_step_callback_t flux_step_callback;
+extern int flux_verbose;
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLUX_HIP_H */

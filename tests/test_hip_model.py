@@ -1,0 +1,188 @@
+"""Whole-model parity of the HIP backend against the CPU oracle and the reference's golden vectors.
+
+Gates (the stated tolerance of the backend): per-forward velocity relative L2 <= 2e-2 and
+cosine >= 0.999 against the fp32 CPU path; final latent PSNR >= 35 dB (peak = range of the
+reference latent).
+"""
+import os
+
+import numpy as np
+import pytest
+
+from metrics import rel_l2, cosine, psnr
+from model_spec import TINY, SMALL, KLEIN_4B, make_weights, normal_f32, write_safetensors
+
+pytestmark = pytest.mark.gpu
+
+REL_L2_MAX, COS_MIN, PSNR_MIN = 2e-2, 0.999, 35.0
+
+
+@pytest.fixture(scope="module")
+def hip():
+    import fluxhip
+    fluxhip.init()
+    fluxhip.lib().flux_hip_linear_force_tile(-1)
+    return fluxhip
+
+
+def gate(got, want, what=""):
+    r, c = rel_l2(got, want), cosine(got, want)
+    print(f"{what}: rel_l2={r:.3e} cos={c:.6f}", flush=True)
+    assert r <= REL_L2_MAX and c >= COS_MIN, (what, r, c)
+
+
+# std 0.02 is the benchmark's literal initialisation; the larger values give the small models the
+# per-layer gain the 4B model has at 0.02, so that attention and modulation shape the output
+# (moving a reference image's RoPE offset then changes the velocity by 5-8 %).
+@pytest.mark.parametrize("cfg,qk,std", [(TINY, "literal", 0.02), (TINY, "sharp", 0.02), (SMALL, "sharp", 0.02),
+                                        (TINY, "sharp", 0.08), (SMALL, "sharp", 0.05)])
+def test_forward_and_refs(hip, oracle_mod, cfg, qk, std):
+    W = make_weights(cfg, 42, std, qk)
+    o = oracle_mod.Oracle(cfg, W)
+    m = hip.Transformer(cfg, W)
+    lat = normal_f32((cfg.channels, 5, 7), 11, 1)
+    txt = normal_f32((40, cfg.text_dim), 11, 2)
+    r1 = (normal_f32((cfg.channels, 3, 4), 11, 3), 3, 4, 10)
+    r2 = (normal_f32((cfg.channels, 2, 5), 11, 4), 2, 5, 20)
+    gate(m.forward(lat, 5, 7, txt, 1.0), o.forward(lat, 5, 7, txt, 1.0), "no refs t=1")
+    gate(m.forward(lat, 5, 7, txt, 0.3), o.forward(lat, 5, 7, txt, 0.3), "no refs t=0.3")
+    gate(m.forward(lat, 5, 7, txt, 0.6, refs=[r1]), o.forward(lat, 5, 7, txt, 0.6, refs=[r1]), "one ref")
+    gate(m.forward(lat, 5, 7, txt, 0.6, refs=[r1, r2]), o.forward(lat, 5, 7, txt, 0.6, refs=[r1, r2]), "two refs")
+    m.close(); o.close()
+
+
+def test_reference_golden_tiny(hip, golden_dir):
+    """Straight against vectors the reference's own C code produced (tests/golden/make_golden.py)."""
+    for qk in ("literal", "sharp"):
+        g = np.load(os.path.join(golden_dir, f"tiny_{qk}.npz"))
+        cfg = TINY
+        m = hip.Transformer(cfg, make_weights(cfg, 42, 0.02, qk))
+        lat = normal_f32((cfg.channels, 4, 4), 7, 100)
+        txt = normal_f32((16, cfg.text_dim), 7, 101)
+        txt_u = normal_f32((12, cfg.text_dim), 7, 102)
+        r1 = (normal_f32((cfg.channels, 2, 3), 7, 103), 2, 3, 10)
+        r2 = (normal_f32((cfg.channels, 3, 2), 7, 104), 3, 2, 20)
+        gate(m.forward(lat, 4, 4, txt, 1.0), g["fwd_t1.0"], f"{qk} fwd t=1")
+        gate(m.forward(lat, 4, 4, txt, 0.37), g["fwd_t0.37"], f"{qk} fwd t=0.37")
+        gate(m.forward(lat, 4, 4, txt, 0.6, refs=[r1]), g["fwd_ref1"], f"{qk} one ref")
+        gate(m.forward(lat, 4, 4, txt, 0.6, refs=[r1, r2]), g["fwd_ref2"], f"{qk} two refs")
+        s3 = hip.schedule("official", 3, 16)
+        for key, kw in (("euler3", {}), ("euler3_ref1", dict(refs=[r1])), ("euler3_ref2", dict(refs=[r1, r2]))):
+            z = m.sample(lat, 4, 4, txt, s3, **kw)
+            assert psnr(z, g[key]) >= PSNR_MIN, (key, psnr(z, g[key]))
+        for key, kw in (("cfg2", {}), ("cfg2_ref1", dict(refs=[r1])), ("cfg2_ref2", dict(refs=[r1, r2]))):
+            z = m.sample(lat, 4, 4, txt, s3[:3], txt_uncond=txt_u, guidance=4.0, **kw)
+            assert psnr(z, g[key]) >= PSNR_MIN, (key, psnr(z, g[key]))
+        m.close()
+
+
+def test_sampler_trace_and_latent(hip, oracle_mod):
+    """Per-step velocities and the final latent of a 4-step schedule, Euler and CFG + reference."""
+    cfg = SMALL
+    W = make_weights(cfg, 42, 0.02, "sharp")
+    o = oracle_mod.Oracle(cfg, W)
+    m = hip.Transformer(cfg, W)
+    h, w = 6, 6
+    z = normal_f32((cfg.channels, h, w), 12, 1)
+    txt = normal_f32((48, cfg.text_dim), 12, 2)
+    txt_u = normal_f32((48, cfg.text_dim), 12, 3)
+    ref = (normal_f32((cfg.channels, h, w), 12, 4), h, w, 10)
+    s = hip.schedule("official", 4, h * w)
+    np.testing.assert_allclose(s, oracle_mod.official_schedule(4, h * w), atol=2e-7)
+    zo, vo = o.sample_euler(z, h, w, txt, s, trace=True)
+    zg, vg = m.sample(z, h, w, txt, s, trace=True)
+    for i in range(4):
+        gate(vg[i], vo[i], f"euler step {i}")
+    assert psnr(zg, zo) >= PSNR_MIN, psnr(zg, zo)
+    zo, vo = o.sample_euler_cfg(z, h, w, txt, txt_u, 4.0, s[:3], refs=[ref], trace=True)
+    zg, vg = m.sample(z, h, w, txt, s[:3], refs=[ref], txt_uncond=txt_u, guidance=4.0, trace=True)
+    for i in range(4):
+        gate(vg[i], vo[i], f"cfg forward {i}")
+    assert psnr(zg, zo) >= PSNR_MIN, psnr(zg, zo)
+    m.close(); o.close()
+
+
+def test_broken_rope_would_be_caught(hip, oracle_mod):
+    """Sensitivity check: against an oracle whose image RoPE is mirrored the gate must fail,
+    otherwise the sharp fixture would say nothing about RoPE in the HIP kernels."""
+    cfg = TINY
+    W = make_weights(cfg, 42, 0.08, "sharp")     # weights large enough for attention to matter
+    o = oracle_mod.Oracle(cfg, W)
+    m = hip.Transformer(cfg, W)
+    lat = normal_f32((cfg.channels, 6, 6), 13, 1)
+    txt = normal_f32((24, cfg.text_dim), 13, 2)
+    good = o.forward(lat, 6, 6, txt, 0.8)
+    wrong = o.forward(lat.reshape(cfg.channels, 6, 6).transpose(0, 2, 1).copy(), 6, 6, txt, 0.8)  # rows<->cols
+    wrong = wrong.transpose(0, 2, 1)
+    got = m.forward(lat, 6, 6, txt, 0.8)
+    gate(got, good, "correct rope")
+    assert rel_l2(got, wrong) > 3 * REL_L2_MAX, rel_l2(got, wrong)
+    # same for the T axis of a reference image: offsets 10 and 20 must be told apart
+    ref = normal_f32((cfg.channels, 6, 6), 13, 3)
+    good = o.forward(lat, 6, 6, txt, 0.8, refs=[(ref, 6, 6, 10)])
+    wrong = o.forward(lat, 6, 6, txt, 0.8, refs=[(ref, 6, 6, 20)])
+    got = m.forward(lat, 6, 6, txt, 0.8, refs=[(ref, 6, 6, 10)])
+    gate(got, good, "ref offset 10")
+    assert rel_l2(got, wrong) > 2 * REL_L2_MAX, rel_l2(got, wrong)
+    m.close(); o.close()
+
+
+def test_safetensors_file_loader(hip, oracle_mod, tmp_path):
+    cfg = TINY
+    W = make_weights(cfg, 42, 0.02, "sharp")
+    p = tmp_path / "tiny.safetensors"
+    write_safetensors(str(p), W)
+    a = hip.Transformer(cfg, path=str(p))
+    b = hip.Transformer(cfg, W)
+    lat = normal_f32((cfg.channels, 4, 4), 14, 1)
+    txt = normal_f32((16, cfg.text_dim), 14, 2)
+    assert np.array_equal(a.forward(lat, 4, 4, txt, 0.5), b.forward(lat, 4, 4, txt, 0.5))
+    a.close(); b.close()
+    # a file with a tensor missing must be refused, not half-loaded
+    W.pop("proj_out.weight")
+    write_safetensors(str(p), W)
+    with pytest.raises(hip.FluxHipError):
+        hip.Transformer(cfg, path=str(p))
+
+
+def test_error_paths(hip):
+    cfg = TINY
+    m = hip.Transformer(cfg)          # no weights yet
+    lat = normal_f32((cfg.channels, 2, 2), 15, 1)
+    txt = normal_f32((8, cfg.text_dim), 15, 2)
+    with pytest.raises(hip.FluxHipError):
+        m.forward(lat, 2, 2, txt, 0.5)
+    with pytest.raises(hip.FluxHipError):
+        m.set_tensor("proj_out.weight", np.zeros(3, np.uint16))        # wrong size
+    with pytest.raises(hip.FluxHipError):
+        m.set_tensor("no.such.tensor", np.zeros(3, np.uint16))
+    m.close()
+
+
+def test_sequence_growth_between_calls(hip, oracle_mod):
+    """Work buffers and RoPE tables are re-made when the token count grows or shrinks."""
+    cfg = TINY
+    W = make_weights(cfg, 42, 0.02, "sharp")
+    o = oracle_mod.Oracle(cfg, W)
+    m = hip.Transformer(cfg, W)
+    for (h, w, nt) in ((2, 2, 8), (9, 11, 70), (3, 3, 5), (9, 11, 70)):
+        lat = normal_f32((cfg.channels, h, w), 16, h * 100 + w)
+        txt = normal_f32((nt, cfg.text_dim), 16, nt)
+        gate(m.forward(lat, h, w, txt, 0.7), o.forward(lat, h, w, txt, 0.7), f"{h}x{w}+{nt}")
+    m.close(); o.close()
+
+
+@pytest.mark.parametrize("qk", ["literal", "sharp"])
+def test_klein4b_c1_against_reference_golden(hip, golden_dir, qk):
+    """Real 4B architecture, 4x4 latent + 64 text tokens, t = 1: the velocity the reference's C
+    code computed for the same seeded weights and inputs (fixture written by make_golden.py --full)."""
+    g = np.load(os.path.join(golden_dir, f"klein4b_c1_{qk}.npz"))
+    cfg = KLEIN_4B
+    m = hip.Transformer(cfg)
+    from model_spec import tensor_shapes
+    for name in tensor_shapes(cfg):            # one tensor at a time keeps the host footprint small
+        m.set_tensor(name, make_weights(cfg, 42, 0.02, qk, only=[name])[name])
+    lat = normal_f32((cfg.channels, 4, 4), 42, 1000)
+    txt = normal_f32((64, cfg.text_dim), 42, 1001)
+    gate(m.forward(lat, 4, 4, txt, 1.0), g["velocity"], f"4B c1 {qk}")
+    m.close()

@@ -1,0 +1,210 @@
+"""Parity of every HIP operator against the CPU oracle, through the C ABI (include/flux_hip.h).
+
+Inputs are rounded to bf16 first, so both sides see identical values; what remains is fp32
+accumulation order and the bf16 rounding of outputs. Tolerances are stated per test.
+"""
+import numpy as np
+import pytest
+
+from metrics import rel_l2
+from model_spec import normal_f32, f32_to_bf16, bf16_to_f32
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+    import fluxhip
+    fluxhip.init()
+    yield fluxhip
+    fluxhip.lib().flux_hip_linear_force_tile(-1)
+
+
+def q(x):
+    """Round to bf16 and come back: the values a bf16 tensor actually holds."""
+    return bf16_to_f32(f32_to_bf16(x))
+
+
+def dev_bf16(hip, x):
+    return hip.DevBuf.from_array(f32_to_bf16(x))
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("M", [1, 37, 130, 300])
+def test_linear_bf16_and_f32(hip, oracle_mod, tile, M):
+    N, K = 512, 192
+    hip.lib().flux_hip_linear_force_tile(tile)
+    x = q(normal_f32((M, K), 3, 1))
+    W = q(normal_f32((N + 64, K), 3, 2, 0.0, 0.1))
+    want = oracle_mod.linear(x, W[64:64 + N])
+    dx, dW = dev_bf16(hip, x), dev_bf16(hip, W)
+    # bf16 output, weight rows start at 64
+    out = hip.DevBuf(M * N * 2)
+    hip.linear(hip.EPI_BF16, [(dx.ptr, dW.ptr, out.ptr, None, M)], N, K, K, K, N, 64, 0)
+    got = bf16_to_f32(out.to_array(np.uint16, (M, N)))
+    assert rel_l2(got, want) < 4e-3          # bf16 output rounding: 2^-9 relative per element
+    # fp32 output is accumulation-order noise only
+    out32 = hip.DevBuf(M * N * 4)
+    hip.linear(hip.EPI_F32, [(dx.ptr, dW.ptr, out32.ptr, None, M)], N, K, K, K, N, 64, 0)
+    assert rel_l2(out32.to_array(np.float32, (M, N)), want) < 2e-6
+    # transposed fp32 output
+    outT = hip.DevBuf(M * N * 4)
+    hip.linear(hip.EPI_F32_T, [(dx.ptr, dW.ptr, outT.ptr, None, M)], N, K, K, K, M, 64, 0)
+    assert rel_l2(outT.to_array(np.float32, (N, M)).T, want) < 2e-6
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2])
+def test_linear_two_parts_resid_and_strides(hip, oracle_mod, tile):
+    """Two row ranges with different weights, strided A (lda > K), gated residual epilogue."""
+    hip.lib().flux_hip_linear_force_tile(tile)
+    M0, M1, N, K, lda = 70, 200, 256, 128, 320
+    a = q(normal_f32((M0 + M1, lda), 4, 1))
+    W0 = q(normal_f32((N, K), 4, 2, 0.0, 0.1))
+    W1 = q(normal_f32((N, K), 4, 3, 0.0, 0.1))
+    res = normal_f32((M0 + M1, N), 4, 4)
+    g0 = normal_f32((N,), 4, 5)
+    g1 = normal_f32((N,), 4, 6)
+    col = 64  # A starts at column 64 of the strided buffer
+    want = res.copy()
+    want[:M0] += g0 * oracle_mod.linear(a[:M0, col:col + K], W0)
+    want[M0:] += g1 * oracle_mod.linear(a[M0:, col:col + K], W1)
+    da, dW0, dW1 = dev_bf16(hip, a), dev_bf16(hip, W0), dev_bf16(hip, W1)
+    dres = hip.DevBuf.from_array(res)
+    dg0, dg1 = hip.DevBuf.from_array(g0), hip.DevBuf.from_array(g1)
+    hip.linear(hip.EPI_RESID, [(da.at(col * 2), dW0.ptr, dres.ptr, dg0.ptr, M0),
+                               (da.at((M0 * lda + col) * 2), dW1.ptr, dres.at(M0 * N * 4), dg1.ptr, M1)],
+               N, K, lda, K, N)
+    assert rel_l2(dres.to_array(np.float32, (M0 + M1, N)), want) < 2e-6
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2])
+def test_linear_swiglu(hip, oracle_mod, tile):
+    """silu(x Wg^T) * (x Wu^T) with gate/up rows at arbitrary offsets and a strided output."""
+    hip.lib().flux_hip_linear_force_tile(tile)
+    M, K, mlp, ldc, r0 = 150, 128, 384, 512, 128
+    x = q(normal_f32((M, K), 5, 1))
+    W = q(normal_f32((r0 + 2 * mlp, K), 5, 2, 0.0, 0.15))
+    g = oracle_mod.linear(x, W[r0:r0 + mlp])
+    u = oracle_mod.linear(x, W[r0 + mlp:])
+    want = oracle_mod.silu(g) * u
+    dx, dW = dev_bf16(hip, x), dev_bf16(hip, W)
+    out = hip.DevBuf.from_array(np.zeros((M, ldc), np.uint16))
+    hip.linear(hip.EPI_SWIGLU, [(dx.ptr, dW.ptr, out.at(64 * 2), None, M)], 2 * mlp, K, K, K, ldc, r0, r0 + mlp)
+    got = bf16_to_f32(out.to_array(np.uint16, (M, ldc)))
+    assert rel_l2(got[:, 64:64 + mlp], want) < 4e-3
+    assert not got[:, :64].any() and not got[:, 64 + mlp:].any()   # nothing written outside
+
+
+def test_linear_rejects_bad_shapes(hip):
+    d = hip.DevBuf(1024)
+    with pytest.raises(hip.FluxHipError):
+        hip.linear(hip.EPI_BF16, [(d.ptr, d.ptr, d.ptr, None, 4)], 128, 100, 100, 100, 128)   # K % 64
+    with pytest.raises(hip.FluxHipError):
+        hip.linear(hip.EPI_BF16, [(d.ptr, d.ptr, d.ptr, None, 4)], 100, 64, 64, 64, 100)      # N % 128
+    with pytest.raises(hip.FluxHipError):
+        hip.linear(hip.EPI_RESID, [(d.ptr, d.ptr, d.ptr, None, 4)], 128, 64, 64, 64, 128)     # no gate
+    hip.linear(hip.EPI_BF16, [(d.ptr, d.ptr, d.ptr, None, 0)], 128, 64, 64, 64, 128)          # empty is a no-op
+
+
+@pytest.mark.parametrize("hidden", [256, 3072])
+def test_adaln(hip, oracle_mod, hidden):
+    rows, split = 45, 17
+    x = normal_f32((rows, hidden), 6, 1, 0.5, 3.0)
+    m = [normal_f32((hidden,), 6, 2 + i, 0.0, 0.5) for i in range(4)]
+    want = np.concatenate([oracle_mod.adaln(x[:split], m[0], m[1]), oracle_mod.adaln(x[split:], m[2], m[3])])
+    dx = hip.DevBuf.from_array(x)
+    dm = [hip.DevBuf.from_array(v) for v in m]
+    out = hip.DevBuf(rows * hidden * 2)
+    hip.check(hip.lib().flux_hip_adaln_norm(out.ptr, hidden, dx.ptr, rows, hidden, split,
+                                            dm[0].ptr, dm[1].ptr, dm[2].ptr, dm[3].ptr, 1e-6))
+    got = bf16_to_f32(out.to_array(np.uint16, (rows, hidden)))
+    assert rel_l2(got, want) < 4e-3           # bf16 output rounding
+    assert np.abs(got - want).max() < 0.05
+
+
+@pytest.mark.parametrize("silu", [0, 1])
+def test_gemv(hip, oracle_mod, silu):
+    M, N, K = 11, 77, 256
+    x = normal_f32((M, K), 7, 1, 0.0, 2.0)
+    W = q(normal_f32((N, K), 7, 2, 0.0, 0.1))
+    want = oracle_mod.linear(oracle_mod.silu(x) if silu else x, W)
+    dx, dW = hip.DevBuf.from_array(x), dev_bf16(hip, W)
+    out = hip.DevBuf(M * N * 4)
+    hip.check(hip.lib().flux_hip_gemv(out.ptr, dx.ptr, dW.ptr, M, N, K, silu))
+    assert rel_l2(out.to_array(np.float32, (M, N)), want) < 5e-6
+
+
+def _attention_case(hip, oracle_mod, n, split, heads, seed, qk_scale=1.0):
+    """qkv buffer -> kv_prepare -> attention, against qk_norm + rope + attention of the oracle."""
+    H = heads * 128
+    qkv = q(normal_f32((n, 3 * H), seed, 1))
+    w = [normal_f32((128,), seed, 2 + i, 1.0, 0.3) * qk_scale for i in range(4)]   # q0 q1 k0 k1
+    ic, isn = oracle_mod.rope_image(1, n - split) if n > split else (np.zeros((0, 128), np.float32),) * 2
+    tc, ts = oracle_mod.rope_text(split)
+    cos = np.concatenate([tc, ic]) if split else ic
+    sin = np.concatenate([ts, isn]) if split else isn
+    Q, K, V = qkv[:, :H].copy(), qkv[:, H:2 * H].copy(), qkv[:, 2 * H:].copy()
+    for lo, hi, qw, kw in ((0, split, w[0], w[2]), (split, n, w[1], w[3])):
+        if hi > lo:
+            Q[lo:hi], K[lo:hi] = oracle_mod.qk_norm(Q[lo:hi], K[lo:hi], qw, kw, heads, 128)
+    Q = oracle_mod.apply_rope(Q, cos, sin, heads, 128)
+    K = oracle_mod.apply_rope(K, cos, sin, heads, 128)
+    want = oracle_mod.attention(Q, K, V, heads, 128)
+
+    dqkv = dev_bf16(hip, qkv)
+    dw = [hip.DevBuf.from_array(v.astype(np.float32)) for v in w]
+    dcos, dsin = hip.DevBuf.from_array(cos), hip.DevBuf.from_array(sin)
+    ldvt = (n + 63) // 64 * 64
+    kn, vt = hip.DevBuf(n * H * 2), hip.DevBuf(H * ldvt * 2)
+    ldo = H + 64
+    out = hip.DevBuf.from_array(np.zeros((n, ldo), np.uint16))
+    L = hip.lib()
+    hip.check(L.flux_hip_kv_prepare(kn.ptr, vt.ptr, ldvt, dqkv.ptr, 3 * H, H, 2 * H, n, heads, split,
+                                    dw[2].ptr, dw[3].ptr, dcos.ptr, dsin.ptr, 1e-6))
+    hip.check(L.flux_hip_attention(out.ptr, ldo, dqkv.ptr, 3 * H, kn.ptr, vt.ptr, ldvt, n, n, heads, split,
+                                   dw[0].ptr, dw[1].ptr, dcos.ptr, dsin.ptr, 1e-6))
+    # prepared K and V^T
+    kn_h = bf16_to_f32(kn.to_array(np.uint16, (n, H)))
+    assert rel_l2(kn_h, K) < 4e-3
+    vt_h = bf16_to_f32(vt.to_array(np.uint16, (H, ldvt)))
+    assert np.array_equal(vt_h[:, :n], V.T) and not vt_h[:, n:].any()
+    got = bf16_to_f32(out.to_array(np.uint16, (n, ldo)))
+    assert not got[:, H:].any()
+    return got[:, :H], want
+
+
+@pytest.mark.parametrize("n,split,heads", [(1, 0, 1), (64, 64, 2), (80, 64, 2), (191, 50, 3), (333, 128, 2), (768, 512, 2)])
+def test_attention(hip, oracle_mod, n, split, heads):
+    got, want = _attention_case(hip, oracle_mod, n, split, heads, 8)
+    # q, k, p are rounded to bf16 inside the kernel and the output is bf16
+    assert rel_l2(got, want) < 1e-2, rel_l2(got, want)
+
+
+def test_attention_sharp_logits(hip, oracle_mod):
+    """Norm weights of 3 give logits of order 10: softmax far from uniform, RoPE decisive."""
+    got, want = _attention_case(hip, oracle_mod, 200, 72, 2, 9, qk_scale=3.0)
+    assert rel_l2(got, want) < 2.5e-2, rel_l2(got, want)
+
+
+def test_layout_edges_and_updates(hip, oracle_mod):
+    C, n = 128, 45
+    lat = normal_f32((C, n), 10, 1)
+    d = hip.DevBuf.from_array(lat)
+    tok = hip.DevBuf(n * C * 2)
+    hip.check(hip.lib().flux_hip_latent_to_tokens(tok.ptr, d.ptr, C, n))
+    assert np.array_equal(tok.to_array(np.uint16, (n, C)), f32_to_bf16(lat.T.copy()))   # bit exact
+    x = normal_f32((1027,), 10, 2)
+    dx = hip.DevBuf.from_array(x)
+    o = hip.DevBuf(1027 * 2)
+    hip.check(hip.lib().flux_hip_f32_to_bf16(o.ptr, dx.ptr, 1027))
+    assert np.array_equal(o.to_array(np.uint16, (1027,)), f32_to_bf16(x))               # RNE, bit exact
+    z = normal_f32((999,), 10, 3)
+    v = normal_f32((999,), 10, 4)
+    vu = normal_f32((999,), 10, 5)
+    dz, dv, dvu = hip.DevBuf.from_array(z), hip.DevBuf.from_array(v), hip.DevBuf.from_array(vu)
+    hip.check(hip.lib().flux_hip_euler_update(dz.ptr, dv.ptr, -0.25, 999))
+    np.testing.assert_allclose(dz.to_array(np.float32, (999,)), z + np.float32(-0.25) * v, rtol=0, atol=1e-6)
+    dz = hip.DevBuf.from_array(z)
+    hip.check(hip.lib().flux_hip_cfg_euler_update(dz.ptr, dvu.ptr, dv.ptr, 4.0, -0.1, 999))
+    want = z + np.float32(-0.1) * (vu + np.float32(4.0) * (v - vu))
+    np.testing.assert_allclose(dz.to_array(np.float32, (999,)), want, rtol=0, atol=2e-6)
