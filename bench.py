@@ -1,0 +1,192 @@
+#!/usr/bin/env python3
+"""Benchmark of the MI355X denoising-transformer backend: denoise steps/s on one GPU.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4]
+
+One "step" is every transformer forward of one Euler step plus the latent update, at the real
+FLUX.2-klein-4B architecture with random-init bf16 weights ~N(0, 0.02) and N(0,1) inputs
+(there are no model files or datasets here). Inputs are resident in HBM before the timed
+region; the host only queues kernels. Prints ONE JSON line.
+
+Also measured in the same run:
+  roofline      the dominant kernel (gate/up projection GEMM with the SiLU*up epilogue) launched
+                alone at the workload's shape and timed with HIP events on the backend's stream
+  cpu_baseline  the CPU oracle (fp32, BLAS when available) on a bounded sample of the same
+                workload: one double-stream and two single-stream blocks at full shape,
+                extrapolated to the 5 + 20 blocks of a step
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "flux2.c_amd"))
+
+import numpy as np  # noqa: E402
+
+import fluxhip  # noqa: E402
+from model_spec import KLEIN_4B, FluxConfig, tensor_shapes, make_weights, normal_f32, normal_bf16, flops_per_forward  # noqa: E402
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA peak (datasheet)
+
+# (latent h, w, text tokens, reference-image latents [(h, w, t_offset)], cfg, schedule steps)
+WORKLOADS = {
+    "c1": dict(h=4, w=4, txt=64, refs=[], cfg=False, desc="64x64: 16 image + 64 text tokens"),
+    "c2": dict(h=16, w=16, txt=512, refs=[], cfg=False, desc="256x256: 256 image + 512 text tokens"),
+    "c3": dict(h=32, w=32, txt=512, refs=[], cfg=False, desc="512x512: 1024 image + 512 text tokens"),
+    "c4": dict(h=64, w=64, txt=512, refs=[], cfg=False, desc="1024x1024: 4096 image + 512 text tokens"),
+    "c5": dict(h=32, w=32, txt=512, refs=[(32, 32, 10)], cfg=True,
+               desc="512x512 CFG + 1 reference image: 2 forwards/step over 2048 image + 512 text tokens"),
+}
+
+
+def load_model(cfg, seed=42, qk="literal"):
+    m = fluxhip.Transformer(cfg)
+    for name in tensor_shapes(cfg):
+        m.set_tensor(name, make_weights(cfg, seed, 0.02, qk, only=[name])[name])
+    return m
+
+
+def time_dominant_kernel(cfg, tokens, launches=20):
+    """Gate/up projection with SwiGLU epilogue at [tokens, hidden] x [2*mlp, hidden]^T, alone."""
+    H, M = cfg.hidden, cfg.mlp
+    a = fluxhip.DevBuf.from_array(normal_bf16((tokens, H), 5, 1))
+    w = fluxhip.DevBuf.from_array(normal_bf16((2 * M, H), 5, 2, 0.0, 0.02))
+    out = fluxhip.DevBuf(tokens * M * 2)
+    L = fluxhip.lib()
+    part = [(a.ptr, w.ptr, out.ptr, None, tokens)]
+    for _ in range(3):
+        fluxhip.linear(fluxhip.EPI_SWIGLU, part, 2 * M, H, H, H, M, 0, M)
+    fluxhip.sync()
+    L.flux_hip_timer_start()
+    for _ in range(launches):
+        fluxhip.linear(fluxhip.EPI_SWIGLU, part, 2 * M, H, H, H, M, 0, M)
+    ms = L.flux_hip_timer_stop() / launches
+    flops = 2.0 * tokens * H * 2 * M
+    for b in (a, w, out):
+        b.free()
+    return ms, flops
+
+
+def cpu_baseline(cfg, n_img, n_txt):
+    """Oracle timing on this host: 1 double + 2 single blocks at full shape -> steps/s."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle as O
+    blas = O.enable_blas()
+    sub = FluxConfig(**{**cfg.as_dict(), "n_double": 1, "n_single": 1})
+    names = [n for n in tensor_shapes(sub) if n.startswith(("transformer_blocks.0.", "single_transformer_blocks.0."))]
+    W = make_weights(sub, 42, 0.02, "literal", only=names)
+    o = O.Oracle(sub, W)
+    del W
+    H = cfg.hidden
+    n = n_img + n_txt
+    ic, isn = O.rope_image(1, n_img)
+    tc, ts = O.rope_text(n_txt)
+    ih, th = normal_f32((n_img, H), 9, 1), normal_f32((n_txt, H), 9, 2)
+    im, tm = normal_f32((6 * H,), 9, 3, 0.0, 0.1), normal_f32((6 * H,), 9, 4, 0.0, 0.1)
+    O.linear(normal_f32((256, 256), 9, 5), normal_f32((256, 256), 9, 6))   # wake the BLAS threads
+    t0 = time.time()
+    o.double_block(0, ih, th, im, tm, ic, isn, tc, ts)
+    t_d = time.time() - t0
+    x = normal_f32((n, H), 9, 7)
+    t_s = []
+    for _ in range(2):
+        t0 = time.time()
+        o.single_block(0, x, im[:3 * H], ic, isn, tc, ts, n_txt)
+        t_s.append(time.time() - t0)
+    o.close()
+    t_step = cfg.n_double * t_d + cfg.n_single * min(t_s)
+    return {
+        "value": 1.0 / t_step, "unit": "steps/s", "cores": int(O.lib().fo_num_threads()), "kind": "port",
+        "sample": f"1 double-stream block ({t_d:.2f} s) + 2 single-stream blocks ({min(t_s):.2f} s each) at full shape "
+                  f"({n} tokens), extrapolated to {cfg.n_double}+{cfg.n_single} blocks; "
+                  f"{'OpenBLAS sgemm ' + os.path.basename(blas) if blas else 'built-in OpenMP loops'}",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=8)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernel-timing", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this backend runs the whole model on ONE GPU (no sharding, no collectives); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    cfg = KLEIN_4B
+    wl = WORKLOADS[args.workload]
+    K, Wm = args.steps, args.warmup
+    h, w, nt = wl["h"], wl["w"], wl["txt"]
+    n_target = h * w
+    n_img = n_target + sum(rh * rw for rh, rw, _ in wl["refs"])
+    forwards = 2 if wl["cfg"] else 1
+
+    fluxhip.init()
+    model = load_model(cfg)
+    z = normal_f32((cfg.channels, h, w), 123, 1)
+    txt = normal_f32((nt, cfg.text_dim), 123, 2)
+    txt_u = normal_f32((nt, cfg.text_dim), 123, 3) if wl["cfg"] else None
+    refs = [(normal_f32((cfg.channels, rh, rw), 123, 10 + i), rh, rw, t) for i, (rh, rw, t) in enumerate(wl["refs"])]
+    sched = fluxhip.schedule("official", K + Wm, n_target)
+    sess = fluxhip.Session(model, z, h, w, txt, sched, refs=refs, txt_uncond=txt_u, guidance=4.0)
+
+    for i in range(Wm):
+        sess.step(i)
+    fluxhip.sync()
+    L = fluxhip.lib()
+    t0 = time.perf_counter()
+    L.flux_hip_timer_start()
+    for i in range(Wm, Wm + K):
+        sess.step(i)
+    ev_ms = L.flux_hip_timer_stop()      # waits for the last kernel
+    fluxhip.sync()
+    wall = time.perf_counter() - t0
+    zf = sess.latent()
+    assert np.isfinite(zf).all(), "latent is not finite"
+    stages = fluxhip.stage_timing()
+    sess.close()
+
+    ms_per_step = wall * 1000.0 / K
+    flops_step = forwards * flops_per_forward(cfg, n_img, nt, n_target)
+    tflops = flops_step / (wall / K) / 1e12
+
+    roof = None
+    if not args.no_kernel_timing:
+        k_ms, k_flops = time_dominant_kernel(cfg, n_img + nt)
+        ach = k_flops / (k_ms * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                "kernel": "gemm_kernel<256,256,2,4,SWIGLU> (gate/up projection + SiLU*up)",
+                "ms_per_launch": round(k_ms, 4), "flops_per_launch": k_flops}
+    model.close()
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(cfg, n_img, nt)
+
+    out = {
+        "metric": "transformer denoise steps/s at 1024^2 (1 GPU); achieved TFLOP/s vs bf16 peak"
+                  if args.workload == "c4" else f"transformer denoise steps/s ({args.workload}, 1 GPU)",
+        "value": round(K / wall, 4), "unit": "steps/s", "n_gpus": 1, "steps": K, "warmup": Wm,
+        "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: FLUX.2-klein-4B transformer, {wl['desc']}, batch 1, "
+                               f"{forwards} forward(s)/step, random-init bf16 weights N(0,0.02)"},
+        "tflops": round(tflops, 1), "frac_of_bf16_peak": round(tflops / PEAK_BF16_TFLOPS, 4),
+        "flops_per_step": flops_step, "device_ms_per_step_events": round(ev_ms / K, 3),
+        "stage_ms_per_step": {"double": round(stages[0] / (K + Wm), 3), "single": round(stages[1] / (K + Wm), 3),
+                              "final": round(stages[2] / (K + Wm), 3)},
+        "roofline": roof, "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -129,11 +129,33 @@ static int upload_ref_tokens(flux_transformer_t *tf, int n_target, const flux_re
     return 1;
 }
 
-float *flux_hip_sample_traced(void *transformer, const float *z, int channels, int h, int w,
-                              const flux_ref_t *refs, int num_refs,
-                              const float *text_emb_cond, int text_seq_cond,
-                              const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
-                              const float *schedule, int num_steps, float *v_trace) {
+/* Device-resident state of one sampling run. */
+struct flux_hip_session {
+    flux_transformer_t *tf;
+    fh_rope *rp_c, *rp_u;
+    int cfg, n_target, num_steps, next_forward;
+    size_t n_lat;
+    float guidance;
+    float *schedule;
+    float *z_dev, *v_c, *v_u;
+    void *txt_c, *txt_u;
+    fh_events *ev;
+};
+
+void flux_hip_session_free(flux_hip_session *s) {
+    if (!s) return;
+    flux_hip_sync();
+    flux_hip_free(s->z_dev); flux_hip_free(s->v_c); flux_hip_free(s->v_u);
+    flux_hip_free(s->txt_c); flux_hip_free(s->txt_u);
+    free(s->schedule);
+    free(s);
+}
+
+flux_hip_session *flux_hip_session_begin(void *transformer, const float *z, int channels, int h, int w,
+                                         const flux_ref_t *refs, int num_refs,
+                                         const float *text_emb_cond, int text_seq_cond,
+                                         const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
+                                         const float *schedule, int num_steps) {
     flux_transformer_t *tf = (flux_transformer_t *)transformer;
     if (!tf || !z || !text_emb_cond || !schedule) { flux_hip_fail("sampler: NULL argument"); return NULL; }
     if (!fh_model_complete(tf)) return NULL;
@@ -142,68 +164,99 @@ float *flux_hip_sample_traced(void *transformer, const float *z, int channels, i
     if (num_refs > 0 && !refs) { flux_hip_fail("sampler: refs is NULL"); return NULL; }
     const int cfg = text_emb_uncond != NULL;
     if (cfg && text_seq_uncond <= 0) { flux_hip_fail("sampler: empty unconditional text"); return NULL; }
-    const int n_target = h * w;
-    const size_t n_lat = (size_t)channels * n_target;
 
-    fh_rope *rp_c = fh_get_rope(tf, text_seq_cond, h, w, refs, num_refs);
-    if (!rp_c) return NULL;
-    fh_rope *rp_u = NULL;
-    int max_tokens = rp_c->n;
+    flux_hip_session *s = (flux_hip_session *)calloc(1, sizeof(*s));
+    if (!s) { flux_hip_fail("out of host memory"); return NULL; }
+    s->tf = tf; s->cfg = cfg; s->n_target = h * w; s->num_steps = num_steps; s->guidance = guidance_scale;
+    s->n_lat = (size_t)channels * s->n_target;
+    s->schedule = (float *)malloc((num_steps + 1) * sizeof(float));
+    if (!s->schedule) { flux_hip_fail("out of host memory"); goto fail; }
+    memcpy(s->schedule, schedule, (num_steps + 1) * sizeof(float));
+
+    s->rp_c = fh_get_rope(tf, text_seq_cond, h, w, refs, num_refs);
+    if (!s->rp_c) goto fail;
+    int max_tokens = s->rp_c->n;
     if (cfg) {
-        rp_u = fh_get_rope(tf, text_seq_uncond, h, w, refs, num_refs);
-        if (!rp_u) return NULL;
+        s->rp_u = fh_get_rope(tf, text_seq_uncond, h, w, refs, num_refs);
+        if (!s->rp_u) goto fail;
         /* the table cache may have recycled the first slot */
-        rp_c = fh_get_rope(tf, text_seq_cond, h, w, refs, num_refs);
-        if (!rp_c) return NULL;
-        if (rp_u->n > max_tokens) max_tokens = rp_u->n;
+        s->rp_c = fh_get_rope(tf, text_seq_cond, h, w, refs, num_refs);
+        if (!s->rp_c) goto fail;
+        if (s->rp_u->n > max_tokens) max_tokens = s->rp_u->n;
     }
-    if (!fh_ensure_workspace(tf, max_tokens)) return NULL;
-    if (num_steps > 0 && !fh_compute_modulation(tf, schedule, num_steps)) return NULL;
+    if (!fh_ensure_workspace(tf, max_tokens)) goto fail;
+    if (num_steps > 0 && !fh_compute_modulation(tf, schedule, num_steps)) goto fail;
 
-    float *out = NULL;
-    float *z_dev = (float *)flux_hip_malloc(n_lat * 4);
-    float *v_c = (float *)flux_hip_malloc(n_lat * 4);
-    float *v_u = cfg ? (float *)flux_hip_malloc(n_lat * 4) : NULL;
-    void *txt_c = upload_as_bf16(text_emb_cond, (size_t)text_seq_cond * tf->c.text_dim);
-    void *txt_u = cfg ? upload_as_bf16(text_emb_uncond, (size_t)text_seq_uncond * tf->c.text_dim) : NULL;
-    fh_events *ev = events_begin(num_steps * (cfg ? 2 : 1));
+    s->z_dev = (float *)flux_hip_malloc(s->n_lat * 4);
+    s->v_c = (float *)flux_hip_malloc(s->n_lat * 4);
+    s->v_u = cfg ? (float *)flux_hip_malloc(s->n_lat * 4) : NULL;
+    s->txt_c = upload_as_bf16(text_emb_cond, (size_t)text_seq_cond * tf->c.text_dim);
+    s->txt_u = cfg ? upload_as_bf16(text_emb_uncond, (size_t)text_seq_uncond * tf->c.text_dim) : NULL;
+    if (!s->z_dev || !s->v_c || !s->txt_c || (cfg && (!s->v_u || !s->txt_u))) goto fail;
+    if (!flux_hip_upload(s->z_dev, z, s->n_lat * 4)) goto fail;
+    if (!upload_ref_tokens(tf, s->n_target, refs, num_refs)) goto fail;
+    s->ev = events_begin(num_steps * (cfg ? 2 : 1));
     flux_reset_timing();
-    if (!z_dev || !v_c || !txt_c || (cfg && (!v_u || !txt_u))) goto done;
-    if (!flux_hip_upload(z_dev, z, n_lat * 4)) goto done;
-    if (!upload_ref_tokens(tf, n_target, refs, num_refs)) goto done;
+    return s;
+fail:
+    flux_hip_session_free(s);
+    return NULL;
+}
 
-    for (int s = 0; s < num_steps; s++) {
-        const float dt = schedule[s + 1] - schedule[s];
-        if (flux_step_callback) flux_step_callback(s + 1, num_steps);
-        if (cfg) {
-            /* unconditional first, then conditional (flux_sample.c:485-493) */
-            if (!fh_forward_device(tf, rp_u, z_dev, n_target, txt_u, s, v_u, ev)) goto done;
-            if (ev) ev->used++;
-            if (!fh_forward_device(tf, rp_c, z_dev, n_target, txt_c, s, v_c, ev)) goto done;
-            if (ev) ev->used++;
-            if (v_trace) {
-                if (!flux_hip_download(v_trace + (size_t)(2 * s) * n_lat, v_u, n_lat * 4)) goto done;
-                if (!flux_hip_download(v_trace + (size_t)(2 * s + 1) * n_lat, v_c, n_lat * 4)) goto done;
-            }
-            if (!flux_hip_cfg_euler_update(z_dev, v_u, v_c, guidance_scale, dt, n_lat)) goto done;
-        } else {
-            if (!fh_forward_device(tf, rp_c, z_dev, n_target, txt_c, s, v_c, ev)) goto done;
-            if (ev) ev->used++;
-            if (v_trace && !flux_hip_download(v_trace + (size_t)s * n_lat, v_c, n_lat * 4)) goto done;
-            if (!flux_hip_euler_update(z_dev, v_c, dt, n_lat)) goto done;
+int flux_hip_session_step(flux_hip_session *s, int step, float *v_trace) {
+    if (!s || step < 0 || step >= s->num_steps) return flux_hip_fail("session step %d out of range", step);
+    flux_transformer_t *tf = s->tf;
+    const float dt = s->schedule[step + 1] - s->schedule[step];
+    const size_t n = s->n_lat;
+    if (flux_step_callback) flux_step_callback(step + 1, s->num_steps);
+    if (s->cfg) {
+        /* unconditional first, then conditional (flux_sample.c:485-493) */
+        if (!fh_forward_device(tf, s->rp_u, s->z_dev, s->n_target, s->txt_u, step, s->v_u, s->ev)) return 0;
+        if (s->ev) s->ev->used++;
+        if (!fh_forward_device(tf, s->rp_c, s->z_dev, s->n_target, s->txt_c, step, s->v_c, s->ev)) return 0;
+        if (s->ev) s->ev->used++;
+        if (v_trace) {
+            if (!flux_hip_download(v_trace, s->v_u, n * 4)) return 0;
+            if (!flux_hip_download(v_trace + n, s->v_c, n * 4)) return 0;
         }
+        return flux_hip_cfg_euler_update(s->z_dev, s->v_u, s->v_c, s->guidance, dt, n);
     }
-    out = (float *)malloc(n_lat * 4);
+    if (!fh_forward_device(tf, s->rp_c, s->z_dev, s->n_target, s->txt_c, step, s->v_c, s->ev)) return 0;
+    if (s->ev) s->ev->used++;
+    if (v_trace && !flux_hip_download(v_trace, s->v_c, n * 4)) return 0;
+    return flux_hip_euler_update(s->z_dev, s->v_c, dt, n);
+}
+
+int flux_hip_session_read_latent(flux_hip_session *s, float *z_out) {
+    if (!s || !z_out) return flux_hip_fail("session: NULL argument");
+    if (!flux_hip_download(z_out, s->z_dev, s->n_lat * 4)) return 0;
+    events_collect(s->ev);
+    if (s->ev) s->ev->used = 0;
+    return 1;
+}
+
+float *flux_hip_sample_traced(void *transformer, const float *z, int channels, int h, int w,
+                              const flux_ref_t *refs, int num_refs,
+                              const float *text_emb_cond, int text_seq_cond,
+                              const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
+                              const float *schedule, int num_steps, float *v_trace) {
+    flux_hip_session *s = flux_hip_session_begin(transformer, z, channels, h, w, refs, num_refs, text_emb_cond,
+                                                 text_seq_cond, text_emb_uncond, text_seq_uncond, guidance_scale,
+                                                 schedule, num_steps);
+    if (!s) return NULL;
+    const size_t per_step = s->n_lat * (s->cfg ? 2 : 1);
+    float *out = NULL;
+    for (int i = 0; i < num_steps; i++)
+        if (!flux_hip_session_step(s, i, v_trace ? v_trace + (size_t)i * per_step : NULL)) goto done;
+    out = (float *)malloc(s->n_lat * 4);
     if (!out) { flux_hip_fail("out of host memory"); goto done; }
-    if (!flux_hip_download(out, z_dev, n_lat * 4)) { free(out); out = NULL; goto done; }
-    events_collect(ev);
+    if (!flux_hip_session_read_latent(s, out)) { free(out); out = NULL; goto done; }
     if (flux_verbose)
         fprintf(stderr, "denoising on device: double %.2f ms, single %.2f ms, final %.2f ms, total %.2f ms\n",
                 flux_timing_transformer_double, flux_timing_transformer_single, flux_timing_transformer_final,
                 flux_timing_transformer_total);
 done:
-    flux_hip_sync();
-    flux_hip_free(z_dev); flux_hip_free(v_c); flux_hip_free(v_u); flux_hip_free(txt_c); flux_hip_free(txt_u);
+    flux_hip_session_free(s);
     return out;
 }
 

@@ -271,12 +271,27 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
     if (np == 0) return 1;
     g.N = N; g.K = K; g.lda = lda; g.ldw = ldw; g.ldc = ldc; g.w_row0 = w_row0; g.w_row1 = w_row1;
 
-    /* Largest tile that still yields a few hundred workgroups for the 256 CUs. */
-    int tile;
-    long total_rows = (long)g.M[0] + g.M[1];
-    if ((N % 256) == 0 && ((total_rows + 255) / 256) * (N / 256) >= 384) tile = 2;
-    else if (((total_rows + 127) / 128) * (N / 128) >= 256 && maxm > 64) tile = 1;
-    else tile = 0;
+    /* Pick the tile with the best estimated throughput: per-tile efficiency (measured on
+     * large shapes) times how evenly the workgroups fill 256 CUs at that tile's occupancy. */
+    int tile = 0;
+    {
+        static const int bm[3] = {64, 128, 256}, bn[3] = {128, 128, 256}, occ[3] = {3, 2, 1};
+        static const double eff[3] = {0.5, 0.8, 1.0};
+        double best = -1.0;
+        for (int t = 0; t < 3; t++) {
+            if (N % bn[t]) continue;
+            long blocks = 0;
+            for (int i = 0; i < np; i++) blocks += (g.M[i] + bm[t] - 1) / bm[t];
+            blocks *= N / bn[t];
+            long slots = 256L * occ[t];
+            long rounds = (blocks + slots - 1) / slots;
+            /* rows of partially filled tiles are wasted work */
+            double fill = 0.0, padded = 0.0;
+            for (int i = 0; i < np; i++) { fill += g.M[i]; padded += (double)((g.M[i] + bm[t] - 1) / bm[t]) * bm[t]; }
+            double score = eff[t] * (fill / padded) * (double)blocks / (double)(rounds * slots);
+            if (score > best) { best = score; tile = t; }
+        }
+    }
     if (g_force_tile >= 0) tile = g_force_tile;
     if (tile == 2 && (N % 256)) tile = 1;
 

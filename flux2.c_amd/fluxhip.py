@@ -93,6 +93,11 @@ def lib():
     L.flux_sample_euler_cfg_with_refs.restype = vp
     L.flux_sample_euler_cfg_with_refs.argtypes = [vp, vp, vp, c_i, c_i, c_i, c_i, vp, c_i, c_i, c_i,
                                                   vp, c_i, vp, c_i, c_f, vp, c_i, vp]
+    L.flux_hip_session_begin.restype = vp
+    L.flux_hip_session_begin.argtypes = [vp, vp, c_i, c_i, c_i, vp, c_i, vp, c_i, vp, c_i, c_f, vp, c_i]
+    L.flux_hip_session_step.argtypes = [vp, c_i, vp]
+    L.flux_hip_session_read_latent.argtypes = [vp, vp]
+    L.flux_hip_session_free.argtypes = [vp]
     for n in ("flux_linear_schedule", "flux_power_schedule", "flux_official_schedule"):
         getattr(L, n).restype = vp
     L.flux_linear_schedule.argtypes = [c_i]
@@ -262,6 +267,51 @@ class Transformer:
             raise FluxHipError(f"sample: {L.flux_hip_last_error().decode()}")
         out = _take_host(p, (self.cfg.channels, h, w))
         return (out, tr) if trace else out
+
+
+class Session:
+    """A device-resident sampling run: begin uploads everything, step() only queues kernels."""
+
+    def __init__(self, model, z, h, w, txt, schedule, refs=None, txt_uncond=None, guidance=0.0):
+        z, txt, schedule = _f32(z), _f32(txt), _f32(schedule)
+        self.model, self.h, self.w = model, h, w
+        self.steps = len(schedule) - 1
+        arr, nr, keep = _refs_array(refs)
+        tu = _f32(txt_uncond) if txt_uncond is not None else None
+        L = lib()
+        self.s = L.flux_hip_session_begin(model.h, z.ctypes.data, model.cfg.channels, h, w, arr, nr,
+                                          txt.ctypes.data, txt.shape[0],
+                                          tu.ctypes.data if tu is not None else None,
+                                          tu.shape[0] if tu is not None else 0, guidance,
+                                          schedule.ctypes.data, self.steps)
+        if not self.s:
+            raise FluxHipError(f"session_begin: {L.flux_hip_last_error().decode()}")
+
+    def step(self, i):
+        check(lib().flux_hip_session_step(self.s, i, None), "session_step")
+
+    def latent(self):
+        out = np.empty((self.model.cfg.channels, self.h, self.w), np.float32)
+        check(lib().flux_hip_session_read_latent(self.s, out.ctypes.data), "session_read_latent")
+        return out
+
+    def close(self):
+        if getattr(self, "s", None):
+            lib().flux_hip_session_free(self.s)
+            self.s = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def stage_timing():
+    """Device milliseconds of the last collected run: (double, single, final, total)."""
+    L = lib()
+    return tuple(ctypes.c_double.in_dll(L, "flux_timing_transformer_" + n).value
+                 for n in ("double", "single", "final", "total"))
 
 
 def schedule(kind, n, arg=None):

@@ -225,6 +225,23 @@ float *flux_hip_sample_traced(void *transformer, const float *z, int channels, i
                               const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
                               const float *schedule, int num_steps, float *v_trace);
 
+/*
+ * The sampling loop in pieces, for callers that drive or time the steps themselves. begin()
+ * uploads latent, text and reference tokens and computes every step's modulation vectors;
+ * step() only queues kernels (no host round trip unless v_trace is given, which receives that
+ * step's velocity or, under CFG, the unconditional then the conditional one); read_latent()
+ * waits and copies the current latent out. The samplers above are built from these.
+ */
+typedef struct flux_hip_session flux_hip_session;
+flux_hip_session *flux_hip_session_begin(void *transformer, const float *z, int channels, int h, int w,
+                                         const flux_ref_t *refs, int num_refs,
+                                         const float *text_emb_cond, int text_seq_cond,
+                                         const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
+                                         const float *schedule, int num_steps);
+int flux_hip_session_step(flux_hip_session *s, int step, float *v_trace);
+int flux_hip_session_read_latent(flux_hip_session *s, float *z_out);
+void flux_hip_session_free(flux_hip_session *s);
+
 /* Per-stage device time of the last sampling call in milliseconds (role of the
  * flux_timing_transformer_* counters, flux_sample.c:29-39). */
 extern double flux_timing_transformer_total;
