@@ -30,6 +30,10 @@ import fluxhip  # noqa: E402
 from model_spec import KLEIN_4B, FluxConfig, tensor_shapes, make_weights, normal_f32, normal_bf16, flops_per_forward  # noqa: E402
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA peak (datasheet)
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# `bench.py --calibrate` (profiles/gemm_swiglu_c4_traffic.txt), scaled by the same counters on a
+# streaming kernel of known size.
+TRAFFIC_BYTES = {"c4": 964_000_000}
 
 # (latent h, w, text tokens, reference-image latents [(h, w, t_offset)], cfg, schedule steps)
 WORKLOADS = {
@@ -114,6 +118,9 @@ def main():
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="launch only a streaming kernel of known size (f32->bf16 over 64 Mi elements: reads 256 MiB, "
+                         "writes 128 MiB) and the dominant GEMM, for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this backend runs the whole model on ONE GPU (no sharding, no collectives); "
@@ -122,6 +129,20 @@ def main():
 
     cfg = KLEIN_4B
     wl = WORKLOADS[args.workload]
+    if args.calibrate:
+        fluxhip.init()
+        n = 64 << 20
+        src = fluxhip.DevBuf(n * 4)
+        dst = fluxhip.DevBuf(n * 2)
+        fluxhip.lib().flux_hip_memset(src.ptr, 0, n * 4)
+        for _ in range(3):
+            fluxhip.check(fluxhip.lib().flux_hip_f32_to_bf16(dst.ptr, src.ptr, n))
+        fluxhip.sync()
+        tokens = wl["h"] * wl["w"] + sum(rh * rw for rh, rw, _ in wl["refs"]) + wl["txt"]
+        ms, fl = time_dominant_kernel(cfg, tokens, launches=5)
+        print(json.dumps({"calibration_copy": {"read_MiB": 256, "write_MiB": 128},
+                          "gemm_ms": ms, "gemm_tflops": fl / ms / 1e9}))
+        return
     K, Wm = args.steps, args.warmup
     h, w, nt = wl["h"], wl["w"], wl["txt"]
     n_target = h * w
@@ -141,6 +162,8 @@ def main():
         sess.step(i)
     fluxhip.sync()
     L = fluxhip.lib()
+    if not args.no_kernel_timing:
+        L.flux_hip_linear_probe(fluxhip.EPI_SWIGLU)   # events around the dominant kernel's launches
     t0 = time.perf_counter()
     L.flux_hip_timer_start()
     for i in range(Wm, Wm + K):
@@ -148,6 +171,10 @@ def main():
     ev_ms = L.flux_hip_timer_stop()      # waits for the last kernel
     fluxhip.sync()
     wall = time.perf_counter() - t0
+    import ctypes
+    k_n, k_ms = ctypes.c_int(0), ctypes.c_float(0.0)
+    L.flux_hip_linear_probe_read(ctypes.byref(k_n), ctypes.byref(k_ms))
+    L.flux_hip_linear_probe(-1)
     zf = sess.latent()
     assert np.isfinite(zf).all(), "latent is not finite"
     stages = fluxhip.stage_timing()
@@ -158,13 +185,17 @@ def main():
     tflops = flops_step / (wall / K) / 1e12
 
     roof = None
-    if not args.no_kernel_timing:
-        k_ms, k_flops = time_dominant_kernel(cfg, n_img + nt)
-        ach = k_flops / (k_ms * 1e-3) / 1e12
+    if not args.no_kernel_timing and k_n.value > 0:
+        # every launch of this kernel in a step has the same cost: [tokens, H] x [2*mlp, H]^T
+        per_ms = k_ms.value / k_n.value
+        k_flops = 2.0 * (n_img + nt) * cfg.hidden * 2 * cfg.mlp
+        ach = k_flops / (per_ms * 1e-3) / 1e12
+        alone_ms, _ = time_dominant_kernel(cfg, n_img + nt)
         roof = {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES.get(args.workload),
                 "kernel": "gemm_kernel<256,256,2,4,SWIGLU> (gate/up projection + SiLU*up)",
-                "ms_per_launch": round(k_ms, 4), "flops_per_launch": k_flops}
+                "launches_timed": k_n.value, "ms_per_launch": round(per_ms, 4), "flops_per_launch": k_flops,
+                "ms_per_launch_back_to_back": round(alone_ms, 4)}
     model.close()
 
     cpu = None
