@@ -8,13 +8,13 @@
  * on q and k. Text and image tokens live in one [text ; image] buffer, so the reference's K/V
  * concatenation (flux_transformer.c:1351-1354) is the buffer itself.
  *
- * Orientation. The kernel computes S^T = K Q^T and O^T = V^T P^T with 32x32x16 bf16 MFMA.
+ * Orientation. The kernel computes S^T = K Q^T and O^T = V^T P^T with bf16 MFMA.
  * In an MFMA accumulator a lane owns one column, so here a lane owns one *query*: the row
- * maximum and row sum of the softmax are reductions over the lane's own registers plus one
- * exchange with lane^32, and the rescale of O is a per-lane scalar. The accumulator of S^T
+ * maximum and row sum of the softmax are reductions over the lane's own registers plus two
+ * lane exchanges, and the rescale of O is a per-lane scalar. The accumulator of S^T
  * also already has the register layout the "B" operand of the second product needs, up to a
- * permutation of keys inside each group of 16, which is applied to the V^T operand instead
- * (two 8-byte LDS reads per fragment).
+ * permutation of keys inside each group of 32, which is applied for free when the K tile is
+ * loaded (the loader picks which key goes to which LDS row).
  */
 #include "common.h"
 #include "../../include/flux_hip.h"
@@ -113,12 +113,23 @@ extern "C" int flux_hip_kv_prepare(void *k_out, void *vt_out, int ld_vt, const v
 }
 
 /* ---------------------------------------------------------------------------------------
- * Flash attention. Workgroup = 4 waves = 128 queries of one head; a wave owns 32 queries and
- * the full head dimension. Keys are walked in tiles of 64 through two LDS stages.
+ * Flash attention. Workgroup = 4 waves = 128 queries of one head; a wave owns 32 queries (two
+ * 16-query MFMA columns) and the full head dimension. Keys are walked in tiles of 64 through
+ * two LDS stages filled by direct global->LDS loads (no register staging).
  *   LDS stage: K tile [64 keys][128 d] (256-byte rows, 16-byte chunks XOR-swizzled by key%16)
  *              V^T tile [128 d][64 keys] (128-byte rows, 16-byte chunks swizzled by (d/2)%8)
+ * MFMA: v_mfma_f32_16x16x32_bf16 (the form that sustains the most under the power limit).
+ *   S^T[key][q]: A = K fragment (lane: key l%16, dims 8(l/16)..+8 of a 32-dim chunk),
+ *                B = Q fragment (lane: query l%16, same dims); accumulator lane: query l%16,
+ *                keys 4(l/16)..+4 of the 16-key block.
+ *   O^T[d][q]:   B = P^T fragment for 32 keys = the accumulators of two 16-row score blocks;
+ *                the K rows are permuted when the tile is loaded so that these are 8
+ *                consecutive keys per lane, and A = V^T fragment is one 16-byte LDS read.
  * --------------------------------------------------------------------------------------- */
 #define ATT_STAGE (64 * 256 + 128 * 128)
+__device__ __forceinline__ int vt_swz(int d) { return ((d >> 1) & 7) ^ ((d & 1) << 2); }
+#define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
+#define LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
 __global__ __launch_bounds__(256, 2) void attention_kernel(bf16 *__restrict__ out, int ldo,
                                                            const bf16 *__restrict__ q, int ldq,
@@ -128,186 +139,244 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(bf16 *__restrict__ ou
                                                            const float *__restrict__ rope_cos,
                                                            const float *__restrict__ rope_sin, float eps) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    const int h = blockIdx.y;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int l31 = lane & 31, lhi = lane >> 5;
+    /* Workgroups are dealt round-robin to the 8 XCDs, each with its own L2. Give every XCD a
+     * contiguous run of (head, query block) pairs, so that all query blocks of a head run on one
+     * XCD and its K / V^T (2.4 MB at 4608 tokens) are fetched from HBM once and then served from
+     * that L2, instead of by all eight. */
+    const int nqb = (seq_q + 127) >> 7;
+    const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    if (logical >= nqb * heads) return;
+    const int h = logical / nqb, qb = logical - h * nqb;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l15 = lane & 15, lq = lane >> 4;
     const int H = heads * HD;
-    const int qrow = blockIdx.x * 128 + wave * 32 + l31;
-    const int qrc = min(qrow, seq_q - 1);
 
-    /* ---- Q fragments: B operand, lane = query, 8 consecutive dims per K-step ---- */
-    bf16x8 qf[8];
-    {
-        const bf16 *qp = q + (size_t)qrc * ldq + h * HD + lhi * 8;
-        float x[8][8];
+    /* ---- tile loader: per-lane global sources (un-swizzled) and per-wave LDS destinations ---- */
+    const int ntiles = (seq_k + 63) >> 6;
+    const bf16 *k_src[4];
+    const bf16 *v_src[4];
+    int k_dst[4], v_dst[4], k_row[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        /* K: one wave instruction covers 4 rows of 256 bytes */
+        int r = wave * 4 + i * 16 + (lane >> 4); /* LDS row */
+        /* LDS row 16 i' + 4 j + e (i' = 2c + b) holds key 32c + 8j + 4b + e of the tile: the
+         * score accumulators of two 16-row blocks then cover 8 consecutive keys per lane */
+        {
+            int ib = r >> 4, jj = (r >> 2) & 3, ee = r & 3;
+            k_row[i] = 32 * (ib >> 1) + 8 * jj + 4 * (ib & 1) + ee;
+        }
+        k_src[i] = k + h * HD + (((lane & 15) ^ (r & 15)) << 3);
+        k_dst[i] = (wave * 4 + i * 16) * 256;
+        /* V^T: one wave instruction covers 8 rows of 128 bytes */
+        int d = wave * 8 + i * 32 + (lane >> 3);
+        v_src[i] = vt + (size_t)(h * HD + d) * ld_vt + (((lane & 7) ^ vt_swz(d)) << 3);
+        v_dst[i] = (wave * 8 + i * 32) * 128;
+    }
+    /* LDS: K ring = 2 slots of 16 KB at 0 and 16 KB; V^T ring = 2 slots of 16 KB at 32 and 48 KB */
+    auto issue_k = [&](int t) {
+        char *base = smem + (t & 1) * (64 * 256);
+        const int key0 = t * 64;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int r = min(key0 + k_row[i], seq_k - 1);
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(k_src[i] + (size_t)r * H), LDS_PTR(base + k_dst[i]), 16, 0, 0);
+        }
+    };
+    auto issue_v = [&](int t) {
+        char *base = smem + 2 * (64 * 256) + (t & 1) * (128 * 128);
+        const int key0 = t * 64;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(v_src[i] + key0), LDS_PTR(base + v_dst[i]), 16, 0, 0);
+    };
+    issue_k(0);
+    issue_v(0);
+    if (ntiles > 1) issue_k(1);
+
+    /* ---- Q fragments (B operand), with RMSNorm * weight, RoPE and the softmax scale ---- */
+    bf16x8 qf[2][4];
+    int qrow[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        qrow[t] = qb * 128 + wave * 32 + t * 16 + l15;
+        const int qrc = min(qrow[t], seq_q - 1);
+        const bf16 *qp = q + (size_t)qrc * ldq + h * HD + lq * 8;
+        float x[4][8];
         float ss = 0.0f;
 #pragma unroll
-        for (int kk = 0; kk < 8; kk++) {
-            bf16x8 v = *(const bf16x8 *)(qp + kk * 16);
+        for (int kk = 0; kk < 4; kk++) {
+            bf16x8 v = *(const bf16x8 *)(qp + kk * 32);
 #pragma unroll
             for (int e = 0; e < 8; e++) { x[kk][e] = (float)v[e]; ss += x[kk][e] * x[kk][e]; }
         }
+        ss += __shfl_xor(ss, 16, 64);
         ss += __shfl_xor(ss, 32, 64);
-        /* fold 1/sqrt(128) and log2(e) into q so that scores are base-2 logits */
         const float inv = 1.0f / sqrtf(ss * (1.0f / HD) + eps);
+        /* 1/sqrt(128) and log2(e) folded into q: scores come out as base-2 logits */
         const float fold = 0.08838834764831845f * 1.44269504088896341f;
-        const float *w = (qrc < split ? q_w0 : q_w1) + lhi * 8;
-        const float *cs = rope_cos + (size_t)qrc * HD + lhi * 8;
-        const float *sn = rope_sin + (size_t)qrc * HD + lhi * 8;
+        const float *w = (qrc < split ? q_w0 : q_w1) + lq * 8;
+        const float *cs = rope_cos + (size_t)qrc * HD + lq * 8;
+        const float *sn = rope_sin + (size_t)qrc * HD + lq * 8;
 #pragma unroll
-        for (int kk = 0; kk < 8; kk++) {
-            f32x4 w0 = *(const f32x4 *)(w + kk * 16), w1 = *(const f32x4 *)(w + kk * 16 + 4);
-            f32x4 c0 = *(const f32x4 *)(cs + kk * 16), c1 = *(const f32x4 *)(cs + kk * 16 + 4);
-            f32x4 s0 = *(const f32x4 *)(sn + kk * 16), s1 = *(const f32x4 *)(sn + kk * 16 + 4);
+        for (int kk = 0; kk < 4; kk++) {
+            f32x4 w0 = *(const f32x4 *)(w + kk * 32), w1 = *(const f32x4 *)(w + kk * 32 + 4);
+            f32x4 c0 = *(const f32x4 *)(cs + kk * 32), c1 = *(const f32x4 *)(cs + kk * 32 + 4);
+            f32x4 s0 = *(const f32x4 *)(sn + kk * 32), s1 = *(const f32x4 *)(sn + kk * 32 + 4);
             float wv[8] = {w0[0], w0[1], w0[2], w0[3], w1[0], w1[1], w1[2], w1[3]};
             float cv[8] = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
             float sv[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
 #pragma unroll
             for (int e = 0; e < 8; e += 2) {
                 float a = x[kk][e] * inv * wv[e], b = x[kk][e + 1] * inv * wv[e + 1];
-                /* round to bf16 first (what the key side does), then apply the folded scale */
-                float ra = a * cv[e] - b * sv[e], rb = b * cv[e] + a * sv[e];
-                qf[kk][e] = (bf16)(ra * fold);
-                qf[kk][e + 1] = (bf16)(rb * fold);
+                qf[t][kk][e] = (bf16)((a * cv[e] - b * sv[e]) * fold);
+                qf[t][kk][e + 1] = (bf16)((b * cv[e] + a * sv[e]) * fold);
             }
         }
     }
 
-    /* ---- tile loader mapping ---- */
-    const int kc = tid & 15, kr = tid >> 4;  /* K: 16 chunks per row, rows kr + 16 i */
-    const int vc = tid & 7, vr = tid >> 3;   /* V^T: 8 chunks per row, rows vr + 32 i */
-    const bf16 *kbase = k + h * HD + kc * 8;
-    const bf16 *vbase = vt + (size_t)(h * HD) * ld_vt + vc * 8;
-    int k_lds[4], v_lds[4];
+    f32x4 o_acc[8][2];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        int r = kr + i * 16;
-        k_lds[i] = r * 256 + ((kc ^ (r & 15)) << 4);
-        int d = vr + i * 32;
-        v_lds[i] = 64 * 256 + d * 128 + ((vc ^ ((d >> 1) & 7)) << 4);
-    }
-    const int ntiles = (seq_k + 63) >> 6;
-    bf16x8 rk[4], rv[4];
-    auto load_tile = [&](int t) {
-        const int key0 = t * 64;
+    for (int i = 0; i < 8; i++)
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            int r = min(key0 + kr + i * 16, seq_k - 1);
-            rk[i] = *(const bf16x8 *)(kbase + (size_t)r * H);
-            rv[i] = *(const bf16x8 *)(vbase + (size_t)(vr + i * 32) * ld_vt + key0);
-        }
-    };
-    auto store_tile = [&](int stage) {
-        char *s = smem + stage * ATT_STAGE;
+        for (int t = 0; t < 2; t++)
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            *(bf16x8 *)(s + k_lds[i]) = rk[i];
-            *(bf16x8 *)(s + v_lds[i]) = rv[i];
-        }
-    };
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
+            for (int e = 0; e < 4; e++) o_acc[i][t][e] = 0.0f;
+    float m_run[2] = {-1e30f, -1e30f}, l_run[2] = {0.0f, 0.0f};
 
-    f32x16 o_acc[4];
+    const int kswz = l15; /* key % 16 of the K rows this lane reads */
+    /* S^T for the 64 keys of tile t against this wave's 32 queries */
+    auto scores = [&](int t, f32x4 (&s_acc)[4][2]) {
+        const char *kt = smem + (t & 1) * (64 * 256);
+        const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+        for (int kk = 0; kk < 4; kk++) {
 #pragma unroll
-        for (int e = 0; e < 16; e++) o_acc[i][e] = 0.0f;
-    float m_run = -1e30f, l_run = 0.0f;
-
-    const int kswz = l31 & 15;
-    for (int t = 0; t < ntiles; t++) {
-        const int cur = t & 1;
-        if (t + 1 < ntiles) load_tile(t + 1);
-        const char *st = smem + cur * ATT_STAGE;
-
-        /* S^T[keys][queries] for 64 keys */
-        f32x16 s_acc[2];
+            for (int i = 0; i < 4; i++) {
+                bf16x8 kf = *(const bf16x8 *)(kt + (i * 16 + l15) * 256 + (((kk * 4 + lq) ^ kswz) << 4));
 #pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) s_acc[i][e] = 0.0f;
-#pragma unroll
-        for (int kk = 0; kk < 8; kk++) {
-#pragma unroll
-            for (int i = 0; i < 2; i++) {
-                bf16x8 kf = *(const bf16x8 *)(st + (i * 32 + l31) * 256 + (((kk * 2 + lhi) ^ kswz) << 4));
-                s_acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s_acc[i], 0, 0, 0);
+                for (int u = 0; u < 2; u++)
+                    s_acc[i][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[u][kk], kk == 0 ? zero : s_acc[i][u], 0, 0, 0);
             }
         }
+    };
+
+    /* Software pipeline inside the wave: the score MFMAs of tile t+1 are issued before the
+     * softmax of tile t, so the matrix pipe works while the VALU does exp/max/sum. K and V^T
+     * therefore live in separate 2-slot rings one tile apart: iteration t reads K(t+1) and
+     * V(t) while K(t+2) and V(t+1) are in flight. */
+    /* One key tile: issue the next loads and the next tile's score MFMAs, then softmax and
+     * P V of the current one. */
+    auto step = [&](int t, f32x4 (&s_cur)[4][2], f32x4 (&s_nxt)[4][2]) {
+        __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): K(t+1) and V(t) parts of this wave are in LDS */
+        __syncthreads();
+        if (t + 1 < ntiles) issue_v(t + 1);
+        if (t + 2 < ntiles) issue_k(t + 2);
+        if (t + 1 < ntiles) scores(t + 1, s_nxt);
+
         if (t == ntiles - 1 && (seq_k & 63)) {
             const int key0 = t * 64;
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int e = 0; e < 16; e++) {
-                    int key = key0 + i * 32 + (e >> 2) * 8 + lhi * 4 + (e & 3);
-                    if (key >= seq_k) s_acc[i][e] = -1e30f;
+                for (int e = 0; e < 4; e++)
+                    if (key0 + 32 * (i >> 1) + 8 * lq + 4 * (i & 1) + e >= seq_k) { s_cur[i][0][e] = -1e30f; s_cur[i][1][e] = -1e30f; }
+        }
+        /* Online softmax; a query's scores sit in lanes l, l^16, l^32, l^48. The reference
+         * maximum is only moved when the true maximum exceeds it by more than 2^8 (scores are
+         * base-2 logits): until then p = 2^(s - m_ref) <= 256 is exact enough in fp32/bf16, the
+         * final division by the row sum cancels the choice of m_ref, and the rescale of O -
+         * 64 multiplies per lane - is skipped for almost every tile. */
+        bool grow = false;
+        float m_new[2];
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            float mx = fmaxf(fmaxf(s_cur[0][u][0], s_cur[0][u][1]), fmaxf(s_cur[0][u][2], s_cur[0][u][3]));
+#pragma unroll
+            for (int i = 1; i < 4; i++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) mx = fmaxf(mx, s_cur[i][u][e]);
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            m_new[u] = mx;
+            grow = grow || (mx > m_run[u] + 8.0f);
+        }
+        if (__any(grow)) {
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                const float m2 = fmaxf(m_run[u], m_new[u]);
+                const float alpha = fast_exp2(m_run[u] - m2);
+                m_run[u] = m2;
+                l_run[u] *= alpha;
+#pragma unroll
+                for (int i = 0; i < 8; i++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o_acc[i][u][e] *= alpha;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            float psum = 0.0f;
+            const float mref = m_run[u];
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    float p = fast_exp2(s_cur[i][u][e] - mref);
+                    s_cur[i][u][e] = p;
+                    psum += p;
                 }
+            l_run[u] += psum;
         }
-        /* online softmax, one query per lane (shared with lane ^ 32) */
-        float mx = s_acc[0][0];
+        /* O^T += V^T P^T over two 32-key chunks */
+        const char *vtile = smem + 2 * (64 * 256) + (t & 1) * (128 * 128);
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int c = 0; c < 2; c++) {
+            bf16x8 pf[2];
 #pragma unroll
-            for (int e = 0; e < 16; e++) mx = fmaxf(mx, s_acc[i][e]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run, mx);
-        const float alpha = fast_exp2(m_run - m_new);
-        m_run = m_new;
-        float psum = 0.0f;
+            for (int u = 0; u < 2; u++)
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+                for (int e = 0; e < 4; e++) {
+                    pf[u][e] = (bf16)s_cur[2 * c][u][e];
+                    pf[u][4 + e] = (bf16)s_cur[2 * c + 1][u][e];
+                }
 #pragma unroll
-            for (int e = 0; e < 16; e++) {
-                float p = fast_exp2(s_acc[i][e] - m_new);
-                s_acc[i][e] = p;
-                psum += p;
+            for (int dt = 0; dt < 8; dt++) {
+                const int d = dt * 16 + l15;
+                bf16x8 vf = *(const bf16x8 *)(vtile + d * 128 + (((4 * c + lq) ^ vt_swz(d)) << 4));
+#pragma unroll
+                for (int u = 0; u < 2; u++)
+                    o_acc[dt][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], o_acc[dt][u], 0, 0, 0);
             }
-        l_run = l_run * alpha + psum;
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) o_acc[i][e] *= alpha;
+        }
+    };
 
-        /* O^T += V^T P^T. Key slot s of lane group j in 16-key chunk c is key
-         * 16c + 8(s/4) + 4j + s%4, on both operands. */
-        bf16x8 pf[4];
-#pragma unroll
-        for (int c = 0; c < 4; c++)
-#pragma unroll
-            for (int s = 0; s < 8; s++) pf[c][s] = (bf16)s_acc[c >> 1][(c & 1) * 8 + s];
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++) {
-            const int d = dt * 32 + l31;
-            const char *vrow = st + 64 * 256 + d * 128 + lhi * 8;
-            const int vs = (d >> 1) & 7;
-#pragma unroll
-            for (int c = 0; c < 4; c++) {
-                bf16x4 lo = *(const bf16x4 *)(vrow + (((c * 2) ^ vs) << 4));
-                bf16x4 hi = *(const bf16x4 *)(vrow + (((c * 2 + 1) ^ vs) << 4));
-                bf16x8 vf = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                o_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[c], o_acc[dt], 0, 0, 0);
-            }
-        }
-        if (t + 1 < ntiles) store_tile(cur ^ 1);
-        __syncthreads();
+    f32x4 s_a[4][2], s_b[4][2];
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    scores(0, s_a);
+    for (int t = 0; t < ntiles; t += 2) {
+        step(t, s_a, s_b);
+        if (t + 1 < ntiles) step(t + 1, s_b, s_a);
     }
 
-    l_run += __shfl_xor(l_run, 32, 64);
-    const float inv_l = 1.0f / l_run;
-    if (qrow < seq_q) {
-        bf16 *op = out + (size_t)qrow * ldo + h * HD + lhi * 4;
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++)
+    for (int u = 0; u < 2; u++) {
+        float l = l_run[u];
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
+        const float inv_l = 1.0f / l;
+        if (qrow[u] < seq_q) {
+            bf16 *op = out + (size_t)qrow[u] * ldo + h * HD + lq * 4;
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
+            for (int dt = 0; dt < 8; dt++) {
                 bf16x4 r;
 #pragma unroll
-                for (int e = 0; e < 4; e++) r[e] = (bf16)(o_acc[dt][g * 4 + e] * inv_l);
-                *(bf16x4 *)(op + dt * 32 + g * 8) = r;
+                for (int e = 0; e < 4; e++) r[e] = (bf16)(o_acc[dt][u][e] * inv_l);
+                *(bf16x4 *)(op + dt * 16) = r;
             }
+        }
     }
 }
 
@@ -325,7 +394,8 @@ extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ld
         HIP_OK(hipFuncSetAttribute((const void *)attention_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
         attr_done = true;
     }
-    hipLaunchKernelGGL(attention_kernel, dim3((seq_q + 127) / 128, heads), dim3(256), 2 * ATT_STAGE, flux_hip_stream_handle(),
+    const int blocks = ((seq_q + 127) / 128) * heads;
+    hipLaunchKernelGGL(attention_kernel, dim3((blocks + 7) & ~7), dim3(256), 2 * ATT_STAGE, flux_hip_stream_handle(),
                        (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,
                        heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps);
     HIP_OK(hipGetLastError());
