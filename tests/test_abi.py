@@ -1,0 +1,76 @@
+"""CPU-side checks of the C ABI library: it loads, exports what include/flux_hip.h declares,
+its host-only functions (schedules) match the reference's golden vectors, and it refuses to
+compute without a GPU instead of falling back to anything."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+import fluxhip
+from model_spec import KLEIN_4B, TINY, tensor_shapes, make_weights, write_safetensors, bf16_to_f32, f32_to_bf16, normal_f32
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = fluxhip.lib()
+    hdr = open(os.path.join(ROOT, "include", "flux_hip.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    funcs = set(re.findall(r"\b(flux_[a-z0-9_]+)\s*\(", hdr))
+    assert len(funcs) > 40
+    for name in sorted(funcs):
+        assert hasattr(L, name), name
+    for var in ("flux_timing_transformer_total", "flux_timing_transformer_double", "flux_timing_transformer_single",
+                "flux_timing_transformer_final"):
+        ctypes.c_double.in_dll(L, var)
+    for var in ("flux_substep_callback", "flux_step_callback"):
+        ctypes.c_void_p.in_dll(L, var)
+    ctypes.c_int.in_dll(L, "flux_verbose")
+
+
+def test_schedules_match_reference_golden(golden_dir):
+    g = np.load(os.path.join(golden_dir, "ops.npz"))
+    for n in (1, 4, 7):
+        np.testing.assert_allclose(fluxhip.schedule("linear", n), g[f"sched_linear_{n}"], atol=1e-7)
+    np.testing.assert_allclose(fluxhip.schedule("power", 5, 2.0), g["sched_power_5_2"], atol=1e-7)
+    for n, sl in ((4, 256), (4, 1024), (4, 4096), (50, 1024), (4, 5000), (1, 16), (28, 4300)):
+        np.testing.assert_allclose(fluxhip.schedule("official", n, sl), g[f"sched_official_{n}_{sl}"], atol=6e-7)   # a few fp32 ulp: expf/powf vs the -ffast-math build
+
+
+def test_no_cpu_fallback():
+    """Without a GPU nothing computes: init fails with a message and model creation raises."""
+    L = fluxhip.lib()
+    if L.flux_hip_init():
+        pytest.skip("a GPU is present")
+    assert b"HIP device" in L.flux_hip_last_error() or L.flux_hip_last_error()
+    assert not L.flux_hip_available()
+    assert not L.flux_hip_malloc(16)
+    with pytest.raises(fluxhip.FluxHipError):
+        fluxhip.Transformer(TINY)
+
+
+def test_model_spec_and_synthetic_tensors(tmp_path):
+    shapes = tensor_shapes(KLEIN_4B)
+    assert len(shapes) == 169                                  # what the reference loader asks for
+    assert sum(int(np.prod(s)) for s in shapes.values()) == 3_875_544_576
+    W = make_weights(TINY, 42, 0.02, "sharp")
+    W2 = make_weights(TINY, 42, 0.02, "sharp", only=["proj_out.weight"])
+    assert np.array_equal(W["proj_out.weight"], W2["proj_out.weight"])      # streams are per tensor
+    w = bf16_to_f32(W["context_embedder.weight"])
+    assert abs(w.std() - 0.02) < 5e-4 and abs(w.mean()) < 5e-4
+    assert np.all(bf16_to_f32(W["transformer_blocks.0.attn.norm_q.weight"]) == 1.0)
+    x = normal_f32((1000,), 1, 1)
+    assert np.array_equal(f32_to_bf16(bf16_to_f32(f32_to_bf16(x))), f32_to_bf16(x))
+    # round to nearest even on the bf16 boundary
+    edge = np.array([1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8], np.float32)
+    assert list(f32_to_bf16(edge)) == [0x3F80, 0x3F82]
+    p = tmp_path / "t.safetensors"
+    write_safetensors(str(p), W)
+    raw = open(p, "rb").read()
+    hlen = int.from_bytes(raw[:8], "little")
+    import json
+    meta = json.loads(raw[8:8 + hlen])
+    assert meta["proj_out.weight"]["dtype"] == "BF16" and meta["proj_out.weight"]["shape"] == [128, 256]
+    assert len(raw) == 8 + hlen + sum(a.size * 2 for a in W.values())
