@@ -1,0 +1,84 @@
+"""Parity at the benchmark's real shapes: FLUX.2-klein-4B architecture, random-init bf16 weights
+N(0, 0.02) seed 42, against the fp32 CPU oracle on the same inputs.
+
+c2: 256 image + 512 text tokens, full 4-step distilled schedule (velocities + final latent)
+c3: 1024 + 512 tokens, first step of the 4-step schedule
+c4: 4096 + 512 tokens (headline shape), first step
+c5: CFG + one reference image, (1024 + 1024) + 512 tokens, first step = two forwards
+The oracle needs seconds to a minute per forward at these sizes, so c3-c5 check one step; the
+remaining steps run the same kernels at the same shapes with other modulation vectors.
+Gates: velocity rel-L2 <= 2e-2, cosine >= 0.999, latent PSNR >= 35 dB.
+"""
+import numpy as np
+import pytest
+
+from metrics import rel_l2, cosine, psnr
+from model_spec import KLEIN_4B, tensor_shapes, make_weights, normal_f32
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def models(oracle_mod):
+    import fluxhip
+    fluxhip.init()
+    fluxhip.lib().flux_hip_linear_force_tile(-1)
+    cfg = KLEIN_4B
+    hip_m = fluxhip.Transformer(cfg)
+    ora = oracle_mod.Oracle(cfg, {})
+    for name in tensor_shapes(cfg):                      # one tensor at a time on the host
+        a = make_weights(cfg, 42, 0.02, "literal", only=[name])[name]
+        hip_m.set_tensor(name, a)
+        rc = oracle_mod.lib().fo_model_set_bf16(ora.h, name.encode(), a.ctypes.data, a.size)
+        assert rc == 0, name
+    yield fluxhip, hip_m, ora
+    hip_m.close()
+    ora.close()
+
+
+def check(vg, vo, what):
+    r, c = rel_l2(vg, vo), cosine(vg, vo)
+    print(f"{what}: rel_l2={r:.3e} cos={c:.6f}", flush=True)
+    assert r <= 2e-2 and c >= 0.999, (what, r, c)
+
+
+def test_c2_full_schedule(models):
+    fluxhip, m, o = models
+    h = w = 16
+    z = normal_f32((128, h, w), 123, 1)
+    txt = normal_f32((512, 7680), 123, 2)
+    s = fluxhip.schedule("official", 4, h * w)
+    zo, vo = o.sample_euler(z, h, w, txt, s, trace=True)
+    zg, vg = m.sample(z, h, w, txt, s, trace=True)
+    for i in range(4):
+        check(vg[i], vo[i], f"c2 step {i}")
+    p = psnr(zg, zo)
+    print(f"c2 final latent PSNR {p:.1f} dB", flush=True)
+    assert p >= 35.0
+
+
+@pytest.mark.parametrize("name,h,w", [("c3", 32, 32), ("c4", 64, 64)])
+def test_first_step(models, name, h, w):
+    fluxhip, m, o = models
+    z = normal_f32((128, h, w), 123, 1)
+    txt = normal_f32((512, 7680), 123, 2)
+    s = fluxhip.schedule("official", 4, h * w)[:2]
+    zo, vo = o.sample_euler(z, h, w, txt, s, trace=True)
+    zg, vg = m.sample(z, h, w, txt, s, trace=True)
+    check(vg[0], vo[0], f"{name} step 0")
+    assert psnr(zg, zo) >= 35.0
+
+
+def test_c5_cfg_with_reference_first_step(models):
+    fluxhip, m, o = models
+    h = w = 32
+    z = normal_f32((128, h, w), 123, 1)
+    txt = normal_f32((512, 7680), 123, 2)
+    txt_u = normal_f32((512, 7680), 123, 3)
+    ref = (normal_f32((128, h, w), 123, 10), h, w, 10)
+    s = fluxhip.schedule("official", 50, h * w)[:2]
+    zo, vo = o.sample_euler_cfg(z, h, w, txt, txt_u, 4.0, s, refs=[ref], trace=True)
+    zg, vg = m.sample(z, h, w, txt, s, refs=[ref], txt_uncond=txt_u, guidance=4.0, trace=True)
+    check(vg[0], vo[0], "c5 uncond")
+    check(vg[1], vo[1], "c5 cond")
+    assert psnr(zg, zo) >= 35.0
