@@ -34,7 +34,15 @@ struct GemmArgs {
     int M[2];
     int mtiles0, mtiles, ntiles, total_tiles;
     int N, K, lda, ldw, ldc, w_row0, w_row1;
+    /* split-K: workgroup (tile, s) multiplies K-steps [s*kt_per, (s+1)*kt_per) and stores its
+     * fp32 partial tile into ws[s][moff[part] + m][n]; a second kernel sums the slices */
+    int ksplit, kt_per;
+    float *ws;
+    int moff[2], ws_rows;
 };
+
+/* internal epilogue: fp32 partial sums of one K slice (see split-K above) */
+#define EPI_PARTIAL 5
 
 __device__ __forceinline__ int lds_swz(int r) { return ((r >> 1) & 7) ^ ((r & 1) << 2); }
 
@@ -60,7 +68,9 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
     int nb = gridDim.x;
     int per_xcd = nb >> 3;
     int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (logical >= g.total_tiles) return;
+    if (logical >= g.total_tiles * g.ksplit) return;
+    const int ks = logical / g.total_tiles;
+    logical -= ks * g.total_tiles;
     int per_group = GROUP_M * g.ntiles;
     int grp = logical / per_group;
     int first_m = grp * GROUP_M;
@@ -116,7 +126,9 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
         for (int i = 0; i < PB; i++)
             __builtin_amdgcn_global_load_lds(GLOBAL_PTR(b_ptr[i] + kt * 64), LDS_PTR(base + b_lds[i]), 16, 0, 0);
     };
-    issue(0, 0);
+    const int kt_begin = ks * g.kt_per;
+    const int KT = min(g.K >> 6, kt_begin + g.kt_per) - kt_begin;
+    issue(kt_begin, 0);
 
     f32x4 acc[TN][TM];
 #pragma unroll
@@ -131,14 +143,13 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
     const int a_frag = (wm * WM + l15) * 128;
     const int b_frag = BM * 128 + (wn * WN + l15) * 128;
 
-    const int KT = g.K >> 6;
     for (int kt = 0; kt < KT; kt++) {
         const int cur = kt & 1;
         /* stage `cur` has landed for this wave; after the barrier it has for all, and everyone
          * is done reading the other stage, which can then be refilled */
         WAIT_VMCNT0();
         __syncthreads();
-        if (kt + 1 < KT) issue(kt + 1, cur ^ 1);
+        if (kt + 1 < KT) issue(kt_begin + kt + 1, cur ^ 1);
         const char *st = smem + cur * STAGE;
 #pragma unroll
         for (int kk = 0; kk < 2; kk++) {
@@ -181,6 +192,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
 #pragma unroll
                     for (int e = 0; e < 4; e++) o[e] = (bf16)acc[i][j][e];
                     *(bf16x4 *)((bf16 *)g.C[prob] + (size_t)m * ldc + n) = o;
+                } else if (EPI == EPI_PARTIAL) {
+                    *(f32x4 *)(g.ws + ((size_t)ks * g.ws_rows + g.moff[prob] + m) * g.N + n) = acc[i][j];
                 } else if (EPI == FLUX_HIP_EPI_F32) {
                     *(f32x4 *)((float *)g.C[prob] + (size_t)m * ldc + n) = acc[i][j];
                 } else if (EPI == FLUX_HIP_EPI_F32_T) {
@@ -216,7 +229,7 @@ static int launch_cfg(GemmArgs &g) {
     g.mtiles = g.mtiles0 + mt1;
     g.ntiles = g.N / BN;
     g.total_tiles = g.mtiles * g.ntiles;
-    int grid = (g.total_tiles + 7) & ~7;
+    int grid = (g.total_tiles * g.ksplit + 7) & ~7;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(T), LDS, flux_hip_stream_handle(), g);
     HIP_OK(hipGetLastError());
     return 1;
@@ -227,12 +240,52 @@ static int launch_epi(GemmArgs &g, int tile) {
     switch (tile) {
         case 2: return launch_cfg<256, 256, 2, 4, EPI>(g);
         case 1: return launch_cfg<128, 128, 2, 2, EPI>(g);
+        case 3: return launch_cfg<64, 64, 2, 2, EPI>(g);
         default: return launch_cfg<64, 128, 2, 2, EPI>(g);
     }
 }
 
+/* x[m, n] += gate[n] * sum_s ws[s][moff + m][n]: second pass of a split-K residual GEMM
+ * (same arithmetic as gated_add, flux_transformer.c:90-97, on the summed product). */
+__global__ __launch_bounds__(256) void splitk_resid_kernel(GemmArgs g) {
+    const int n4 = g.N >> 2;
+    const size_t total = (size_t)(g.M[0] + g.M[1]) * n4;
+    size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= total) return;
+    int row = (int)(idx / n4), n = (int)(idx - (size_t)row * n4) << 2;
+    int prob = row >= g.M[0] ? 1 : 0;
+    int m = prob ? row - g.M[0] : row;
+    f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int s = 0; s < g.ksplit; s++) {
+        f32x4 v = *(const f32x4 *)(g.ws + ((size_t)s * g.ws_rows + g.moff[prob] + m) * g.N + n);
+#pragma unroll
+        for (int e = 0; e < 4; e++) sum[e] += v[e];
+    }
+    float *p = (float *)g.C[prob] + (size_t)m * g.ldc + n;
+    f32x4 x = *(f32x4 *)p;
+    f32x4 gt = *(const f32x4 *)(g.gate[prob] + n);
+#pragma unroll
+    for (int e = 0; e < 4; e++) x[e] += gt[e] * sum[e];
+    *(f32x4 *)p = x;
+}
+
+static float *g_ws = nullptr;
+static size_t g_ws_bytes = 0;
+static int ensure_ws(size_t bytes) {
+    if (bytes <= g_ws_bytes) return 1;
+    HIP_OK(hipStreamSynchronize(flux_hip_stream_handle()));
+    if (g_ws) hipFree(g_ws);
+    g_ws = nullptr;
+    g_ws_bytes = 0;
+    HIP_OK(hipMalloc((void **)&g_ws, bytes));
+    g_ws_bytes = bytes;
+    return 1;
+}
+
 static int g_force_tile = -1;
+static int g_splitk_enabled = 1;
 extern "C" void flux_hip_linear_force_tile(int tile) { g_force_tile = tile; }
+extern "C" void flux_hip_linear_enable_splitk(int on) { g_splitk_enabled = on; }
 
 /* Launch probe: HIP events around every launch with one chosen epilogue, so a benchmark can
  * read that kernel's average duration inside its timed region. */
@@ -303,29 +356,57 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
     if (np == 0) return 1;
     g.N = N; g.K = K; g.lda = lda; g.ldw = ldw; g.ldc = ldc; g.w_row0 = w_row0; g.w_row1 = w_row1;
 
-    /* Pick the tile with the best estimated throughput: per-tile efficiency (measured on
-     * large shapes) times how evenly the workgroups fill 256 CUs at that tile's occupancy. */
-    int tile = 0;
+    /* Choose tile and K split with a small cost model: workgroups run in rounds over
+     * 256 CUs x occupancy; a workgroup's time is its FLOPs at the tile's measured rate plus a
+     * fixed prologue/epilogue cost; the launch cannot beat the time to stream its operands,
+     * which depends on how many bytes the resident workgroups keep in flight. */
+    static const int bm[4] = {64, 128, 256, 64}, bn[4] = {128, 128, 256, 64}, occ[4] = {3, 2, 1, 4};
+    static const double rate[4] = {2.0e12, 2.9e12, 4.1e12, 1.5e12}; /* FLOP/s of one CU running this tile */
+    const int kt_total = K >> 6;
+    int tile = 1, best_split = 1;
     {
-        static const int bm[3] = {64, 128, 256}, bn[3] = {128, 128, 256}, occ[3] = {3, 2, 1};
-        static const double eff[3] = {0.5, 0.8, 1.0};
-        double best = -1.0;
-        for (int t = 0; t < 3; t++) {
+        double best = 1e30;
+        static const int splits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
+        const bool can_split = epilogue == FLUX_HIP_EPI_RESID && g_splitk_enabled;
+        double rows = 0.0;
+        for (int i = 0; i < np; i++) rows += g.M[i];
+        for (int t = 0; t < 4; t++) {
             if (N % bn[t]) continue;
-            long blocks = 0;
-            for (int i = 0; i < np; i++) blocks += (g.M[i] + bm[t] - 1) / bm[t];
-            blocks *= N / bn[t];
-            long slots = 256L * occ[t];
-            long rounds = (blocks + slots - 1) / slots;
-            /* rows of partially filled tiles are wasted work */
-            double fill = 0.0, padded = 0.0;
-            for (int i = 0; i < np; i++) { fill += g.M[i]; padded += (double)((g.M[i] + bm[t] - 1) / bm[t]) * bm[t]; }
-            double score = eff[t] * (fill / padded) * (double)blocks / (double)(rounds * slots);
-            if (score > best) { best = score; tile = t; }
+            if (g_force_tile >= 0 && t != g_force_tile) continue;
+            long tiles = 0;
+            for (int i = 0; i < np; i++) tiles += (g.M[i] + bm[t] - 1) / bm[t];
+            tiles *= N / bn[t];
+            for (int si = 0; si < 10; si++) {
+                const int sp = splits[si];
+                if (sp > 1 && (!can_split || kt_total / sp < 4)) break;
+                const int per = (kt_total + sp - 1) / sp;
+                const long blocks = tiles * ((kt_total + per - 1) / per);
+                const long slots = 256L * occ[t];
+                const long rounds = (blocks + slots - 1) / slots;
+                const long resident = blocks < slots ? blocks : slots;
+                const long per_cu = (resident + 255) / 256;          /* workgroups sharing one CU */
+                const double t_block = 2.0 * bm[t] * bn[t] * 64.0 * per / (rate[t] / per_cu) + 2.5e-6;
+                double t_compute = rounds * t_block;
+                const double bytes = (rows + N) * (double)K * 2.0;
+                double bw = 5.5e12 * (double)(resident * (bm[t] + bn[t]) * 128) / 12.0e6;
+                if (bw > 5.5e12) bw = 5.5e12;
+                double est = t_compute > bytes / bw ? t_compute : bytes / bw;
+                if (sp > 1) est += 3.0e-6 + (sp + 2.0) * rows * N * 4.0 / 4.0e12;
+                if (est < best) { best = est; tile = t; best_split = sp; }
+            }
         }
     }
-    if (g_force_tile >= 0) tile = g_force_tile;
-    if (tile == 2 && (N % 256)) tile = 1;
+    g.ksplit = 1;
+    g.kt_per = kt_total;
+    if (best_split > 1) {
+        g.kt_per = (kt_total + best_split - 1) / best_split;
+        g.ksplit = (kt_total + g.kt_per - 1) / g.kt_per;
+        g.moff[0] = 0;
+        g.moff[1] = g.M[0];
+        g.ws_rows = g.M[0] + g.M[1];
+        if (!ensure_ws((size_t)g.ksplit * g.ws_rows * N * sizeof(float))) return 0;
+        g.ws = g_ws;
+    }
 
     const int slot = probe_slot(epilogue);
     if (slot >= 0) hipEventRecord(g_probe_ev[slot][0], flux_hip_stream_handle());
@@ -334,7 +415,19 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
         case FLUX_HIP_EPI_BF16: ok = launch_epi<FLUX_HIP_EPI_BF16>(g, tile); break;
         case FLUX_HIP_EPI_F32: ok = launch_epi<FLUX_HIP_EPI_F32>(g, tile); break;
         case FLUX_HIP_EPI_F32_T: ok = launch_epi<FLUX_HIP_EPI_F32_T>(g, tile); break;
-        case FLUX_HIP_EPI_RESID: ok = launch_epi<FLUX_HIP_EPI_RESID>(g, tile); break;
+        case FLUX_HIP_EPI_RESID:
+            if (g.ksplit > 1) {
+                ok = launch_epi<EPI_PARTIAL>(g, tile);
+                if (ok) {
+                    size_t total = (size_t)(g.M[0] + g.M[1]) * (N >> 2);
+                    hipLaunchKernelGGL(splitk_resid_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                                       flux_hip_stream_handle(), g);
+                    ok = hipGetLastError() == hipSuccess ? 1 : flux_hip_fail("split-K reduction launch failed");
+                }
+            } else {
+                ok = launch_epi<FLUX_HIP_EPI_RESID>(g, tile);
+            }
+            break;
         case FLUX_HIP_EPI_SWIGLU: ok = launch_epi<FLUX_HIP_EPI_SWIGLU>(g, tile); break;
         default: return flux_hip_fail("flux_hip_linear: unknown epilogue %d", epilogue);
     }

@@ -88,11 +88,12 @@ typedef struct {
 int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
                     int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1);
 
-/* Measurement hooks. force_tile: 0/1/2 pins the GEMM tile (64x128, 128x128, 256x256), -1
- * restores the automatic choice. probe(epilogue) records HIP events around every later
+/* Measurement hooks. force_tile: 0/1/2/3 pins the GEMM tile (64x128, 128x128, 256x256, 64x64),
+ * -1 restores the automatic choice; enable_splitk(0) turns the split-K path off. probe(epilogue) records HIP events around every later
  * flux_hip_linear launch with that epilogue (-1 stops); probe_read waits for them and returns
  * their count and summed duration. */
 void flux_hip_linear_force_tile(int tile);
+void flux_hip_linear_enable_splitk(int on);
 int flux_hip_linear_probe(int epilogue);
 int flux_hip_linear_probe_read(int *launches, float *total_ms);
 

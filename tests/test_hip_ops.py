@@ -29,7 +29,7 @@ def dev_bf16(hip, x):
     return hip.DevBuf.from_array(f32_to_bf16(x))
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
 @pytest.mark.parametrize("M", [1, 37, 130, 300])
 def test_linear_bf16_and_f32(hip, oracle_mod, tile, M):
     N, K = 512, 192
@@ -53,7 +53,7 @@ def test_linear_bf16_and_f32(hip, oracle_mod, tile, M):
     assert rel_l2(outT.to_array(np.float32, (N, M)).T, want) < 2e-6
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
 def test_linear_two_parts_resid_and_strides(hip, oracle_mod, tile):
     """Two row ranges with different weights, strided A (lda > K), gated residual epilogue."""
     hip.lib().flux_hip_linear_force_tile(tile)
@@ -77,7 +77,7 @@ def test_linear_two_parts_resid_and_strides(hip, oracle_mod, tile):
     assert rel_l2(dres.to_array(np.float32, (M0 + M1, N)), want) < 2e-6
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
 def test_linear_swiglu(hip, oracle_mod, tile):
     """silu(x Wg^T) * (x Wu^T) with gate/up rows at arbitrary offsets and a strided output."""
     hip.lib().flux_hip_linear_force_tile(tile)
@@ -93,6 +93,44 @@ def test_linear_swiglu(hip, oracle_mod, tile):
     got = bf16_to_f32(out.to_array(np.uint16, (M, ldc)))
     assert rel_l2(got[:, 64:64 + mlp], want) < 4e-3
     assert not got[:, :64].any() and not got[:, 64 + mlp:].any()   # nothing written outside
+
+
+@pytest.mark.parametrize("tile", [-1, 0, 3])
+def test_linear_split_k(hip, oracle_mod, tile):
+    """Long K, few output tiles: the residual epilogue splits K over workgroups (two passes through a
+    workspace, fixed summation order). Two row ranges, repeated runs must agree bit for bit."""
+    hip.lib().flux_hip_linear_force_tile(tile)
+    M0, M1, N, K = 64, 16, 256, 4096
+    a = q(normal_f32((M0 + M1, K), 20, 1))
+    W0 = q(normal_f32((N, K), 20, 2, 0.0, 0.05))
+    W1 = q(normal_f32((N, K), 20, 3, 0.0, 0.05))
+    res = normal_f32((M0 + M1, N), 20, 4)
+    g0, g1 = normal_f32((N,), 20, 5), normal_f32((N,), 20, 6)
+    want = res.copy()
+    want[:M0] += g0 * oracle_mod.linear(a[:M0], W0)
+    want[M0:] += g1 * oracle_mod.linear(a[M0:], W1)
+    da, dW0, dW1 = dev_bf16(hip, a), dev_bf16(hip, W0), dev_bf16(hip, W1)
+    dg0, dg1 = hip.DevBuf.from_array(g0), hip.DevBuf.from_array(g1)
+    outs = []
+    for on in (1, 1, 0):
+        hip.lib().flux_hip_linear_enable_splitk(on)
+        dres = hip.DevBuf.from_array(res)
+        hip.linear(hip.EPI_RESID, [(da.ptr, dW0.ptr, dres.ptr, dg0.ptr, M0),
+                                   (da.at(M0 * K * 2), dW1.ptr, dres.at(M0 * N * 4), dg1.ptr, M1)], N, K, K, K, N)
+        outs.append(dres.to_array(np.float32, (M0 + M1, N)))
+    hip.lib().flux_hip_linear_enable_splitk(1)
+    assert np.array_equal(outs[0], outs[1])            # deterministic
+    for o in outs:
+        assert rel_l2(o, want) < 2e-6
+    # one-part, ragged K slices (K/64 = 25 steps does not divide evenly)
+    K2 = 1600
+    x = q(normal_f32((40, K2), 20, 7))
+    W = q(normal_f32((128, K2), 20, 8, 0.0, 0.05))
+    r = normal_f32((40, 128), 20, 9)
+    dres = hip.DevBuf.from_array(r)
+    dx, dW = dev_bf16(hip, x), dev_bf16(hip, W)
+    hip.linear(hip.EPI_RESID, [(dx.ptr, dW.ptr, dres.ptr, dg0.ptr, 40)], 128, K2, K2, K2, 128)
+    assert rel_l2(dres.to_array(np.float32, (40, 128)), r + g0[:128] * oracle_mod.linear(x, W)) < 2e-6
 
 
 def test_linear_rejects_bad_shapes(hip):
