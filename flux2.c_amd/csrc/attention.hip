@@ -131,7 +131,8 @@ __device__ __forceinline__ int vt_swz(int d) { return ((d >> 1) & 7) ^ ((d & 1) 
 #define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
-__global__ __launch_bounds__(256, 2) void attention_kernel(bf16 *__restrict__ out, int ldo,
+template <int NW>
+__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf16 *__restrict__ out, int ldo,
                                                            const bf16 *__restrict__ q, int ldq,
                                                            const bf16 *__restrict__ k, const bf16 *__restrict__ vt, int ld_vt,
                                                            int seq_q, int seq_k, int heads, int split,
@@ -143,7 +144,9 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(bf16 *__restrict__ ou
      * contiguous run of (head, query block) pairs, so that all query blocks of a head run on one
      * XCD and its K / V^T (2.4 MB at 4608 tokens) are fetched from HBM once and then served from
      * that L2, instead of by all eight. */
-    const int nqb = (seq_q + 127) >> 7;
+    constexpr int BQ = NW * 32;  /* queries per workgroup */
+    constexpr int LP = 16 / NW;  /* wave-wide load instructions per wave and tile, for K and for V^T */
+    const int nqb = (seq_q + BQ - 1) / BQ;
     const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
     if (logical >= nqb * heads) return;
     const int h = logical / nqb, qb = logical - h * nqb;
@@ -154,13 +157,13 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(bf16 *__restrict__ ou
 
     /* ---- tile loader: per-lane global sources (un-swizzled) and per-wave LDS destinations ---- */
     const int ntiles = (seq_k + 63) >> 6;
-    const bf16 *k_src[4];
-    const bf16 *v_src[4];
-    int k_dst[4], v_dst[4], k_row[4];
+    const bf16 *k_src[LP];
+    const bf16 *v_src[LP];
+    int k_dst[LP], v_dst[LP], k_row[LP];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < LP; i++) {
         /* K: one wave instruction covers 4 rows of 256 bytes */
-        int r = wave * 4 + i * 16 + (lane >> 4); /* LDS row */
+        int r = wave * 4 + i * (NW * 4) + (lane >> 4); /* LDS row */
         /* LDS row 16 i' + 4 j + e (i' = 2c + b) holds key 32c + 8j + 4b + e of the tile: the
          * score accumulators of two 16-row blocks then cover 8 consecutive keys per lane */
         {
@@ -168,18 +171,18 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(bf16 *__restrict__ ou
             k_row[i] = 32 * (ib >> 1) + 8 * jj + 4 * (ib & 1) + ee;
         }
         k_src[i] = k + h * HD + (((lane & 15) ^ (r & 15)) << 3);
-        k_dst[i] = (wave * 4 + i * 16) * 256;
+        k_dst[i] = (wave * 4 + i * (NW * 4)) * 256;
         /* V^T: one wave instruction covers 8 rows of 128 bytes */
-        int d = wave * 8 + i * 32 + (lane >> 3);
+        int d = wave * 8 + i * (NW * 8) + (lane >> 3);
         v_src[i] = vt + (size_t)(h * HD + d) * ld_vt + (((lane & 7) ^ vt_swz(d)) << 3);
-        v_dst[i] = (wave * 8 + i * 32) * 128;
+        v_dst[i] = (wave * 8 + i * (NW * 8)) * 128;
     }
     /* LDS: K ring = 2 slots of 16 KB at 0 and 16 KB; V^T ring = 2 slots of 16 KB at 32 and 48 KB */
     auto issue_k = [&](int t) {
         char *base = smem + (t & 1) * (64 * 256);
         const int key0 = t * 64;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < LP; i++) {
             int r = min(key0 + k_row[i], seq_k - 1);
             __builtin_amdgcn_global_load_lds(GLOBAL_PTR(k_src[i] + (size_t)r * H), LDS_PTR(base + k_dst[i]), 16, 0, 0);
         }
@@ -188,7 +191,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(bf16 *__restrict__ ou
         char *base = smem + 2 * (64 * 256) + (t & 1) * (128 * 128);
         const int key0 = t * 64;
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < LP; i++)
             __builtin_amdgcn_global_load_lds(GLOBAL_PTR(v_src[i] + key0), LDS_PTR(base + v_dst[i]), 16, 0, 0);
     };
     issue_k(0);
@@ -200,7 +203,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(bf16 *__restrict__ ou
     int qrow[2];
 #pragma unroll
     for (int t = 0; t < 2; t++) {
-        qrow[t] = qb * 128 + wave * 32 + t * 16 + l15;
+        qrow[t] = qb * BQ + wave * 32 + t * 16 + l15;
         const int qrc = min(qrow[t], seq_q - 1);
         const bf16 *qp = q + (size_t)qrc * ldq + h * HD + lq * 8;
         float x[4][8];
@@ -380,6 +383,9 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(bf16 *__restrict__ ou
     }
 }
 
+static int g_att_force = -1;
+extern "C" void flux_hip_attention_force_variant(int v) { g_att_force = v; }
+
 extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ldq, const void *k, const void *vt,
                                   int ld_vt, int seq_q, int seq_k, int heads, int split, const float *q_w0,
                                   const float *q_w1, const float *rope_cos, const float *rope_sin, float eps) {
@@ -389,15 +395,26 @@ extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ld
     if (split < seq_q && !q_w1) return flux_hip_fail("flux_hip_attention: second weight missing");
     if ((ldo & 3) || (ldq & 7) || (ld_vt & 7) || ld_vt < (seq_k + 63) / 64 * 64)
         return flux_hip_fail("flux_hip_attention: bad leading dimensions (ldo=%d ldq=%d ld_vt=%d)", ldo, ldq, ld_vt);
+    /* 256-query workgroups (8 waves) share each K / V^T tile among twice as many queries;
+     * 128-query workgroups (two per CU) balance better when there are few of them. */
+    const int big = g_att_force >= 0 ? g_att_force : (((seq_q + 255) / 256) * heads >= 256);
     static bool attr_done = false;
     if (!attr_done) {
-        HIP_OK(hipFuncSetAttribute((const void *)attention_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
+        HIP_OK(hipFuncSetAttribute((const void *)attention_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
+        HIP_OK(hipFuncSetAttribute((const void *)attention_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
         attr_done = true;
     }
-    const int blocks = ((seq_q + 127) / 128) * heads;
-    hipLaunchKernelGGL(attention_kernel, dim3((blocks + 7) & ~7), dim3(256), 2 * ATT_STAGE, flux_hip_stream_handle(),
-                       (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,
-                       heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps);
+    if (big) {
+        const int blocks = ((seq_q + 255) / 256) * heads;
+        hipLaunchKernelGGL(attention_kernel<8>, dim3((blocks + 7) & ~7), dim3(512), 2 * ATT_STAGE, flux_hip_stream_handle(),
+                           (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,
+                           heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps);
+    } else {
+        const int blocks = ((seq_q + 127) / 128) * heads;
+        hipLaunchKernelGGL(attention_kernel<4>, dim3((blocks + 7) & ~7), dim3(256), 2 * ATT_STAGE, flux_hip_stream_handle(),
+                           (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,
+                           heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps);
+    }
     HIP_OK(hipGetLastError());
     return 1;
 }

@@ -274,7 +274,7 @@ static size_t g_ws_bytes = 0;
 static int ensure_ws(size_t bytes) {
     if (bytes <= g_ws_bytes) return 1;
     HIP_OK(hipStreamSynchronize(flux_hip_stream_handle()));
-    if (g_ws) hipFree(g_ws);
+    if (g_ws) (void)hipFree(g_ws);
     g_ws = nullptr;
     g_ws_bytes = 0;
     HIP_OK(hipMalloc((void **)&g_ws, bytes));
@@ -409,7 +409,7 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
     }
 
     const int slot = probe_slot(epilogue);
-    if (slot >= 0) hipEventRecord(g_probe_ev[slot][0], flux_hip_stream_handle());
+    if (slot >= 0) (void)hipEventRecord(g_probe_ev[slot][0], flux_hip_stream_handle());
     int ok;
     switch (epilogue) {
         case FLUX_HIP_EPI_BF16: ok = launch_epi<FLUX_HIP_EPI_BF16>(g, tile); break;
@@ -431,6 +431,6 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
         case FLUX_HIP_EPI_SWIGLU: ok = launch_epi<FLUX_HIP_EPI_SWIGLU>(g, tile); break;
         default: return flux_hip_fail("flux_hip_linear: unknown epilogue %d", epilogue);
     }
-    if (slot >= 0) hipEventRecord(g_probe_ev[slot][1], flux_hip_stream_handle());
+    if (slot >= 0) (void)hipEventRecord(g_probe_ev[slot][1], flux_hip_stream_handle());
     return ok;
 }

@@ -47,10 +47,10 @@ extern "C" int flux_hip_available(void) { return g_ready || flux_hip_init(); }
 
 extern "C" void flux_hip_cleanup(void) {
     if (!g_ready) return;
-    hipStreamSynchronize(g_stream);
-    hipEventDestroy(g_ev0);
-    hipEventDestroy(g_ev1);
-    hipStreamDestroy(g_stream);
+    (void)hipStreamSynchronize(g_stream);
+    (void)hipEventDestroy(g_ev0);
+    (void)hipEventDestroy(g_ev1);
+    (void)hipStreamDestroy(g_stream);
     g_stream = nullptr;
     g_ready = 0;
 }
@@ -73,7 +73,7 @@ extern "C" void *flux_hip_malloc(size_t bytes) {
 }
 
 extern "C" void flux_hip_free(void *p) {
-    if (p) hipFree(p);
+    if (p) (void)hipFree(p);
 }
 
 extern "C" int flux_hip_upload(void *dst, const void *src, size_t bytes) {

@@ -94,6 +94,8 @@ int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
  * their count and summed duration. */
 void flux_hip_linear_force_tile(int tile);
 void flux_hip_linear_enable_splitk(int on);
+/* 0 = 128-query workgroups, 1 = 256-query workgroups, -1 = automatic */
+void flux_hip_attention_force_variant(int v);
 int flux_hip_linear_probe(int epilogue);
 int flux_hip_linear_probe_read(int *launches, float *total_ms);
 

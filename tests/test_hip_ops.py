@@ -246,3 +246,15 @@ def test_layout_edges_and_updates(hip, oracle_mod):
     hip.check(hip.lib().flux_hip_cfg_euler_update(dz.ptr, dvu.ptr, dv.ptr, 4.0, -0.1, 999))
     want = z + np.float32(-0.1) * (vu + np.float32(4.0) * (v - vu))
     np.testing.assert_allclose(dz.to_array(np.float32, (999,)), want, rtol=0, atol=2e-6)
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+def test_attention_workgroup_variants(hip, oracle_mod, variant):
+    """Both workgroup sizes (128 and 256 queries) give the same answer on ragged lengths."""
+    hip.lib().flux_hip_attention_force_variant(variant)
+    try:
+        for n, split, heads in ((300, 100, 2), (513, 512, 1)):
+            got, want = _attention_case(hip, oracle_mod, n, split, heads, 30 + variant)
+            assert rel_l2(got, want) < 1e-2, (n, rel_l2(got, want))
+    finally:
+        hip.lib().flux_hip_attention_force_variant(-1)
