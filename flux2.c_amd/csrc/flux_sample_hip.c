@@ -61,6 +61,64 @@ float *flux_official_schedule(int num_steps, int image_seq_len) {
     return s;
 }
 
+/* ------------------------------------------------------------------ initial noise */
+
+/* Host RNG of the reference: SplitMix64-seeded xoshiro256** and Box-Muller (flux_kernels.c:45-102).
+ * When the process also links the reference's flux_kernels.c its generator is used, so that an
+ * unseeded call continues the stream the application seeded (main.c:254); otherwise the same
+ * algorithm runs here. */
+extern void flux_rng_seed(uint64_t seed) __attribute__((weak));
+extern void flux_randn(float *out, int n) __attribute__((weak));
+
+static uint64_t rng_s[4] = {0x853c49e6748fea9bULL, 0xda3e39cb94b95bdbULL, 0x647c4677a2884327ULL, 0xc6e7918d2e2969f5ULL};
+static uint64_t rotl64(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }
+static uint64_t rng_next(void) {
+    const uint64_t r = rotl64(rng_s[1] * 5, 7) * 9, t = rng_s[1] << 17;
+    rng_s[2] ^= rng_s[0]; rng_s[3] ^= rng_s[1]; rng_s[1] ^= rng_s[2]; rng_s[0] ^= rng_s[3];
+    rng_s[2] ^= t; rng_s[3] = rotl64(rng_s[3], 45);
+    return r;
+}
+static void own_seed(uint64_t seed) {
+    for (int i = 0; i < 4; i++) {
+        seed += 0x9e3779b97f4a7c15ULL;
+        uint64_t z = seed;
+        z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ULL;
+        z = (z ^ (z >> 27)) * 0x94d049bb133111ebULL;
+        rng_s[i] = z ^ (z >> 31);
+    }
+}
+static float own_uniform(void) { return (rng_next() >> 11) * (1.0 / 9007199254740992.0); }
+static void own_randn(float *out, int n) {
+    for (int i = 0; i < n; i++) {
+        float u1 = own_uniform(), u2 = own_uniform();
+        while (u1 == 0.0f) u1 = own_uniform();
+        out[i] = sqrtf(-2.0f * logf(u1)) * cosf(2.0f * 3.14159265358979323846f * u2);
+    }
+}
+
+/* Noise is drawn at 112 x 112 and subsampled (nearest) so that a seed gives similar compositions
+ * at every resolution (flux_sample.c:837-877). Returns malloc'd [batch, channels, h, w]. */
+float *flux_init_noise(int batch, int channels, int h, int w, int64_t seed) {
+    const int MAXD = 112;
+    void (*seedf)(uint64_t) = flux_rng_seed ? flux_rng_seed : own_seed;
+    void (*randn)(float *, int) = flux_randn ? flux_randn : own_randn;
+    const int n = batch * channels * h * w;
+    float *noise = (float *)malloc((size_t)n * sizeof(float));
+    if (!noise) return NULL;
+    if (seed >= 0) seedf((uint64_t)seed);
+    if (h >= MAXD && w >= MAXD) { randn(noise, n); return noise; }
+    const int big_n = batch * channels * MAXD * MAXD;
+    float *big = (float *)malloc((size_t)big_n * sizeof(float));
+    if (!big) { free(noise); return NULL; }
+    randn(big, big_n);
+    for (int bc = 0; bc < batch * channels; bc++)
+        for (int y = 0; y < h; y++)
+            for (int x = 0; x < w; x++)
+                noise[((size_t)bc * h + y) * w + x] = big[((size_t)bc * MAXD + y * MAXD / h) * MAXD + x * MAXD / w];
+    free(big);
+    return noise;
+}
+
 /* ------------------------------------------------------------------ stage timing */
 
 #define EV_MAX_FORWARDS 512

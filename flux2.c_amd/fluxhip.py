@@ -102,6 +102,8 @@ def lib():
     L.flux_hip_session_step.argtypes = [vp, c_i, vp]
     L.flux_hip_session_read_latent.argtypes = [vp, vp]
     L.flux_hip_session_free.argtypes = [vp]
+    L.flux_init_noise.restype = vp
+    L.flux_init_noise.argtypes = [c_i, c_i, c_i, c_i, ctypes.c_int64]
     for n in ("flux_linear_schedule", "flux_power_schedule", "flux_official_schedule"):
         getattr(L, n).restype = vp
     L.flux_linear_schedule.argtypes = [c_i]
@@ -316,6 +318,11 @@ def stage_timing():
     L = lib()
     return tuple(ctypes.c_double.in_dll(L, "flux_timing_transformer_" + n).value
                  for n in ("double", "single", "final", "total"))
+
+
+def init_noise(channels, h, w, seed):
+    p = lib().flux_init_noise(1, channels, h, w, seed)
+    return _take_host(p, (channels, h, w))
 
 
 def schedule(kind, n, arg=None):

@@ -228,6 +228,10 @@ float *flux_linear_schedule(int num_steps);
 float *flux_power_schedule(int num_steps, float alpha);
 float *flux_official_schedule(int num_steps, int image_seq_len);
 
+/* Initial latent noise from the reference's host RNG (flux_sample.c:837-877); malloc'd
+ * [batch, channels, h, w], caller frees. seed < 0 continues the current stream. */
+float *flux_init_noise(int batch, int channels, int h, int w, int64_t seed);
+
 /* Same sampling loops, additionally copying every forward's velocity (in call order,
  * [forwards, channels*h*w] f32) to v_trace when it is not NULL. For parity tests. */
 float *flux_hip_sample_traced(void *transformer, const float *z, int channels, int h, int w,
