@@ -186,3 +186,54 @@ def test_klein4b_c1_against_reference_golden(hip, golden_dir, qk):
     txt = normal_f32((64, cfg.text_dim), 42, 1001)
     gate(m.forward(lat, 4, 4, txt, 1.0), g["velocity"], f"4B c1 {qk}")
     m.close()
+
+
+def test_reference_loader_entry_point(hip, golden_dir, tmp_path):
+    """flux_transformer_load_safetensors_mmap() fed with the handle the reference's own
+    safetensors_open() returns (its C code compiled in place, oracle/_ref): checks the mirrored
+    struct layout, the name mapping and ownership on the real 4B file layout."""
+    import ctypes
+    ref_so = os.path.join(os.path.dirname(golden_dir), "..", "oracle", "_ref", "libfluxref.so")
+    if not os.path.exists(ref_so):
+        pytest.skip("oracle/_ref/libfluxref.so is not built")
+    from model_spec import tensor_shapes
+    cfg = KLEIN_4B
+    path = "/dev/shm/flux_hip_test_4b.safetensors" if os.path.isdir("/dev/shm") else str(tmp_path / "m.safetensors")
+    try:
+        # stream the 7.75 GB file tensor by tensor
+        import json
+        shapes = tensor_shapes(cfg)
+        header, off = {}, 0
+        for name, shp in shapes.items():
+            nb = int(np.prod(shp)) * 2
+            header[name] = {"dtype": "BF16", "shape": list(shp), "data_offsets": [off, off + nb]}
+            off += nb
+        hj = json.dumps(header, separators=(",", ":")).encode()
+        hj += b" " * ((8 - len(hj) % 8) % 8)
+        with open(path, "wb") as f:
+            f.write(len(hj).to_bytes(8, "little"))
+            f.write(hj)
+            for name in shapes:
+                f.write(make_weights(cfg, 42, 0.02, "sharp", only=[name])[name].tobytes())
+        R = ctypes.CDLL(os.path.realpath(ref_so))
+        R.safetensors_open.restype = ctypes.c_void_p
+        R.safetensors_open.argtypes = [ctypes.c_char_p]
+        sf = R.safetensors_open(path.encode())
+        assert sf
+        L = hip.lib()
+        L.flux_transformer_load_safetensors_mmap.restype = ctypes.c_void_p
+        L.flux_transformer_load_safetensors_mmap.argtypes = [ctypes.c_void_p]
+        tf = L.flux_transformer_load_safetensors_mmap(sf)
+        assert tf, L.flux_hip_last_error()
+        lat = normal_f32((cfg.channels, 4, 4), 42, 1000)
+        txt = normal_f32((64, cfg.text_dim), 42, 1001)
+        p = L.flux_transformer_forward(tf, lat.ctypes.data, 4, 4, txt.ctypes.data, 64, 1.0)
+        assert p, L.flux_hip_last_error()
+        v = np.ctypeslib.as_array(ctypes.cast(p, ctypes.POINTER(ctypes.c_float)), shape=(cfg.channels * 16,)).copy()
+        hip.libc_free(p)
+        g = np.load(os.path.join(golden_dir, "klein4b_c1_sharp.npz"))
+        gate(v, g["velocity"], "4B c1 through the reference loader entry point")
+        L.flux_transformer_free(tf)      # also closes sf (mmap mode owns the handle)
+    finally:
+        if os.path.exists(path):
+            os.remove(path)
