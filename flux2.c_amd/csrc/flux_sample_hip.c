@@ -293,19 +293,21 @@ int flux_hip_session_read_latent(flux_hip_session *s, float *z_out) {
     return 1;
 }
 
-float *flux_hip_sample_traced(void *transformer, const float *z, int channels, int h, int w,
-                              const flux_ref_t *refs, int num_refs,
-                              const float *text_emb_cond, int text_seq_cond,
-                              const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
-                              const float *schedule, int num_steps, float *v_trace) {
+static float *sample_impl(void *transformer, const float *z, int channels, int h, int w,
+                          const flux_ref_t *refs, int num_refs,
+                          const float *text_emb_cond, int text_seq_cond,
+                          const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
+                          const float *schedule, int num_steps, float *v_trace, void (*progress)(int, int)) {
     flux_hip_session *s = flux_hip_session_begin(transformer, z, channels, h, w, refs, num_refs, text_emb_cond,
                                                  text_seq_cond, text_emb_uncond, text_seq_uncond, guidance_scale,
                                                  schedule, num_steps);
     if (!s) return NULL;
     const size_t per_step = s->n_lat * (s->cfg ? 2 : 1);
     float *out = NULL;
-    for (int i = 0; i < num_steps; i++)
+    for (int i = 0; i < num_steps; i++) {
         if (!flux_hip_session_step(s, i, v_trace ? v_trace + (size_t)i * per_step : NULL)) goto done;
+        if (progress) progress(i + 1, num_steps); /* the step has been queued (flux_sample.c:254) */
+    }
     out = (float *)malloc(s->n_lat * 4);
     if (!out) { flux_hip_fail("out of host memory"); goto done; }
     if (!flux_hip_session_read_latent(s, out)) { free(out); out = NULL; goto done; }
@@ -318,17 +320,22 @@ done:
     return out;
 }
 
+float *flux_hip_sample_traced(void *transformer, const float *z, int channels, int h, int w,
+                              const flux_ref_t *refs, int num_refs,
+                              const float *text_emb_cond, int text_seq_cond,
+                              const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
+                              const float *schedule, int num_steps, float *v_trace) {
+    return sample_impl(transformer, z, channels, h, w, refs, num_refs, text_emb_cond, text_seq_cond, text_emb_uncond,
+                       text_seq_uncond, guidance_scale, schedule, num_steps, v_trace, NULL);
+}
+
 /* ------------------------------------------------------------------ reference-named entry points */
 
 static float *run(void *tf, float *z, int batch, int channels, int h, int w, const flux_ref_t *refs, int num_refs,
                   const float *tc, int sc, const float *tu, int su, float g, const float *schedule, int steps,
                   void (*progress)(int, int)) {
     if (batch != 1) { flux_hip_fail("sampler: batch=%d (the pipeline always passes 1)", batch); return NULL; }
-    /* progress fires per step at queue time through flux_step_callback-style notification */
-    float *out = flux_hip_sample_traced(tf, z, channels, h, w, refs, num_refs, tc, sc, tu, su, g, schedule, steps, NULL);
-    if (out && progress)
-        for (int s = 0; s < steps; s++) progress(s + 1, steps);
-    return out;
+    return sample_impl(tf, z, channels, h, w, refs, num_refs, tc, sc, tu, su, g, schedule, steps, NULL, progress);
 }
 
 float *flux_sample_euler(void *transformer, void *text_encoder, float *z, int batch, int channels, int h, int w,

@@ -188,6 +188,19 @@ def test_klein4b_c1_against_reference_golden(hip, golden_dir, qk):
     m.close()
 
 
+def test_long_ragged_sequence(hip, oracle_mod):
+    """8000 image tokens (100 x 80, beyond the 1024^2 case) + 333 text tokens on the small model:
+    many 256-wide tiles, a ragged tail in every kernel, the 256-query attention workgroups."""
+    cfg = SMALL
+    W = make_weights(cfg, 42, 0.05, "sharp")
+    o = oracle_mod.Oracle(cfg, W)
+    m = hip.Transformer(cfg, W)
+    lat = normal_f32((cfg.channels, 100, 80), 17, 1)
+    txt = normal_f32((333, cfg.text_dim), 17, 2)
+    gate(m.forward(lat, 100, 80, txt, 0.9), o.forward(lat, 100, 80, txt, 0.9), "100x80 + 333")
+    m.close(); o.close()
+
+
 def test_reference_loader_entry_point(hip, golden_dir, tmp_path):
     """flux_transformer_load_safetensors_mmap() fed with the handle the reference's own
     safetensors_open() returns (its C code compiled in place, oracle/_ref): checks the mirrored
@@ -237,3 +250,40 @@ def test_reference_loader_entry_point(hip, golden_dir, tmp_path):
     finally:
         if os.path.exists(path):
             os.remove(path)
+
+
+def test_callbacks_fire_in_order(hip):
+    """Step, sub-step and progress callbacks (flux_kernels.h:245-256, flux_sample.c:240,254) fire on
+    the calling thread in the reference's order."""
+    import ctypes
+    cfg = TINY
+    m = hip.Transformer(cfg, make_weights(cfg, 42, 0.02, "sharp"))
+    L = hip.lib()
+    log = []
+    STEP = ctypes.CFUNCTYPE(None, ctypes.c_int, ctypes.c_int)
+    SUB = ctypes.CFUNCTYPE(None, ctypes.c_int, ctypes.c_int, ctypes.c_int)
+    step_cb = STEP(lambda s, n: log.append(("step", s, n)))
+    sub_cb = SUB(lambda t, i, n: log.append(("sub", t, i, n)))
+    prog_cb = STEP(lambda s, n: log.append(("progress", s, n)))
+    ctypes.c_void_p.in_dll(L, "flux_step_callback").value = ctypes.cast(step_cb, ctypes.c_void_p).value
+    ctypes.c_void_p.in_dll(L, "flux_substep_callback").value = ctypes.cast(sub_cb, ctypes.c_void_p).value
+    try:
+        z = normal_f32((cfg.channels, 2, 2), 18, 1)
+        txt = normal_f32((8, cfg.text_dim), 18, 2)
+        sched = hip.schedule("linear", 2)
+        L.flux_sample_euler.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 4 + [ctypes.c_void_p, ctypes.c_int,
+                                                                                     ctypes.c_void_p, ctypes.c_int, STEP]
+        p = L.flux_sample_euler(m.h, None, z.ctypes.data, 1, cfg.channels, 2, 2, txt.ctypes.data, 8,
+                                sched.ctypes.data, 2, prog_cb)
+        assert p
+        hip.libc_free(p)
+    finally:
+        ctypes.c_void_p.in_dll(L, "flux_step_callback").value = None
+        ctypes.c_void_p.in_dll(L, "flux_substep_callback").value = None
+    per_step = [("sub", 0, i, cfg.n_double) for i in range(cfg.n_double)] + \
+               [("sub", 1, i, cfg.n_single) for i in range(cfg.n_single)] + [("sub", 2, 0, 1)]
+    want = []
+    for s in (1, 2):
+        want += [("step", s, 2)] + per_step + [("progress", s, 2)]
+    assert log == want
+    m.close()
