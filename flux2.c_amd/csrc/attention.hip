@@ -105,6 +105,8 @@ extern "C" int flux_hip_kv_prepare(void *k_out, void *vt_out, int ld_vt, const v
     const int padded = (rows + 63) / 64 * 64;
     if (ld_vt < padded || (ld_vt & 7)) return flux_hip_fail("flux_hip_kv_prepare: ld_vt=%d must be >= %d and a multiple of 8", ld_vt, padded);
     if ((ld & 7) || (k_col & 7) || (v_col & 7)) return flux_hip_fail("flux_hip_kv_prepare: ld/k_col/v_col must be multiples of 8");
+    if (((uintptr_t)k_out | (uintptr_t)vt_out | (uintptr_t)qkv | (uintptr_t)k_w0 | (uintptr_t)k_w1 | (uintptr_t)rope_cos | (uintptr_t)rope_sin) & 15)
+        return flux_hip_fail("flux_hip_kv_prepare: operands must be 16-byte aligned");
     hipLaunchKernelGGL(kv_prepare_kernel, dim3(padded / 64, heads), dim3(256), 0, flux_hip_stream_handle(),
                        (bf16 *)k_out, (bf16 *)vt_out, ld_vt, (const bf16 *)qkv, ld, k_col, v_col, rows, heads, split,
                        k_w0, k_w1 ? k_w1 : k_w0, rope_cos, rope_sin, eps);
@@ -393,6 +395,9 @@ extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ld
     if (seq_k <= 0) return flux_hip_fail("flux_hip_attention: seq_k=%d", seq_k);
     if (!out_bf16 || !q || !k || !vt || !q_w0 || !rope_cos || !rope_sin) return flux_hip_fail("flux_hip_attention: NULL argument");
     if (split < seq_q && !q_w1) return flux_hip_fail("flux_hip_attention: second weight missing");
+    if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)vt | (uintptr_t)q_w0 | (uintptr_t)q_w1 | (uintptr_t)rope_cos | (uintptr_t)rope_sin) & 15) ||
+        ((uintptr_t)out_bf16 & 7))
+        return flux_hip_fail("flux_hip_attention: operands must be 16-byte aligned (output 8-byte)");
     if ((ldo & 3) || (ldq & 7) || (ld_vt & 7) || ld_vt < (seq_k + 63) / 64 * 64)
         return flux_hip_fail("flux_hip_attention: bad leading dimensions (ldo=%d ldq=%d ld_vt=%d)", ldo, ldq, ld_vt);
     /* 256-query workgroups (8 waves) share each K / V^T tile among twice as many queries;

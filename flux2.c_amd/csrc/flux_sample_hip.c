@@ -198,6 +198,7 @@ struct flux_hip_session {
     float *z_dev, *v_c, *v_u;
     void *txt_c, *txt_u;
     fh_events *ev;
+    int owns_tf;
 };
 
 void flux_hip_session_free(flux_hip_session *s) {
@@ -206,6 +207,7 @@ void flux_hip_session_free(flux_hip_session *s) {
     flux_hip_free(s->z_dev); flux_hip_free(s->v_c); flux_hip_free(s->v_u);
     flux_hip_free(s->txt_c); flux_hip_free(s->txt_u);
     free(s->schedule);
+    if (s->tf && s->owns_tf) s->tf->session_active = 0;
     free(s);
 }
 
@@ -223,8 +225,11 @@ flux_hip_session *flux_hip_session_begin(void *transformer, const float *z, int 
     const int cfg = text_emb_uncond != NULL;
     if (cfg && text_seq_uncond <= 0) { flux_hip_fail("sampler: empty unconditional text"); return NULL; }
 
+    if (tf->session_active) { flux_hip_fail("sampler: another run is active on this transformer"); return NULL; }
     flux_hip_session *s = (flux_hip_session *)calloc(1, sizeof(*s));
     if (!s) { flux_hip_fail("out of host memory"); return NULL; }
+    tf->session_active = 1;
+    s->owns_tf = 1;
     s->tf = tf; s->cfg = cfg; s->n_target = h * w; s->num_steps = num_steps; s->guidance = guidance_scale;
     s->n_lat = (size_t)channels * s->n_target;
     s->schedule = (float *)malloc((num_steps + 1) * sizeof(float));

@@ -269,6 +269,7 @@ __global__ __launch_bounds__(256) void splitk_resid_kernel(GemmArgs g) {
     *(f32x4 *)p = x;
 }
 
+extern "C" void flux_hip_linear_release(void);
 static float *g_ws = nullptr;
 static size_t g_ws_bytes = 0;
 static int ensure_ws(size_t bytes) {
@@ -280,6 +281,12 @@ static int ensure_ws(size_t bytes) {
     HIP_OK(hipMalloc((void **)&g_ws, bytes));
     g_ws_bytes = bytes;
     return 1;
+}
+
+extern "C" void flux_hip_linear_release(void) {
+    if (g_ws) (void)hipFree(g_ws);
+    g_ws = nullptr;
+    g_ws_bytes = 0;
 }
 
 static int g_force_tile = -1;
@@ -340,6 +347,9 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
             return flux_hip_fail("flux_hip_linear: NULL operand");
         if (epilogue == FLUX_HIP_EPI_RESID && parts[i].M > 0 && !parts[i].gate)
             return flux_hip_fail("flux_hip_linear: residual epilogue needs a gate vector");
+        if (parts[i].M > 0 && ((((uintptr_t)parts[i].A | (uintptr_t)parts[i].W | (uintptr_t)parts[i].gate) & 15) ||
+                               ((uintptr_t)parts[i].C & (epilogue == FLUX_HIP_EPI_F32_T ? 3 : epilogue == FLUX_HIP_EPI_BF16 || epilogue == FLUX_HIP_EPI_SWIGLU ? 7 : 15))))
+            return flux_hip_fail("flux_hip_linear: operands must be 16-byte aligned (bf16 outputs 8-byte)");
     }
     /* drop empty parts */
     int np = 0;

@@ -52,6 +52,7 @@ struct flux_transformer {
     float *mod, *temb, *sincos;
     int mod_cap, mod_steps;
     void *owned_sf; /* reference safetensors handle owned in mmap mode */
+    int session_active; /* work buffers, RoPE tables and modulation belong to one run at a time */
 };
 
 /* Four HIP events per forward: start, after double blocks, after single blocks, end. */

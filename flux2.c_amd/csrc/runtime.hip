@@ -45,9 +45,12 @@ extern "C" int flux_hip_init(void) {
 
 extern "C" int flux_hip_available(void) { return g_ready || flux_hip_init(); }
 
+extern "C" void flux_hip_linear_release(void);
+
 extern "C" void flux_hip_cleanup(void) {
     if (!g_ready) return;
     (void)hipStreamSynchronize(g_stream);
+    flux_hip_linear_release();
     (void)hipEventDestroy(g_ev0);
     (void)hipEventDestroy(g_ev1);
     (void)hipStreamDestroy(g_stream);
