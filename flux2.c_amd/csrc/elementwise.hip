@@ -209,6 +209,36 @@ __global__ __launch_bounds__(256) void cfg_euler_kernel(float *__restrict__ z, c
     }
 }
 
+/* Heun (flux_sample.c:780-796): predictor out = z + dt v1 into a second buffer, corrector
+ * z += dt/2 (v1 + v2). */
+__global__ __launch_bounds__(256) void axpy_out_kernel(float *__restrict__ out, const float *__restrict__ z,
+                                                       const float *__restrict__ v, float dt, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = z[i] + dt * v[i];
+}
+
+__global__ __launch_bounds__(256) void heun_kernel(float *__restrict__ z, const float *__restrict__ v1,
+                                                   const float *__restrict__ v2, float dt, size_t n) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) z[i] += 0.5f * dt * (v1[i] + v2[i]);
+}
+
+extern "C" int flux_hip_euler_predict(float *out, const float *z, const float *v, float dt, size_t n) {
+    if (!n) return 1;
+    if (!out || !z || !v) return flux_hip_fail("flux_hip_euler_predict: NULL argument");
+    hipLaunchKernelGGL(axpy_out_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, flux_hip_stream_handle(), out, z, v, dt, n);
+    HIP_OK(hipGetLastError());
+    return 1;
+}
+
+extern "C" int flux_hip_heun_update(float *z, const float *v1, const float *v2, float dt, size_t n) {
+    if (!n) return 1;
+    if (!z || !v1 || !v2) return flux_hip_fail("flux_hip_heun_update: NULL argument");
+    hipLaunchKernelGGL(heun_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, flux_hip_stream_handle(), z, v1, v2, dt, n);
+    HIP_OK(hipGetLastError());
+    return 1;
+}
+
 extern "C" int flux_hip_euler_update(float *z, const float *v, float dt, size_t n) {
     if (!n) return 1;
     if (!z || !v) return flux_hip_fail("flux_hip_euler_update: NULL argument");

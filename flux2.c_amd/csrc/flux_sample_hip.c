@@ -1,8 +1,10 @@
 /*
- * flux_sample_hip.c - Euler / CFG samplers and the single-forward entry points on MI355X.
+ * flux_sample_hip.c - samplers and the single-forward entry points on MI355X.
  *
- * Exports the reference's sampler functions (flux_sample.c:212, 303, 381, 457, 534, 615) and
- * schedules (flux_sample.c:49, 62, 145) with their signatures. The loop itself is device
+ * Exports everything the reference's flux_sample.c exports, with the same signatures: the
+ * Euler / CFG samplers (flux_sample.c:212, 303, 381, 457, 534, 615), the noise-injecting and
+ * Heun samplers (:697, :760), the schedules (:49, 62, 75, 96, 145), flux_init_noise (:837),
+ * flux_generate_latent (:891) and the timing and progress globals. The loop itself is device
  * resident: latent, text and reference tokens are uploaded once, every step's latent update
  * runs as a kernel (z += dt v, or the CFG combine), and the latent comes back once at the end.
  * The host thread only queues work; step callbacks therefore fire at queue time.
@@ -61,15 +63,34 @@ float *flux_official_schedule(int num_steps, int image_seq_len) {
     return s;
 }
 
+/* 1 - sigmoid(10 (i/n - 1/2) + shift), endpoints forced to 1 and 0 (flux_sample.c:75-91). */
+float *flux_sigmoid_schedule(int num_steps, float shift) {
+    float *s = (float *)malloc((num_steps + 1) * sizeof(float));
+    for (int i = 0; i <= num_steps; i++) {
+        float x = ((float)i / (float)num_steps - 0.5f) * 10.0f + shift;
+        s[i] = 1.0f - 1.0f / (1.0f + expf(-x));
+    }
+    s[0] = 1.0f;
+    s[num_steps] = 0.0f;
+    return s;
+}
+
+/* 1 - (i/n)^(1 + shift/2) with shift 1 from 1024x1024 pixels up, 0.5 from 512x512 up, else 0
+ * (flux_sample.c:96-116). */
+float *flux_resolution_schedule(int num_steps, int height, int width) {
+    const int pixels = height * width;
+    const float shift = pixels >= 1024 * 1024 ? 1.0f : pixels >= 512 * 512 ? 0.5f : 0.0f;
+    float *s = (float *)malloc((num_steps + 1) * sizeof(float));
+    for (int i = 0; i <= num_steps; i++) s[i] = 1.0f - powf((float)i / (float)num_steps, 1.0f + shift * 0.5f);
+    return s;
+}
+
 /* ------------------------------------------------------------------ initial noise */
 
-/* Host RNG of the reference: SplitMix64-seeded xoshiro256** and Box-Muller (flux_kernels.c:45-102).
- * When the process also links the reference's flux_kernels.c its generator is used, so that an
- * unseeded call continues the stream the application seeded (main.c:254); otherwise the same
- * algorithm runs here. */
-extern void flux_rng_seed(uint64_t seed) __attribute__((weak));
-extern void flux_randn(float *out, int n) __attribute__((weak));
-
+/* Host RNG of the reference: SplitMix64-seeded xoshiro256** and Box-Muller (flux_kernels.c:45-102),
+ * exported under the reference's names. In a process that also links the reference's
+ * flux_kernels.c the executable's definitions take precedence at load time, here too, so an
+ * unseeded call continues the stream the application seeded (main.c:254). */
 static uint64_t rng_s[4] = {0x853c49e6748fea9bULL, 0xda3e39cb94b95bdbULL, 0x647c4677a2884327ULL, 0xc6e7918d2e2969f5ULL};
 static uint64_t rotl64(uint64_t x, int k) { return (x << k) | (x >> (64 - k)); }
 static uint64_t rng_next(void) {
@@ -78,7 +99,7 @@ static uint64_t rng_next(void) {
     rng_s[2] ^= t; rng_s[3] = rotl64(rng_s[3], 45);
     return r;
 }
-static void own_seed(uint64_t seed) {
+void flux_rng_seed(uint64_t seed) {
     for (int i = 0; i < 4; i++) {
         seed += 0x9e3779b97f4a7c15ULL;
         uint64_t z = seed;
@@ -87,11 +108,11 @@ static void own_seed(uint64_t seed) {
         rng_s[i] = z ^ (z >> 31);
     }
 }
-static float own_uniform(void) { return (rng_next() >> 11) * (1.0 / 9007199254740992.0); }
-static void own_randn(float *out, int n) {
+static float rng_uniform(void) { return (rng_next() >> 11) * (1.0 / 9007199254740992.0); }
+void flux_randn(float *out, int n) {
     for (int i = 0; i < n; i++) {
-        float u1 = own_uniform(), u2 = own_uniform();
-        while (u1 == 0.0f) u1 = own_uniform();
+        float u1 = rng_uniform(), u2 = rng_uniform();
+        while (u1 == 0.0f) u1 = rng_uniform();
         out[i] = sqrtf(-2.0f * logf(u1)) * cosf(2.0f * 3.14159265358979323846f * u2);
     }
 }
@@ -100,17 +121,15 @@ static void own_randn(float *out, int n) {
  * at every resolution (flux_sample.c:837-877). Returns malloc'd [batch, channels, h, w]. */
 float *flux_init_noise(int batch, int channels, int h, int w, int64_t seed) {
     const int MAXD = 112;
-    void (*seedf)(uint64_t) = flux_rng_seed ? flux_rng_seed : own_seed;
-    void (*randn)(float *, int) = flux_randn ? flux_randn : own_randn;
     const int n = batch * channels * h * w;
     float *noise = (float *)malloc((size_t)n * sizeof(float));
     if (!noise) return NULL;
-    if (seed >= 0) seedf((uint64_t)seed);
-    if (h >= MAXD && w >= MAXD) { randn(noise, n); return noise; }
+    if (seed >= 0) flux_rng_seed((uint64_t)seed);
+    if (h >= MAXD && w >= MAXD) { flux_randn(noise, n); return noise; }
     const int big_n = batch * channels * MAXD * MAXD;
     float *big = (float *)malloc((size_t)big_n * sizeof(float));
     if (!big) { free(noise); return NULL; }
-    randn(big, big_n);
+    flux_randn(big, big_n);
     for (int bc = 0; bc < batch * channels; bc++)
         for (int y = 0; y < h; y++)
             for (int x = 0; x < w; x++)
@@ -191,7 +210,7 @@ static int upload_ref_tokens(flux_transformer_t *tf, int n_target, const flux_re
 struct flux_hip_session {
     flux_transformer_t *tf;
     fh_rope *rp_c, *rp_u;
-    int cfg, n_target, num_steps, next_forward;
+    int cfg, n_target, num_steps, next_forward, h, w;
     size_t n_lat;
     float guidance;
     float *schedule;
@@ -231,6 +250,7 @@ flux_hip_session *flux_hip_session_begin(void *transformer, const float *z, int 
     tf->session_active = 1;
     s->owns_tf = 1;
     s->tf = tf; s->cfg = cfg; s->n_target = h * w; s->num_steps = num_steps; s->guidance = guidance_scale;
+    s->h = h; s->w = w;
     s->n_lat = (size_t)channels * s->n_target;
     s->schedule = (float *)malloc((num_steps + 1) * sizeof(float));
     if (!s->schedule) { flux_hip_fail("out of host memory"); goto fail; }
@@ -298,6 +318,40 @@ int flux_hip_session_read_latent(flux_hip_session *s, float *z_out) {
     return 1;
 }
 
+/* Intermediate-image hook of the reference (flux_sample.c:258-266): when the application has set
+ * flux_step_image_callback and flux_step_image_vae (flux.c:161-164), every step but the last
+ * hands the current latent to the application's own VAE decoder and the image to the callback.
+ * All four symbols belong to the application (flux_kernels.c:35-36, flux_vae.c, flux_image.c);
+ * they are weak here, and without them the hook does nothing. Each use waits for the device. */
+struct flux_image;
+typedef void (*fh_step_image_cb)(int step, int total, const struct flux_image *img);
+extern fh_step_image_cb flux_step_image_callback __attribute__((weak));
+extern void *flux_step_image_vae __attribute__((weak));
+extern struct flux_image *flux_vae_decode(void *vae, const float *latent, int batch, int latent_h, int latent_w) __attribute__((weak));
+extern void flux_image_free(struct flux_image *img) __attribute__((weak));
+
+static void step_image_hook(flux_hip_session *s, int step) {
+    if (!&flux_step_image_callback || !&flux_step_image_vae || !flux_vae_decode || !flux_image_free) return;
+    if (!flux_step_image_callback || !flux_step_image_vae || step + 1 >= s->num_steps) return;
+    float *z = (float *)malloc(s->n_lat * 4);
+    if (!z) return;
+    if (flux_hip_download(z, s->z_dev, s->n_lat * 4)) {
+        struct flux_image *img = flux_vae_decode(flux_step_image_vae, z, 1, s->h, s->w);
+        if (img) {
+            flux_step_image_callback(step + 1, s->num_steps, img);
+            flux_image_free(img);
+        }
+    }
+    free(z);
+}
+
+static void print_stage_times(void) {
+    if (flux_verbose)
+        fprintf(stderr, "denoising on device: double %.2f ms, single %.2f ms, final %.2f ms, total %.2f ms\n",
+                flux_timing_transformer_double, flux_timing_transformer_single, flux_timing_transformer_final,
+                flux_timing_transformer_total);
+}
+
 static float *sample_impl(void *transformer, const float *z, int channels, int h, int w,
                           const flux_ref_t *refs, int num_refs,
                           const float *text_emb_cond, int text_seq_cond,
@@ -312,15 +366,100 @@ static float *sample_impl(void *transformer, const float *z, int channels, int h
     for (int i = 0; i < num_steps; i++) {
         if (!flux_hip_session_step(s, i, v_trace ? v_trace + (size_t)i * per_step : NULL)) goto done;
         if (progress) progress(i + 1, num_steps); /* the step has been queued (flux_sample.c:254) */
+        step_image_hook(s, i);
     }
     out = (float *)malloc(s->n_lat * 4);
     if (!out) { flux_hip_fail("out of host memory"); goto done; }
     if (!flux_hip_session_read_latent(s, out)) { free(out); out = NULL; goto done; }
-    if (flux_verbose)
-        fprintf(stderr, "denoising on device: double %.2f ms, single %.2f ms, final %.2f ms, total %.2f ms\n",
-                flux_timing_transformer_double, flux_timing_transformer_single, flux_timing_transformer_final,
-                flux_timing_transformer_total);
+    print_stage_times();
 done:
+    flux_hip_session_free(s);
+    return out;
+}
+
+/* Heun (flux_sample.c:760-826): v1 = f(z, t_i); z' = z + dt v1; v2 = f(z', t_{i+1});
+ * z += dt/2 (v1 + v2); the last step is a plain Euler step. The modulation vectors of t_{i+1}
+ * are those the next step uses, so they exist already. v_trace (optional) receives v1, v2 of
+ * every step in call order: 2 * num_steps - 1 velocities. */
+float *flux_hip_sample_heun_traced(void *transformer, const float *z, int channels, int h, int w,
+                                   const float *text_emb, int text_seq, const float *schedule, int num_steps,
+                                   float *v_trace, void (*progress)(int, int)) {
+    flux_hip_session *s = flux_hip_session_begin(transformer, z, channels, h, w, NULL, 0, text_emb, text_seq, NULL, 0,
+                                                 0.0f, schedule, num_steps);
+    if (!s) return NULL;
+    const size_t n = s->n_lat;
+    float *out = NULL, *z_pred = NULL;
+    size_t k = 0;
+    s->ev = events_begin(2 * num_steps);
+    z_pred = (float *)flux_hip_malloc(n * 4);
+    s->v_u = (float *)flux_hip_malloc(n * 4); /* second velocity; released with the session */
+    if (!z_pred || !s->v_u) goto done;
+    for (int i = 0; i < num_steps; i++) {
+        const float dt = schedule[i + 1] - schedule[i];
+        if (!fh_forward_device(s->tf, s->rp_c, s->z_dev, s->n_target, s->txt_c, i, s->v_c, s->ev)) goto done;
+        if (s->ev) s->ev->used++;
+        if (v_trace && !flux_hip_download(v_trace + (k++) * n, s->v_c, n * 4)) goto done;
+        if (i < num_steps - 1) {
+            if (!flux_hip_euler_predict(z_pred, s->z_dev, s->v_c, dt, n)) goto done;
+            if (!fh_forward_device(s->tf, s->rp_c, z_pred, s->n_target, s->txt_c, i + 1, s->v_u, s->ev)) goto done;
+            if (s->ev) s->ev->used++;
+            if (v_trace && !flux_hip_download(v_trace + (k++) * n, s->v_u, n * 4)) goto done;
+            if (!flux_hip_heun_update(s->z_dev, s->v_c, s->v_u, dt, n)) goto done;
+        } else if (!flux_hip_euler_update(s->z_dev, s->v_c, dt, n)) {
+            goto done;
+        }
+        if (progress) progress(i + 1, num_steps);
+        step_image_hook(s, i);
+    }
+    out = (float *)malloc(n * 4);
+    if (!out) { flux_hip_fail("out of host memory"); goto done; }
+    if (!flux_hip_session_read_latent(s, out)) { free(out); out = NULL; goto done; }
+    print_stage_times();
+done:
+    flux_hip_free(z_pred);
+    flux_hip_session_free(s);
+    return out;
+}
+
+/* Euler with noise injection (flux_sample.c:697-748): after every step but the last,
+ * z += eta sqrt(|dt|) N(0,1). The normals come from the host generator flux_randn, in the
+ * order the reference draws them (nothing else draws during a run), but all at once before the
+ * loop so that the loop itself never waits for the host. */
+float *flux_hip_sample_ancestral_traced(void *transformer, const float *z, int channels, int h, int w,
+                                        const float *text_emb, int text_seq, const float *schedule, int num_steps,
+                                        float eta, float *v_trace, void (*progress)(int, int)) {
+    flux_hip_session *s = flux_hip_session_begin(transformer, z, channels, h, w, NULL, 0, text_emb, text_seq, NULL, 0,
+                                                 0.0f, schedule, num_steps);
+    if (!s) return NULL;
+    const size_t n = s->n_lat;
+    const int draws = (eta > 0 && num_steps > 1) ? num_steps - 1 : 0;
+    float *out = NULL, *noise_dev = NULL;
+    if (draws) {
+        if (n > 0x7fffffff) { flux_hip_fail("ancestral sampler: latent too large"); goto done; }
+        float *noise = (float *)malloc((size_t)draws * n * 4);
+        noise_dev = (float *)flux_hip_malloc((size_t)draws * n * 4);
+        if (!noise || !noise_dev) { free(noise); flux_hip_fail("ancestral sampler: out of memory"); goto done; }
+        for (int i = 0; i < draws; i++) flux_randn(noise + (size_t)i * n, (int)n);
+        int ok = flux_hip_upload(noise_dev, noise, (size_t)draws * n * 4);
+        free(noise);
+        if (!ok) goto done;
+    }
+    for (int i = 0; i < num_steps; i++) {
+        const float dt = schedule[i + 1] - schedule[i];
+        if (!fh_forward_device(s->tf, s->rp_c, s->z_dev, s->n_target, s->txt_c, i, s->v_c, s->ev)) goto done;
+        if (s->ev) s->ev->used++;
+        if (v_trace && !flux_hip_download(v_trace + (size_t)i * n, s->v_c, n * 4)) goto done;
+        if (!flux_hip_euler_update(s->z_dev, s->v_c, dt, n)) goto done;
+        if (i < draws && !flux_hip_euler_update(s->z_dev, noise_dev + (size_t)i * n, eta * sqrtf(fabsf(dt)), n)) goto done;
+        if (progress) progress(i + 1, num_steps);
+        step_image_hook(s, i);
+    }
+    out = (float *)malloc(n * 4);
+    if (!out) { flux_hip_fail("out of host memory"); goto done; }
+    if (!flux_hip_session_read_latent(s, out)) { free(out); out = NULL; goto done; }
+    print_stage_times();
+done:
+    flux_hip_free(noise_dev);
     flux_hip_session_free(s);
     return out;
 }
@@ -400,6 +539,43 @@ float *flux_sample_euler_cfg_with_multi_refs(void *transformer, void *text_encod
     return run(transformer, z, batch, channels, h, w, refs, refs ? num_refs : 0, text_emb_cond, text_seq_cond, text_emb_uncond,
                text_seq_uncond, guidance_scale, schedule, num_steps, progress_callback);
 }
+
+float *flux_sample_heun(void *transformer, float *z, int batch, int channels, int h, int w,
+                        const float *text_emb, int text_seq, const float *schedule, int num_steps,
+                        void (*progress_callback)(int step, int total)) {
+    if (batch != 1) { flux_hip_fail("sampler: batch=%d (the pipeline always passes 1)", batch); return NULL; }
+    return flux_hip_sample_heun_traced(transformer, z, channels, h, w, text_emb, text_seq, schedule, num_steps, NULL,
+                                       progress_callback);
+}
+
+float *flux_sample_euler_ancestral(void *transformer, float *z, int batch, int channels, int h, int w,
+                                   const float *text_emb, int text_seq, const float *schedule, int num_steps,
+                                   float eta, void (*progress_callback)(int step, int total)) {
+    if (batch != 1) { flux_hip_fail("sampler: batch=%d (the pipeline always passes 1)", batch); return NULL; }
+    return flux_hip_sample_ancestral_traced(transformer, z, channels, h, w, text_emb, text_seq, schedule, num_steps, eta,
+                                            NULL, progress_callback);
+}
+
+/* Noise, linear schedule and the Euler sampler in one call (flux_sample.c:891-919). As in the
+ * reference, the first argument is handed to the sampler as the transformer. */
+float *flux_generate_latent(void *ctx_ptr, const float *text_emb, int text_seq, int height, int width, int num_steps,
+                            int64_t seed, void (*progress_callback)(int step, int total)) {
+    const int lh = height / 16, lw = width / 16, channels = 128;
+    if (lh <= 0 || lw <= 0 || num_steps <= 0) { flux_hip_fail("flux_generate_latent: bad sizes"); return NULL; }
+    float *z = flux_init_noise(1, channels, lh, lw, seed);
+    float *schedule = flux_linear_schedule(num_steps);
+    float *latent = (z && schedule) ? flux_sample_euler(ctx_ptr, NULL, z, 1, channels, lh, lw, text_emb, text_seq, schedule,
+                                                        num_steps, progress_callback)
+                                    : NULL;
+    free(z);
+    free(schedule);
+    return latent;
+}
+
+/* Legacy step-progress global kept for source compatibility (flux_sample.c:926-930); the
+ * reference never calls it either. */
+void (*flux_progress_callback)(int, int) = NULL;
+void flux_set_progress_callback(void (*callback)(int, int)) { flux_progress_callback = callback; }
 
 /* One forward = a one-step schedule whose velocity is returned instead of applied
  * (flux_transformer.c:3115, 3605, 3815; used by flux_denoise_step, flux.c:1109). */

@@ -104,8 +104,21 @@ def lib():
     L.flux_hip_session_free.argtypes = [vp]
     L.flux_init_noise.restype = vp
     L.flux_init_noise.argtypes = [c_i, c_i, c_i, c_i, ctypes.c_int64]
-    for n in ("flux_linear_schedule", "flux_power_schedule", "flux_official_schedule"):
+    for n in ("flux_linear_schedule", "flux_power_schedule", "flux_official_schedule", "flux_sigmoid_schedule",
+              "flux_resolution_schedule", "flux_hip_sample_heun_traced", "flux_hip_sample_ancestral_traced",
+              "flux_sample_heun", "flux_sample_euler_ancestral", "flux_generate_latent"):
         getattr(L, n).restype = vp
+    L.flux_sigmoid_schedule.argtypes = [c_i, c_f]
+    L.flux_resolution_schedule.argtypes = [c_i, c_i, c_i]
+    L.flux_hip_sample_heun_traced.argtypes = [vp, vp, c_i, c_i, c_i, vp, c_i, vp, c_i, vp, vp]
+    L.flux_hip_sample_ancestral_traced.argtypes = [vp, vp, c_i, c_i, c_i, vp, c_i, vp, c_i, c_f, vp, vp]
+    L.flux_sample_heun.argtypes = [vp, vp, c_i, c_i, c_i, c_i, vp, c_i, vp, c_i, vp]
+    L.flux_sample_euler_ancestral.argtypes = [vp, vp, c_i, c_i, c_i, c_i, vp, c_i, vp, c_i, c_f, vp]
+    L.flux_generate_latent.argtypes = [vp, vp, c_i, c_i, c_i, c_i, ctypes.c_int64, vp]
+    L.flux_rng_seed.argtypes = [ctypes.c_uint64]
+    L.flux_rng_seed.restype = None
+    L.flux_randn.argtypes = [vp, c_i]
+    L.flux_randn.restype = None
     L.flux_linear_schedule.argtypes = [c_i]
     L.flux_power_schedule.argtypes = [c_i, c_f]
     L.flux_official_schedule.argtypes = [c_i, c_i]
@@ -275,6 +288,38 @@ class Transformer:
         return (out, tr) if trace else out
 
 
+    def sample_heun(self, z, h, w, txt, schedule, trace=False):
+        """Heun sampling loop; the trace holds v1, v2 of every step in call order (2*steps - 1 rows)."""
+        z, txt, schedule = _f32(z), _f32(txt), _f32(schedule)
+        steps = len(schedule) - 1
+        n = self.cfg.channels * h * w
+        tr = np.zeros((max(2 * steps - 1, 0), n), np.float32) if trace else None
+        L = lib()
+        p = L.flux_hip_sample_heun_traced(self.h, z.ctypes.data, self.cfg.channels, h, w, txt.ctypes.data, txt.shape[0],
+                                          schedule.ctypes.data, steps, tr.ctypes.data if trace else None, None)
+        if not p:
+            raise FluxHipError(f"sample_heun: {L.flux_hip_last_error().decode()}")
+        out = _take_host(p, (self.cfg.channels, h, w))
+        return (out, tr) if trace else out
+
+    def sample_ancestral(self, z, h, w, txt, schedule, eta, seed=None, trace=False):
+        """Euler with noise injection; `seed` (if given) seeds the host generator first."""
+        z, txt, schedule = _f32(z), _f32(txt), _f32(schedule)
+        steps = len(schedule) - 1
+        n = self.cfg.channels * h * w
+        tr = np.zeros((steps, n), np.float32) if trace else None
+        L = lib()
+        if seed is not None:
+            L.flux_rng_seed(seed)
+        p = L.flux_hip_sample_ancestral_traced(self.h, z.ctypes.data, self.cfg.channels, h, w, txt.ctypes.data,
+                                               txt.shape[0], schedule.ctypes.data, steps, eta,
+                                               tr.ctypes.data if trace else None, None)
+        if not p:
+            raise FluxHipError(f"sample_ancestral: {L.flux_hip_last_error().decode()}")
+        out = _take_host(p, (self.cfg.channels, h, w))
+        return (out, tr) if trace else out
+
+
 class Session:
     """A device-resident sampling run: begin uploads everything, step() only queues kernels."""
 
@@ -325,12 +370,27 @@ def init_noise(channels, h, w, seed):
     return _take_host(p, (channels, h, w))
 
 
-def schedule(kind, n, arg=None):
+def schedule(kind, n, arg=None, arg2=None):
     L = lib()
     if kind == "linear":
         p = L.flux_linear_schedule(n)
     elif kind == "power":
         p = L.flux_power_schedule(n, arg)
-    else:
+    elif kind == "sigmoid":
+        p = L.flux_sigmoid_schedule(n, arg)
+    elif kind == "resolution":
+        p = L.flux_resolution_schedule(n, arg, arg2)
+    elif kind == "official":
         p = L.flux_official_schedule(n, arg)
+    else:
+        raise ValueError(f"unknown schedule {kind!r}")
     return _take_host(p, (n + 1,))
+
+
+def randn(n, seed=None):
+    """n normals from the library's host generator (seeded first when `seed` is given)."""
+    if seed is not None:
+        lib().flux_rng_seed(seed)
+    out = np.empty(n, np.float32)
+    lib().flux_randn(out.ctypes.data, n)
+    return out

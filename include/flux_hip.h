@@ -147,6 +147,9 @@ int flux_hip_f32_to_bf16(void *out_bf16, const float *in, size_t n);
 int flux_hip_euler_update(float *z, const float *v, float dt, size_t n);
 /* z += dt * (vu + g * (vc - vu))   (flux_sample.c:496-499) */
 int flux_hip_cfg_euler_update(float *z, const float *v_uncond, const float *v_cond, float guidance, float dt, size_t n);
+/* Heun: out = z + dt * v (predictor, flux_sample.c:780-782); z += dt/2 * (v1 + v2) (corrector, :789-792) */
+int flux_hip_euler_predict(float *out, const float *z, const float *v, float dt, size_t n);
+int flux_hip_heun_update(float *z, const float *v1, const float *v2, float dt, size_t n);
 
 /* -------------------------------------------------------------------- model */
 
@@ -223,14 +226,36 @@ float *flux_sample_euler_cfg_with_multi_refs(void *transformer, void *text_encod
                                              const float *schedule, int num_steps,
                                              void (*progress_callback)(int step, int total));
 
-/* Schedules (flux_sample.c:49, 62, 145); malloc'd [num_steps + 1], caller frees. */
+/* Second-order and noise-injecting samplers (flux_sample.c:760, 697): text-only conditioning,
+ * no reference images, as in the reference. Heun runs 2 * num_steps - 1 forwards. The noise of
+ * the ancestral sampler comes from flux_randn in its current state. */
+float *flux_sample_heun(void *transformer, float *z, int batch, int channels, int h, int w,
+                        const float *text_emb, int text_seq, const float *schedule, int num_steps,
+                        void (*progress_callback)(int step, int total));
+float *flux_sample_euler_ancestral(void *transformer, float *z, int batch, int channels, int h, int w,
+                                   const float *text_emb, int text_seq, const float *schedule, int num_steps,
+                                   float eta, void (*progress_callback)(int step, int total));
+
+/* Schedules (flux_sample.c:49, 62, 75, 96, 145); malloc'd [num_steps + 1], caller frees. */
 float *flux_linear_schedule(int num_steps);
 float *flux_power_schedule(int num_steps, float alpha);
+float *flux_sigmoid_schedule(int num_steps, float shift);
+float *flux_resolution_schedule(int num_steps, int height, int width);
 float *flux_official_schedule(int num_steps, int image_seq_len);
 
-/* Initial latent noise from the reference's host RNG (flux_sample.c:837-877); malloc'd
- * [batch, channels, h, w], caller frees. seed < 0 continues the current stream. */
+/* Host generator of the reference (flux_kernels.c:45-102: xoshiro256** seeded through
+ * SplitMix64, Box-Muller), and the initial latent noise drawn from it (flux_sample.c:837-877):
+ * malloc'd [batch, channels, h, w], caller frees; seed < 0 continues the current stream. */
+void flux_rng_seed(uint64_t seed);
+void flux_randn(float *out, int n);
 float *flux_init_noise(int batch, int channels, int h, int w, int64_t seed);
+
+/* Noise + linear schedule + Euler sampler for a height x width image (flux_sample.c:891-919);
+ * the first argument is the transformer. */
+float *flux_generate_latent(void *ctx_ptr, const float *text_emb, int text_seq, int height, int width, int num_steps,
+                            int64_t seed, void (*progress_callback)(int step, int total));
+extern void (*flux_progress_callback)(int, int);
+void flux_set_progress_callback(void (*callback)(int, int));
 
 /* Same sampling loops, additionally copying every forward's velocity (in call order,
  * [forwards, channels*h*w] f32) to v_trace when it is not NULL. For parity tests. */
@@ -239,6 +264,13 @@ float *flux_hip_sample_traced(void *transformer, const float *z, int channels, i
                               const float *text_emb_cond, int text_seq_cond,
                               const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
                               const float *schedule, int num_steps, float *v_trace);
+/* Heun: v_trace holds v1, v2 of every step in call order (2 * num_steps - 1 velocities). */
+float *flux_hip_sample_heun_traced(void *transformer, const float *z, int channels, int h, int w,
+                                   const float *text_emb, int text_seq, const float *schedule, int num_steps,
+                                   float *v_trace, void (*progress)(int, int));
+float *flux_hip_sample_ancestral_traced(void *transformer, const float *z, int channels, int h, int w,
+                                        const float *text_emb, int text_seq, const float *schedule, int num_steps,
+                                        float eta, float *v_trace, void (*progress)(int, int));
 
 /*
  * The sampling loop in pieces, for callers that drive or time the steps themselves. begin()

@@ -16,7 +16,8 @@
  *   fo_timestep_embedding, fo_time_mlp, fo_rope_image, fo_rope_text,
  *   fo_apply_rope, fo_adaln, fo_qk_norm, fo_linear, fo_attention,
  *   fo_double_block, fo_single_block, fo_forward (0/1/2 references),
- *   fo_sample_euler, fo_sample_euler_cfg, schedules, fo_init_noise:
+ *   fo_sample_euler, fo_sample_euler_cfg, fo_sample_heun, fo_sample_euler_ancestral,
+ *   schedules (linear, power, sigmoid, resolution, official), fo_init_noise:
  *   pinned against golden vectors produced by the reference's own C code
  *   compiled from its sources (oracle/ref_probe.c -> oracle/_ref/), and
  *   against closed forms / brute force in tests/test_oracle_math.py.
@@ -686,6 +687,24 @@ void fo_power_schedule(float *s, int n, float alpha) {
     for (int i = 0; i <= n; i++) s[i] = 1.0f - powf((float)i / (float)n, alpha);
 }
 
+/* Shifted sigmoid, endpoints forced to 1 and 0 (flux_sample.c:75-91). */
+void fo_sigmoid_schedule(float *s, int n, float shift) {
+    for (int i = 0; i <= n; i++) {
+        float x = ((float)i / (float)n - 0.5f) * 10.0f + shift;
+        s[i] = 1.0f - 1.0f / (1.0f + expf(-x));
+    }
+    s[0] = 1.0f;
+    s[n] = 0.0f;
+}
+
+/* 1 - (i/n)^(1 + shift/2), shift 1 from 1024x1024 pixels, 0.5 from 512x512, else 0
+ * (flux_sample.c:96-116). */
+void fo_resolution_schedule(float *s, int n, int height, int width) {
+    int pixels = height * width;
+    float shift = pixels >= 1024 * 1024 ? 1.0f : pixels >= 512 * 512 ? 0.5f : 0.0f;
+    for (int i = 0; i <= n; i++) s[i] = 1.0f - powf((float)i / (float)n, 1.0f + shift * 0.5f);
+}
+
 static float empirical_mu(int seq_len, int steps) {
     const float a1 = 8.73809524e-05f, b1 = 1.89833333f;
     const float a2 = 0.00016927f, b2 = 0.45666666f;
@@ -754,6 +773,63 @@ float *fo_sample_euler_cfg(const fo_model *m, const float *z, int h, int w,
         }
         free(vu); free(vc);
     }
+    return zc;
+}
+
+/* Heun (flux_sample.c:760-826): v1 at (z, t_s); predictor zp = z + dt v1; v2 at (zp, t_{s+1});
+ * z += dt/2 (v1 + v2); the last step is a plain Euler step. v_trace gets v1, v2 of every step
+ * in call order (2*num_steps - 1 velocities). */
+float *fo_sample_heun(const fo_model *m, const float *z, int h, int w,
+                      const float *txt, int txt_seq,
+                      const float *schedule, int num_steps, float *v_trace) {
+    int n = m->c.channels * h * w;
+    float *zc = (float *)malloc(sizeof(float) * n);
+    float *zp = (float *)malloc(sizeof(float) * n);
+    memcpy(zc, z, sizeof(float) * n);
+    size_t k = 0;
+    for (int s = 0; s < num_steps; s++) {
+        float dt = schedule[s + 1] - schedule[s];
+        float *v1 = fo_forward(m, zc, h, w, NULL, 0, txt, txt_seq, schedule[s]);
+        if (v_trace) memcpy(v_trace + (k++) * n, v1, sizeof(float) * n);
+        if (s < num_steps - 1) {
+            for (int i = 0; i < n; i++) zp[i] = zc[i] + dt * v1[i];
+            float *v2 = fo_forward(m, zp, h, w, NULL, 0, txt, txt_seq, schedule[s + 1]);
+            if (v_trace) memcpy(v_trace + (k++) * n, v2, sizeof(float) * n);
+            for (int i = 0; i < n; i++) zc[i] += 0.5f * dt * (v1[i] + v2[i]);
+            free(v2);
+        } else {
+            for (int i = 0; i < n; i++) zc[i] += dt * v1[i];
+        }
+        free(v1);
+    }
+    free(zp);
+    return zc;
+}
+
+void fo_randn(float *out, int64_t n);
+
+/* Euler with noise injection (flux_sample.c:697-748): after every step but the last,
+ * z += eta sqrt(|dt|) * N(0,1) drawn from the global generator in its current state. */
+float *fo_sample_euler_ancestral(const fo_model *m, const float *z, int h, int w,
+                                 const float *txt, int txt_seq,
+                                 const float *schedule, int num_steps, float eta, float *v_trace) {
+    int n = m->c.channels * h * w;
+    float *zc = (float *)malloc(sizeof(float) * n);
+    float *noise = (float *)malloc(sizeof(float) * n);
+    memcpy(zc, z, sizeof(float) * n);
+    for (int s = 0; s < num_steps; s++) {
+        float dt = schedule[s + 1] - schedule[s];
+        float *v = fo_forward(m, zc, h, w, NULL, 0, txt, txt_seq, schedule[s]);
+        if (v_trace) memcpy(v_trace + (size_t)s * n, v, sizeof(float) * n);
+        for (int i = 0; i < n; i++) zc[i] += dt * v[i];
+        if (eta > 0 && s < num_steps - 1) {
+            float sigma = eta * sqrtf(fabsf(dt));
+            fo_randn(noise, n);
+            for (int i = 0; i < n; i++) zc[i] += sigma * noise[i];
+        }
+        free(v);
+    }
+    free(noise);
     return zc;
 }
 

@@ -53,6 +53,10 @@ def lib():
     L.fo_sample_euler.restype = vp
     L.fo_sample_euler_cfg.argtypes = [vp, vp, c_i, c_i, vp, c_i, vp, c_i, vp, c_i, c_f, vp, c_i, vp]
     L.fo_sample_euler_cfg.restype = vp
+    L.fo_sample_heun.argtypes = [vp, vp, c_i, c_i, vp, c_i, vp, c_i, vp]
+    L.fo_sample_heun.restype = vp
+    L.fo_sample_euler_ancestral.argtypes = [vp, vp, c_i, c_i, vp, c_i, vp, c_i, c_f, vp]
+    L.fo_sample_euler_ancestral.restype = vp
     L.fo_double_block.argtypes = [vp, c_i, vp, vp, vp, vp, vp, vp, vp, vp, c_i, c_i]
     L.fo_single_block.argtypes = [vp, c_i, vp, vp, vp, vp, vp, vp, c_i, c_i]
     L.fo_timestep_embedding.argtypes = [vp, c_f, c_i, c_f]
@@ -70,6 +74,8 @@ def lib():
     L.fo_linear_schedule.argtypes = [vp, c_i]
     L.fo_power_schedule.argtypes = [vp, c_i, c_f]
     L.fo_official_schedule.argtypes = [vp, c_i, c_i]
+    L.fo_sigmoid_schedule.argtypes = [vp, c_i, c_f]
+    L.fo_resolution_schedule.argtypes = [vp, c_i, c_i, c_i]
     L.fo_init_noise.argtypes = [vp, c_i, c_i, c_i, ctypes.c_int64]
     L.fo_rng_seed.argtypes = [ctypes.c_uint64]
     L.fo_randn.argtypes = [vp, ctypes.c_int64]
@@ -170,6 +176,30 @@ class Oracle:
         p = lib().fo_sample_euler_cfg(self.h, z.ctypes.data, h, w, arr, nr, tc.ctypes.data, tc.shape[0],
                                       tu.ctypes.data, tu.shape[0], guidance, schedule.ctypes.data, steps,
                                       tr.ctypes.data if trace else None)
+        out = self._take(p, n).reshape(self.cfg.channels, h, w)
+        return (out, tr) if trace else out
+
+    def sample_heun(self, z, h, w, txt, schedule, trace=False):
+        """Heun sampler; the trace holds v1, v2 of every step in call order (2*steps - 1 rows)."""
+        z, txt, schedule = _f32(z), _f32(txt), _f32(schedule)
+        steps = len(schedule) - 1
+        n = self.cfg.channels * h * w
+        tr = np.zeros((max(2 * steps - 1, 0), n), np.float32) if trace else None
+        p = lib().fo_sample_heun(self.h, z.ctypes.data, h, w, txt.ctypes.data, txt.shape[0],
+                                 schedule.ctypes.data, steps, tr.ctypes.data if trace else None)
+        out = self._take(p, n).reshape(self.cfg.channels, h, w)
+        return (out, tr) if trace else out
+
+    def sample_euler_ancestral(self, z, h, w, txt, schedule, eta, seed=None, trace=False):
+        """Euler with noise injection; `seed` (if given) seeds the oracle's generator first."""
+        z, txt, schedule = _f32(z), _f32(txt), _f32(schedule)
+        steps = len(schedule) - 1
+        n = self.cfg.channels * h * w
+        if seed is not None:
+            lib().fo_rng_seed(seed)
+        tr = np.zeros((steps, n), np.float32) if trace else None
+        p = lib().fo_sample_euler_ancestral(self.h, z.ctypes.data, h, w, txt.ctypes.data, txt.shape[0],
+                                            schedule.ctypes.data, steps, eta, tr.ctypes.data if trace else None)
         out = self._take(p, n).reshape(self.cfg.channels, h, w)
         return (out, tr) if trace else out
 
@@ -284,6 +314,18 @@ def power_schedule(n, alpha):
 def official_schedule(n, image_seq_len):
     s = np.empty(n + 1, np.float32)
     lib().fo_official_schedule(s.ctypes.data, n, image_seq_len)
+    return s
+
+
+def sigmoid_schedule(n, shift):
+    s = np.empty(n + 1, np.float32)
+    lib().fo_sigmoid_schedule(s.ctypes.data, n, shift)
+    return s
+
+
+def resolution_schedule(n, height, width):
+    s = np.empty(n + 1, np.float32)
+    lib().fo_resolution_schedule(s.ctypes.data, n, height, width)
     return s
 
 

@@ -46,7 +46,9 @@ def load():
                  "flux_sample_euler_with_refs", "flux_sample_euler_with_multi_refs",
                  "flux_sample_euler_cfg", "flux_sample_euler_cfg_with_refs",
                  "flux_sample_euler_cfg_with_multi_refs", "flux_linear_schedule",
-                 "flux_power_schedule", "flux_official_schedule", "flux_init_noise"):
+                 "flux_power_schedule", "flux_official_schedule", "flux_init_noise",
+                 "flux_sigmoid_schedule", "flux_resolution_schedule", "flux_sample_heun",
+                 "flux_sample_euler_ancestral"):
         getattr(L, name).restype = vp
     L.flux_transformer_forward.argtypes = [vp, vp, c_i, c_i, vp, c_i, c_f]
     L.flux_transformer_forward_with_refs.argtypes = [vp, vp, c_i, c_i, vp, c_i, c_i, c_i, vp, c_i, c_f]
@@ -59,6 +61,10 @@ def load():
                                                   vp, c_i, vp, c_i, c_f, vp, c_i, vp]
     L.flux_sample_euler_cfg_with_multi_refs.argtypes = [vp, vp, vp, c_i, c_i, c_i, c_i, vp, c_i,
                                                         vp, c_i, vp, c_i, c_f, vp, c_i, vp]
+    L.flux_sample_heun.argtypes = [vp, vp, c_i, c_i, c_i, c_i, vp, c_i, vp, c_i, vp]
+    L.flux_sample_euler_ancestral.argtypes = [vp, vp, c_i, c_i, c_i, c_i, vp, c_i, vp, c_i, c_f, vp]
+    L.flux_sigmoid_schedule.argtypes = [c_i, c_f]
+    L.flux_resolution_schedule.argtypes = [c_i, c_i, c_i]
     L.flux_linear_schedule.argtypes = [c_i]
     L.flux_power_schedule.argtypes = [c_i, c_f]
     L.flux_official_schedule.argtypes = [c_i, c_i]
@@ -118,6 +124,8 @@ def refs_array(refs):
 
 # Seeds / shapes shared with tests/test_oracle_golden.py -------------------------------------------
 SEED = 7
+ANCESTRAL_SEED = 99     # flux_rng_seed() value set right before the ancestral sampler runs
+ANCESTRAL_ETA = 0.7
 
 
 def case_inputs(cfg):
@@ -187,6 +195,10 @@ def ops_golden():
     g["sched_power_5_2"] = take(L.flux_power_schedule(5, 2.0), (6,))
     for n, sl in ((4, 256), (4, 1024), (4, 4096), (50, 1024), (4, 5000), (1, 16), (28, 4300)):
         g[f"sched_official_{n}_{sl}"] = take(L.flux_official_schedule(n, sl), (n + 1,))
+    for n, sh in ((4, 0.0), (7, 1.5), (1, -2.0)):
+        g[f"sched_sigmoid_{n}_{sh}"] = take(L.flux_sigmoid_schedule(n, sh), (n + 1,))
+    for n, hh, ww in ((4, 256, 256), (6, 512, 512), (5, 1024, 1024), (3, 2048, 256), (4, 768, 1024)):
+        g[f"sched_resolution_{n}_{hh}_{ww}"] = take(L.flux_resolution_schedule(n, hh, ww), (n + 1,))
     # rng + noise
     L.flux_rng_seed(42); o = np.empty(64, np.float32); L.flux_randn(P(o), 64); g["randn_42"] = o
     g["noise_42_4x4"] = take(L.flux_init_noise(1, 128, 4, 4, 42), (128, 4, 4))
@@ -254,6 +266,16 @@ def model_golden(cfg, qk):
     g["cfg2_ref2"] = take(L.flux_sample_euler_cfg_with_multi_refs(m, None, P(z), 1, cfg.channels, 4, 4, ra, 2,
                                                                   P(txt), 16, P(txt_u), 12, 4.0, P(s3), 2, None),
                           (cfg.channels, 4, 4))
+    # second-order and stochastic samplers (no reference-image variants exist for these)
+    g["heun3"] = take(L.flux_sample_heun(m, P(z), 1, cfg.channels, 4, 4, P(txt), 16, P(s3), 3, None),
+                      (cfg.channels, 4, 4))
+    g["heun1"] = take(L.flux_sample_heun(m, P(z), 1, cfg.channels, 4, 4, P(txt), 16, P(s3), 1, None),
+                      (cfg.channels, 4, 4))
+    L.flux_rng_seed(ANCESTRAL_SEED)
+    g["ancestral3"] = take(L.flux_sample_euler_ancestral(m, P(z), 1, cfg.channels, 4, 4, P(txt), 16, P(s3), 3,
+                                                         ANCESTRAL_ETA, None), (cfg.channels, 4, 4))
+    g["ancestral3_eta0"] = take(L.flux_sample_euler_ancestral(m, P(z), 1, cfg.channels, 4, 4, P(txt), 16, P(s3), 3,
+                                                              0.0, None), (cfg.channels, 4, 4))
     L.ref_model_free(m)
     return g
 

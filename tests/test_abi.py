@@ -37,6 +37,18 @@ def test_schedules_match_reference_golden(golden_dir):
     np.testing.assert_allclose(fluxhip.schedule("power", 5, 2.0), g["sched_power_5_2"], atol=1e-7)
     for n, sl in ((4, 256), (4, 1024), (4, 4096), (50, 1024), (4, 5000), (1, 16), (28, 4300)):
         np.testing.assert_allclose(fluxhip.schedule("official", n, sl), g[f"sched_official_{n}_{sl}"], atol=6e-7)   # a few fp32 ulp: expf/powf vs the -ffast-math build
+    for n, sh in ((4, 0.0), (7, 1.5), (1, -2.0)):
+        np.testing.assert_allclose(fluxhip.schedule("sigmoid", n, sh), g[f"sched_sigmoid_{n}_{sh}"], atol=6e-7)
+    for n, hh, ww in ((4, 256, 256), (6, 512, 512), (5, 1024, 1024), (3, 2048, 256), (4, 768, 1024)):
+        np.testing.assert_allclose(fluxhip.schedule("resolution", n, hh, ww), g[f"sched_resolution_{n}_{hh}_{ww}"], atol=6e-7)
+
+
+def test_host_generator_matches_reference_golden(golden_dir):
+    g = np.load(os.path.join(golden_dir, "ops.npz"))
+    np.testing.assert_allclose(fluxhip.randn(64, seed=42), g["randn_42"], atol=1e-6)
+    a = fluxhip.randn(8)                              # continues the stream
+    assert not np.array_equal(a, g["randn_42"][:8])
+    np.testing.assert_allclose(fluxhip.randn(64, seed=42), g["randn_42"], atol=1e-6)
 
 
 def test_init_noise_matches_reference_golden(golden_dir):

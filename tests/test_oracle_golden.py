@@ -101,6 +101,10 @@ def test_schedules(oracle_mod, ops):
     np.testing.assert_allclose(oracle_mod.power_schedule(5, 2.0), ops["sched_power_5_2"], atol=1e-7)
     for n, sl in ((4, 256), (4, 1024), (4, 4096), (50, 1024), (4, 5000), (1, 16), (28, 4300)):
         np.testing.assert_allclose(oracle_mod.official_schedule(n, sl), ops[f"sched_official_{n}_{sl}"], atol=2e-7)
+    for n, sh in ((4, 0.0), (7, 1.5), (1, -2.0)):
+        np.testing.assert_allclose(oracle_mod.sigmoid_schedule(n, sh), ops[f"sched_sigmoid_{n}_{sh}"], atol=2e-7)
+    for n, hh, ww in ((4, 256, 256), (6, 512, 512), (5, 1024, 1024), (3, 2048, 256), (4, 768, 1024)):
+        np.testing.assert_allclose(oracle_mod.resolution_schedule(n, hh, ww), ops[f"sched_resolution_{n}_{hh}_{ww}"], atol=2e-7)
 
 
 def test_rng_and_noise(oracle_mod, ops):
@@ -168,6 +172,14 @@ def test_tiny_model(oracle_mod, golden_dir, qk):
     close(m.sample_euler_cfg(d["lat"], 4, 4, d["txt"], d["txt_u"], 4.0, s3[:3]), g["cfg2"])
     close(m.sample_euler_cfg(d["lat"], 4, 4, d["txt"], d["txt_u"], 4.0, s3[:3], refs=[r1]), g["cfg2_ref1"])
     close(m.sample_euler_cfg(d["lat"], 4, 4, d["txt"], d["txt_u"], 4.0, s3[:3], refs=[r1, r2]), g["cfg2_ref2"])
+    # Heun (a one-step run is plain Euler) and the noise-injecting sampler; for the latter the reference's
+    # generator was seeded with 99 right before the call and eta was 0.7 (tests/golden/make_golden.py)
+    close(m.sample_heun(d["lat"], 4, 4, d["txt"], s3), g["heun3"])
+    close(m.sample_heun(d["lat"], 4, 4, d["txt"], s3[:2]), g["heun1"])
+    close(m.sample_euler_ancestral(d["lat"], 4, 4, d["txt"], s3, 0.7, seed=99), g["ancestral3"])
+    close(m.sample_euler_ancestral(d["lat"], 4, 4, d["txt"], s3, 0.0), g["ancestral3_eta0"])
+    close(g["ancestral3_eta0"], g["euler3"])
+    assert rel_l2(g["heun3"], g["euler3"]) > 1e-4 and rel_l2(g["ancestral3"], g["euler3"]) > 1e-2
     m.close()
 
 
