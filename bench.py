@@ -202,7 +202,7 @@ def main():
         alone_ms, _ = time_dominant_kernel(cfg, n_img + nt)
         roof = {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES.get(args.workload),
-                "kernel": "gemm_kernel<256,256,2,4,SWIGLU> (gate/up projection + SiLU*up)",
+                "kernel": "gemm256_kernel<SWIGLU> (gate/up projection + SiLU*up; 256x256 tile, 4 waves)",
                 "launches_timed": k_n.value, "ms_per_launch": round(per_ms, 4), "flops_per_launch": k_flops,
                 "ms_per_launch_back_to_back": round(alone_ms, 4)}
     model.close()

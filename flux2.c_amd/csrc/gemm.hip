@@ -18,6 +18,17 @@
  * so that in the accumulator a lane holds one token (m) and four consecutive output features
  * (n): epilogues use 8/16-byte accesses and pair gate/up columns inside a lane.
  *
+ * Two kernels share the tile decode and the epilogues. gemm_kernel<BM,BN,WGM,WGN> (8 or 4
+ * waves, two waves per SIMD) serves the small tiles. gemm256_kernel is the 256 x 256 tile for the
+ * large projections: 4 waves, one per SIMD, each owning 128 x 128 of the tile with its 256
+ * accumulator registers pinned to AGPRs. A 128 x 128 wave tile needs 16 fragment reads per 64
+ * MFMAs instead of 12 per 32, i.e. a third less LDS traffic per FLOP, which under the power
+ * limit is what buys throughput (1020 -> 1145 TFLOP/s sustained back to back on the
+ * 4608 x 18432 x 3072 projection). With a single wave per SIMD nothing hides latency for free,
+ * so the loop is software-pipelined by hand: fragments are double-buffered in registers, every
+ * fourth MFMA is followed by one LDS read for the next half-step and (in the second half) one
+ * global->LDS load for the stage after next, and there is one barrier per 64-wide K step.
+ *
  * LDS rows are 128 bytes (64 bf16); the 16-byte chunk index is XOR-swizzled with a function of
  * the row so that the 16 rows a fragment read touches spread over all banks. A direct-to-LDS
  * load writes lane i's 16 bytes at (wave base + 16 i), so the swizzle is applied on the global
@@ -52,6 +63,92 @@ __device__ __forceinline__ int lds_swz(int r) { return ((r >> 1) & 7) ^ ((r & 1)
 /* s_waitcnt vmcnt(0) only (expcnt and lgkmcnt fields left at their maxima) */
 #define WAIT_VMCNT0() __builtin_amdgcn_s_waitcnt(0x0F70)
 
+/* Which tile (and K slice) a workgroup owns. Workgroups are dealt round-robin to the 8 XCDs;
+ * each XCD gets a contiguous run of tiles so that its L2 sees the reuse, and tiles are walked in
+ * groups of GROUP_M rows. */
+struct TileId {
+    int ks, tm, tn, prob, tml;
+};
+__device__ __forceinline__ bool decode_tile(const GemmArgs &g, TileId &t) {
+    int nb = gridDim.x;
+    int per_xcd = nb >> 3;
+    int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if (logical >= g.total_tiles * g.ksplit) return false;
+    t.ks = logical / g.total_tiles;
+    logical -= t.ks * g.total_tiles;
+    int per_group = GROUP_M * g.ntiles;
+    int grp = logical / per_group;
+    int first_m = grp * GROUP_M;
+    int gsz = min(g.mtiles - first_m, GROUP_M);
+    int in_grp = logical - grp * per_group;
+    t.tm = first_m + in_grp % gsz;
+    t.tn = in_grp / gsz;
+    t.prob = t.tm >= g.mtiles0 ? 1 : 0;
+    t.tml = t.prob ? t.tm - g.mtiles0 : t.tm;
+    return true;
+}
+
+/* Weight row that feeds column v of the tile. For the SwiGLU epilogue 16-column blocks alternate
+ * gate, up so that a lane ends up holding matching pairs. */
+template <int BN, int WN, int EPI>
+__device__ __forceinline__ int weight_row(const GemmArgs &g, int tn, int v) {
+    if (EPI == FLUX_HIP_EPI_SWIGLU) {
+        int wv = v / WN, blk = (v % WN) >> 4;
+        int idx = wv * (WN / 2) + (blk >> 1) * 16 + (v & 15);
+        return ((blk & 1) ? g.w_row1 : g.w_row0) + tn * (BN / 2) + idx;
+    }
+    return g.w_row0 + tn * BN + v;
+}
+
+/* Accumulator element e of block (i, j): feature n = 4*(lane/16) + e of the 16-column block,
+ * token m = lane%16 of the 16-row block. */
+template <int BN, int WM, int WN, int EPI>
+__device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f32x4 (&acc)[WN / 16][WM / 16], int m0, int M,
+                                           int wm, int wn, int l15, int lq) {
+    constexpr int TM = WM / 16, TN = WN / 16;
+    const int ldc = g.ldc, prob = t.prob, tn = t.tn, n0 = tn * BN, ks = t.ks;
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+        const int m = m0 + wm * WM + j * 16 + l15;
+        if (m >= M) continue;
+        if (EPI == FLUX_HIP_EPI_SWIGLU) {
+            bf16 *C = (bf16 *)g.C[prob] + (size_t)m * ldc + tn * (BN / 2) + wn * (WN / 2) + lq * 4;
+#pragma unroll
+            for (int i = 0; i < TN; i += 2) {
+                bf16x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[e] = (bf16)(silu_f(acc[i][j][e]) * acc[i + 1][j][e]);
+                *(bf16x4 *)(C + (i >> 1) * 16) = o;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < TN; i++) {
+                const int n = n0 + wn * WN + i * 16 + lq * 4;
+                if (EPI == FLUX_HIP_EPI_BF16) {
+                    bf16x4 o;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o[e] = (bf16)acc[i][j][e];
+                    *(bf16x4 *)((bf16 *)g.C[prob] + (size_t)m * ldc + n) = o;
+                } else if (EPI == EPI_PARTIAL) {
+                    *(f32x4 *)(g.ws + ((size_t)ks * g.ws_rows + g.moff[prob] + m) * g.N + n) = acc[i][j];
+                } else if (EPI == FLUX_HIP_EPI_F32) {
+                    *(f32x4 *)((float *)g.C[prob] + (size_t)m * ldc + n) = acc[i][j];
+                } else if (EPI == FLUX_HIP_EPI_F32_T) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) ((float *)g.C[prob])[(size_t)(n + e) * ldc + m] = acc[i][j][e];
+                } else if (EPI == FLUX_HIP_EPI_RESID) {
+                    float *p = (float *)g.C[prob] + (size_t)m * ldc + n;
+                    f32x4 x = *(f32x4 *)p;
+                    f32x4 gt = *(const f32x4 *)(g.gate[prob] + n);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) x[e] += gt[e] * acc[i][j][e];
+                    *(f32x4 *)p = x;
+                }
+            }
+        }
+    }
+}
+
 template <int BM, int BN, int WGM, int WGN, int EPI>
 __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
     constexpr int T = WGM * WGN * 64;
@@ -63,28 +160,13 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
     static_assert(EPI != FLUX_HIP_EPI_SWIGLU || (TN % 2 == 0), "swiglu pairs 16-column blocks");
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
-    /* Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous run of tiles
-     * so that its L2 sees the reuse, then walk tiles in groups of GROUP_M rows. */
-    int nb = gridDim.x;
-    int per_xcd = nb >> 3;
-    int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if (logical >= g.total_tiles * g.ksplit) return;
-    const int ks = logical / g.total_tiles;
-    logical -= ks * g.total_tiles;
-    int per_group = GROUP_M * g.ntiles;
-    int grp = logical / per_group;
-    int first_m = grp * GROUP_M;
-    int gsz = min(g.mtiles - first_m, GROUP_M);
-    int in_grp = logical - grp * per_group;
-    int tm = first_m + in_grp % gsz;
-    int tn = in_grp / gsz;
-
-    int prob = tm >= g.mtiles0 ? 1 : 0;
-    int tml = prob ? tm - g.mtiles0 : tm;
+    TileId t;
+    if (!decode_tile(g, t)) return;
+    const int ks = t.ks, tn = t.tn, prob = t.prob;
     const bf16 *__restrict__ A = g.A[prob];
     const bf16 *__restrict__ W = g.W[prob];
     const int M = g.M[prob];
-    const int m0 = tml * BM, n0 = tn * BN;
+    const int m0 = t.tml * BM;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -105,15 +187,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
 #pragma unroll
     for (int i = 0; i < PB; i++) {
         int v = lrow + i * RPP; /* column of the tile */
-        int wrow;
-        if (EPI == FLUX_HIP_EPI_SWIGLU) {
-            /* 16-column blocks alternate gate, up so a lane ends up holding matching pairs */
-            int wv = v / WN, blk = (v % WN) >> 4;
-            int idx = wv * (WN / 2) + (blk >> 1) * 16 + (v & 15);
-            wrow = ((blk & 1) ? g.w_row1 : g.w_row0) + tn * (BN / 2) + idx;
-        } else {
-            wrow = g.w_row0 + n0 + v;
-        }
+        int wrow = weight_row<BN, WN, EPI>(g, tn, v);
         b_ptr[i] = W + (size_t)wrow * g.ldw + ((lchunk ^ lds_swz(v)) << 3);
         b_lds[i] = BM * 128 + (wave * 8 + i * RPP) * 128;
     }
@@ -167,49 +241,127 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
         }
     }
 
-    /* Accumulator element e of block (i, j): feature n = 4*(lane/16) + e of the 16-column
-     * block, token m = lane%16 of the 16-row block. */
-    const int ldc = g.ldc;
+    store_tile<BN, WM, WN, EPI>(g, t, acc, m0, M, wm, wn, l15, lq);
+}
+
+/* The 256 x 256 tile: 4 waves (2 x 2), 128 x 128 per wave, see the file comment. The MFMA is
+ * issued through inline asm so that the accumulator stays in one AGPR quad for the whole loop
+ * (left to the register allocator, accumulators migrate between VGPRs and AGPRs with hundreds of
+ * copies per K step). Statements with side effects keep their program order, which is what
+ * places the LDS reads and global->LDS loads between the MFMAs. */
+#define MFMA_AGPR(acc, a, b) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b))
+
+template <bool V> struct BoolC { static constexpr bool value = V; };
+
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
+    constexpr int BM = 256, BN = 256, WGN = 2, WM = 128, WN = 128, TM = 8, TN = 8;
+    constexpr int RPP = 32, PA = 8, PB = 8, STAGE = (BM + BN) * 128;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    TileId t;
+    if (!decode_tile(g, t)) return;
+    const int tn = t.tn, prob = t.prob;
+    const bf16 *__restrict__ A = g.A[prob];
+    const bf16 *__restrict__ W = g.W[prob];
+    const int M = g.M[prob];
+    const int m0 = t.tml * BM;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int lrow = tid >> 3, lchunk = tid & 7;
+
+    /* Per-lane global sources, K offset of this slice included. Rows RPP apart share a swizzle. */
+    const int kt_begin = t.ks * g.kt_per;
+    const int KT = min(g.K >> 6, kt_begin + g.kt_per) - kt_begin;
+    const int chunk = ((lchunk ^ lds_swz(lrow)) << 3) + kt_begin * 64;
+    const bf16 *src[PA + PB];
 #pragma unroll
-    for (int j = 0; j < TM; j++) {
-        const int m = m0 + wm * WM + j * 16 + l15;
-        if (m >= M) continue;
-        if (EPI == FLUX_HIP_EPI_SWIGLU) {
-            bf16 *C = (bf16 *)g.C[prob] + (size_t)m * ldc + tn * (BN / 2) + wn * (WN / 2) + lq * 4;
+    for (int i = 0; i < PA; i++) src[i] = A + (size_t)min(m0 + lrow + i * RPP, M - 1) * g.lda + chunk;
 #pragma unroll
-            for (int i = 0; i < TN; i += 2) {
-                bf16x4 o;
+    for (int i = 0; i < PB; i++) src[PA + i] = W + (size_t)weight_row<BN, WN, EPI>(g, tn, lrow + i * RPP) * g.ldw + chunk;
+    static_assert(PA * RPP == BM, "load i of a stage lands at tile row wave*8 + i*RPP: activation rows, then weight rows");
+    auto issue1 = [&](int kt, int stage, int i) {
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src[i] + kt * 64),
+                                         LDS_PTR(smem + stage * STAGE + (wave * 8 + i * RPP) * 128),
+                                         16, 0, 0);
+    };
 #pragma unroll
-                for (int e = 0; e < 4; e++) o[e] = (bf16)(silu_f(acc[i][j][e]) * acc[i + 1][j][e]);
-                *(bf16x4 *)(C + (i >> 1) * 16) = o;
-            }
-        } else {
+    for (int i = 0; i < PA + PB; i++) issue1(0, 0, i);
+
+    f32x4 acc[TN][TM];
 #pragma unroll
-            for (int i = 0; i < TN; i++) {
-                const int n = n0 + wn * WN + i * 16 + lq * 4;
-                if (EPI == FLUX_HIP_EPI_BF16) {
-                    bf16x4 o;
+    for (int i = 0; i < TN; i++)
 #pragma unroll
-                    for (int e = 0; e < 4; e++) o[e] = (bf16)acc[i][j][e];
-                    *(bf16x4 *)((bf16 *)g.C[prob] + (size_t)m * ldc + n) = o;
-                } else if (EPI == EPI_PARTIAL) {
-                    *(f32x4 *)(g.ws + ((size_t)ks * g.ws_rows + g.moff[prob] + m) * g.N + n) = acc[i][j];
-                } else if (EPI == FLUX_HIP_EPI_F32) {
-                    *(f32x4 *)((float *)g.C[prob] + (size_t)m * ldc + n) = acc[i][j];
-                } else if (EPI == FLUX_HIP_EPI_F32_T) {
+        for (int j = 0; j < TM; j++)
 #pragma unroll
-                    for (int e = 0; e < 4; e++) ((float *)g.C[prob])[(size_t)(n + e) * ldc + m] = acc[i][j][e];
-                } else if (EPI == FLUX_HIP_EPI_RESID) {
-                    float *p = (float *)g.C[prob] + (size_t)m * ldc + n;
-                    f32x4 x = *(f32x4 *)p;
-                    f32x4 gt = *(const f32x4 *)(g.gate[prob] + n);
+            for (int e = 0; e < 4; e++) acc[i][j][e] = 0.0f;
+
+    const int l15 = lane & 15, lq = lane >> 4;
+    const int swzl = lds_swz(l15);
+    const int a_frag = (wm * WM + l15) * 128;
+    const int b_frag = BM * 128 + (wn * WN + l15) * 128;
+    const int coff0 = (lq ^ swzl) << 4, coff1 = ((4 + lq) ^ swzl) << 4;
+    /* fragment q of a half-step: 0..7 weight side (MFMA A operand), 8..15 activation side */
+    auto frag = [&](const char *st, int coff, int q) -> bf16x8 {
+        return q < TN ? *(const bf16x8 *)(st + b_frag + q * 2048 + coff) : *(const bf16x8 *)(st + a_frag + (q - TN) * 2048 + coff);
+    };
+    bf16x8 f0[TN + TM], f1[TN + TM];
+
+    WAIT_VMCNT0();
+    __syncthreads();
+    if (KT > 1) {
 #pragma unroll
-                    for (int e = 0; e < 4; e++) x[e] += gt[e] * acc[i][j][e];
-                    *(f32x4 *)p = x;
-                }
+        for (int i = 0; i < PA + PB; i++) issue1(1, 1, i);
+    }
+#pragma unroll
+    for (int q = 0; q < TN + TM; q++) f0[q] = frag(smem, coff0, q);
+
+    auto step = [&](int kt, auto more_c, auto more2_c) {
+        constexpr bool more = decltype(more_c)::value, more2 = decltype(more2_c)::value;
+        const int cur = kt & 1;
+        const char *st = smem + cur * STAGE;
+        const char *nx = smem + (cur ^ 1) * STAGE;
+        /* first K half of the stage from f0, while the second half's fragments arrive in f1 */
+#pragma unroll
+        for (int q = 0; q < 16; q++) {
+            f1[q] = frag(st, coff1, q);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int b = q * 4 + r, j = b >> 3, i = b & 7;
+                MFMA_AGPR(acc[i][j], f0[i], f0[TN + j]);
             }
         }
+        if (more) {
+            /* the next stage has landed for this wave; past the barrier it has for all, and
+             * everyone has finished reading this stage, which is refilled below */
+            WAIT_VMCNT0();
+            __syncthreads();
+        }
+#pragma unroll
+        for (int q = 0; q < 16; q++) {
+            if (more) f0[q] = frag(nx, coff0, q);
+            if (more2) issue1(kt + 2, cur, q);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int b = q * 4 + r, j = b >> 3, i = b & 7;
+                MFMA_AGPR(acc[i][j], f1[i], f1[TN + j]);
+            }
+        }
+    };
+    int kt = 0;
+    for (; kt < KT - 2; kt++) step(kt, BoolC<true>{}, BoolC<true>{});
+    if (kt < KT - 1) {
+        step(kt, BoolC<true>{}, BoolC<false>{});
+        kt++;
     }
+    step(kt, BoolC<false>{}, BoolC<false>{});
+    /* the MFMAs above are opaque to the compiler's hazard handling: let the last results retire
+     * before the accumulators are read */
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+
+    store_tile<BN, WM, WN, EPI>(g, t, acc, m0, M, wm, wn, l15, lq);
 }
 
 /* ------------------------------------------------------------------ host side */
@@ -236,9 +388,30 @@ static int launch_cfg(GemmArgs &g) {
 }
 
 template <int EPI>
+static int launch_256(GemmArgs &g) {
+    constexpr int LDS = 2 * 512 * 128;
+    static bool attr_done = false;
+    auto kern = gemm256_kernel<EPI>;
+    if (!attr_done) {
+        HIP_OK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+        attr_done = true;
+    }
+    g.mtiles0 = (g.M[0] + 255) / 256;
+    int mt1 = g.M[1] > 0 ? (g.M[1] + 255) / 256 : 0;
+    g.mtiles = g.mtiles0 + mt1;
+    g.ntiles = g.N / 256;
+    g.total_tiles = g.mtiles * g.ntiles;
+    int grid = (g.total_tiles * g.ksplit + 7) & ~7;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), LDS, flux_hip_stream_handle(), g);
+    HIP_OK(hipGetLastError());
+    return 1;
+}
+
+template <int EPI>
 static int launch_epi(GemmArgs &g, int tile) {
     switch (tile) {
-        case 2: return launch_cfg<256, 256, 2, 4, EPI>(g);
+        case 2: return launch_256<EPI>(g);
+        case 4: return launch_cfg<256, 256, 2, 4, EPI>(g); /* 8-wave form of the same tile, for comparison runs */
         case 1: return launch_cfg<128, 128, 2, 2, EPI>(g);
         case 3: return launch_cfg<64, 64, 2, 2, EPI>(g);
         default: return launch_cfg<64, 128, 2, 2, EPI>(g);
@@ -382,7 +555,7 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
         for (int i = 0; i < np; i++) rows += g.M[i];
         for (int t = 0; t < 4; t++) {
             if (N % bn[t]) continue;
-            if (g_force_tile >= 0 && t != g_force_tile) continue;
+            if (g_force_tile >= 0 && t != (g_force_tile == 4 ? 2 : g_force_tile)) continue;
             long tiles = 0;
             for (int i = 0; i < np; i++) tiles += (g.M[i] + bm[t] - 1) / bm[t];
             tiles *= N / bn[t];
@@ -406,6 +579,7 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
             }
         }
     }
+    if (g_force_tile == 4 && tile == 2) tile = 4;
     g.ksplit = 1;
     g.kt_per = kt_total;
     if (best_split > 1) {

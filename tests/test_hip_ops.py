@@ -29,7 +29,7 @@ def dev_bf16(hip, x):
     return hip.DevBuf.from_array(f32_to_bf16(x))
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
 @pytest.mark.parametrize("M", [1, 37, 130, 300])
 def test_linear_bf16_and_f32(hip, oracle_mod, tile, M):
     N, K = 512, 192
@@ -53,7 +53,7 @@ def test_linear_bf16_and_f32(hip, oracle_mod, tile, M):
     assert rel_l2(outT.to_array(np.float32, (N, M)).T, want) < 2e-6
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
 def test_linear_two_parts_resid_and_strides(hip, oracle_mod, tile):
     """Two row ranges with different weights, strided A (lda > K), gated residual epilogue."""
     hip.lib().flux_hip_linear_force_tile(tile)
@@ -77,7 +77,7 @@ def test_linear_two_parts_resid_and_strides(hip, oracle_mod, tile):
     assert rel_l2(dres.to_array(np.float32, (M0 + M1, N)), want) < 2e-6
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
 def test_linear_swiglu(hip, oracle_mod, tile):
     """silu(x Wg^T) * (x Wu^T) with gate/up rows at arbitrary offsets and a strided output."""
     hip.lib().flux_hip_linear_force_tile(tile)
@@ -95,7 +95,23 @@ def test_linear_swiglu(hip, oracle_mod, tile):
     assert not got[:, :64].any() and not got[:, 64 + mlp:].any()   # nothing written outside
 
 
-@pytest.mark.parametrize("tile", [-1, 0, 3])
+@pytest.mark.parametrize("K", [64, 128, 192, 256, 448])
+def test_linear_256_tile_k_steps(hip, oracle_mod, K):
+    """The 256 x 256 tile's hand-pipelined loop peels its last two K steps: every count from one step
+    up, with a ragged row count and several tiles in both directions."""
+    hip.lib().flux_hip_linear_force_tile(2)
+    M, N = 300, 768
+    x = q(normal_f32((M, K), 31, 1))
+    W = q(normal_f32((N, K), 31, 2, 0.0, 0.1))
+    want = oracle_mod.linear(x, W)
+    dx, dW = dev_bf16(hip, x), dev_bf16(hip, W)
+    out32 = hip.DevBuf(M * N * 4)
+    hip.linear(hip.EPI_F32, [(dx.ptr, dW.ptr, out32.ptr, None, M)], N, K, K, K, N, 0, 0)
+    assert rel_l2(out32.to_array(np.float32, (M, N)), want) < 2e-6
+    hip.lib().flux_hip_linear_force_tile(-1)
+
+
+@pytest.mark.parametrize("tile", [-1, 0, 2, 3])
 def test_linear_split_k(hip, oracle_mod, tile):
     """Long K, few output tiles: the residual epilogue splits K over workgroups (two passes through a
     workspace, fixed summation order). Two row ranges, repeated runs must agree bit for bit."""
