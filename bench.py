@@ -118,6 +118,8 @@ def main():
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
+    ap.add_argument("--tile-mask", type=lambda v: int(v, 0), default=0,
+                    help="restrict the GEMM tiles the backend may choose (bit t = tile id t), for A/B runs")
     ap.add_argument("--calibrate", action="store_true",
                     help="launch only a streaming kernel of known size (f32->bf16 over 64 Mi elements: reads 256 MiB, "
                          "writes 128 MiB) and the dominant GEMM, for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
@@ -150,6 +152,8 @@ def main():
     forwards = 2 if wl["cfg"] else 1
 
     fluxhip.init()
+    if args.tile_mask:
+        fluxhip.lib().flux_hip_linear_tile_mask(args.tile_mask)
     model = load_model(cfg)
     z = normal_f32((cfg.channels, h, w), 123, 1)
     txt = normal_f32((nt, cfg.text_dim), 123, 2)
@@ -202,7 +206,7 @@ def main():
         alone_ms, _ = time_dominant_kernel(cfg, n_img + nt)
         roof = {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES.get(args.workload),
-                "kernel": "gemm256_kernel<SWIGLU> (gate/up projection + SiLU*up; 256x256 tile, 4 waves)",
+                "kernel": "gemm4w_kernel<9,6,SWIGLU> (gate/up projection + SiLU*up; 288x192 tile, 4 waves)",
                 "launches_timed": k_n.value, "ms_per_launch": round(per_ms, 4), "flops_per_launch": k_flops,
                 "ms_per_launch_back_to_back": round(alone_ms, 4)}
     model.close()

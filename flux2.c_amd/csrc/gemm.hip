@@ -19,9 +19,10 @@
  * (n): epilogues use 8/16-byte accesses and pair gate/up columns inside a lane.
  *
  * Two kernels share the tile decode and the epilogues. gemm_kernel<BM,BN,WGM,WGN> (8 or 4
- * waves, two waves per SIMD) serves the small tiles. gemm256_kernel is the 256 x 256 tile for the
- * large projections: 4 waves, one per SIMD, each owning 128 x 128 of the tile with its 256
- * accumulator registers pinned to AGPRs. A 128 x 128 wave tile needs 16 fragment reads per 64
+ * waves, two waves per SIMD) serves the small tiles. gemm4w_kernel<TM,TN> is for the
+ * large projections, as a 256 x 256 or a 288 x 192 tile (the second divides 4608-token problems
+ * into a whole number of rounds over 256 CUs): 4 waves, one per SIMD, each owning 128 x 128
+ * (144 x 96) of the tile with its 256 (216) accumulator registers pinned to AGPRs. A 128 x 128 wave tile needs 16 fragment reads per 64
  * MFMAs instead of 12 per 32, i.e. a third less LDS traffic per FLOP, which under the power
  * limit is what buys throughput (1020 -> 1145 TFLOP/s sustained back to back on the
  * 4608 x 18432 x 3072 projection). With a single wave per SIMD nothing hides latency for free,
@@ -244,19 +245,44 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
     store_tile<BN, WM, WN, EPI>(g, t, acc, m0, M, wm, wn, l15, lq);
 }
 
-/* The 256 x 256 tile: 4 waves (2 x 2), 128 x 128 per wave, see the file comment. The MFMA is
- * issued through inline asm so that the accumulator stays in one AGPR quad for the whole loop
- * (left to the register allocator, accumulators migrate between VGPRs and AGPRs with hundreds of
- * copies per K step). Statements with side effects keep their program order, which is what
- * places the LDS reads and global->LDS loads between the MFMAs. */
+/* The large tiles: 4 waves (2 x 2), one per SIMD, each owning a (16 TM) x (16 TN) part of a
+ * (32 TM) x (32 TN) tile, see the file comment. The MFMA is issued through inline asm so that the
+ * accumulator stays in one AGPR quad for the whole loop (left to the register allocator,
+ * accumulators migrate between VGPRs and AGPRs with hundreds of copies per K step). Statements with
+ * side effects keep their program order, which is what places the LDS reads and global->LDS
+ * loads between the MFMAs. */
 #define MFMA_AGPR(acc, a, b) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b))
+
+/* The compiler neither sees those MFMAs' register hazards nor keeps plain register moves in order
+ * around them. acc_fence passes every accumulator through an empty asm statement that is ordered
+ * with the MFMAs: accumulator writes before it stay before it, reads after it stay after it.
+ * Idle cycles for the hazards are placed explicitly next to it. */
+template <int TM, int TN>
+__device__ __forceinline__ void acc_fence(f32x4 (&acc)[TN][TM]) {
+    static_assert(TN == 8 || TN == 6, "one asm statement per accumulator column");
+#pragma unroll
+    for (int j = 0; j < TM; j++) {
+        if constexpr (TN == 8)
+            asm volatile("" : "+a"(acc[0][j]), "+a"(acc[1][j]), "+a"(acc[2][j]), "+a"(acc[3][j]),
+                              "+a"(acc[4][j]), "+a"(acc[5][j]), "+a"(acc[6][j]), "+a"(acc[7][j]));
+        else
+            asm volatile("" : "+a"(acc[0][j]), "+a"(acc[1][j]), "+a"(acc[2][j]), "+a"(acc[3][j]),
+                              "+a"(acc[4][j]), "+a"(acc[5][j]));
+    }
+}
 
 template <bool V> struct BoolC { static constexpr bool value = V; };
 
-template <int EPI>
-__global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
-    constexpr int BM = 256, BN = 256, WGN = 2, WM = 128, WN = 128, TM = 8, TN = 8;
-    constexpr int RPP = 32, PA = 8, PB = 8, STAGE = (BM + BN) * 128;
+template <int TM, int TN, int EPI>
+__global__ __launch_bounds__(256) void gemm4w_kernel(GemmArgs g) {
+    constexpr int BM = 32 * TM, BN = 32 * TN, WGN = 2, WM = 16 * TM, WN = 16 * TN;
+    constexpr int NL = TM + TN;     /* global->LDS loads per wave and stage: 8 tile rows each */
+    constexpr int NF = TM + TN;     /* fragments per K half-step: TN weight side, TM activation side */
+    constexpr int NM = TM * TN;     /* MFMAs per K half-step */
+    constexpr int RD = NM / NF;     /* one LDS read (and one load) every RD MFMAs */
+    constexpr int STAGE = (BM + BN) * 128;
+    static_assert(EPI != FLUX_HIP_EPI_SWIGLU || (TN % 2 == 0), "swiglu pairs 16-column blocks");
+    static_assert(RD >= 2 && RD * (NF - 1) + 1 < NM, "reads and loads must fit between the MFMAs");
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     TileId t;
@@ -272,23 +298,22 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
     const int wm = wave / WGN, wn = wave % WGN;
     const int lrow = tid >> 3, lchunk = tid & 7;
 
-    /* Per-lane global sources, K offset of this slice included. Rows RPP apart share a swizzle. */
+    /* Load i of a stage by this wave covers tile rows lrow + 32 i (8 rows of 128 bytes per wave
+     * instruction): activation rows for i < TM, weight rows after. Rows 32 apart share a swizzle.
+     * The K offset of this workgroup's slice is folded into the per-lane sources. */
     const int kt_begin = t.ks * g.kt_per;
     const int KT = min(g.K >> 6, kt_begin + g.kt_per) - kt_begin;
     const int chunk = ((lchunk ^ lds_swz(lrow)) << 3) + kt_begin * 64;
-    const bf16 *src[PA + PB];
+    const bf16 *src[NL];
 #pragma unroll
-    for (int i = 0; i < PA; i++) src[i] = A + (size_t)min(m0 + lrow + i * RPP, M - 1) * g.lda + chunk;
+    for (int i = 0; i < TM; i++) src[i] = A + (size_t)min(m0 + lrow + i * 32, M - 1) * g.lda + chunk;
 #pragma unroll
-    for (int i = 0; i < PB; i++) src[PA + i] = W + (size_t)weight_row<BN, WN, EPI>(g, tn, lrow + i * RPP) * g.ldw + chunk;
-    static_assert(PA * RPP == BM, "load i of a stage lands at tile row wave*8 + i*RPP: activation rows, then weight rows");
+    for (int i = 0; i < TN; i++) src[TM + i] = W + (size_t)weight_row<BN, WN, EPI>(g, tn, lrow + i * 32) * g.ldw + chunk;
     auto issue1 = [&](int kt, int stage, int i) {
-        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src[i] + kt * 64),
-                                         LDS_PTR(smem + stage * STAGE + (wave * 8 + i * RPP) * 128),
-                                         16, 0, 0);
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src[i] + kt * 64), LDS_PTR(smem + stage * STAGE + (lrow - (lane >> 3) + i * 32) * 128), 16, 0, 0);
     };
 #pragma unroll
-    for (int i = 0; i < PA + PB; i++) issue1(0, 0, i);
+    for (int i = 0; i < NL; i++) issue1(0, 0, i);
 
     f32x4 acc[TN][TM];
 #pragma unroll
@@ -297,41 +322,40 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
         for (int j = 0; j < TM; j++)
 #pragma unroll
             for (int e = 0; e < 4; e++) acc[i][j][e] = 0.0f;
+    acc_fence<TM, TN>(acc); /* the zeroes are written, and a few cycles pass, before the first MFMA reads them */
+    asm volatile("s_nop 7" ::: "memory");
 
     const int l15 = lane & 15, lq = lane >> 4;
     const int swzl = lds_swz(l15);
     const int a_frag = (wm * WM + l15) * 128;
     const int b_frag = BM * 128 + (wn * WN + l15) * 128;
     const int coff0 = (lq ^ swzl) << 4, coff1 = ((4 + lq) ^ swzl) << 4;
-    /* fragment q of a half-step: 0..7 weight side (MFMA A operand), 8..15 activation side */
+    /* fragment q of a half-step: 0..TN-1 weight side (MFMA A operand), then activation side */
     auto frag = [&](const char *st, int coff, int q) -> bf16x8 {
         return q < TN ? *(const bf16x8 *)(st + b_frag + q * 2048 + coff) : *(const bf16x8 *)(st + a_frag + (q - TN) * 2048 + coff);
     };
-    bf16x8 f0[TN + TM], f1[TN + TM];
+    bf16x8 f0[NF], f1[NF];
 
     WAIT_VMCNT0();
     __syncthreads();
     if (KT > 1) {
 #pragma unroll
-        for (int i = 0; i < PA + PB; i++) issue1(1, 1, i);
+        for (int i = 0; i < NL; i++) issue1(1, 1, i);
     }
 #pragma unroll
-    for (int q = 0; q < TN + TM; q++) f0[q] = frag(smem, coff0, q);
+    for (int q = 0; q < NF; q++) f0[q] = frag(smem, coff0, q);
 
     auto step = [&](int kt, auto more_c, auto more2_c) {
         constexpr bool more = decltype(more_c)::value, more2 = decltype(more2_c)::value;
+        auto &accr = acc;
         const int cur = kt & 1;
         const char *st = smem + cur * STAGE;
         const char *nx = smem + (cur ^ 1) * STAGE;
         /* first K half of the stage from f0, while the second half's fragments arrive in f1 */
 #pragma unroll
-        for (int q = 0; q < 16; q++) {
-            f1[q] = frag(st, coff1, q);
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int b = q * 4 + r, j = b >> 3, i = b & 7;
-                MFMA_AGPR(acc[i][j], f0[i], f0[TN + j]);
-            }
+        for (int b = 0; b < NM; b++) {
+            if (b % RD == 0 && b / RD < NF) f1[b / RD] = frag(st, coff1, b / RD);
+            MFMA_AGPR(accr[b % TN][b / TN], f0[b % TN], f0[TN + b / TN]);
         }
         if (more) {
             /* the next stage has landed for this wave; past the barrier it has for all, and
@@ -339,15 +363,13 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
             WAIT_VMCNT0();
             __syncthreads();
         }
+        /* second half from f1, while the next stage's first fragments arrive in f0 and the stage
+         * after next is requested; at most one other instruction between two MFMAs */
 #pragma unroll
-        for (int q = 0; q < 16; q++) {
-            if (more) f0[q] = frag(nx, coff0, q);
-            if (more2) issue1(kt + 2, cur, q);
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int b = q * 4 + r, j = b >> 3, i = b & 7;
-                MFMA_AGPR(acc[i][j], f1[i], f1[TN + j]);
-            }
+        for (int b = 0; b < NM; b++) {
+            if (more && b % RD == 0 && b / RD < NF) f0[b / RD] = frag(nx, coff0, b / RD);
+            if (more2 && b % RD == 1 && b / RD < NL) issue1(kt + 2, cur, b / RD);
+            MFMA_AGPR(accr[b % TN][b / TN], f1[b % TN], f1[TN + b / TN]);
         }
     };
     int kt = 0;
@@ -357,9 +379,8 @@ __global__ __launch_bounds__(256) void gemm256_kernel(GemmArgs g) {
         kt++;
     }
     step(kt, BoolC<false>{}, BoolC<false>{});
-    /* the MFMAs above are opaque to the compiler's hazard handling: let the last results retire
-     * before the accumulators are read */
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); /* the last MFMA results retire before they are read */
+    acc_fence<TM, TN>(acc);
 
     store_tile<BN, WM, WN, EPI>(g, t, acc, m0, M, wm, wn, l15, lq);
 }
@@ -387,19 +408,19 @@ static int launch_cfg(GemmArgs &g) {
     return 1;
 }
 
-template <int EPI>
-static int launch_256(GemmArgs &g) {
-    constexpr int LDS = 2 * 512 * 128;
+template <int TM, int TN, int EPI>
+static int launch_4w(GemmArgs &g) {
+    constexpr int BM = 32 * TM, BN = 32 * TN, LDS = 2 * (BM + BN) * 128;
     static bool attr_done = false;
-    auto kern = gemm256_kernel<EPI>;
+    auto kern = gemm4w_kernel<TM, TN, EPI>;
     if (!attr_done) {
         HIP_OK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
         attr_done = true;
     }
-    g.mtiles0 = (g.M[0] + 255) / 256;
-    int mt1 = g.M[1] > 0 ? (g.M[1] + 255) / 256 : 0;
+    g.mtiles0 = (g.M[0] + BM - 1) / BM;
+    int mt1 = g.M[1] > 0 ? (g.M[1] + BM - 1) / BM : 0;
     g.mtiles = g.mtiles0 + mt1;
-    g.ntiles = g.N / 256;
+    g.ntiles = g.N / BN;
     g.total_tiles = g.mtiles * g.ntiles;
     int grid = (g.total_tiles * g.ksplit + 7) & ~7;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256), LDS, flux_hip_stream_handle(), g);
@@ -410,7 +431,8 @@ static int launch_256(GemmArgs &g) {
 template <int EPI>
 static int launch_epi(GemmArgs &g, int tile) {
     switch (tile) {
-        case 2: return launch_256<EPI>(g);
+        case 2: return launch_4w<8, 8, EPI>(g);
+        case 5: return launch_4w<9, 6, EPI>(g);
         case 4: return launch_cfg<256, 256, 2, 4, EPI>(g); /* 8-wave form of the same tile, for comparison runs */
         case 1: return launch_cfg<128, 128, 2, 2, EPI>(g);
         case 3: return launch_cfg<64, 64, 2, 2, EPI>(g);
@@ -463,8 +485,10 @@ extern "C" void flux_hip_linear_release(void) {
 }
 
 static int g_force_tile = -1;
+static unsigned g_tile_mask = 0x2F; /* tiles the automatic choice may use: all but the 8-wave comparison form */
 static int g_splitk_enabled = 1;
 extern "C" void flux_hip_linear_force_tile(int tile) { g_force_tile = tile; }
+extern "C" void flux_hip_linear_tile_mask(unsigned mask) { g_tile_mask = mask ? mask : 0x2F; }
 extern "C" void flux_hip_linear_enable_splitk(int on) { g_splitk_enabled = on; }
 
 /* Launch probe: HIP events around every launch with one chosen epilogue, so a benchmark can
@@ -543,8 +567,10 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
      * 256 CUs x occupancy; a workgroup's time is its FLOPs at the tile's measured rate plus a
      * fixed prologue/epilogue cost; the launch cannot beat the time to stream its operands,
      * which depends on how many bytes the resident workgroups keep in flight. */
-    static const int bm[4] = {64, 128, 256, 64}, bn[4] = {128, 128, 256, 64}, occ[4] = {3, 2, 1, 4};
-    static const double rate[4] = {2.0e12, 2.9e12, 4.1e12, 1.5e12}; /* FLOP/s of one CU running this tile */
+    /* tile ids: 0..3 the small tiles and 256 x 256, 4 = the 8-wave form of 256 x 256 (only when
+     * forced, for comparison runs), 5 = 288 x 192 */
+    static const int bm[6] = {64, 128, 256, 64, 256, 288}, bn[6] = {128, 128, 256, 64, 256, 192}, occ[6] = {3, 2, 1, 4, 1, 1};
+    static const double rate[6] = {2.0e12, 2.9e12, 5.3e12, 1.5e12, 4.6e12, 5.0e12}; /* FLOP/s of one CU running this tile */
     const int kt_total = K >> 6;
     int tile = 1, best_split = 1;
     {
@@ -553,9 +579,9 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
         const bool can_split = epilogue == FLUX_HIP_EPI_RESID && g_splitk_enabled;
         double rows = 0.0;
         for (int i = 0; i < np; i++) rows += g.M[i];
-        for (int t = 0; t < 4; t++) {
+        for (int t = 0; t < 6; t++) {
             if (N % bn[t]) continue;
-            if (g_force_tile >= 0 && t != (g_force_tile == 4 ? 2 : g_force_tile)) continue;
+            if (g_force_tile >= 0 ? t != g_force_tile : !((g_tile_mask >> t) & 1)) continue;
             long tiles = 0;
             for (int i = 0; i < np; i++) tiles += (g.M[i] + bm[t] - 1) / bm[t];
             tiles *= N / bn[t];
@@ -579,7 +605,6 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
             }
         }
     }
-    if (g_force_tile == 4 && tile == 2) tile = 4;
     g.ksplit = 1;
     g.kt_per = kt_total;
     if (best_split > 1) {
