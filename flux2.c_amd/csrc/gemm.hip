@@ -496,6 +496,7 @@ extern "C" void flux_hip_linear_enable_splitk(int on) { g_splitk_enabled = on; }
 #define PROBE_MAX 4096
 static int g_probe_epi = -1, g_probe_n = 0;
 static hipEvent_t g_probe_ev[PROBE_MAX][2];
+static unsigned char g_probe_tile[PROBE_MAX];
 static int g_probe_created = 0;
 
 extern "C" int flux_hip_linear_probe(int epilogue) {
@@ -504,18 +505,26 @@ extern "C" int flux_hip_linear_probe(int epilogue) {
     return 1;
 }
 
-extern "C" int flux_hip_linear_probe_read(int *launches, float *total_ms) {
+/* Count and summed duration of the recorded launches that used `tile` (-1: all of them). The
+ * record is kept until the next flux_hip_linear_probe call. */
+extern "C" int flux_hip_linear_probe_read_tile(int tile, int *launches, float *total_ms) {
     float sum = 0.0f;
+    int n = 0;
     for (int i = 0; i < g_probe_n; i++) {
+        if (tile >= 0 && g_probe_tile[i] != tile) continue;
         float ms = 0.0f;
         HIP_OK(hipEventSynchronize(g_probe_ev[i][1]));
         HIP_OK(hipEventElapsedTime(&ms, g_probe_ev[i][0], g_probe_ev[i][1]));
         sum += ms;
+        n++;
     }
-    if (launches) *launches = g_probe_n;
+    if (launches) *launches = n;
     if (total_ms) *total_ms = sum;
-    g_probe_n = 0;
     return 1;
+}
+
+extern "C" int flux_hip_linear_probe_read(int *launches, float *total_ms) {
+    return flux_hip_linear_probe_read_tile(-1, launches, total_ms);
 }
 
 static int probe_slot(int epilogue) {
@@ -618,6 +627,7 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
     }
 
     const int slot = probe_slot(epilogue);
+    if (slot >= 0) g_probe_tile[slot] = (unsigned char)tile;
     if (slot >= 0) (void)hipEventRecord(g_probe_ev[slot][0], flux_hip_stream_handle());
     int ok;
     switch (epilogue) {

@@ -66,6 +66,7 @@ def lib():
     L.flux_hip_attention_force_variant.argtypes = [c_i]
     L.flux_hip_linear_probe.argtypes = [c_i]
     L.flux_hip_linear_probe_read.argtypes = [ctypes.POINTER(c_i), ctypes.POINTER(c_f)]
+    L.flux_hip_linear_probe_read_tile.argtypes = [c_i, ctypes.POINTER(c_i), ctypes.POINTER(c_f)]
     L.flux_hip_adaln_norm.argtypes = [vp, c_i, vp, c_i, c_i, c_i, vp, vp, vp, vp, c_f]
     L.flux_hip_kv_prepare.argtypes = [vp, vp, c_i, vp, c_i, c_i, c_i, c_i, c_i, c_i, vp, vp, vp, vp, c_f]
     L.flux_hip_attention.argtypes = [vp, c_i, vp, c_i, vp, vp, c_i, c_i, c_i, c_i, c_i, vp, vp, vp, vp, c_f]

@@ -101,6 +101,8 @@ void flux_hip_linear_enable_splitk(int on);
 void flux_hip_attention_force_variant(int v);
 int flux_hip_linear_probe(int epilogue);
 int flux_hip_linear_probe_read(int *launches, float *total_ms);
+/* the same for the recorded launches that used one tile id (see force_tile) */
+int flux_hip_linear_probe_read_tile(int tile, int *launches, float *total_ms);
 
 /*
  * out = (1 + scale) * LayerNorm(x) + shift per row, x f32 [rows, hidden], out bf16.
