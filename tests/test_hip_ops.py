@@ -29,10 +29,10 @@ def dev_bf16(hip, x):
     return hip.DevBuf.from_array(f32_to_bf16(x))
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("M", [1, 37, 130, 300])
 def test_linear_bf16_and_f32(hip, oracle_mod, tile, M):
-    N, K = (768 if tile == 5 else 512), 192        # the 288 x 192 tile needs N % 192 == 0
+    N, K = (768 if tile >= 5 else 512), 192        # the 192-wide tiles need N % 192 == 0
     hip.lib().flux_hip_linear_force_tile(tile)
     x = q(normal_f32((M, K), 3, 1))
     W = q(normal_f32((N + 64, K), 3, 2, 0.0, 0.1))
@@ -53,11 +53,11 @@ def test_linear_bf16_and_f32(hip, oracle_mod, tile, M):
     assert rel_l2(outT.to_array(np.float32, (N, M)).T, want) < 2e-6
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6])
 def test_linear_two_parts_resid_and_strides(hip, oracle_mod, tile):
     """Two row ranges with different weights, strided A (lda > K), gated residual epilogue."""
     hip.lib().flux_hip_linear_force_tile(tile)
-    M0, M1, N, K, lda = 70, 200, (768 if tile == 5 else 256), 128, 320
+    M0, M1, N, K, lda = 70, 200, (768 if tile >= 5 else 256), 128, 320
     a = q(normal_f32((M0 + M1, lda), 4, 1))
     W0 = q(normal_f32((N, K), 4, 2, 0.0, 0.1))
     W1 = q(normal_f32((N, K), 4, 3, 0.0, 0.1))
@@ -77,7 +77,7 @@ def test_linear_two_parts_resid_and_strides(hip, oracle_mod, tile):
     assert rel_l2(dres.to_array(np.float32, (M0 + M1, N)), want) < 2e-6
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6])
 def test_linear_swiglu(hip, oracle_mod, tile):
     """silu(x Wg^T) * (x Wu^T) with gate/up rows at arbitrary offsets and a strided output."""
     hip.lib().flux_hip_linear_force_tile(tile)
@@ -95,7 +95,7 @@ def test_linear_swiglu(hip, oracle_mod, tile):
     assert not got[:, :64].any() and not got[:, 64 + mlp:].any()   # nothing written outside
 
 
-@pytest.mark.parametrize("tile", [2, 5])
+@pytest.mark.parametrize("tile", [2, 5, 6])
 @pytest.mark.parametrize("K", [64, 128, 192, 256, 448])
 def test_linear_large_tile_k_steps(hip, oracle_mod, K, tile):
     """The hand-pipelined loop of the 4-wave tiles peels its last two K steps: every count from one
@@ -112,12 +112,12 @@ def test_linear_large_tile_k_steps(hip, oracle_mod, K, tile):
     hip.lib().flux_hip_linear_force_tile(-1)
 
 
-@pytest.mark.parametrize("tile", [-1, 0, 2, 3, 5])
+@pytest.mark.parametrize("tile", [-1, 0, 2, 3, 5, 6])
 def test_linear_split_k(hip, oracle_mod, tile):
     """Long K, few output tiles: the residual epilogue splits K over workgroups (two passes through a
     workspace, fixed summation order). Two row ranges, repeated runs must agree bit for bit."""
     hip.lib().flux_hip_linear_force_tile(tile)
-    M0, M1, N, K = 64, 16, (768 if tile == 5 else 256), 4096
+    M0, M1, N, K = 64, 16, (768 if tile >= 5 else 256), 4096
     a = q(normal_f32((M0 + M1, K), 20, 1))
     W0 = q(normal_f32((N, K), 20, 2, 0.0, 0.05))
     W1 = q(normal_f32((N, K), 20, 3, 0.0, 0.05))
@@ -267,10 +267,11 @@ def test_layout_edges_and_updates(hip, oracle_mod):
 
 @pytest.mark.parametrize("variant", [0, 1])
 def test_attention_workgroup_variants(hip, oracle_mod, variant):
-    """Both workgroup sizes (128 and 256 queries) give the same answer on ragged lengths."""
+    """Both workgroup sizes (128 and 256 queries) give the same answer on ragged lengths, from a
+    single key tile up."""
     hip.lib().flux_hip_attention_force_variant(variant)
     try:
-        for n, split, heads in ((300, 100, 2), (513, 512, 1)):
+        for n, split, heads in ((300, 100, 2), (513, 512, 1), (40, 16, 2), (64, 64, 1), (130, 0, 3)):
             got, want = _attention_case(hip, oracle_mod, n, split, heads, 30 + variant)
             assert rel_l2(got, want) < 1e-2, (n, rel_l2(got, want))
     finally:
