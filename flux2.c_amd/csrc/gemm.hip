@@ -441,28 +441,55 @@ static int launch_epi(GemmArgs &g, int tile) {
     }
 }
 
-/* x[m, n] += gate[n] * sum_s ws[s][moff + m][n]: second pass of a split-K residual GEMM
- * (same arithmetic as gated_add, flux_transformer.c:90-97, on the summed product). */
-__global__ __launch_bounds__(256) void splitk_resid_kernel(GemmArgs g) {
-    const int n4 = g.N >> 2;
+/* Second pass of a split-K GEMM: sums the K slices ws[s][moff + m][n] in a fixed order and
+ * applies the epilogue to the sum (for the residual form the same arithmetic as gated_add,
+ * flux_transformer.c:90-97). For SwiGLU the workspace holds plain columns - gate features in
+ * [0, N/2), up features in [N/2, N) - and thread n4 combines column n with column N/2 + n. */
+template <int EPI>
+__global__ __launch_bounds__(256) void splitk_finish_kernel(GemmArgs g) {
+    const int ncols = EPI == FLUX_HIP_EPI_SWIGLU ? g.N >> 1 : g.N;
+    const int n4 = ncols >> 2;
     const size_t total = (size_t)(g.M[0] + g.M[1]) * n4;
     size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
     int row = (int)(idx / n4), n = (int)(idx - (size_t)row * n4) << 2;
     int prob = row >= g.M[0] ? 1 : 0;
     int m = prob ? row - g.M[0] : row;
-    f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+    f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f}, sum2 = {0.0f, 0.0f, 0.0f, 0.0f};
     for (int s = 0; s < g.ksplit; s++) {
-        f32x4 v = *(const f32x4 *)(g.ws + ((size_t)s * g.ws_rows + g.moff[prob] + m) * g.N + n);
+        const float *w = g.ws + ((size_t)s * g.ws_rows + g.moff[prob] + m) * g.N + n;
+        f32x4 v = *(const f32x4 *)w;
 #pragma unroll
         for (int e = 0; e < 4; e++) sum[e] += v[e];
-    }
-    float *p = (float *)g.C[prob] + (size_t)m * g.ldc + n;
-    f32x4 x = *(f32x4 *)p;
-    f32x4 gt = *(const f32x4 *)(g.gate[prob] + n);
+        if (EPI == FLUX_HIP_EPI_SWIGLU) {
+            f32x4 u = *(const f32x4 *)(w + ncols);
 #pragma unroll
-    for (int e = 0; e < 4; e++) x[e] += gt[e] * sum[e];
-    *(f32x4 *)p = x;
+            for (int e = 0; e < 4; e++) sum2[e] += u[e];
+        }
+    }
+    if (EPI == FLUX_HIP_EPI_RESID) {
+        float *p = (float *)g.C[prob] + (size_t)m * g.ldc + n;
+        f32x4 x = *(f32x4 *)p;
+        f32x4 gt = *(const f32x4 *)(g.gate[prob] + n);
+#pragma unroll
+        for (int e = 0; e < 4; e++) x[e] += gt[e] * sum[e];
+        *(f32x4 *)p = x;
+    } else if (EPI == FLUX_HIP_EPI_F32) {
+        *(f32x4 *)((float *)g.C[prob] + (size_t)m * g.ldc + n) = sum;
+    } else {
+        bf16x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; e++) o[e] = (bf16)(EPI == FLUX_HIP_EPI_SWIGLU ? silu_f(sum[e]) * sum2[e] : sum[e]);
+        *(bf16x4 *)((bf16 *)g.C[prob] + (size_t)m * g.ldc + n) = o;
+    }
+}
+
+template <int EPI>
+static int launch_split(GemmArgs &g, int tile) {
+    if (!launch_epi<EPI_PARTIAL>(g, tile)) return 0;
+    const size_t total = (size_t)(g.M[0] + g.M[1]) * ((EPI == FLUX_HIP_EPI_SWIGLU ? g.N >> 1 : g.N) >> 2);
+    hipLaunchKernelGGL(splitk_finish_kernel<EPI>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, flux_hip_stream_handle(), g);
+    return hipGetLastError() == hipSuccess ? 1 : flux_hip_fail("split-K reduction launch failed");
 }
 
 extern "C" void flux_hip_linear_release(void);
@@ -587,7 +614,11 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
     {
         double best = 1e30;
         static const int splits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
-        const bool can_split = epilogue == FLUX_HIP_EPI_RESID && g_splitk_enabled;
+        /* every epilogue but the transposed store can run as K slices + a finishing pass; for
+         * SwiGLU the gate and up rows must be one contiguous block of the weight matrix */
+        const bool can_split = g_splitk_enabled &&
+                               (epilogue == FLUX_HIP_EPI_RESID || epilogue == FLUX_HIP_EPI_BF16 || epilogue == FLUX_HIP_EPI_F32 ||
+                                (epilogue == FLUX_HIP_EPI_SWIGLU && w_row1 == w_row0 + N / 2));
         double rows = 0.0;
         for (int i = 0; i < np; i++) rows += g.M[i];
         for (int t = 0; t < NT; t++) {
@@ -632,24 +663,13 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
     if (slot >= 0) g_probe_tile[slot] = (unsigned char)tile;
     if (slot >= 0) (void)hipEventRecord(g_probe_ev[slot][0], flux_hip_stream_handle());
     int ok;
+    const bool split = g.ksplit > 1;
     switch (epilogue) {
-        case FLUX_HIP_EPI_BF16: ok = launch_epi<FLUX_HIP_EPI_BF16>(g, tile); break;
-        case FLUX_HIP_EPI_F32: ok = launch_epi<FLUX_HIP_EPI_F32>(g, tile); break;
+        case FLUX_HIP_EPI_BF16: ok = split ? launch_split<FLUX_HIP_EPI_BF16>(g, tile) : launch_epi<FLUX_HIP_EPI_BF16>(g, tile); break;
+        case FLUX_HIP_EPI_F32: ok = split ? launch_split<FLUX_HIP_EPI_F32>(g, tile) : launch_epi<FLUX_HIP_EPI_F32>(g, tile); break;
         case FLUX_HIP_EPI_F32_T: ok = launch_epi<FLUX_HIP_EPI_F32_T>(g, tile); break;
-        case FLUX_HIP_EPI_RESID:
-            if (g.ksplit > 1) {
-                ok = launch_epi<EPI_PARTIAL>(g, tile);
-                if (ok) {
-                    size_t total = (size_t)(g.M[0] + g.M[1]) * (N >> 2);
-                    hipLaunchKernelGGL(splitk_resid_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
-                                       flux_hip_stream_handle(), g);
-                    ok = hipGetLastError() == hipSuccess ? 1 : flux_hip_fail("split-K reduction launch failed");
-                }
-            } else {
-                ok = launch_epi<FLUX_HIP_EPI_RESID>(g, tile);
-            }
-            break;
-        case FLUX_HIP_EPI_SWIGLU: ok = launch_epi<FLUX_HIP_EPI_SWIGLU>(g, tile); break;
+        case FLUX_HIP_EPI_RESID: ok = split ? launch_split<FLUX_HIP_EPI_RESID>(g, tile) : launch_epi<FLUX_HIP_EPI_RESID>(g, tile); break;
+        case FLUX_HIP_EPI_SWIGLU: ok = split ? launch_split<FLUX_HIP_EPI_SWIGLU>(g, tile) : launch_epi<FLUX_HIP_EPI_SWIGLU>(g, tile); break;
         default: return flux_hip_fail("flux_hip_linear: unknown epilogue %d", epilogue);
     }
     if (slot >= 0) (void)hipEventRecord(g_probe_ev[slot][1], flux_hip_stream_handle());

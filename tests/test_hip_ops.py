@@ -112,6 +112,40 @@ def test_linear_large_tile_k_steps(hip, oracle_mod, K, tile):
     hip.lib().flux_hip_linear_force_tile(-1)
 
 
+@pytest.mark.parametrize("tile", [-1, 0, 1, 6])
+def test_linear_split_k_other_epilogues(hip, oracle_mod, tile):
+    """Few rows, long K: the bf16, fp32 and SwiGLU epilogues also run as K slices plus a finishing pass
+    (SwiGLU only when gate and up rows are adjacent). Same answer with the split switched off."""
+    hip.lib().flux_hip_linear_force_tile(tile)
+    M, K, mlp, r0 = 80, 3072, 384, 64
+    x = q(normal_f32((M, K), 33, 1))
+    W = q(normal_f32((r0 + 2 * mlp, K), 33, 2, 0.0, 0.05))
+    lin = oracle_mod.linear(x, W[r0:])
+    want_sw = oracle_mod.silu(lin[:, :mlp]) * lin[:, mlp:]
+    dx, dW = dev_bf16(hip, x), dev_bf16(hip, W)
+    res = {}
+    for on in (1, 0):
+        hip.lib().flux_hip_linear_enable_splitk(on)
+        o_bf = hip.DevBuf(M * 2 * mlp * 2)
+        hip.linear(hip.EPI_BF16, [(dx.ptr, dW.ptr, o_bf.ptr, None, M)], 2 * mlp, K, K, K, 2 * mlp, r0, 0)
+        o_f = hip.DevBuf(M * 2 * mlp * 4)
+        hip.linear(hip.EPI_F32, [(dx.ptr, dW.ptr, o_f.ptr, None, M)], 2 * mlp, K, K, K, 2 * mlp, r0, 0)
+        o_sw = hip.DevBuf(M * mlp * 2)
+        hip.linear(hip.EPI_SWIGLU, [(dx.ptr, dW.ptr, o_sw.ptr, None, M)], 2 * mlp, K, K, K, mlp, r0, r0 + mlp)
+        res[on] = (bf16_to_f32(o_bf.to_array(np.uint16, (M, 2 * mlp))), o_f.to_array(np.float32, (M, 2 * mlp)),
+                   bf16_to_f32(o_sw.to_array(np.uint16, (M, mlp))))
+    hip.lib().flux_hip_linear_enable_splitk(1)
+    for on in (1, 0):
+        assert rel_l2(res[on][0], lin) < 4e-3
+        assert rel_l2(res[on][1], lin) < 2e-6
+        assert rel_l2(res[on][2], want_sw) < 4e-3
+    # gate and up rows not adjacent: must still be right (no split possible)
+    o_sw = hip.DevBuf(M * 128 * 2)
+    hip.linear(hip.EPI_SWIGLU, [(dx.ptr, dW.ptr, o_sw.ptr, None, M)], 256, K, K, K, 128, r0, r0 + 2 * mlp - 128)
+    want = oracle_mod.silu(lin[:, :128]) * lin[:, 2 * mlp - 128:]
+    assert rel_l2(bf16_to_f32(o_sw.to_array(np.uint16, (M, 128))), want) < 4e-3
+
+
 @pytest.mark.parametrize("tile", [-1, 0, 2, 3, 5, 6])
 def test_linear_split_k(hip, oracle_mod, tile):
     """Long K, few output tiles: the residual epilogue splits K over workgroups (two passes through a
