@@ -115,9 +115,9 @@ extern "C" int flux_hip_kv_prepare(void *k_out, void *vt_out, int ld_vt, const v
 }
 
 /* ---------------------------------------------------------------------------------------
- * Flash attention. Workgroup = 4 waves = 128 queries of one head; a wave owns 32 queries (two
- * 16-query MFMA columns) and the full head dimension. Keys are walked in tiles of 64 through
- * two LDS stages filled by direct global->LDS loads (no register staging).
+ * Flash attention. Workgroup = 4 or 8 waves = 128 or 256 queries of one head; a wave owns 32
+ * queries (two 16-query MFMA columns) and the full head dimension. Keys are walked in tiles of 64
+ * through two LDS stages filled by direct global->LDS loads (no register staging).
  *   LDS stage: K tile [64 keys][128 d] (256-byte rows, 16-byte chunks XOR-swizzled by key%16)
  *              V^T tile [128 d][64 keys] (128-byte rows, 16-byte chunks swizzled by (d/2)%8)
  * MFMA: v_mfma_f32_16x16x32_bf16 (the form that sustains the most under the power limit).
@@ -198,7 +198,6 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
     };
     issue_k(0);
     issue_v(0);
-    if (ntiles > 1) issue_k(1);
 
     /* ---- Q fragments (B operand), with RMSNorm * weight, RoPE and the softmax scale ---- */
     bf16x8 qf[2][4];
@@ -248,37 +247,62 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
         for (int t = 0; t < 2; t++)
 #pragma unroll
             for (int e = 0; e < 4; e++) o_acc[i][t][e] = 0.0f;
-    float m_run[2] = {-1e30f, -1e30f}, l_run[2] = {0.0f, 0.0f};
+    /* m_run: reference maximum of the online softmax (base-2 logits). The score accumulators of
+     * a tile are *initialised* with -m_run, so the MFMAs deliver s - m_run and the exponent needs
+     * no subtraction; the first tile starts from 0 and is re-based when it is processed. */
+    float m_run[2] = {0.0f, 0.0f}, l_run[2] = {0.0f, 0.0f};
+    f32x4 s_acc[4][2];
 
-    const int kswz = l15; /* key % 16 of the K rows this lane reads */
-    /* S^T for the 64 keys of tile t against this wave's 32 queries */
-    auto scores = [&](int t, f32x4 (&s_acc)[4][2]) {
+    /* One key tile: S^T = K Q^T - m_run (32 MFMAs), online softmax, O^T += V^T P^T (32 MFMAs).
+     * K(t) and V^T(t) sit in slot t%2 of their rings; the loads of tile t+1 are issued at the
+     * top of the step and awaited at the top of the next one. Fragments are read from LDS one
+     * block of four (8 MFMAs) ahead of their use; the first V^T block is requested before the
+     * softmax so that its latency hides behind the exponentials. */
+    auto step = [&](int t) {
+        __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): this wave's parts of K(t), V(t) are in LDS */
+        __syncthreads();
+        if (t + 1 < ntiles) {
+            issue_k(t + 1);
+            issue_v(t + 1);
+        }
         const char *kt = smem + (t & 1) * (64 * 256);
-        const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+        const char *vtile = smem + 2 * (64 * 256) + (t & 1) * (128 * 128);
+        auto kread = [&](int kk, bf16x8 (&dst)[4]) { /* 32 head dims, key blocks 0..3 */
 #pragma unroll
-        for (int kk = 0; kk < 4; kk++) {
+            for (int i = 0; i < 4; i++) dst[i] = *(const bf16x8 *)(kt + (i * 16 + l15) * 256 + (((kk * 4 + lq) ^ l15) << 4));
+        };
+        auto vread = [&](int b, bf16x8 (&dst)[4]) { /* 32-key chunk b/2, head-dim blocks 4(b%2) .. +3 */
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                bf16x8 kf = *(const bf16x8 *)(kt + (i * 16 + l15) * 256 + (((kk * 4 + lq) ^ kswz) << 4));
+            for (int f = 0; f < 4; f++) {
+                const int d = ((b & 1) * 4 + f) * 16 + l15;
+                dst[f] = *(const bf16x8 *)(vtile + d * 128 + (((4 * (b >> 1) + lq) ^ vt_swz(d)) << 4));
+            }
+        };
+        bf16x8 fa[4], fb[4];
+        {
+            f32x4 init[2];
 #pragma unroll
-                for (int u = 0; u < 2; u++)
-                    s_acc[i][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[u][kk], kk == 0 ? zero : s_acc[i][u], 0, 0, 0);
+            for (int u = 0; u < 2; u++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) init[u][e] = -m_run[u];
+            kread(0, fa);
+            kread(1, fb);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                bf16x8 (&cur)[4] = (kk & 1) ? fb : fa;
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int u = 0; u < 2; u++)
+                        s_acc[i][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[i], qf[u][kk], kk == 0 ? init[u] : s_acc[i][u], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0); /* keep the read distance: nothing moves across */
+                if (kk + 2 < 4) kread(kk + 2, cur);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-    };
-
-    /* Software pipeline inside the wave: the score MFMAs of tile t+1 are issued before the
-     * softmax of tile t, so the matrix pipe works while the VALU does exp/max/sum. K and V^T
-     * therefore live in separate 2-slot rings one tile apart: iteration t reads K(t+1) and
-     * V(t) while K(t+2) and V(t+1) are in flight. */
-    /* One key tile: issue the next loads and the next tile's score MFMAs, then softmax and
-     * P V of the current one. */
-    auto step = [&](int t, f32x4 (&s_cur)[4][2], f32x4 (&s_nxt)[4][2]) {
-        __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): K(t+1) and V(t) parts of this wave are in LDS */
-        __syncthreads();
-        if (t + 1 < ntiles) issue_v(t + 1);
-        if (t + 2 < ntiles) issue_k(t + 2);
-        if (t + 1 < ntiles) scores(t + 1, s_nxt);
+        vread(0, fa); /* in flight during the softmax */
+        __builtin_amdgcn_sched_barrier(0);
 
         if (t == ntiles - 1 && (seq_k & 63)) {
             const int key0 = t * 64;
@@ -286,85 +310,83 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
             for (int i = 0; i < 4; i++)
 #pragma unroll
                 for (int e = 0; e < 4; e++)
-                    if (key0 + 32 * (i >> 1) + 8 * lq + 4 * (i & 1) + e >= seq_k) { s_cur[i][0][e] = -1e30f; s_cur[i][1][e] = -1e30f; }
+                    if (key0 + 32 * (i >> 1) + 8 * lq + 4 * (i & 1) + e >= seq_k) { s_acc[i][0][e] = -1e30f; s_acc[i][1][e] = -1e30f; }
         }
         /* Online softmax; a query's scores sit in lanes l, l^16, l^32, l^48. The reference
-         * maximum is only moved when the true maximum exceeds it by more than 2^8 (scores are
-         * base-2 logits): until then p = 2^(s - m_ref) <= 256 is exact enough in fp32/bf16, the
-         * final division by the row sum cancels the choice of m_ref, and the rescale of O -
-         * 64 multiplies per lane - is skipped for almost every tile. */
-        bool grow = false;
+         * maximum is only moved when a tile's maximum exceeds it by more than 2^8 (scores are
+         * base-2 logits): until then p = 2^(s - m_run) <= 256 is exact enough in fp32/bf16, the
+         * final division by the row sum cancels the choice of m_run, and the rescale of O -
+         * 64 multiplies per lane - is skipped for almost every tile. The first tile takes its
+         * own maximum as the reference. */
+        bool grow = t == 0;
         float m_new[2];
 #pragma unroll
         for (int u = 0; u < 2; u++) {
-            float mx = fmaxf(fmaxf(s_cur[0][u][0], s_cur[0][u][1]), fmaxf(s_cur[0][u][2], s_cur[0][u][3]));
+            float mx = fmaxf(fmaxf(s_acc[0][u][0], s_acc[0][u][1]), fmaxf(s_acc[0][u][2], s_acc[0][u][3]));
 #pragma unroll
-            for (int i = 1; i < 4; i++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) mx = fmaxf(mx, s_cur[i][u][e]);
+            for (int i = 1; i < 4; i++) mx = fmaxf(fmaxf(mx, fmaxf(s_acc[i][u][0], s_acc[i][u][1])), fmaxf(s_acc[i][u][2], s_acc[i][u][3]));
             mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            m_new[u] = mx;
-            grow = grow || (mx > m_run[u] + 8.0f);
+            m_new[u] = mx; /* relative to m_run */
+            grow = grow || (mx > 8.0f);
         }
         if (__any(grow)) {
 #pragma unroll
             for (int u = 0; u < 2; u++) {
-                const float m2 = fmaxf(m_run[u], m_new[u]);
-                const float alpha = fast_exp2(m_run[u] - m2);
-                m_run[u] = m2;
+                const float d = t == 0 ? m_new[u] : fmaxf(m_new[u], 0.0f);
+                const float alpha = fast_exp2(-d);
+                m_run[u] += d;
                 l_run[u] *= alpha;
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) s_acc[i][u][e] -= d;
 #pragma unroll
                 for (int i = 0; i < 8; i++)
 #pragma unroll
                     for (int e = 0; e < 4; e++) o_acc[i][u][e] *= alpha;
             }
         }
+        bf16x8 pf[2][2]; /* P^T as MFMA B fragments: [32-key chunk][query block] */
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             float psum = 0.0f;
-            const float mref = m_run[u];
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    float p = fast_exp2(s_cur[i][u][e] - mref);
-                    s_cur[i][u][e] = p;
+                    float p = fast_exp2(s_acc[i][u][e]);
+                    s_acc[i][u][e] = p;
                     psum += p;
                 }
             l_run[u] += psum;
-        }
-        /* O^T += V^T P^T over two 32-key chunks */
-        const char *vtile = smem + 2 * (64 * 256) + (t & 1) * (128 * 128);
 #pragma unroll
-        for (int c = 0; c < 2; c++) {
-            bf16x8 pf[2];
-#pragma unroll
-            for (int u = 0; u < 2; u++)
+            for (int c = 0; c < 2; c++)
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    pf[u][e] = (bf16)s_cur[2 * c][u][e];
-                    pf[u][4 + e] = (bf16)s_cur[2 * c + 1][u][e];
+                    pf[c][u][e] = (bf16)s_acc[2 * c][u][e];
+                    pf[c][u][4 + e] = (bf16)s_acc[2 * c + 1][u][e];
                 }
+        }
+        /* O^T += V^T P^T over two 32-key chunks, four blocks of 8 MFMAs */
+        __builtin_amdgcn_sched_barrier(0);
+        vread(1, fb);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int dt = 0; dt < 8; dt++) {
-                const int d = dt * 16 + l15;
-                bf16x8 vf = *(const bf16x8 *)(vtile + d * 128 + (((4 * c + lq) ^ vt_swz(d)) << 4));
+        for (int b = 0; b < 4; b++) {
+            bf16x8 (&cur)[4] = (b & 1) ? fb : fa;
+#pragma unroll
+            for (int f = 0; f < 4; f++)
 #pragma unroll
                 for (int u = 0; u < 2; u++)
-                    o_acc[dt][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[u], o_acc[dt][u], 0, 0, 0);
-            }
+                    o_acc[(b & 1) * 4 + f][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur[f], pf[b >> 1][u], o_acc[(b & 1) * 4 + f][u], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (b + 2 < 4) vread(b + 2, cur);
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
-    f32x4 s_a[4][2], s_b[4][2];
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-    scores(0, s_a);
-    for (int t = 0; t < ntiles; t += 2) {
-        step(t, s_a, s_b);
-        if (t + 1 < ntiles) step(t + 1, s_b, s_a);
-    }
+    for (int t = 0; t < ntiles; t++) step(t);
 
 #pragma unroll
     for (int u = 0; u < 2; u++) {
