@@ -133,6 +133,8 @@ __device__ __forceinline__ int vt_swz(int d) { return ((d >> 1) & 7) ^ ((d & 1) 
 #define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
+template <bool V> struct AttFlag { static constexpr bool value = V; };
+
 template <int NW>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf16 *__restrict__ out, int ldo,
                                                            const bf16 *__restrict__ q, int ldq,
@@ -250,15 +252,27 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
     /* m_run: reference maximum of the online softmax (base-2 logits). The score accumulators of
      * a tile are *initialised* with -m_run, so the MFMAs deliver s - m_run and the exponent needs
      * no subtraction; the first tile starts from 0 and is re-based when it is processed. */
-    float m_run[2] = {0.0f, 0.0f}, l_run[2] = {0.0f, 0.0f};
+    float m_run[2] = {0.0f, 0.0f};
     f32x4 s_acc[4][2];
+    /* Row sums of P come from the matrix pipe too: one more 16-row block of "V^T" that is all
+     * ones, so that every accumulator element of a lane is the sum, over the keys seen so far, of
+     * the bf16 probabilities that also multiply V (4 MFMAs per tile instead of 32 additions). */
+    f32x4 l_acc[2];
+    bf16x8 ones;
+#pragma unroll
+    for (int e = 0; e < 8; e++) ones[e] = (bf16)1.0f;
+#pragma unroll
+    for (int u = 0; u < 2; u++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) l_acc[u][e] = 0.0f;
 
     /* One key tile: S^T = K Q^T - m_run (32 MFMAs), online softmax, O^T += V^T P^T (32 MFMAs).
      * K(t) and V^T(t) sit in slot t%2 of their rings; the loads of tile t+1 are issued at the
      * top of the step and awaited at the top of the next one. Fragments are read from LDS one
      * block of four (8 MFMAs) ahead of their use; the first V^T block is requested before the
      * softmax so that its latency hides behind the exponentials. */
-    auto step = [&](int t) {
+    auto step = [&](int t, auto edge_c) {
+        constexpr bool EDGE = decltype(edge_c)::value; /* first or last tile: re-base the maximum, mask the ragged end */
         __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): this wave's parts of K(t), V(t) are in LDS */
         __syncthreads();
         if (t + 1 < ntiles) {
@@ -304,7 +318,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
         vread(0, fa); /* in flight during the softmax */
         __builtin_amdgcn_sched_barrier(0);
 
-        if (t == ntiles - 1 && (seq_k & 63)) {
+        if (EDGE && t == ntiles - 1 && (seq_k & 63)) {
             const int key0 = t * 64;
 #pragma unroll
             for (int i = 0; i < 4; i++)
@@ -318,7 +332,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
          * final division by the row sum cancels the choice of m_run, and the rescale of O -
          * 64 multiplies per lane - is skipped for almost every tile. The first tile takes its
          * own maximum as the reference. */
-        bool grow = t == 0;
+        bool grow = EDGE && t == 0;
         float m_new[2];
 #pragma unroll
         for (int u = 0; u < 2; u++) {
@@ -333,10 +347,11 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
         if (__any(grow)) {
 #pragma unroll
             for (int u = 0; u < 2; u++) {
-                const float d = t == 0 ? m_new[u] : fmaxf(m_new[u], 0.0f);
+                const float d = (EDGE && t == 0) ? m_new[u] : fmaxf(m_new[u], 0.0f);
                 const float alpha = fast_exp2(-d);
                 m_run[u] += d;
-                l_run[u] *= alpha;
+#pragma unroll
+                for (int e = 0; e < 4; e++) l_acc[u][e] *= alpha;
 #pragma unroll
                 for (int i = 0; i < 4; i++)
 #pragma unroll
@@ -350,16 +365,10 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
         bf16x8 pf[2][2]; /* P^T as MFMA B fragments: [32-key chunk][query block] */
 #pragma unroll
         for (int u = 0; u < 2; u++) {
-            float psum = 0.0f;
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    float p = fast_exp2(s_acc[i][u][e]);
-                    s_acc[i][u][e] = p;
-                    psum += p;
-                }
-            l_run[u] += psum;
+                for (int e = 0; e < 4; e++) s_acc[i][u][e] = fast_exp2(s_acc[i][u][e]);
 #pragma unroll
             for (int c = 0; c < 2; c++)
 #pragma unroll
@@ -368,7 +377,11 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
                     pf[c][u][4 + e] = (bf16)s_acc[2 * c + 1][u][e];
                 }
         }
-        /* O^T += V^T P^T over two 32-key chunks, four blocks of 8 MFMAs */
+        /* O^T += V^T P^T over two 32-key chunks, four blocks of 8 MFMAs; row sums first */
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int u = 0; u < 2; u++) l_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, pf[c][u], l_acc[u], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         vread(1, fb);
         __builtin_amdgcn_sched_barrier(0);
@@ -386,14 +399,13 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
         }
     };
 
-    for (int t = 0; t < ntiles; t++) step(t);
+    step(0, AttFlag<true>{});
+    for (int t = 1; t < ntiles - 1; t++) step(t, AttFlag<false>{});
+    if (ntiles > 1) step(ntiles - 1, AttFlag<true>{});
 
 #pragma unroll
     for (int u = 0; u < 2; u++) {
-        float l = l_run[u];
-        l += __shfl_xor(l, 16, 64);
-        l += __shfl_xor(l, 32, 64);
-        const float inv_l = 1.0f / l;
+        const float inv_l = 1.0f / l_acc[u][0];
         if (qrow[u] < seq_q) {
             bf16 *op = out + (size_t)qrow[u] * ldo + h * HD + lq * 4;
 #pragma unroll
