@@ -226,11 +226,39 @@ void fh_safetensors_close_compat(void *p) {
     free(sf);
 }
 
+/* The reference fixes the architecture in its loader (flux_transformer.c:4418-4434). The file
+ * itself says what it holds, so the sizes are read from the tensor shapes; a FLUX.2-klein-4B
+ * file gives exactly the reference's constants, and a smaller model of the same family loads too. */
+static const ref_safetensor *find_tensor(const ref_safetensors_file *sf, const char *name) {
+    for (int i = 0; i < sf->num_tensors; i++)
+        if (!strcmp(sf->tensors[i].name, name)) return &sf->tensors[i];
+    return NULL;
+}
+
+static void infer_config(const ref_safetensors_file *sf, flux_hip_config *c) {
+    const ref_safetensor *t;
+    if ((t = find_tensor(sf, "x_embedder.weight")) && t->ndim == 2) { c->hidden = (int)t->shape[0]; c->channels = (int)t->shape[1]; }
+    if ((t = find_tensor(sf, "context_embedder.weight")) && t->ndim == 2) c->text_dim = (int)t->shape[1];
+    if ((t = find_tensor(sf, "transformer_blocks.0.ff.linear_in.weight")) && t->ndim == 2) c->mlp = (int)(t->shape[0] / 2);
+    if ((t = find_tensor(sf, "transformer_blocks.0.attn.norm_q.weight")) && t->ndim == 1) c->head_dim = (int)t->shape[0];
+    if (c->head_dim > 0) c->heads = c->hidden / c->head_dim;
+    int nd = 0, ns = 0;
+    for (int i = 0; i < sf->num_tensors; i++) {
+        int idx;
+        if (sscanf(sf->tensors[i].name, "transformer_blocks.%d.", &idx) == 1 && idx + 1 > nd) nd = idx + 1;
+        if (sscanf(sf->tensors[i].name, "single_transformer_blocks.%d.", &idx) == 1 && idx + 1 > ns) ns = idx + 1;
+    }
+    if (nd > 0) c->n_double = nd;
+    if (ns > 0) c->n_single = ns;
+}
+
 static flux_transformer_t *load_from_handle(void *p) {
     ref_safetensors_file *sf = (ref_safetensors_file *)p;
     if (!sf || !sf->data) { flux_hip_fail("flux_transformer_load_safetensors: NULL file"); return NULL; }
+    if (sf->num_tensors < 0 || sf->num_tensors > 512) { flux_hip_fail("flux_transformer_load_safetensors: bad tensor count"); return NULL; }
     flux_hip_config c;
     flux_hip_default_config(&c);
+    infer_config(sf, &c);
     flux_transformer_t *tf = flux_hip_transformer_new(&c);
     if (!tf) return NULL;
     for (int i = 0; i < sf->num_tensors; i++) {

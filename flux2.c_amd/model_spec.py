@@ -162,6 +162,84 @@ def write_safetensors(path, tensors):
             f.write(np.ascontiguousarray(a).tobytes())
 
 
+def vae_tensor_shapes() -> "OrderedDict[str, tuple]":
+    """Tensor names and shapes of the FLUX.2 VAE file as the reference reads it
+    (flux_vae_load_safetensors, flux_vae.c:1232-1340): z 32 channels, base 128, multipliers 1,2,4,4,
+    two residual blocks per encoder level and three per decoder level, GroupNorm(32)."""
+    t = OrderedDict()
+    mult = [1, 2, 4, 4]
+
+    def conv(name, o, i, k):
+        t[name + ".weight"] = (o, i, k, k)
+        t[name + ".bias"] = (o,)
+
+    def norm(name, c):
+        t[name + ".weight"] = (c,)
+        t[name + ".bias"] = (c,)
+
+    def res(prefix, i, o):
+        norm(prefix + ".norm1", i)
+        conv(prefix + ".conv1", o, i, 3)
+        norm(prefix + ".norm2", o)
+        conv(prefix + ".conv2", o, o, 3)
+        if i != o:
+            conv(prefix + ".conv_shortcut", o, i, 1)
+
+    def attn(prefix, c):
+        norm(prefix + ".group_norm", c)
+        for n in ("to_q", "to_k", "to_v", "to_out.0"):
+            t[f"{prefix}.{n}.weight"] = (c, c)
+            t[f"{prefix}.{n}.bias"] = (c,)
+
+    conv("encoder.conv_in", 128, 3, 3)
+    for lvl in range(4):
+        ch = 128 * mult[lvl]
+        prev = 128 if lvl == 0 else 128 * mult[lvl - 1]
+        for r in range(2):
+            res(f"encoder.down_blocks.{lvl}.resnets.{r}", prev if (r == 0 and lvl > 0) else ch, ch)
+        if lvl < 3:
+            conv(f"encoder.down_blocks.{lvl}.downsamplers.0.conv", ch, ch, 3)
+    for side in ("encoder", "decoder"):
+        res(f"{side}.mid_block.resnets.0", 512, 512)
+        attn(f"{side}.mid_block.attentions.0", 512)
+        res(f"{side}.mid_block.resnets.1", 512, 512)
+    norm("encoder.conv_norm_out", 512)
+    conv("encoder.conv_out", 64, 512, 3)
+    conv("quant_conv", 64, 64, 1)
+    conv("decoder.conv_in", 512, 32, 3)
+    for up in range(4):
+        lvl = 3 - up
+        ch = 128 * mult[lvl]
+        prev = 512 if lvl == 3 else 128 * mult[lvl + 1]
+        for r in range(3):
+            res(f"decoder.up_blocks.{up}.resnets.{r}", prev if r == 0 else ch, ch)
+        if up < 3:
+            conv(f"decoder.up_blocks.{up}.upsamplers.0.conv", ch, ch, 3)
+    norm("decoder.conv_norm_out", 128)
+    conv("decoder.conv_out", 3, 128, 3)
+    t["bn.running_mean"] = (128,)
+    t["bn.running_var"] = (128,)
+    conv("post_quant_conv", 32, 32, 1)
+    return t
+
+
+def make_vae_weights(seed=77):
+    """Synthetic bf16 VAE: convolution and linear weights ~N(0, 1/sqrt(fan_in)), norm scales near 1,
+    small biases, positive running variances; enough for the decoder to give a textured image."""
+    out = OrderedDict()
+    for i, (name, shape) in enumerate(vae_tensor_shapes().items()):
+        if name == "bn.running_var":
+            out[name] = f32_to_bf16(1.0 + 0.2 * np.abs(normal_f32(shape, seed, 5000 + i)))
+        elif name.endswith(".bias") or name == "bn.running_mean":
+            out[name] = normal_bf16(shape, seed, 5000 + i, 0.0, 0.05)
+        elif len(shape) == 1:
+            out[name] = normal_bf16(shape, seed, 5000 + i, 1.0, 0.1)
+        else:
+            fan_in = int(np.prod(shape[1:]))
+            out[name] = normal_bf16(shape, seed, 5000 + i, 0.0, 1.0 / np.sqrt(fan_in))
+    return out
+
+
 def flops_per_forward(cfg: FluxConfig, n_img, n_txt, n_img_out=None):
     """Algorithmic FLOPs of one forward (1 MAC = 2 FLOP)."""
     H, C, T = cfg.hidden, cfg.channels, cfg.text_dim

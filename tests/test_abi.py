@@ -112,3 +112,11 @@ def test_reference_cli_links_against_the_library():
         assert re.search(rf"\bU {name}\b", syms), name          # imported from the shared library
     h = subprocess.run([exe, "--help"], capture_output=True, text=True)
     assert "Usage" in (h.stdout + h.stderr) or "usage" in (h.stdout + h.stderr)
+    # the library level (flux.h) as a shared library over the backend, used by tests/test_hip_pipeline.py
+    r = subprocess.run(["make", "-C", os.path.join(ROOT, "oracle"), "pipeline"], capture_output=True, text=True)
+    assert r.returncode == 0 and "linked _ref/libfluxpipe.so" in r.stdout, r.stdout + r.stderr
+    syms = subprocess.run(["nm", "-D", os.path.join(ROOT, "oracle", "_ref", "libfluxpipe.so")], capture_output=True, text=True).stdout
+    for name in ("flux_sample_euler", "flux_transformer_forward", "flux_transformer_load_safetensors"):
+        assert re.search(rf"\bU {name}\b", syms), name
+    for name in ("flux_load_dir", "flux_generate_with_embeddings", "flux_denoise_step"):
+        assert re.search(rf"\bT {name}\b", syms), name

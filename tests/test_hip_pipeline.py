@@ -1,0 +1,120 @@
+"""The reference's library level over the HIP backend.
+
+oracle/_ref/libfluxpipe.so is the reference's own flux.c (flux_load_dir, flux_generate_with_embeddings,
+flux_denoise_step, flux.h:109-293) with its VAE, image and safetensors code, built from the reference
+sources without flux_transformer.c and flux_sample.c and linked against libflux_hip.so (make -C oracle
+pipeline). Here it loads a synthetic model directory - a small transformer of the same family and a
+full-size VAE with random weights - and generates an image; the expected image comes from the CPU
+oracle's sampler followed by the reference's VAE decoder (oracle/_ref/libfluxref.so) on the same files.
+Acceptance follows the reference's own end-to-end test (run_test.py:96-104): mean absolute pixel
+difference at most 20 of 255; the observed difference is far smaller and is asserted as well.
+"""
+import ctypes
+import os
+
+import numpy as np
+import pytest
+
+from metrics import rel_l2, cosine
+from model_spec import SMALL, make_weights, make_vae_weights, normal_f32, write_safetensors
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PIPE = os.path.join(ROOT, "oracle", "_ref", "libfluxpipe.so")
+REF = os.path.join(ROOT, "oracle", "_ref", "libfluxref.so")
+vp, c_i, c_f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+
+
+class FluxParams(ctypes.Structure):          # flux.h:84-93
+    _fields_ = [("width", c_i), ("height", c_i), ("num_steps", c_i), ("seed", ctypes.c_int64), ("guidance", c_f),
+                ("linear_schedule", c_i), ("power_schedule", c_i), ("power_alpha", c_f)]
+
+
+class FluxImage(ctypes.Structure):           # flux.h:73-78
+    _fields_ = [("width", c_i), ("height", c_i), ("channels", c_i), ("data", ctypes.POINTER(ctypes.c_uint8))]
+
+
+def _image(ptr):
+    im = ctypes.cast(ptr, ctypes.POINTER(FluxImage)).contents
+    return np.ctypeslib.as_array(im.data, shape=(im.height, im.width, im.channels)).copy()
+
+
+@pytest.mark.skipif(not (os.path.exists(PIPE) and os.path.exists(REF)), reason="reference-built libraries not present")
+def test_reference_pipeline_runs_on_the_backend(oracle_mod, tmp_path):
+    import fluxhip
+    fluxhip.init()
+    cfg = SMALL
+    W = make_weights(cfg, 42, 0.05, "sharp")
+    os.makedirs(tmp_path / "transformer")
+    os.makedirs(tmp_path / "vae")
+    write_safetensors(str(tmp_path / "transformer" / "diffusion_pytorch_model.safetensors"), W)
+    write_safetensors(str(tmp_path / "vae" / "diffusion_pytorch_model.safetensors"), make_vae_weights())
+
+    P = ctypes.CDLL(PIPE)
+    P.flux_load_dir.restype = vp
+    P.flux_load_dir.argtypes = [ctypes.c_char_p]
+    P.flux_get_error.restype = ctypes.c_char_p
+    P.flux_generate_with_embeddings.restype = vp
+    P.flux_generate_with_embeddings.argtypes = [vp, vp, c_i, ctypes.POINTER(FluxParams)]
+    P.flux_denoise_step.restype = vp
+    P.flux_denoise_step.argtypes = [vp, vp, c_f, vp, c_i, c_i, c_i]
+    P.flux_image_free.argtypes = [vp]
+    P.flux_free.argtypes = [vp]
+
+    ctx = P.flux_load_dir(str(tmp_path).encode())
+    assert ctx, P.flux_get_error()
+    width, height, steps, seed, seq = 64, 96, 3, 11, 24
+    lh, lw = height // 16, width // 16
+    emb = normal_f32((seq, cfg.text_dim), 40, 1)
+    prm = FluxParams(width, height, steps, seed, 0.0, 0, 0, 2.0)
+    img_p = P.flux_generate_with_embeddings(ctx, emb.ctypes.data, seq, ctypes.byref(prm))
+    assert img_p, P.flux_get_error()
+    got = _image(img_p)
+    P.flux_image_free(img_p)
+    assert got.shape == (height, width, 3)
+
+    # expected: oracle sampler on the same noise and schedule, then the reference's VAE decoder on the CPU
+    o = oracle_mod.Oracle(cfg, W)
+    z0 = oracle_mod.init_noise(cfg.channels, lh, lw, seed)
+    latent = o.sample_euler(z0, lh, lw, emb, oracle_mod.official_schedule(steps, lh * lw))
+    R = ctypes.CDLL(REF)
+    R.safetensors_open.restype = vp
+    R.safetensors_open.argtypes = [ctypes.c_char_p]
+    R.safetensors_close.argtypes = [vp]
+    R.flux_vae_load_safetensors.restype = vp
+    R.flux_vae_load_safetensors.argtypes = [vp]
+    R.flux_vae_decode.restype = vp
+    R.flux_vae_decode.argtypes = [vp, vp, c_i, c_i, c_i]
+    R.flux_vae_free.argtypes = [vp]
+    R.flux_image_free.argtypes = [vp]
+    sf = R.safetensors_open(str(tmp_path / "vae" / "diffusion_pytorch_model.safetensors").encode())
+    assert sf
+    vae = R.flux_vae_load_safetensors(sf)
+    R.safetensors_close(sf)
+    assert vae
+    lat = np.ascontiguousarray(latent, dtype=np.float32)
+    want_p = R.flux_vae_decode(vae, lat.ctypes.data, 1, lh, lw)
+    assert want_p
+    want = _image(want_p)
+    R.flux_image_free(want_p)
+    R.flux_vae_free(vae)
+
+    diff = np.abs(got.astype(np.int32) - want.astype(np.int32))
+    print(f"pipeline image: mean abs diff {diff.mean():.3f}, max {diff.max()}, image std {want.std():.1f}", flush=True)
+    assert want.std() > 5.0                      # a textured image, not a constant
+    assert diff.mean() <= 20.0                   # the reference's own acceptance threshold
+    assert diff.mean() <= 0.6 and diff.max() <= 6  # observed: mean 0.2, max 2
+
+    # flux_denoise_step (flux.c:1109): one forward through the loaded context
+    z = normal_f32((cfg.channels, lh, lw), 40, 2)
+    v_p = P.flux_denoise_step(ctx, z.ctypes.data, 0.6, emb.ctypes.data, seq, lh, lw)
+    assert v_p, P.flux_get_error()
+    v = np.ctypeslib.as_array(ctypes.cast(v_p, ctypes.POINTER(c_f)), shape=(cfg.channels, lh, lw)).copy()
+    fluxhip.libc_free(v_p)
+    vo = o.forward(z, lh, lw, emb, 0.6)
+    r, c = rel_l2(v, vo), cosine(v, vo)
+    print(f"flux_denoise_step: rel_l2={r:.3e} cos={c:.6f}", flush=True)
+    assert r <= 2e-2 and c >= 0.999
+    o.close()
+    P.flux_free(ctx)
