@@ -180,7 +180,8 @@ def main():
     # the gate/up projection runs under more than one tile shape in a step (single-stream blocks
     # and two-part double-stream blocks); the dominant kernel is the shape with the most time
     TILE_NAMES = {0: "gemm_kernel<64,128,2,2,SWIGLU>", 1: "gemm_kernel<128,128,2,2,SWIGLU>", 2: "gemm4w_kernel<8,8,SWIGLU> (256x256 tile)",
-                  3: "gemm_kernel<64,64,2,2,SWIGLU>", 4: "gemm_kernel<256,256,2,4,SWIGLU>", 5: "gemm4w_kernel<9,6,SWIGLU> (288x192 tile)", 6: "gemm4w_kernel<6,6,SWIGLU> (192x192 tile)"}
+                  3: "gemm_kernel<64,64,2,2,SWIGLU>", 4: "gemm_kernel<256,256,2,4,SWIGLU>", 5: "gemm4w_kernel<9,6,SWIGLU> (288x192 tile)", 6: "gemm4w_kernel<6,6,SWIGLU> (192x192 tile)",
+                  7: "gemm4w_kernel<8,6,SWIGLU> (256x192 tile)"}
     k_tile = -1
     for tile in TILE_NAMES:
         n_t, ms_t = ctypes.c_int(0), ctypes.c_float(0.0)

@@ -434,6 +434,7 @@ static int launch_epi(GemmArgs &g, int tile) {
         case 2: return launch_4w<8, 8, EPI>(g);
         case 5: return launch_4w<9, 6, EPI>(g);
         case 6: return launch_4w<6, 6, EPI>(g);
+        case 7: return launch_4w<8, 6, EPI>(g);
         case 4: return launch_cfg<256, 256, 2, 4, EPI>(g); /* 8-wave form of the same tile, for comparison runs */
         case 1: return launch_cfg<128, 128, 2, 2, EPI>(g);
         case 3: return launch_cfg<64, 64, 2, 2, EPI>(g);
@@ -513,10 +514,10 @@ extern "C" void flux_hip_linear_release(void) {
 }
 
 static int g_force_tile = -1;
-static unsigned g_tile_mask = 0x6F; /* tiles the automatic choice may use: all but the 8-wave comparison form */
+static unsigned g_tile_mask = 0xEF; /* tiles the automatic choice may use: all but the 8-wave comparison form */
 static int g_splitk_enabled = 1;
 extern "C" void flux_hip_linear_force_tile(int tile) { g_force_tile = tile; }
-extern "C" void flux_hip_linear_tile_mask(unsigned mask) { g_tile_mask = mask ? mask : 0x6F; }
+extern "C" void flux_hip_linear_tile_mask(unsigned mask) { g_tile_mask = mask ? mask : 0xEF; }
 extern "C" void flux_hip_linear_enable_splitk(int on) { g_splitk_enabled = on; }
 
 /* Launch probe: HIP events around every launch with one chosen epilogue, so a benchmark can
@@ -605,10 +606,10 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
      * fixed prologue/epilogue cost; the launch cannot beat the time to stream its operands,
      * which depends on how many bytes the resident workgroups keep in flight. */
     /* tile ids: 0..3 the small tiles and 256 x 256, 4 = the 8-wave form of 256 x 256 (only when
-     * forced, for comparison runs), 5 = 288 x 192, 6 = 192 x 192 */
-    constexpr int NT = 7;
-    static const int bm[NT] = {64, 128, 256, 64, 256, 288, 192}, bn[NT] = {128, 128, 256, 64, 256, 192, 192}, occ[NT] = {3, 2, 1, 4, 1, 1, 1};
-    static const double rate[NT] = {2.0e12, 2.9e12, 5.3e12, 1.5e12, 4.6e12, 5.0e12, 4.0e12}; /* FLOP/s of one CU running this tile */
+     * forced, for comparison runs), 5 = 288 x 192, 6 = 192 x 192, 7 = 256 x 192 */
+    constexpr int NT = 8;
+    static const int bm[NT] = {64, 128, 256, 64, 256, 288, 192, 256}, bn[NT] = {128, 128, 256, 64, 256, 192, 192, 192}, occ[NT] = {3, 2, 1, 4, 1, 1, 1, 1};
+    static const double rate[NT] = {2.0e12, 2.9e12, 5.3e12, 1.5e12, 4.6e12, 5.0e12, 4.0e12, 4.9e12}; /* FLOP/s of one CU running this tile */
     const int kt_total = K >> 6;
     int tile = 1, best_split = 1;
     {

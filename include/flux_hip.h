@@ -88,13 +88,13 @@ typedef struct {
 int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
                     int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1);
 
-/* Measurement hooks. force_tile: 0/1/2/3/5/6 pins the GEMM tile (64x128, 128x128, 256x256, 64x64,
- * 288x192, 192x192; 4 = 256x256 in its 8-wave form, never chosen automatically), -1 restores the automatic
+/* Measurement hooks. force_tile: 0/1/2/3/5/6/7 pins the GEMM tile (64x128, 128x128, 256x256, 64x64,
+ * 288x192, 192x192, 256x192; 4 = 256x256 in its 8-wave form, never chosen automatically), -1 restores the automatic
  * choice (a tile whose width does not divide N is skipped; if none is left the call fails); enable_splitk(0) turns the split-K path off. probe(epilogue) records HIP events around every later
  * flux_hip_linear launch with that epilogue (-1 stops); probe_read waits for them and returns
  * their count and summed duration. */
 void flux_hip_linear_force_tile(int tile);
-/* bit t set = the automatic choice may use tile t (default 0x6F: all but tile 4; 0 restores it) */
+/* bit t set = the automatic choice may use tile t (default 0xEF: all but tile 4; 0 restores it) */
 void flux_hip_linear_tile_mask(unsigned mask);
 void flux_hip_linear_enable_splitk(int on);
 /* 0 = 128-query workgroups, 1 = 256-query workgroups, -1 = automatic */

@@ -29,7 +29,7 @@ def dev_bf16(hip, x):
     return hip.DevBuf.from_array(f32_to_bf16(x))
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7])
 @pytest.mark.parametrize("M", [1, 37, 130, 300])
 def test_linear_bf16_and_f32(hip, oracle_mod, tile, M):
     N, K = (768 if tile >= 5 else 512), 192        # the 192-wide tiles need N % 192 == 0
@@ -53,7 +53,7 @@ def test_linear_bf16_and_f32(hip, oracle_mod, tile, M):
     assert rel_l2(outT.to_array(np.float32, (N, M)).T, want) < 2e-6
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7])
 def test_linear_two_parts_resid_and_strides(hip, oracle_mod, tile):
     """Two row ranges with different weights, strided A (lda > K), gated residual epilogue."""
     hip.lib().flux_hip_linear_force_tile(tile)
@@ -77,7 +77,7 @@ def test_linear_two_parts_resid_and_strides(hip, oracle_mod, tile):
     assert rel_l2(dres.to_array(np.float32, (M0 + M1, N)), want) < 2e-6
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7])
 def test_linear_swiglu(hip, oracle_mod, tile):
     """silu(x Wg^T) * (x Wu^T) with gate/up rows at arbitrary offsets and a strided output."""
     hip.lib().flux_hip_linear_force_tile(tile)
@@ -95,7 +95,7 @@ def test_linear_swiglu(hip, oracle_mod, tile):
     assert not got[:, :64].any() and not got[:, 64 + mlp:].any()   # nothing written outside
 
 
-@pytest.mark.parametrize("tile", [2, 5, 6])
+@pytest.mark.parametrize("tile", [2, 5, 6, 7])
 @pytest.mark.parametrize("K", [64, 128, 192, 256, 448])
 def test_linear_large_tile_k_steps(hip, oracle_mod, K, tile):
     """The hand-pipelined loop of the 4-wave tiles peels its last two K steps: every count from one
@@ -146,7 +146,7 @@ def test_linear_split_k_other_epilogues(hip, oracle_mod, tile):
     assert rel_l2(bf16_to_f32(o_sw.to_array(np.uint16, (M, 128))), want) < 4e-3
 
 
-@pytest.mark.parametrize("tile", [-1, 0, 2, 3, 5, 6])
+@pytest.mark.parametrize("tile", [-1, 0, 2, 3, 5, 6, 7])
 def test_linear_split_k(hip, oracle_mod, tile):
     """Long K, few output tiles: the residual epilogue splits K over workgroups (two passes through a
     workspace, fixed summation order). Two row ranges, repeated runs must agree bit for bit."""
