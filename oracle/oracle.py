@@ -81,6 +81,17 @@ def lib():
     L.fo_randn.argtypes = [vp, ctypes.c_int64]
     L.fo_num_threads.restype = c_i
     L.fo_has_blas.restype = c_i
+    L.fo_conv2d.argtypes = [vp, vp, vp, vp, c_i, c_i, c_i, c_i, c_i, c_i]
+    L.fo_group_norm.argtypes = [vp, vp, vp, vp, c_i, c_i, c_i, c_i, c_f]
+    L.fo_upsample_nearest.argtypes = [vp, vp, c_i, c_i, c_i]
+    L.fo_unpatchify.argtypes = [vp, vp, c_i, c_i, c_i, c_i]
+    L.fo_vae_new.argtypes = [c_i]
+    L.fo_vae_new.restype = vp
+    L.fo_vae_free.argtypes = [vp]
+    L.fo_vae_set.argtypes = [vp, ctypes.c_char_p, vp, ctypes.c_int64]
+    L.fo_vae_set.restype = c_i
+    L.fo_vae_decode.argtypes = [vp, vp, c_i, c_i, vp, vp]
+    L.fo_vae_decode.restype = c_i
     _lib = L
     return L
 
@@ -340,3 +351,74 @@ def randn(n, seed):
     lib().fo_rng_seed(seed)
     lib().fo_randn(out.ctypes.data, n)
     return out
+
+
+# ---- VAE decoder (oracle/vae_oracle.c) ----
+
+def conv2d(x, w, bias, pad):
+    """x [cin, H, W], w [cout, cin, k, k] -> [cout, H, W] (stride 1, zero padding)."""
+    x, w = _f32(x), _f32(w)
+    b = None if bias is None else _f32(bias)
+    out = np.empty((w.shape[0], x.shape[1], x.shape[2]), np.float32)
+    lib().fo_conv2d(out.ctypes.data, x.ctypes.data, w.ctypes.data, None if b is None else b.ctypes.data,
+                    x.shape[0], w.shape[0], x.shape[1], x.shape[2], w.shape[2], pad)
+    return out
+
+
+def group_norm(x, gamma, beta, groups=32, eps=1e-4):
+    x, gamma, beta = _f32(x), _f32(gamma), _f32(beta)
+    out = np.empty_like(x)
+    lib().fo_group_norm(out.ctypes.data, x.ctypes.data, gamma.ctypes.data, beta.ctypes.data,
+                        x.shape[0], x.shape[1], x.shape[2], groups, eps)
+    return out
+
+
+def upsample_nearest(x):
+    x = _f32(x)
+    out = np.empty((x.shape[0], 2 * x.shape[1], 2 * x.shape[2]), np.float32)
+    lib().fo_upsample_nearest(out.ctypes.data, x.ctypes.data, x.shape[0], x.shape[1], x.shape[2])
+    return out
+
+
+def unpatchify(x, p=2):
+    x = _f32(x)
+    c = x.shape[0] // (p * p)
+    out = np.empty((c, p * x.shape[1], p * x.shape[2]), np.float32)
+    lib().fo_unpatchify(out.ctypes.data, x.ctypes.data, c, x.shape[1], x.shape[2], p)
+    return out
+
+
+class VaeOracle:
+    """The decoder half of the VAE. `weights` maps tensor name -> uint16 (bf16) or float32 array."""
+
+    def __init__(self, weights, base_channels=128):
+        from model_spec import bf16_to_f32
+        self._L = lib()
+        self._v = self._L.fo_vae_new(base_channels)
+        for name, a in weights.items():
+            if not (name.startswith("decoder.") or name.startswith("bn.") or name.startswith("post_quant_conv")):
+                continue
+            a = _f32(bf16_to_f32(a) if a.dtype == np.uint16 else a)
+            rc = self._L.fo_vae_set(self._v, name.encode(), a.ctypes.data, a.size)
+            if rc != 0:
+                raise ValueError(f"vae oracle rejected tensor {name}")
+
+    def close(self):
+        if self._v:
+            self._L.fo_vae_free(self._v)
+            self._v = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def decode(self, latent, h, w):
+        """latent [128, h, w] -> (float image [3, 16h, 16w] in about [-1, 1], uint8 image [16h, 16w, 3])."""
+        latent = _f32(latent)
+        f = np.empty((3, 16 * h, 16 * w), np.float32)
+        u = np.empty((16 * h, 16 * w, 3), np.uint8)
+        if self._L.fo_vae_decode(self._v, latent.ctypes.data, h, w, f.ctypes.data, u.ctypes.data) != 0:
+            raise RuntimeError("vae oracle: decode failed (missing tensor)")
+        return f, u

@@ -20,7 +20,8 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 sys.path.insert(0, os.path.join(ROOT, "flux2.c_amd"))
-from model_spec import TINY, KLEIN_4B, make_weights, normal_f32, bf16_to_f32  # noqa: E402
+from model_spec import (TINY, KLEIN_4B, make_weights, make_vae_weights, write_safetensors, normal_f32,  # noqa: E402
+                        bf16_to_f32)
 
 c_f, c_i, vp = ctypes.c_float, ctypes.c_int, ctypes.c_void_p
 
@@ -280,6 +281,80 @@ def model_golden(cfg, qk):
     return g
 
 
+class FluxImage(ctypes.Structure):           # flux.h:73-78
+    _fields_ = [("width", c_i), ("height", c_i), ("channels", c_i), ("data", ctypes.POINTER(ctypes.c_uint8))]
+
+
+# shapes shared with tests/test_oracle_golden.py
+VAE_OP_SEED = 21
+VAE_DECODE_CASES = ((2, 2, 301), (3, 2, 302))     # latent h, w, seed
+
+
+def vae_golden():
+    """The reference's convolution, group norm, upsample and unpatchify (flux_kernels.c) on small
+    seeded tensors, and its VAE decoder (flux_vae_decode, flux_vae.c:690) on the synthetic
+    full-size VAE of model_spec.make_vae_weights."""
+    import tempfile
+    g = {}
+    for fn in ("flux_conv2d", "flux_group_norm", "flux_upsample_nearest", "flux_unpatchify"):
+        getattr(L, fn).restype = None
+    L.flux_conv2d.argtypes = [vp, vp, vp, vp] + [c_i] * 9
+    L.flux_group_norm.argtypes = [vp, vp, vp, vp, c_i, c_i, c_i, c_i, c_i, c_f]
+    L.flux_upsample_nearest.argtypes = [vp, vp] + [c_i] * 6
+    L.flux_unpatchify.argtypes = [vp, vp] + [c_i] * 5
+    x = normal_f32((5, 7, 6), VAE_OP_SEED, 1)
+    w3 = normal_f32((4, 5, 3, 3), VAE_OP_SEED, 2, 0.0, 0.2)
+    w1 = normal_f32((4, 5, 1, 1), VAE_OP_SEED, 3, 0.0, 0.4)
+    b = normal_f32((4,), VAE_OP_SEED, 4)
+    o = np.empty((4, 7, 6), np.float32)
+    L.flux_conv2d(P(o), P(x), P(w3), P(b), 1, 5, 4, 7, 6, 3, 3, 1, 1)
+    g["conv3x3"] = o.copy()
+    L.flux_conv2d(P(o), P(x), P(w1), P(b), 1, 5, 4, 7, 6, 1, 1, 1, 0)
+    g["conv1x1"] = o.copy()
+    L.flux_conv2d(P(o), P(x), P(w3), None, 1, 5, 4, 7, 6, 3, 3, 1, 1)
+    g["conv3x3_nobias"] = o.copy()
+    xg = normal_f32((64, 5, 3), VAE_OP_SEED, 5, 0.3, 2.0)
+    gm, bt = normal_f32((64,), VAE_OP_SEED, 6, 1.0, 0.2), normal_f32((64,), VAE_OP_SEED, 7)
+    og = np.empty_like(xg)
+    L.flux_group_norm(P(og), P(xg), P(gm), P(bt), 1, 64, 5, 3, 32, 1e-4)
+    g["group_norm"] = og
+    xu = normal_f32((3, 4, 5), VAE_OP_SEED, 8)
+    ou = np.empty((3, 8, 10), np.float32)
+    L.flux_upsample_nearest(P(ou), P(xu), 1, 3, 4, 5, 2, 2)
+    g["upsample"] = ou
+    xp = normal_f32((12, 3, 2), VAE_OP_SEED, 9)
+    op = np.empty((3, 6, 4), np.float32)
+    L.flux_unpatchify(P(op), P(xp), 1, 3, 3, 2, 2)
+    g["unpatchify"] = op
+
+    L.safetensors_open.restype = vp
+    L.safetensors_open.argtypes = [ctypes.c_char_p]
+    L.safetensors_close.argtypes = [vp]
+    L.flux_vae_load_safetensors.restype = vp
+    L.flux_vae_load_safetensors.argtypes = [vp]
+    L.flux_vae_decode.restype = vp
+    L.flux_vae_decode.argtypes = [vp, vp, c_i, c_i, c_i]
+    L.flux_vae_free.argtypes = [vp]
+    L.flux_image_free.argtypes = [vp]
+    with tempfile.TemporaryDirectory() as d:
+        path = os.path.join(d, "vae.safetensors")
+        write_safetensors(path, make_vae_weights())
+        sf = L.safetensors_open(path.encode())
+        vae = L.flux_vae_load_safetensors(sf)
+        L.safetensors_close(sf)
+        assert vae
+        for h, w, seed in VAE_DECODE_CASES:
+            lat = normal_f32((128, h, w), seed, 1)
+            ip = L.flux_vae_decode(vae, P(lat), 1, h, w)
+            assert ip
+            im = ctypes.cast(ip, ctypes.POINTER(FluxImage)).contents
+            g[f"decode_{h}x{w}"] = np.ctypeslib.as_array(im.data, shape=(im.height, im.width, im.channels)).copy()
+            L.flux_image_free(ip)
+            print("vae decode", h, w, "std", g[f"decode_{h}x{w}"].std(), flush=True)
+        L.flux_vae_free(vae)
+    return g
+
+
 def full_c1(qk):
     """Config c1 of the benchmark at the real 4B architecture: 4x4 latent, 64 text tokens, t=1."""
     cfg = KLEIN_4B
@@ -296,8 +371,12 @@ def full_c1(qk):
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--full", action="store_true")
+    ap.add_argument("--only-vae", action="store_true", help="rewrite vae.npz only")
     args = ap.parse_args()
     L = load()
+    np.savez_compressed(os.path.join(HERE, "vae.npz"), **vae_golden())
+    if args.only_vae:
+        sys.exit(0)
     np.savez_compressed(os.path.join(HERE, "ops.npz"), **ops_golden())
     for qk in ("literal", "sharp"):
         np.savez_compressed(os.path.join(HERE, f"tiny_{qk}.npz"), **model_golden(TINY, qk))

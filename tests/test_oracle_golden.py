@@ -214,3 +214,46 @@ def test_klein4b_c1(oracle_mod, golden_dir, qk):
     txt = normal_f32((64, cfg.text_dim), 42, 1001)
     close(m.forward(lat, 4, 4, txt, 1.0), g["velocity"], 5e-5)
     m.close()
+
+
+# ---- VAE decoder (oracle/vae_oracle.c) against the reference's flux_kernels.c / flux_vae.c ----
+VAE_OP_SEED = 21
+VAE_DECODE_CASES = ((2, 2, 301), (3, 2, 302))
+
+
+@pytest.fixture(scope="module")
+def vae_gold(golden_dir):
+    return np.load(os.path.join(golden_dir, "vae.npz"))
+
+
+def test_vae_operators(oracle_mod, vae_gold):
+    x = normal_f32((5, 7, 6), VAE_OP_SEED, 1)
+    w3 = normal_f32((4, 5, 3, 3), VAE_OP_SEED, 2, 0.0, 0.2)
+    w1 = normal_f32((4, 5, 1, 1), VAE_OP_SEED, 3, 0.0, 0.4)
+    b = normal_f32((4,), VAE_OP_SEED, 4)
+    close(oracle_mod.conv2d(x, w3, b, 1), vae_gold["conv3x3"], 2e-6)
+    close(oracle_mod.conv2d(x, w1, b, 0), vae_gold["conv1x1"], 2e-6)
+    close(oracle_mod.conv2d(x, w3, None, 1), vae_gold["conv3x3_nobias"], 2e-6)
+    xg = normal_f32((64, 5, 3), VAE_OP_SEED, 5, 0.3, 2.0)
+    gm, bt = normal_f32((64,), VAE_OP_SEED, 6, 1.0, 0.2), normal_f32((64,), VAE_OP_SEED, 7)
+    close(oracle_mod.group_norm(xg, gm, bt, 32, 1e-4), vae_gold["group_norm"], 2e-6)
+    np.testing.assert_array_equal(oracle_mod.upsample_nearest(normal_f32((3, 4, 5), VAE_OP_SEED, 8)), vae_gold["upsample"])
+    np.testing.assert_array_equal(oracle_mod.unpatchify(normal_f32((12, 3, 2), VAE_OP_SEED, 9)), vae_gold["unpatchify"])
+
+
+def test_vae_decode_images(oracle_mod, vae_gold):
+    """Whole decoder on the synthetic full-size VAE: the 8-bit image must equal the reference's
+    except where a value sits on a rounding boundary (both sides truncate (v+1)*127.5)."""
+    from model_spec import make_vae_weights
+    o = oracle_mod.VaeOracle(make_vae_weights())
+    for h, w, seed in VAE_DECODE_CASES:
+        f, u = o.decode(normal_f32((128, h, w), seed, 1), h, w)
+        want = vae_gold[f"decode_{h}x{w}"]
+        assert u.shape == want.shape == (16 * h, 16 * w, 3)
+        diff = np.abs(u.astype(np.int32) - want.astype(np.int32))
+        assert want.std() > 20.0                    # a textured image
+        assert diff.max() <= 1 and (diff > 0).mean() < 0.01, (diff.max(), (diff > 0).mean())
+        # the float image is consistent with the 8-bit one
+        q = np.clip((f.transpose(1, 2, 0) + 1.0) * 127.5, 0, 255).astype(np.uint8)
+        np.testing.assert_array_equal(q, u)
+    o.close()

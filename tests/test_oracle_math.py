@@ -120,3 +120,41 @@ def test_silu_softmax(oracle_mod):
     p = oracle_mod.softmax(m)
     np.testing.assert_allclose(p.sum(1), 1, atol=1e-5)
     np.testing.assert_allclose(p, np_softmax(m), atol=1e-6)
+
+
+# ---- VAE operators ----
+
+def test_conv2d_closed_forms(oracle_mod):
+    x = normal_f32((3, 6, 5), 2, 1)
+    # a kernel that is 1 at the centre of its own channel reproduces the input
+    w = np.zeros((3, 3, 3, 3), np.float32)
+    for c in range(3):
+        w[c, c, 1, 1] = 1.0
+    np.testing.assert_array_equal(oracle_mod.conv2d(x, w, None, 1), x)
+    # a kernel that is 1 at (ky, kx) = (0, 2) reads the pixel one up and one to the right, zero outside
+    w = np.zeros((1, 3, 3, 3), np.float32)
+    w[0, 1, 0, 2] = 1.0
+    want = np.zeros((6, 5), np.float32)
+    want[1:, :-1] = x[1, :-1, 1:]
+    np.testing.assert_array_equal(oracle_mod.conv2d(x, w, None, 1)[0], want)
+    # all-ones 3x3 over a constant image counts the taps inside the image; bias adds on top
+    ones = np.ones((1, 4, 4), np.float32)
+    y = oracle_mod.conv2d(ones, np.ones((1, 1, 3, 3), np.float32), np.array([0.5], np.float32), 1)[0]
+    assert y[0, 0] == 4.5 and y[0, 1] == 6.5 and y[1, 1] == 9.5 and y[3, 3] == 4.5
+    # against a direct numpy evaluation
+    w = normal_f32((4, 3, 3, 3), 2, 2)
+    xp = np.pad(x.astype(np.float64), ((0, 0), (1, 1), (1, 1)))
+    ref = np.zeros((4, 6, 5))
+    for ky in range(3):
+        for kx in range(3):
+            ref += np.einsum("oc,chw->ohw", w[:, :, ky, kx].astype(np.float64), xp[:, ky:ky + 6, kx:kx + 5])
+    assert rel_l2(oracle_mod.conv2d(x, w, None, 1), ref) < 1e-6
+
+
+def test_group_norm_statistics(oracle_mod):
+    x = normal_f32((64, 6, 7), 2, 3, 1.5, 3.0)
+    y = oracle_mod.group_norm(x, np.ones(64, np.float32), np.zeros(64, np.float32), 32, 1e-6)
+    g = y.reshape(32, -1)
+    assert np.abs(g.mean(axis=1)).max() < 1e-5 and np.abs(g.var(axis=1) - 1.0).max() < 1e-4
+    gm, bt = normal_f32((64,), 2, 4), normal_f32((64,), 2, 5)
+    assert rel_l2(oracle_mod.group_norm(x, gm, bt, 32, 1e-6), y * gm[:, None, None] + bt[:, None, None]) < 1e-6
