@@ -45,7 +45,7 @@ static float f16_to_f32(uint16_t h) {
     return f;
 }
 
-enum { DT_F32 = 0, DT_F16 = 1, DT_BF16 = 2 };
+enum { DT_F32 = FH_DT_F32, DT_F16 = FH_DT_F16, DT_BF16 = FH_DT_BF16 };
 
 static int set_from(flux_transformer_t *tf, const char *name, int dtype, const void *data, int64_t numel) {
     if (dtype == DT_BF16) return flux_hip_transformer_set_tensor(tf, name, (const uint16_t *)data, numel);
@@ -97,23 +97,20 @@ static const char *skip_value(const char *p, const char *e) {
     return p;
 }
 
-flux_transformer_t *flux_hip_transformer_load_file(const char *path, const flux_hip_config *cfg) {
-    flux_hip_config c;
-    if (cfg) c = *cfg; else flux_hip_default_config(&c);
+/* Walks a .safetensors file: calls cb(ctx, name, dtype, data, numel) for every tensor, in file
+ * order. cb returns 0 to abort (after recording an error). Returns 1 when every call did. */
+int fh_safetensors_walk(const char *path, fh_tensor_cb cb, void *ctx) {
     int fd = open(path, O_RDONLY);
-    if (fd < 0) { flux_hip_fail("cannot open %s", path); return NULL; }
+    if (fd < 0) return flux_hip_fail("cannot open %s", path);
     struct stat sb;
-    if (fstat(fd, &sb) != 0 || sb.st_size < 8) { close(fd); flux_hip_fail("%s: not a safetensors file", path); return NULL; }
+    if (fstat(fd, &sb) != 0 || sb.st_size < 8) { close(fd); return flux_hip_fail("%s: not a safetensors file", path); }
     size_t fsize = (size_t)sb.st_size;
     char *map = (char *)mmap(NULL, fsize, PROT_READ, MAP_PRIVATE, fd, 0);
     close(fd);
-    if (map == MAP_FAILED) { flux_hip_fail("%s: mmap failed", path); return NULL; }
+    if (map == MAP_FAILED) return flux_hip_fail("%s: mmap failed", path);
     uint64_t hlen = 0;
     memcpy(&hlen, map, 8);
-    flux_transformer_t *tf = NULL;
     if (hlen == 0 || hlen > fsize - 8) { flux_hip_fail("%s: bad header length", path); goto fail; }
-    tf = flux_hip_transformer_new(&c);
-    if (!tf) goto fail;
     {
         const char *p = map + 8, *e = map + 8 + hlen, *data = e;
         size_t dsize = fsize - 8 - hlen;
@@ -181,19 +178,33 @@ flux_transformer_t *flux_hip_transformer_load_file(const char *path, const flux_
                     flux_hip_fail("%s: tensor %s has inconsistent offsets", path, name);
                     goto fail;
                 }
-                if (!set_from(tf, name, dt, data + off0, numel)) goto fail;
+                if (!cb(ctx, name, dt, data + off0, numel)) goto fail;
             }
             p = skip_ws(p, e);
             if (p < e && *p == ',') p++;
         }
     }
-    if (!fh_model_complete(tf)) goto fail;
     munmap(map, fsize);
-    return tf;
+    return 1;
 fail:
     munmap(map, fsize);
-    flux_transformer_free(tf);
-    return NULL;
+    return 0;
+}
+
+static int transformer_tensor_cb(void *ctx, const char *name, int dtype, const void *data, int64_t numel) {
+    return set_from((flux_transformer_t *)ctx, name, dtype, data, numel);
+}
+
+flux_transformer_t *flux_hip_transformer_load_file(const char *path, const flux_hip_config *cfg) {
+    flux_hip_config c;
+    if (cfg) c = *cfg; else flux_hip_default_config(&c);
+    flux_transformer_t *tf = flux_hip_transformer_new(&c);
+    if (!tf) return NULL;
+    if (!fh_safetensors_walk(path, transformer_tensor_cb, tf) || !fh_model_complete(tf)) {
+        flux_transformer_free(tf);
+        return NULL;
+    }
+    return tf;
 }
 
 /* ---- the reference's parsed-file handle (flux_safetensors.h:31-49) ---- */
@@ -224,6 +235,28 @@ void fh_safetensors_close_compat(void *p) {
     free(sf->path);
     free(sf->header_json);
     free(sf);
+}
+
+int fh_safetensors_walk_handle(void *p, fh_tensor_cb cb, void *ctx) {
+    ref_safetensors_file *sf = (ref_safetensors_file *)p;
+    if (!sf || !sf->data) return flux_hip_fail("safetensors handle is NULL");
+    if (sf->num_tensors < 0 || sf->num_tensors > 512) return flux_hip_fail("safetensors handle: bad tensor count");
+    for (int i = 0; i < sf->num_tensors; i++) {
+        const ref_safetensor *t = &sf->tensors[i];
+        int64_t numel = 1;
+        for (int d = 0; d < t->ndim; d++) numel *= t->shape[d];
+        if (!cb(ctx, t->name, t->dtype, (const char *)sf->data + 8 + sf->header_size + t->data_offset, numel)) return 0;
+    }
+    return 1;
+}
+
+float fh_tensor_value(int dtype, const void *data, int64_t i) {
+    if (dtype == DT_F32) return ((const float *)data)[i];
+    if (dtype == DT_F16) return f16_to_f32(((const uint16_t *)data)[i]);
+    uint32_t u = (uint32_t)((const uint16_t *)data)[i] << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
 }
 
 /* The reference fixes the architecture in its loader (flux_transformer.c:4418-4434). The file

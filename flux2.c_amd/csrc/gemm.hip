@@ -51,7 +51,28 @@ struct GemmArgs {
     int ksplit, kt_per;
     float *ws;
     int moff[2], ws_rows;
+    /* convolution epilogues (see flux_hip_conv): rows are the positions of a zero-bordered
+     * conv_hp x conv_wp image with channels contiguous. With 9 taps K runs tap-major over
+     * 9 x cin and K step kt reads the activation rows shifted by its tap's (dy, dx);
+     * conv_kshift = log2(cin / 64) */
+    int conv_taps, conv_kshift, conv_wp, conv_hp;
+    const float *bias, *res;
 };
+
+template <int EPI> struct IsConv { static constexpr bool value = EPI == FLUX_HIP_EPI_CONV_BF16 || EPI == FLUX_HIP_EPI_CONV_F32; };
+
+/* Element offset of K step kt within an activation row. Plain GEMM: kt * 64. 3x3 convolution:
+ * tap = kt / (cin/64) selects a neighbour dy*Wp + dx rows away (uniform for the whole launch,
+ * because border positions are rows of the matrix too), the remainder a 64-channel slice. */
+template <int EPI>
+__device__ __forceinline__ int a_step_offset(const GemmArgs &g, int kt) {
+    if (IsConv<EPI>::value && g.conv_taps == 9) {
+        const int tap = kt >> g.conv_kshift, kc = kt - (tap << g.conv_kshift);
+        const int dy = (tap * 11) >> 5, dx = tap - dy * 3; /* tap / 3, tap % 3 for tap < 9 */
+        return ((dy - 1) * g.conv_wp + (dx - 1)) * g.lda + kc * 64;
+    }
+    return kt * 64;
+}
 
 /* internal epilogue: fp32 partial sums of one K slice (see split-K above) */
 #define EPI_PARTIAL 5
@@ -112,6 +133,11 @@ __device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f
     for (int j = 0; j < TM; j++) {
         const int m = m0 + wm * WM + j * 16 + l15;
         if (m >= M) continue;
+        bool inside = true; /* convolutions: border positions of the image are written as zeros */
+        if (IsConv<EPI>::value && g.conv_wp > 0) {
+            const int y = m / g.conv_wp, x = m - y * g.conv_wp;
+            inside = y >= 1 && y < g.conv_hp - 1 && x >= 1 && x < g.conv_wp - 1;
+        }
         if (EPI == FLUX_HIP_EPI_SWIGLU) {
             bf16 *C = (bf16 *)g.C[prob] + (size_t)m * ldc + tn * (BN / 2) + wn * (WN / 2) + lq * 4;
 #pragma unroll
@@ -144,6 +170,19 @@ __device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f
 #pragma unroll
                     for (int e = 0; e < 4; e++) x[e] += gt[e] * acc[i][j][e];
                     *(f32x4 *)p = x;
+                } else if (EPI == FLUX_HIP_EPI_CONV_BF16) {
+                    const f32x4 bv = *(const f32x4 *)(g.bias + n);
+                    bf16x4 o;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o[e] = (bf16)(inside ? acc[i][j][e] + bv[e] : 0.0f);
+                    *(bf16x4 *)((bf16 *)g.C[prob] + (size_t)m * ldc + n) = o;
+                } else if (EPI == FLUX_HIP_EPI_CONV_F32) {
+                    const f32x4 bv = *(const f32x4 *)(g.bias + n);
+                    f32x4 r = {0.0f, 0.0f, 0.0f, 0.0f};
+                    if (g.res) r = *(const f32x4 *)(g.res + (size_t)m * ldc + n);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) r[e] = inside ? r[e] + acc[i][j][e] + bv[e] : 0.0f;
+                    *(f32x4 *)((float *)g.C[prob] + (size_t)m * ldc + n) = r;
                 }
             }
         }
@@ -194,9 +233,10 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
     }
     auto issue = [&](int kt, int stage) {
         char *base = smem + stage * STAGE;
+        const int aoff = a_step_offset<EPI>(g, kt);
 #pragma unroll
         for (int i = 0; i < PA; i++)
-            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(a_ptr[i] + kt * 64), LDS_PTR(base + a_lds[i]), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(a_ptr[i] + aoff), LDS_PTR(base + a_lds[i]), 16, 0, 0);
 #pragma unroll
         for (int i = 0; i < PB; i++)
             __builtin_amdgcn_global_load_lds(GLOBAL_PTR(b_ptr[i] + kt * 64), LDS_PTR(base + b_lds[i]), 16, 0, 0);
@@ -309,8 +349,10 @@ __global__ __launch_bounds__(256) void gemm4w_kernel(GemmArgs g) {
     for (int i = 0; i < TM; i++) src[i] = A + (size_t)min(m0 + lrow + i * 32, M - 1) * g.lda + chunk;
 #pragma unroll
     for (int i = 0; i < TN; i++) src[TM + i] = W + (size_t)weight_row<BN, WN, EPI>(g, tn, lrow + i * 32) * g.ldw + chunk;
+    /* (convolutions never split K, so for them kt below is the absolute K step) */
     auto issue1 = [&](int kt, int stage, int i) {
-        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src[i] + kt * 64), LDS_PTR(smem + stage * STAGE + (lrow - (lane >> 3) + i * 32) * 128), 16, 0, 0);
+        const int off = i < TM ? a_step_offset<EPI>(g, kt) : kt * 64;
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src[i] + off), LDS_PTR(smem + stage * STAGE + (lrow - (lane >> 3) + i * 32) * 128), 16, 0, 0);
     };
 #pragma unroll
     for (int i = 0; i < NL; i++) issue1(0, 0, i);
@@ -442,6 +484,18 @@ static int launch_epi(GemmArgs &g, int tile) {
     }
 }
 
+/* The convolution epilogues exist for the tiles whose width divides 64, 128, 256 or 512 output
+ * channels. */
+template <int EPI>
+static int launch_conv(GemmArgs &g, int tile) {
+    switch (tile) {
+        case 2: return launch_4w<8, 8, EPI>(g);
+        case 1: return launch_cfg<128, 128, 2, 2, EPI>(g);
+        case 3: return launch_cfg<64, 64, 2, 2, EPI>(g);
+        default: return launch_cfg<64, 128, 2, 2, EPI>(g);
+    }
+}
+
 /* Second pass of a split-K GEMM: sums the K slices ws[s][moff + m][n] in a fixed order and
  * applies the epilogue to the sum (for the residual form the same arithmetic as gated_add,
  * flux_transformer.c:90-97). For SwiGLU the workspace holds plain columns - gate features in
@@ -566,8 +620,91 @@ static int probe_slot(int epilogue) {
     return g_probe_n++;
 }
 
+/* Tile and K-split choice, then the launch; `allowed` has bit t set for every tile id that may be used. */
+static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed) {
+    /* Choose tile and K split with a small cost model: workgroups run in rounds over
+     * 256 CUs x occupancy; a workgroup's time is its FLOPs at the tile's measured rate plus a
+     * fixed prologue/epilogue cost; the launch cannot beat the time to stream its operands,
+     * which depends on how many bytes the resident workgroups keep in flight. */
+    /* tile ids: 0..3 the small tiles and 256 x 256, 4 = the 8-wave form of 256 x 256 (only when
+     * forced, for comparison runs), 5 = 288 x 192, 6 = 192 x 192, 7 = 256 x 192 */
+    constexpr int NT = 8;
+    static const int bm[NT] = {64, 128, 256, 64, 256, 288, 192, 256}, bn[NT] = {128, 128, 256, 64, 256, 192, 192, 192}, occ[NT] = {3, 2, 1, 4, 1, 1, 1, 1};
+    static const double rate[NT] = {2.0e12, 2.9e12, 5.3e12, 1.5e12, 4.6e12, 5.0e12, 4.0e12, 4.9e12}; /* FLOP/s of one CU running this tile */
+    const int kt_total = g.K >> 6;
+    int tile = -1, best_split = 1;
+    {
+        double best = 1e30;
+        static const int splits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
+        /* every epilogue but the transposed store can run as K slices + a finishing pass; for
+         * SwiGLU the gate and up rows must be one contiguous block of the weight matrix */
+        const int N = g.N, K = g.K, w_row0 = g.w_row0, w_row1 = g.w_row1;
+        const bool can_split = g_splitk_enabled &&
+                               (epilogue == FLUX_HIP_EPI_RESID || epilogue == FLUX_HIP_EPI_BF16 || epilogue == FLUX_HIP_EPI_F32 ||
+                                (epilogue == FLUX_HIP_EPI_SWIGLU && w_row1 == w_row0 + N / 2));
+        double rows = 0.0;
+        for (int i = 0; i < np; i++) rows += g.M[i];
+        for (int t = 0; t < NT; t++) {
+            if (N % bn[t]) continue;
+            if (!((allowed >> t) & 1)) continue;
+            long tiles = 0;
+            for (int i = 0; i < np; i++) tiles += (g.M[i] + bm[t] - 1) / bm[t];
+            tiles *= N / bn[t];
+            for (int si = 0; si < 10; si++) {
+                const int sp = splits[si];
+                if (sp > 1 && (!can_split || kt_total / sp < 4)) break;
+                const int per = (kt_total + sp - 1) / sp;
+                const long blocks = tiles * ((kt_total + per - 1) / per);
+                const long slots = 256L * occ[t];
+                const long rounds = (blocks + slots - 1) / slots;
+                const long resident = blocks < slots ? blocks : slots;
+                const long per_cu = (resident + 255) / 256;          /* workgroups sharing one CU */
+                const double t_block = 2.0 * bm[t] * bn[t] * 64.0 * per / (rate[t] / per_cu) + 2.5e-6;
+                double t_compute = rounds * t_block;
+                const double bytes = (rows + N) * (double)K * 2.0;
+                double bw = 5.5e12 * (double)(resident * (bm[t] + bn[t]) * 128) / 12.0e6;
+                if (bw > 5.5e12) bw = 5.5e12;
+                double est = t_compute > bytes / bw ? t_compute : bytes / bw;
+                if (sp > 1) est += 3.0e-6 + (sp + 2.0) * rows * N * 4.0 / 4.0e12;
+                if (est < best) { best = est; tile = t; best_split = sp; }
+            }
+        }
+    }
+    if (tile < 0) return flux_hip_fail("flux_hip_linear: no permitted tile width divides N=%d", g.N);
+    g.ksplit = 1;
+    g.kt_per = kt_total;
+    if (best_split > 1) {
+        g.kt_per = (kt_total + best_split - 1) / best_split;
+        g.ksplit = (kt_total + g.kt_per - 1) / g.kt_per;
+        g.moff[0] = 0;
+        g.moff[1] = g.M[0];
+        g.ws_rows = g.M[0] + g.M[1];
+        if (!ensure_ws((size_t)g.ksplit * g.ws_rows * g.N * sizeof(float))) return 0;
+        g.ws = g_ws;
+    }
+
+    const int slot = probe_slot(epilogue);
+    if (slot >= 0) g_probe_tile[slot] = (unsigned char)tile;
+    if (slot >= 0) (void)hipEventRecord(g_probe_ev[slot][0], flux_hip_stream_handle());
+    int ok;
+    const bool split = g.ksplit > 1;
+    switch (epilogue) {
+        case FLUX_HIP_EPI_BF16: ok = split ? launch_split<FLUX_HIP_EPI_BF16>(g, tile) : launch_epi<FLUX_HIP_EPI_BF16>(g, tile); break;
+        case FLUX_HIP_EPI_F32: ok = split ? launch_split<FLUX_HIP_EPI_F32>(g, tile) : launch_epi<FLUX_HIP_EPI_F32>(g, tile); break;
+        case FLUX_HIP_EPI_F32_T: ok = launch_epi<FLUX_HIP_EPI_F32_T>(g, tile); break;
+        case FLUX_HIP_EPI_RESID: ok = split ? launch_split<FLUX_HIP_EPI_RESID>(g, tile) : launch_epi<FLUX_HIP_EPI_RESID>(g, tile); break;
+        case FLUX_HIP_EPI_SWIGLU: ok = split ? launch_split<FLUX_HIP_EPI_SWIGLU>(g, tile) : launch_epi<FLUX_HIP_EPI_SWIGLU>(g, tile); break;
+        case FLUX_HIP_EPI_CONV_BF16: ok = launch_conv<FLUX_HIP_EPI_CONV_BF16>(g, tile); break;
+        case FLUX_HIP_EPI_CONV_F32: ok = launch_conv<FLUX_HIP_EPI_CONV_F32>(g, tile); break;
+        default: return flux_hip_fail("flux_hip_linear: unknown epilogue %d", epilogue);
+    }
+    if (slot >= 0) (void)hipEventRecord(g_probe_ev[slot][1], flux_hip_stream_handle());
+    return ok;
+}
+
 extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
                                int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1) {
+    if (epilogue < FLUX_HIP_EPI_BF16 || epilogue > FLUX_HIP_EPI_SWIGLU) return flux_hip_fail("flux_hip_linear: unknown epilogue %d", epilogue);
     if (nparts < 1 || nparts > 2) return flux_hip_fail("flux_hip_linear: nparts=%d (1 or 2)", nparts);
     if (K <= 0 || (K & 63)) return flux_hip_fail("flux_hip_linear: K=%d must be a positive multiple of 64", K);
     if (N <= 0 || (N & 127)) return flux_hip_fail("flux_hip_linear: N=%d must be a positive multiple of 128", N);
@@ -600,79 +737,36 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
     }
     if (np == 0) return 1;
     g.N = N; g.K = K; g.lda = lda; g.ldw = ldw; g.ldc = ldc; g.w_row0 = w_row0; g.w_row1 = w_row1;
+    return gemm_dispatch(g, np, epilogue, g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask);
+}
 
-    /* Choose tile and K split with a small cost model: workgroups run in rounds over
-     * 256 CUs x occupancy; a workgroup's time is its FLOPs at the tile's measured rate plus a
-     * fixed prologue/epilogue cost; the launch cannot beat the time to stream its operands,
-     * which depends on how many bytes the resident workgroups keep in flight. */
-    /* tile ids: 0..3 the small tiles and 256 x 256, 4 = the 8-wave form of 256 x 256 (only when
-     * forced, for comparison runs), 5 = 288 x 192, 6 = 192 x 192, 7 = 256 x 192 */
-    constexpr int NT = 8;
-    static const int bm[NT] = {64, 128, 256, 64, 256, 288, 192, 256}, bn[NT] = {128, 128, 256, 64, 256, 192, 192, 192}, occ[NT] = {3, 2, 1, 4, 1, 1, 1, 1};
-    static const double rate[NT] = {2.0e12, 2.9e12, 5.3e12, 1.5e12, 4.6e12, 5.0e12, 4.0e12, 4.9e12}; /* FLOP/s of one CU running this tile */
-    const int kt_total = K >> 6;
-    int tile = 1, best_split = 1;
-    {
-        double best = 1e30;
-        static const int splits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
-        /* every epilogue but the transposed store can run as K slices + a finishing pass; for
-         * SwiGLU the gate and up rows must be one contiguous block of the weight matrix */
-        const bool can_split = g_splitk_enabled &&
-                               (epilogue == FLUX_HIP_EPI_RESID || epilogue == FLUX_HIP_EPI_BF16 || epilogue == FLUX_HIP_EPI_F32 ||
-                                (epilogue == FLUX_HIP_EPI_SWIGLU && w_row1 == w_row0 + N / 2));
-        double rows = 0.0;
-        for (int i = 0; i < np; i++) rows += g.M[i];
-        for (int t = 0; t < NT; t++) {
-            if (N % bn[t]) continue;
-            if (g_force_tile >= 0 ? t != g_force_tile : !((g_tile_mask >> t) & 1)) continue;
-            long tiles = 0;
-            for (int i = 0; i < np; i++) tiles += (g.M[i] + bm[t] - 1) / bm[t];
-            tiles *= N / bn[t];
-            for (int si = 0; si < 10; si++) {
-                const int sp = splits[si];
-                if (sp > 1 && (!can_split || kt_total / sp < 4)) break;
-                const int per = (kt_total + sp - 1) / sp;
-                const long blocks = tiles * ((kt_total + per - 1) / per);
-                const long slots = 256L * occ[t];
-                const long rounds = (blocks + slots - 1) / slots;
-                const long resident = blocks < slots ? blocks : slots;
-                const long per_cu = (resident + 255) / 256;          /* workgroups sharing one CU */
-                const double t_block = 2.0 * bm[t] * bn[t] * 64.0 * per / (rate[t] / per_cu) + 2.5e-6;
-                double t_compute = rounds * t_block;
-                const double bytes = (rows + N) * (double)K * 2.0;
-                double bw = 5.5e12 * (double)(resident * (bm[t] + bn[t]) * 128) / 12.0e6;
-                if (bw > 5.5e12) bw = 5.5e12;
-                double est = t_compute > bytes / bw ? t_compute : bytes / bw;
-                if (sp > 1) est += 3.0e-6 + (sp + 2.0) * rows * N * 4.0 / 4.0e12;
-                if (est < best) { best = est; tile = t; best_split = sp; }
-            }
-        }
-    }
-    g.ksplit = 1;
-    g.kt_per = kt_total;
-    if (best_split > 1) {
-        g.kt_per = (kt_total + best_split - 1) / best_split;
-        g.ksplit = (kt_total + g.kt_per - 1) / g.kt_per;
-        g.moff[0] = 0;
-        g.moff[1] = g.M[0];
-        g.ws_rows = g.M[0] + g.M[1];
-        if (!ensure_ws((size_t)g.ksplit * g.ws_rows * N * sizeof(float))) return 0;
-        g.ws = g_ws;
-    }
-
-    const int slot = probe_slot(epilogue);
-    if (slot >= 0) g_probe_tile[slot] = (unsigned char)tile;
-    if (slot >= 0) (void)hipEventRecord(g_probe_ev[slot][0], flux_hip_stream_handle());
-    int ok;
-    const bool split = g.ksplit > 1;
-    switch (epilogue) {
-        case FLUX_HIP_EPI_BF16: ok = split ? launch_split<FLUX_HIP_EPI_BF16>(g, tile) : launch_epi<FLUX_HIP_EPI_BF16>(g, tile); break;
-        case FLUX_HIP_EPI_F32: ok = split ? launch_split<FLUX_HIP_EPI_F32>(g, tile) : launch_epi<FLUX_HIP_EPI_F32>(g, tile); break;
-        case FLUX_HIP_EPI_F32_T: ok = launch_epi<FLUX_HIP_EPI_F32_T>(g, tile); break;
-        case FLUX_HIP_EPI_RESID: ok = split ? launch_split<FLUX_HIP_EPI_RESID>(g, tile) : launch_epi<FLUX_HIP_EPI_RESID>(g, tile); break;
-        case FLUX_HIP_EPI_SWIGLU: ok = split ? launch_split<FLUX_HIP_EPI_SWIGLU>(g, tile) : launch_epi<FLUX_HIP_EPI_SWIGLU>(g, tile); break;
-        default: return flux_hip_fail("flux_hip_linear: unknown epilogue %d", epilogue);
-    }
-    if (slot >= 0) (void)hipEventRecord(g_probe_ev[slot][1], flux_hip_stream_handle());
-    return ok;
+/* Convolution over a zero-bordered channels-last image as one GEMM, see the header. */
+extern "C" int flux_hip_conv(int epilogue, const void *in, const void *w, const float *bias, const float *res,
+                             void *out, int rows, int wp, int cin, int cout, int taps) {
+    if (epilogue != FLUX_HIP_EPI_CONV_BF16 && epilogue != FLUX_HIP_EPI_CONV_F32)
+        return flux_hip_fail("flux_hip_conv: epilogue %d is not a convolution epilogue", epilogue);
+    if (taps != 1 && taps != 9) return flux_hip_fail("flux_hip_conv: taps=%d (1 or 9)", taps);
+    if (rows <= 0 || cin <= 0 || (cin & 63) || cout <= 0 || (cout & 63))
+        return flux_hip_fail("flux_hip_conv: rows=%d cin=%d cout=%d (channels must be multiples of 64)", rows, cin, cout);
+    int kshift = 0;
+    while ((64 << kshift) < cin) kshift++;
+    if (taps == 9 && ((64 << kshift) != cin || wp < 3 || rows % wp || rows / wp < 3))
+        return flux_hip_fail("flux_hip_conv: a 3x3 convolution needs cin = 64 * 2^k and a bordered image (rows=%d wp=%d cin=%d)", rows, wp, cin);
+    if (wp > 0 && rows % wp) return flux_hip_fail("flux_hip_conv: rows=%d is not a multiple of the image width %d", rows, wp);
+    if (!in || !w || !bias || !out) return flux_hip_fail("flux_hip_conv: NULL operand");
+    if ((((uintptr_t)in | (uintptr_t)w | (uintptr_t)bias | (uintptr_t)res | (uintptr_t)out) & 15))
+        return flux_hip_fail("flux_hip_conv: operands must be 16-byte aligned");
+    if (res && epilogue != FLUX_HIP_EPI_CONV_F32) return flux_hip_fail("flux_hip_conv: only the fp32 epilogue adds a residual");
+    GemmArgs g = {};
+    g.A[0] = (const bf16 *)in;
+    g.W[0] = (const bf16 *)w;
+    g.C[0] = out;
+    g.M[0] = rows;
+    g.N = cout; g.K = taps * cin; g.lda = cin; g.ldw = taps * cin; g.ldc = cout;
+    g.conv_taps = taps; g.conv_kshift = kshift; g.conv_wp = wp; g.conv_hp = wp > 0 ? rows / wp : 0;
+    g.bias = bias; g.res = res;
+    const unsigned conv_tiles = 0x0F; /* 64x128, 128x128, 256x256 (4 waves), 64x64 */
+    unsigned allowed = g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask;
+    if (!(allowed & conv_tiles)) allowed = conv_tiles;
+    return gemm_dispatch(g, 1, epilogue, allowed & conv_tiles);
 }

@@ -67,6 +67,15 @@ int fh_forward_device(flux_transformer_t *tf, const fh_rope *rp, const float *z_
                       const void *txt_dev, int step, float *v_dev, fh_events *ev);
 int flux_hip_fail(const char *fmt, ...);
 
+/* safetensors access shared by the transformer and VAE loaders (flux_loader_hip.c) */
+enum { FH_DT_F32 = 0, FH_DT_F16 = 1, FH_DT_BF16 = 2 }; /* the reference's numbering, flux_safetensors.h:20-28 */
+typedef int (*fh_tensor_cb)(void *ctx, const char *name, int dtype, const void *data, int64_t numel);
+int fh_safetensors_walk(const char *path, fh_tensor_cb cb, void *ctx);
+/* the same over the reference's parsed-file handle (safetensors_file_t, flux_safetensors.h:31-49) */
+int fh_safetensors_walk_handle(void *sf, fh_tensor_cb cb, void *ctx);
+/* element i of a tensor of the given dtype as fp32 */
+float fh_tensor_value(int dtype, const void *data, int64_t i);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,309 @@
+/*
+ * vae.hip - the memory-bound kernels of the VAE decoder (reference: flux_vae_decode,
+ * flux_vae.c:690-837); its convolutions and attention products run as MFMA GEMMs (gemm.hip).
+ *
+ * Images are channels-last with a one-pixel zero border: position p = y * Wp + x over the
+ * (H+2) x (W+2) grid, channels contiguous. That makes a 3x3 convolution one GEMM whose K steps
+ * read the same rows shifted by a constant (flux_hip_conv), and every kernel here keeps the
+ * border at zero so that the next convolution sees its padding. The residual stream is fp32;
+ * what feeds an MFMA is bf16.
+ */
+#include "common.h"
+#include "../../include/flux_hip.h"
+#include <math.h>
+
+#define LAUNCH_OK(what)                                                                         \
+    do {                                                                                        \
+        hipError_t e_ = hipGetLastError();                                                      \
+        if (e_ != hipSuccess) return flux_hip_fail("%s launch failed: %s", what, hipGetErrorString(e_)); \
+    } while (0)
+
+__device__ __forceinline__ bool interior(int p, int hp, int wp) {
+    const int y = p / wp, x = p - y * wp;
+    return y >= 1 && y < hp - 1 && x >= 1 && x < wp - 1;
+}
+
+/* latent [128, h, w] fp32 -> x * sqrt(var + eps) + mean per latent channel (flux_vae.c:718-728),
+ * 2x2 unpatchify to 32 channels at (2h, 2w) (flux_kernels.c:1067-1097), 1x1 post-quant
+ * convolution 32 -> 32 (flux_vae.c:739-741); written as bf16 [Hp*Wp, 64] with channels 32..63
+ * zero (the first 3x3 convolution wants a multiple of 64 input channels). One workgroup of 64
+ * threads per position. */
+__global__ __launch_bounds__(64) void vae_latent_kernel(bf16 *__restrict__ out, const float *__restrict__ latent,
+                                                        const float *__restrict__ bn_mean, const float *__restrict__ bn_var,
+                                                        const float *__restrict__ pq_w, const float *__restrict__ pq_b,
+                                                        int h, int w, float eps) {
+    const int hp = 2 * h + 2, wp = 2 * w + 2;
+    const int p = blockIdx.x, c = threadIdx.x;
+    const int y = p / wp, x = p - y * wp;
+    float v = 0.0f;
+    if (c < 32 && y >= 1 && y < hp - 1 && x >= 1 && x < wp - 1) {
+        const int ph = (y - 1) >> 1, pi = (y - 1) & 1, pw = (x - 1) >> 1, pj = (x - 1) & 1;
+        v = pq_b[c];
+        for (int ci = 0; ci < 32; ci++) {
+            const int lc = ci * 4 + pi * 2 + pj;
+            const float z = latent[((size_t)lc * h + ph) * w + pw] * sqrtf(bn_var[lc] + eps) + bn_mean[lc];
+            v += pq_w[c * 32 + ci] * z;
+        }
+    }
+    out[(size_t)p * 64 + c] = (bf16)v;
+}
+
+/* ---- group norm (flux_group_norm, flux_kernels.c:511-553): 32 groups of C/32 adjacent channels,
+ * statistics over the whole image. Three kernels: per-block partial sums, their combination in
+ * double precision, and the normalisation itself. Border positions hold zeros and add nothing
+ * to the sums; the element count is the interior's. ---- */
+#define GN_ROWS 256 /* positions per workgroup of the partial-sum pass */
+
+__global__ __launch_bounds__(256) void gn_partial_kernel(float *__restrict__ partial, const float *__restrict__ x, int rows, int C) {
+    __shared__ float sh[256][2];
+    const int quads = C >> 2, rpi = 256 / quads; /* C is 128, 256 or 512: 32, 64 or 128 quads */
+    const int q = threadIdx.x % quads, r0 = threadIdx.x / quads;
+    const int row_begin = blockIdx.x * GN_ROWS, row_end = min(rows, row_begin + GN_ROWS);
+    float s = 0.0f, ss = 0.0f;
+    for (int r = row_begin + r0; r < row_end; r += rpi) {
+        const f32x4 v = *(const f32x4 *)(x + (size_t)r * C + q * 4);
+#pragma unroll
+        for (int e = 0; e < 4; e++) { s += v[e]; ss += v[e] * v[e]; }
+    }
+    sh[threadIdx.x][0] = s;
+    sh[threadIdx.x][1] = ss;
+    __syncthreads();
+    if (threadIdx.x < 32) {
+        /* group g owns quads [g * qpg, (g+1) * qpg) of every thread row; fixed summation order */
+        const int g = threadIdx.x, qpg = quads >> 5;
+        float a = 0.0f, b = 0.0f;
+        for (int r = 0; r < rpi; r++)
+            for (int k = 0; k < qpg; k++) {
+                a += sh[r * quads + g * qpg + k][0];
+                b += sh[r * quads + g * qpg + k][1];
+            }
+        partial[((size_t)blockIdx.x * 32 + g) * 2 + 0] = a;
+        partial[((size_t)blockIdx.x * 32 + g) * 2 + 1] = b;
+    }
+}
+
+/* one workgroup per group: mean and 1/sqrt(var + eps) with the biased variance */
+__global__ __launch_bounds__(256) void gn_finalize_kernel(float *__restrict__ stats, const float *__restrict__ partial, int nblocks,
+                                                          double count, float eps) {
+    __shared__ double sh[256][2];
+    const int g = blockIdx.x;
+    double a = 0.0, b = 0.0;
+    for (int i = threadIdx.x; i < nblocks; i += 256) {
+        a += (double)partial[((size_t)i * 32 + g) * 2 + 0];
+        b += (double)partial[((size_t)i * 32 + g) * 2 + 1];
+    }
+    sh[threadIdx.x][0] = a;
+    sh[threadIdx.x][1] = b;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if (threadIdx.x < s) {
+            sh[threadIdx.x][0] += sh[threadIdx.x + s][0];
+            sh[threadIdx.x][1] += sh[threadIdx.x + s][1];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const double mean = sh[0][0] / count;
+        double var = sh[0][1] / count - mean * mean;
+        if (var < 0.0) var = 0.0;
+        stats[g * 2 + 0] = (float)mean;
+        stats[g * 2 + 1] = (float)(1.0 / sqrt(var + (double)eps));
+    }
+}
+
+/* out bf16 = [swish](gamma * (x - mean) * rstd + beta), zeros on the border; raw (optional)
+ * receives x itself as bf16, the input of a residual block's 1x1 shortcut convolution */
+__global__ __launch_bounds__(256) void gn_apply_kernel(bf16 *__restrict__ out, bf16 *__restrict__ raw, const float *__restrict__ x,
+                                                       const float *__restrict__ stats, const float *__restrict__ gamma,
+                                                       const float *__restrict__ beta, int rows, int C, int hp, int wp, int swish) {
+    const int quads = C >> 2;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)rows * quads) return;
+    const int r = (int)(idx / quads), q = (int)(idx - (size_t)r * quads);
+    const int g = (q * 4) / (C >> 5);
+    const f32x4 v = *(const f32x4 *)(x + (size_t)r * C + q * 4);
+    const bool in = interior(r, hp, wp);
+    const float mean = stats[g * 2], rstd = stats[g * 2 + 1];
+    const f32x4 gm = *(const f32x4 *)(gamma + q * 4), bt = *(const f32x4 *)(beta + q * 4);
+    bf16x4 o, rw;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        float y = gm[e] * ((v[e] - mean) * rstd) + bt[e];
+        if (swish) y = silu_f(y);
+        o[e] = (bf16)(in ? y : 0.0f);
+        rw[e] = (bf16)v[e];
+    }
+    *(bf16x4 *)(out + (size_t)r * C + q * 4) = o;
+    if (raw) *(bf16x4 *)(raw + (size_t)r * C + q * 4) = rw;
+}
+
+/* nearest-neighbour 2x upsample (flux_upsample_nearest, flux_kernels.c:1017-1036): fp32
+ * [hp*wp, C] -> bf16 [(2H+2)*(2W+2), C] with a fresh zero border */
+__global__ __launch_bounds__(256) void vae_upsample_kernel(bf16 *__restrict__ out, const float *__restrict__ x, int hp, int wp, int C) {
+    const int quads = C >> 2;
+    const int H2 = 2 * (hp - 2), W2 = 2 * (wp - 2), hp2 = H2 + 2, wp2 = W2 + 2;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)hp2 * wp2 * quads) return;
+    const int p = (int)(idx / quads), q = (int)(idx - (size_t)p * quads);
+    const int y = p / wp2, xx = p - y * wp2;
+    bf16x4 o = {(bf16)0.0f, (bf16)0.0f, (bf16)0.0f, (bf16)0.0f};
+    if (y >= 1 && y <= H2 && xx >= 1 && xx <= W2) {
+        const int sy = 1 + ((y - 1) >> 1), sx = 1 + ((xx - 1) >> 1);
+        const f32x4 v = *(const f32x4 *)(x + ((size_t)sy * wp + sx) * C + q * 4);
+#pragma unroll
+        for (int e = 0; e < 4; e++) o[e] = (bf16)v[e];
+    }
+    *(bf16x4 *)(out + (size_t)p * C + q * 4) = o;
+}
+
+/* ---- attention over all positions with one head (attnblock_forward, flux_vae.c:223-313).
+ * Scores are materialised, as in the reference: S = q k^T (GEMM), P = softmax(S * scale + bias)
+ * (below), O = P v (GEMM against v^T). Keys run over the bordered grid plus padding up to a
+ * multiple of 128; key_bias is 0 for real pixels and -inf for border and padding columns. ---- */
+__global__ __launch_bounds__(256) void vae_key_bias_kernel(float *__restrict__ bias, int n, int rows, int hp, int wp) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    bias[i] = (i < rows && interior(i, hp, wp)) ? 0.0f : -INFINITY;
+}
+
+__global__ __launch_bounds__(256) void vae_softmax_kernel(bf16 *__restrict__ P, const float *__restrict__ S, const float *__restrict__ key_bias,
+                                                          int ld, float scale) {
+    __shared__ float red[4];
+    const float *s = S + (size_t)blockIdx.x * ld;
+    bf16 *p = P + (size_t)blockIdx.x * ld;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float mx = -INFINITY;
+    for (int i = threadIdx.x * 4; i < ld; i += 1024) {
+        const f32x4 v = *(const f32x4 *)(s + i), kb = *(const f32x4 *)(key_bias + i);
+#pragma unroll
+        for (int e = 0; e < 4; e++) mx = fmaxf(mx, v[e] * scale + kb[e]);
+    }
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    if (lane == 0) red[wave] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float sum = 0.0f;
+    for (int i = threadIdx.x * 4; i < ld; i += 1024) {
+        const f32x4 v = *(const f32x4 *)(s + i), kb = *(const f32x4 *)(key_bias + i);
+#pragma unroll
+        for (int e = 0; e < 4; e++) sum += __expf(v[e] * scale + kb[e] - mx);
+    }
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+    if (lane == 0) red[wave] = sum;
+    __syncthreads();
+    const float inv = 1.0f / (red[0] + red[1] + red[2] + red[3]);
+    for (int i = threadIdx.x * 4; i < ld; i += 1024) {
+        const f32x4 v = *(const f32x4 *)(s + i), kb = *(const f32x4 *)(key_bias + i);
+        bf16x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; e++) o[e] = (bf16)(__expf(v[e] * scale + kb[e] - mx) * inv);
+        *(bf16x4 *)(p + i) = o;
+    }
+}
+
+/* vt[c][j] = v[j][c] for j < rows, 0 for rows <= j < ld: the value matrix as the "weight" operand
+ * of the second attention GEMM. 64 x 64 tiles through LDS. */
+__global__ __launch_bounds__(256) void vae_transpose_kernel(bf16 *__restrict__ vt, int ld, const bf16 *__restrict__ v, int ldv, int rows) {
+    __shared__ bf16 tile[64][66];
+    const int j0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int jj = i >> 6, cc = i & 63;
+        tile[jj][cc] = (j0 + jj < rows) ? v[(size_t)(j0 + jj) * ldv + c0 + cc] : (bf16)0.0f;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int cc = i >> 6, jj = i & 63;
+        if (j0 + jj < ld) vt[(size_t)(c0 + cc) * ld + j0 + jj] = tile[jj][cc];
+    }
+}
+
+/* decoder output fp32 [hp*wp, ldx] (channels 0..2 used) -> image: 8-bit [H, W, 3] with the
+ * reference's conversion (v + 1) * 0.5 * 255, clamped, truncated (flux_vae.c:820-833), and
+ * optionally the unquantised values as [3, H, W] */
+__global__ __launch_bounds__(256) void vae_image_kernel(uint8_t *__restrict__ rgb, float *__restrict__ rgb_f32, const float *__restrict__ x,
+                                                        int ldx, int H, int W) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= H * W) return;
+    const int y = i / W, xx = i - y * W;
+    const float *src = x + ((size_t)(y + 1) * (W + 2) + xx + 1) * ldx;
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+        const float v = src[c];
+        float val = (v + 1.0f) * 0.5f * 255.0f;
+        val = val < 0.0f ? 0.0f : val > 255.0f ? 255.0f : val;
+        if (rgb) rgb[(size_t)i * 3 + c] = (uint8_t)val;
+        if (rgb_f32) rgb_f32[(size_t)c * H * W + i] = v;
+    }
+}
+
+/* ------------------------------------------------------------------ host entry points */
+
+extern "C" int flux_hip_vae_latent_in(void *out_bf16, const float *latent, const float *bn_mean, const float *bn_var,
+                                      const float *pq_w, const float *pq_b, int h, int w, float eps) {
+    if (h <= 0 || w <= 0) return flux_hip_fail("flux_hip_vae_latent_in: bad size %d x %d", h, w);
+    const int positions = (2 * h + 2) * (2 * w + 2);
+    hipLaunchKernelGGL(vae_latent_kernel, dim3(positions), dim3(64), 0, flux_hip_stream_handle(), (bf16 *)out_bf16, latent, bn_mean, bn_var,
+                       pq_w, pq_b, h, w, eps);
+    LAUNCH_OK("vae_latent_kernel");
+    return 1;
+}
+
+extern "C" int flux_hip_group_norm(void *out_bf16, void *raw_bf16, const float *x, const float *gamma, const float *beta,
+                                   float *scratch, int hp, int wp, int C, float eps, int swish) {
+    if (C != 128 && C != 256 && C != 512) return flux_hip_fail("flux_hip_group_norm: C=%d (128, 256 or 512)", C);
+    if (hp < 3 || wp < 3) return flux_hip_fail("flux_hip_group_norm: bad image %d x %d", hp, wp);
+    const int rows = hp * wp, nblocks = (rows + GN_ROWS - 1) / GN_ROWS;
+    float *partial = scratch + 64, *stats = scratch;
+    hipStream_t st = flux_hip_stream_handle();
+    hipLaunchKernelGGL(gn_partial_kernel, dim3(nblocks), dim3(256), 0, st, partial, x, rows, C);
+    LAUNCH_OK("gn_partial_kernel");
+    const double count = (double)(hp - 2) * (wp - 2) * (C / 32);
+    hipLaunchKernelGGL(gn_finalize_kernel, dim3(32), dim3(256), 0, st, stats, partial, nblocks, count, eps);
+    LAUNCH_OK("gn_finalize_kernel");
+    const size_t total = (size_t)rows * (C / 4);
+    hipLaunchKernelGGL(gn_apply_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, (bf16 *)out_bf16, (bf16 *)raw_bf16, x, stats,
+                       gamma, beta, rows, C, hp, wp, swish);
+    LAUNCH_OK("gn_apply_kernel");
+    return 1;
+}
+
+extern "C" size_t flux_hip_group_norm_scratch_floats(int hp, int wp) {
+    return 64 + (size_t)((hp * wp + GN_ROWS - 1) / GN_ROWS) * 64;
+}
+
+extern "C" int flux_hip_upsample2x(void *out_bf16, const float *x, int hp, int wp, int C) {
+    if (C <= 0 || (C & 3) || hp < 3 || wp < 3) return flux_hip_fail("flux_hip_upsample2x: bad shape");
+    const size_t total = (size_t)(2 * (hp - 2) + 2) * (2 * (wp - 2) + 2) * (C / 4);
+    hipLaunchKernelGGL(vae_upsample_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, flux_hip_stream_handle(), (bf16 *)out_bf16, x, hp,
+                       wp, C);
+    LAUNCH_OK("vae_upsample_kernel");
+    return 1;
+}
+
+extern "C" int flux_hip_vae_key_bias(float *bias, int n, int hp, int wp) {
+    hipLaunchKernelGGL(vae_key_bias_kernel, dim3((n + 255) / 256), dim3(256), 0, flux_hip_stream_handle(), bias, n, hp * wp, hp, wp);
+    LAUNCH_OK("vae_key_bias_kernel");
+    return 1;
+}
+
+extern "C" int flux_hip_softmax_rows(void *p_bf16, const float *s, const float *key_bias, int rows, int ld, float scale) {
+    if (rows <= 0 || ld <= 0 || (ld & 3)) return flux_hip_fail("flux_hip_softmax_rows: bad shape %d x %d", rows, ld);
+    hipLaunchKernelGGL(vae_softmax_kernel, dim3(rows), dim3(256), 0, flux_hip_stream_handle(), (bf16 *)p_bf16, s, key_bias, ld, scale);
+    LAUNCH_OK("vae_softmax_kernel");
+    return 1;
+}
+
+extern "C" int flux_hip_transpose_bf16(void *vt, int ld, const void *v, int ldv, int rows, int cols) {
+    if (cols <= 0 || (cols & 63) || ld < rows) return flux_hip_fail("flux_hip_transpose_bf16: bad shape");
+    hipLaunchKernelGGL(vae_transpose_kernel, dim3((ld + 63) / 64, cols / 64), dim3(256), 0, flux_hip_stream_handle(), (bf16 *)vt, ld, (const bf16 *)v,
+                       ldv, rows);
+    LAUNCH_OK("vae_transpose_kernel");
+    return 1;
+}
+
+extern "C" int flux_hip_vae_image_out(uint8_t *rgb, float *rgb_f32, const float *x, int ldx, int H, int W) {
+    hipLaunchKernelGGL(vae_image_kernel, dim3((H * W + 255) / 256), dim3(256), 0, flux_hip_stream_handle(), rgb, rgb_f32, x, ldx, H, W);
+    LAUNCH_OK("vae_image_kernel");
+    return 1;
+}

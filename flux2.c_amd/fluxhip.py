@@ -14,6 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 c_f, c_i, vp, c_sz = ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
 
 EPI_BF16, EPI_F32, EPI_F32_T, EPI_RESID, EPI_SWIGLU = range(5)
+EPI_CONV_BF16, EPI_CONV_F32 = 6, 7
 
 
 class _Cfg(ctypes.Structure):
@@ -123,6 +124,19 @@ def lib():
     L.flux_linear_schedule.argtypes = [c_i]
     L.flux_power_schedule.argtypes = [c_i, c_f]
     L.flux_official_schedule.argtypes = [c_i, c_i]
+    L.flux_hip_conv.argtypes = [c_i, vp, vp, vp, vp, vp, c_i, c_i, c_i, c_i, c_i]
+    L.flux_hip_group_norm.argtypes = [vp, vp, vp, vp, vp, vp, c_i, c_i, c_i, c_f, c_i]
+    L.flux_hip_group_norm_scratch_floats.restype = c_sz
+    L.flux_hip_group_norm_scratch_floats.argtypes = [c_i, c_i]
+    L.flux_hip_upsample2x.argtypes = [vp, vp, c_i, c_i, c_i]
+    L.flux_hip_softmax_rows.argtypes = [vp, vp, vp, c_i, c_i, c_f]
+    L.flux_hip_transpose_bf16.argtypes = [vp, c_i, vp, c_i, c_i, c_i]
+    L.flux_hip_vae_new.restype = vp
+    L.flux_hip_vae_load_file.restype = vp
+    L.flux_hip_vae_load_file.argtypes = [ctypes.c_char_p]
+    L.flux_hip_vae_set_tensor.argtypes = [vp, ctypes.c_char_p, c_i, vp, ctypes.c_int64]
+    L.flux_hip_vae_free.argtypes = [vp]
+    L.flux_hip_vae_decode.argtypes = [vp, vp, c_i, c_i, vp, vp]
     _lib = L
     return L
 
@@ -395,3 +409,43 @@ def randn(n, seed=None):
     out = np.empty(n, np.float32)
     lib().flux_randn(out.ctypes.data, n)
     return out
+
+
+class Vae:
+    """The VAE decoder on the GPU, built from named tensors (uint16 = bf16, float32) or a safetensors file."""
+
+    def __init__(self, weights=None, path=None):
+        init()
+        L = lib()
+        if path is not None:
+            self.h = L.flux_hip_vae_load_file(os.fsencode(path))
+            if not self.h:
+                raise FluxHipError(f"vae load_file: {L.flux_hip_last_error().decode()}")
+            return
+        self.h = L.flux_hip_vae_new()
+        if not self.h:
+            raise FluxHipError(f"vae_new: {L.flux_hip_last_error().decode()}")
+        for name, a in (weights or {}).items():
+            a = np.ascontiguousarray(a)
+            dt = {np.dtype(np.float32): 0, np.dtype(np.float16): 1, np.dtype(np.uint16): 2}[a.dtype]
+            check(L.flux_hip_vae_set_tensor(self.h, name.encode(), dt, a.ctypes.data, a.size), f"vae set_tensor({name})")
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().flux_hip_vae_free(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def decode(self, latent, h, w):
+        """latent [128, h, w] -> (float image [3, 16h, 16w], uint8 image [16h, 16w, 3])."""
+        latent = _f32(latent)
+        assert latent.size == 128 * h * w
+        f = np.empty((3, 16 * h, 16 * w), np.float32)
+        u = np.empty((16 * h, 16 * w, 3), np.uint8)
+        check(lib().flux_hip_vae_decode(self.h, latent.ctypes.data, h, w, u.ctypes.data, f.ctypes.data), "flux_hip_vae_decode")
+        return f, u

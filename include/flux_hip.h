@@ -63,7 +63,10 @@ enum {
     FLUX_HIP_EPI_F32 = 1,     /* C f32  [M, ldc] = A W^T */
     FLUX_HIP_EPI_F32_T = 2,   /* C f32  [N, ldc] = (A W^T)^T  (token-major -> channel-major) */
     FLUX_HIP_EPI_RESID = 3,   /* C f32  [M, ldc] += gate[n] * (A W^T)      gated_add, flux_transformer.c:90 */
-    FLUX_HIP_EPI_SWIGLU = 4   /* C bf16 [M, ldc] = silu(A Wg^T) * (A Wu^T) swiglu, flux_transformer.c:1749-1757 */
+    FLUX_HIP_EPI_SWIGLU = 4,  /* C bf16 [M, ldc] = silu(A Wg^T) * (A Wu^T) swiglu, flux_transformer.c:1749-1757 */
+    /* 5 is used inside the library */
+    FLUX_HIP_EPI_CONV_BF16 = 6, /* flux_hip_conv: out bf16 = conv + bias, zeros on the image border */
+    FLUX_HIP_EPI_CONV_F32 = 7   /* flux_hip_conv: out f32 = [res +] conv + bias, zeros on the image border */
 };
 
 /* One row range of a linear layer. */
@@ -87,6 +90,23 @@ typedef struct {
  */
 int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
                     int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1);
+
+/*
+ * 3x3 (taps = 9, padding 1, stride 1) or 1x1 (taps = 1) convolution with bias as one MFMA GEMM
+ * over a channels-last image. Replaces flux_conv2d (flux_kernels.c:342-470; im2col + sgemm
+ * there) for the VAE decoder's layers, with the residual add of resblock_forward /
+ * attnblock_forward (flux_vae.c:218, 311) in the fp32 epilogue.
+ *   in   bf16 [rows, cin]: the image including a one-pixel zero border, rows = (H+2) * (W+2)
+ *        positions in row-major order, wp = W+2. With 9 taps the kernel reads up to wp+1 rows
+ *        before `in` and after its end: the allocation must extend that far (contents there
+ *        only reach border outputs, which are written as zeros).
+ *   w    bf16 [cout, taps * cin], tap-major: w[o][(ky*3+kx) * cin + c]
+ *   bias f32 [cout]; res f32 [rows, cout] or NULL (may be `out` itself); out [rows, cout]
+ * Border positions of `out` are written as zeros, so it can feed the next convolution. wp = 0
+ * (1x1 only) treats every row as interior. cin, cout: multiples of 64; 9 taps: cin = 64 * 2^k.
+ */
+int flux_hip_conv(int epilogue, const void *in, const void *w, const float *bias, const float *res,
+                  void *out, int rows, int wp, int cin, int cout, int taps);
 
 /* Measurement hooks. force_tile: 0/1/2/3/5/6/7 pins the GEMM tile (64x128, 128x128, 256x256, 64x64,
  * 288x192, 192x192, 256x192; 4 = 256x256 in its 8-wave form, never chosen automatically), -1 restores the automatic
@@ -276,6 +296,43 @@ float *flux_hip_sample_heun_traced(void *transformer, const float *z, int channe
 float *flux_hip_sample_ancestral_traced(void *transformer, const float *z, int channels, int h, int w,
                                         const float *text_emb, int text_seq, const float *schedule, int num_steps,
                                         float eta, float *v_trace, void (*progress)(int, int));
+
+/* ---------------------------------------------------------------- VAE decoder
+ * The step after the sampling loop: final latent -> RGB image (flux_vae_decode,
+ * flux_vae.c:690-837; the reference's device path is vae_decode_gpu, flux_vae.c:505). Images on
+ * the device are channels-last with a one-pixel zero border, positions in row-major order over
+ * the (H+2) x (W+2) grid: hp = H+2, wp = W+2 below. */
+
+/*
+ * GroupNorm(32 groups, statistics over the whole image) with optional swish, x f32
+ * [hp*wp, C] -> out bf16, zeros on the border. raw (optional) receives x itself as bf16.
+ * scratch: flux_hip_group_norm_scratch_floats(hp, wp) floats. C is 128, 256 or 512.
+ * Replaces flux_group_norm (flux_kernels.c:511-553) + flux_silu (flux_kernels.c:581).
+ */
+int flux_hip_group_norm(void *out_bf16, void *raw_bf16, const float *x, const float *gamma, const float *beta,
+                        float *scratch, int hp, int wp, int C, float eps, int swish);
+size_t flux_hip_group_norm_scratch_floats(int hp, int wp);
+/* nearest-neighbour 2x: x f32 [hp*wp, C] -> out bf16 [(2H+2)*(2W+2), C] (flux_upsample_nearest, flux_kernels.c:1017) */
+int flux_hip_upsample2x(void *out_bf16, const float *x, int hp, int wp, int C);
+/* P bf16 [rows, ld] = softmax over each row of (S * scale + key_bias), S f32 [rows, ld], key_bias f32 [ld]
+ * (0 or -inf); flux_softmax, flux_kernels.c:596, with the scale of flux_vae.c:247 */
+int flux_hip_softmax_rows(void *p_bf16, const float *s, const float *key_bias, int rows, int ld, float scale);
+/* vt bf16 [cols, ld] = v^T for v bf16 [rows, ldv] (first `cols` columns), zero-filled for columns rows..ld-1 */
+int flux_hip_transpose_bf16(void *vt, int ld, const void *v, int ldv, int rows, int cols);
+
+typedef struct flux_hip_vae flux_hip_vae;
+/* Decoder weights from a VAE .safetensors file (tensor names as flux_vae_load_safetensors reads
+ * them, flux_vae.c:1232-1330; encoder tensors are skipped), or from the reference's parsed-file
+ * handle (safetensors_file_t *). NULL on failure. */
+flux_hip_vae *flux_hip_vae_load_file(const char *path);
+flux_hip_vae *flux_hip_vae_load_safetensors(void *safetensors_file);
+/* Piecewise construction: new, then one set_tensor per tensor (dtype 0 = f32, 1 = f16, 2 = bf16). */
+flux_hip_vae *flux_hip_vae_new(void);
+int flux_hip_vae_set_tensor(flux_hip_vae *v, const char *name, int dtype, const void *data, int64_t numel);
+void flux_hip_vae_free(flux_hip_vae *v);
+/* latent f32 [128, h, w] (host) -> rgb u8 [16h, 16w, 3] and/or rgb_f32 [3, 16h, 16w] (decoder output
+ * before the conversion to 8 bits); either may be NULL. h, w <= 128. 1 = ok, 0 = failed. */
+int flux_hip_vae_decode(flux_hip_vae *v, const float *latent, int h, int w, uint8_t *rgb, float *rgb_f32);
 
 /*
  * The sampling loop in pieces, for callers that drive or time the steps themselves. begin()

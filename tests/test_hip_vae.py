@@ -1,0 +1,263 @@
+"""GPU parity tests of the VAE decoder: its operators through the C ABI against the CPU oracle
+(oracle/vae_oracle.c), and the whole decoder against the oracle and against the images the
+reference's own flux_vae_decode produced (tests/golden/vae.npz).
+
+Tolerances. Operators take bf16 inputs (the same rounded values go to the oracle) and accumulate in
+fp32: 2e-6 relative for fp32 outputs, 4e-3 for bf16 outputs (one rounding, 2^-9 per element).
+The decoder keeps its residual stream in fp32 and rounds what feeds each convolution to bf16
+(about 30 layers): the unquantised image must agree with the fp32 oracle to 2e-2 relative L2,
+the 8-bit image to a mean absolute difference of 1.5 levels (the reference's own end-to-end threshold
+is 20, run_test.py:96-104).
+"""
+import os
+
+import numpy as np
+import pytest
+
+from metrics import rel_l2
+from model_spec import normal_f32, f32_to_bf16, bf16_to_f32, make_vae_weights
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+    import fluxhip
+    fluxhip.init()
+    yield fluxhip
+    fluxhip.lib().flux_hip_linear_force_tile(-1)
+
+
+def q(x):
+    return bf16_to_f32(f32_to_bf16(x))
+
+
+def to_padded(x):
+    """[C, H, W] -> [(H+2)*(W+2), C] with a zero border."""
+    C, H, W = x.shape
+    p = np.zeros((H + 2, W + 2, C), np.float32)
+    p[1:-1, 1:-1] = x.transpose(1, 2, 0)
+    return p.reshape(-1, C)
+
+
+def from_padded(p, H, W):
+    C = p.shape[1]
+    return p.reshape(H + 2, W + 2, C)[1:-1, 1:-1].transpose(2, 0, 1)
+
+
+def border_is_zero(p, H, W):
+    g = p.reshape(H + 2, W + 2, -1)
+    return not (g[0].any() or g[-1].any() or g[:, 0].any() or g[:, -1].any())
+
+
+class Guarded:
+    """bf16 image on the device with the slack rows flux_hip_conv may read around it."""
+
+    def __init__(self, hip, padded, wp):
+        rows, C = padded.shape
+        g = wp + 2
+        buf = np.full((rows + 2 * g, C), 7.0, np.float32)      # non-zero slack: it must not reach kept outputs
+        buf[g:g + rows] = padded
+        self.buf = hip.DevBuf.from_array(f32_to_bf16(buf))
+        self.ptr = self.buf.at(g * C * 2)
+
+
+def conv_weight(w):
+    """[cout, cin, k, k] -> bf16 [cout, k*k*cin], tap-major."""
+    co, ci, k, _ = w.shape
+    return f32_to_bf16(np.ascontiguousarray(w.transpose(0, 2, 3, 1)).reshape(co, k * k * ci))
+
+
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3])
+@pytest.mark.parametrize("shape", [(9, 7, 64, 256), (5, 12, 128, 256), (20, 17, 256, 256)])
+def test_conv3x3(hip, oracle_mod, tile, shape):
+    H, W, cin, cout = shape
+    hip.lib().flux_hip_linear_force_tile(tile)
+    x = q(normal_f32((cin, H, W), 51, 1))
+    w = q(normal_f32((cout, cin, 3, 3), 51, 2, 0.0, 0.05))
+    b = normal_f32((cout,), 51, 3)
+    res = normal_f32((cout, H, W), 51, 4)
+    want = oracle_mod.conv2d(x, w, b, 1)
+    rows, wp = (H + 2) * (W + 2), W + 2
+    din = Guarded(hip, to_padded(x), wp)
+    dw, db = hip.DevBuf.from_array(conv_weight(w)), hip.DevBuf.from_array(b)
+    # fp32 output, no residual
+    out = hip.DevBuf.from_array(np.full((rows, cout), 3.0, np.float32))
+    hip.check(hip.lib().flux_hip_conv(hip.EPI_CONV_F32, din.ptr, dw.ptr, db.ptr, None, out.ptr, rows, wp, cin, cout, 9))
+    got = out.to_array(np.float32, (rows, cout))
+    assert border_is_zero(got, H, W)
+    assert rel_l2(from_padded(got, H, W), want) < 2e-6
+    # residual added in place
+    dres = hip.DevBuf.from_array(to_padded(res))
+    hip.check(hip.lib().flux_hip_conv(hip.EPI_CONV_F32, din.ptr, dw.ptr, db.ptr, dres.ptr, dres.ptr, rows, wp, cin, cout, 9))
+    got = dres.to_array(np.float32, (rows, cout))
+    assert border_is_zero(got, H, W)
+    assert rel_l2(from_padded(got, H, W), want + res) < 2e-6
+    # bf16 output
+    outb = hip.DevBuf.from_array(np.full((rows, cout), 0x4040, np.uint16))
+    hip.check(hip.lib().flux_hip_conv(hip.EPI_CONV_BF16, din.ptr, dw.ptr, db.ptr, None, outb.ptr, rows, wp, cin, cout, 9))
+    got = bf16_to_f32(outb.to_array(np.uint16, (rows, cout)))
+    assert border_is_zero(got, H, W)
+    assert rel_l2(from_padded(got, H, W), want) < 4e-3
+    hip.lib().flux_hip_linear_force_tile(-1)
+
+
+def test_conv_output_widths(hip, oracle_mod):
+    """64 output channels (the padded conv_out) and 512 (mid block), automatic tile."""
+    for cin, cout, H, W in ((128, 64, 11, 6), (512, 512, 6, 6)):
+        x = q(normal_f32((cin, H, W), 52, 1))
+        w = q(normal_f32((cout, cin, 3, 3), 52, 2, 0.0, 0.03))
+        b = normal_f32((cout,), 52, 3)
+        rows, wp = (H + 2) * (W + 2), W + 2
+        din = Guarded(hip, to_padded(x), wp)
+        dw, db = hip.DevBuf.from_array(conv_weight(w)), hip.DevBuf.from_array(b)
+        out = hip.DevBuf(rows * cout * 4)
+        hip.check(hip.lib().flux_hip_conv(hip.EPI_CONV_F32, din.ptr, dw.ptr, db.ptr, None, out.ptr, rows, wp, cin, cout, 9))
+        got = out.to_array(np.float32, (rows, cout))
+        assert border_is_zero(got, H, W)
+        assert rel_l2(from_padded(got, H, W), oracle_mod.conv2d(x, w, b, 1)) < 2e-6
+
+
+def test_conv1x1(hip, oracle_mod):
+    H, W, cin, cout = 7, 9, 512, 256
+    x = q(normal_f32((cin, H, W), 53, 1))
+    w = q(normal_f32((cout, cin, 1, 1), 53, 2, 0.0, 0.05))
+    b = normal_f32((cout,), 53, 3)
+    want = oracle_mod.conv2d(x, w, b, 0)
+    rows, wp = (H + 2) * (W + 2), W + 2
+    din = hip.DevBuf.from_array(f32_to_bf16(to_padded(x)))
+    dw, db = hip.DevBuf.from_array(conv_weight(w)), hip.DevBuf.from_array(b)
+    out = hip.DevBuf(rows * cout * 4)
+    hip.check(hip.lib().flux_hip_conv(hip.EPI_CONV_F32, din.ptr, dw.ptr, db.ptr, None, out.ptr, rows, wp, cin, cout, 1))
+    got = out.to_array(np.float32, (rows, cout))
+    assert border_is_zero(got, H, W)
+    assert rel_l2(from_padded(got, H, W), want) < 2e-6
+    # wp = 0: every row is a plain row (border rows get the bias)
+    hip.check(hip.lib().flux_hip_conv(hip.EPI_CONV_F32, din.ptr, dw.ptr, db.ptr, None, out.ptr, rows, 0, cin, cout, 1))
+    got = out.to_array(np.float32, (rows, cout))
+    assert rel_l2(from_padded(got, H, W), want) < 2e-6
+    np.testing.assert_allclose(got[0], b, rtol=1e-6)
+
+
+def test_conv_rejects_bad_arguments(hip):
+    L = hip.lib()
+    d = hip.DevBuf(1 << 16)
+    assert L.flux_hip_conv(hip.EPI_CONV_F32, d.ptr, d.ptr, d.ptr, None, d.ptr, 30, 6, 96, 64, 9) == 0     # cin not 64 * 2^k
+    assert L.flux_hip_conv(hip.EPI_CONV_F32, d.ptr, d.ptr, d.ptr, None, d.ptr, 30, 6, 192, 64, 9) == 0
+    assert L.flux_hip_conv(hip.EPI_CONV_F32, d.ptr, d.ptr, d.ptr, None, d.ptr, 31, 6, 64, 64, 9) == 0     # rows not a multiple of wp
+    assert L.flux_hip_conv(hip.EPI_BF16, d.ptr, d.ptr, d.ptr, None, d.ptr, 30, 6, 64, 64, 9) == 0         # not a conv epilogue
+    assert L.flux_hip_conv(hip.EPI_CONV_F32, d.ptr, d.ptr, None, None, d.ptr, 30, 6, 64, 64, 9) == 0      # bias is required
+    assert L.flux_hip_linear(hip.EPI_CONV_F32, 1, None, 128, 64, 64, 64, 128, 0, 0) == 0
+
+
+@pytest.mark.parametrize("C", [128, 256, 512])
+@pytest.mark.parametrize("swish", [0, 1])
+def test_group_norm(hip, oracle_mod, C, swish):
+    H, W = 19, 23                                    # 525 positions: more than one block of the partial-sum pass
+    x = normal_f32((C, H, W), 54, 1, 0.4, 1.7)
+    gm, bt = normal_f32((C,), 54, 2, 1.0, 0.2), normal_f32((C,), 54, 3)
+    want = oracle_mod.group_norm(x, gm, bt, 32, 1e-4)
+    if swish:
+        want = oracle_mod.silu(want)
+    rows = (H + 2) * (W + 2)
+    dx = hip.DevBuf.from_array(to_padded(x))
+    dg, db = hip.DevBuf.from_array(gm), hip.DevBuf.from_array(bt)
+    out, raw = hip.DevBuf(rows * C * 2), hip.DevBuf(rows * C * 2)
+    scratch = hip.DevBuf(hip.lib().flux_hip_group_norm_scratch_floats(H + 2, W + 2) * 4)
+    hip.check(hip.lib().flux_hip_group_norm(out.ptr, raw.ptr, dx.ptr, dg.ptr, db.ptr, scratch.ptr, H + 2, W + 2, C, 1e-4, swish))
+    got = bf16_to_f32(out.to_array(np.uint16, (rows, C)))
+    assert border_is_zero(got, H, W)
+    assert rel_l2(from_padded(got, H, W), want) < 4e-3
+    np.testing.assert_array_equal(raw.to_array(np.uint16, (rows, C)), f32_to_bf16(to_padded(x)))
+
+
+def test_upsample(hip, oracle_mod):
+    C, H, W = 128, 5, 7
+    x = normal_f32((C, H, W), 55, 1)
+    dx = hip.DevBuf.from_array(to_padded(x))
+    rows2 = (2 * H + 2) * (2 * W + 2)
+    out = hip.DevBuf.from_array(np.full((rows2, C), 0x4040, np.uint16))
+    hip.check(hip.lib().flux_hip_upsample2x(out.ptr, dx.ptr, H + 2, W + 2, C))
+    got = bf16_to_f32(out.to_array(np.uint16, (rows2, C)))
+    assert border_is_zero(got, 2 * H, 2 * W)
+    np.testing.assert_array_equal(from_padded(got, 2 * H, 2 * W), q(oracle_mod.upsample_nearest(x)))
+
+
+def test_softmax_rows_and_transpose(hip, oracle_mod):
+    rows, ld, valid = 37, 384, 300
+    s = normal_f32((rows, ld), 56, 1, 0.0, 6.0)
+    kb = np.zeros(ld, np.float32)
+    kb[valid:] = -np.inf
+    kb[5] = -np.inf
+    scale = 0.37
+    keep = np.isfinite(kb)
+    want = np.zeros((rows, ld), np.float32)
+    want[:, keep] = oracle_mod.softmax(s[:, keep] * np.float32(scale))
+    ds, dk = hip.DevBuf.from_array(s), hip.DevBuf.from_array(kb)
+    out = hip.DevBuf(rows * ld * 2)
+    hip.check(hip.lib().flux_hip_softmax_rows(out.ptr, ds.ptr, dk.ptr, rows, ld, scale))
+    got = bf16_to_f32(out.to_array(np.uint16, (rows, ld)))
+    assert not got[:, ~keep].any()
+    assert rel_l2(got, want) < 4e-3
+    assert np.abs(got.sum(axis=1) - 1.0).max() < 4e-3
+    # transpose of a column slice of a wider matrix, zero-filled to ld
+    v = f32_to_bf16(normal_f32((100, 192), 56, 2))
+    dv = hip.DevBuf.from_array(v)
+    vt = hip.DevBuf.from_array(np.full((128, 128), 0x4040, np.uint16))
+    hip.check(hip.lib().flux_hip_transpose_bf16(vt.ptr, 128, dv.at(64 * 2), 192, 100, 128))
+    got = vt.to_array(np.uint16, (128, 128))
+    np.testing.assert_array_equal(got[:, :100], v[:, 64:192].T)
+    assert not got[:, 100:].any()
+
+
+@pytest.fixture(scope="module")
+def vae_pair(hip, oracle_mod):
+    W = make_vae_weights()
+    dev = hip.Vae(W)
+    cpu = oracle_mod.VaeOracle(W)
+    yield dev, cpu
+    dev.close()
+    cpu.close()
+
+
+@pytest.mark.parametrize("case", [(2, 2, 301), (3, 2, 302), (4, 5, 303)])
+def test_vae_decode(vae_pair, golden_dir, case):
+    dev, cpu = vae_pair
+    h, w, seed = case
+    lat = normal_f32((128, h, w), seed, 1)
+    f, u = dev.decode(lat, h, w)
+    fo, uo = cpu.decode(lat, h, w)
+    r = rel_l2(f, fo)
+    diff = np.abs(u.astype(np.int32) - uo.astype(np.int32))
+    print(f"vae decode {h}x{w}: rel_l2={r:.3e} mean|d|={diff.mean():.3f} max|d|={diff.max()} std={uo.std():.1f}", flush=True)
+    assert uo.std() > 20.0
+    assert r <= 2e-2
+    assert diff.mean() <= 1.5
+    gold = np.load(os.path.join(golden_dir, "vae.npz"))
+    key = f"decode_{h}x{w}"
+    if key in gold:                      # the reference's own decoder output for this latent
+        dg = np.abs(u.astype(np.int32) - gold[key].astype(np.int32))
+        assert dg.mean() <= 1.5
+
+
+def test_vae_decode_smaller_after_larger(vae_pair):
+    """Work buffers sized for a larger image serve a smaller one; the result does not depend on what ran before."""
+    dev, cpu = vae_pair
+    lat = normal_f32((128, 2, 3), 304, 1)
+    f1, u1 = dev.decode(lat, 2, 3)
+    dev.decode(normal_f32((128, 5, 4), 305, 1), 5, 4)
+    f2, u2 = dev.decode(lat, 2, 3)
+    np.testing.assert_array_equal(f1, f2)
+    np.testing.assert_array_equal(u1, u2)
+    assert rel_l2(f1, cpu.decode(lat, 2, 3)[0]) <= 2e-2
+
+
+def test_vae_missing_tensor_fails(hip):
+    W = make_vae_weights()
+    del W["decoder.mid_block.attentions.0.to_k.bias"]
+    v = hip.Vae(W)
+    out = np.empty((32, 32, 3), np.uint8)
+    lat = np.zeros((128, 2, 2), np.float32)
+    assert hip.lib().flux_hip_vae_decode(v.h, lat.ctypes.data, 2, 2, out.ctypes.data, None) == 0
+    assert b"to_k.bias" in hip.lib().flux_hip_last_error()
+    v.close()
