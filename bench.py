@@ -14,6 +14,9 @@ Also measured in the same run:
   cpu_baseline  the CPU oracle (fp32, BLAS when available) on a bounded sample of the same
                 workload: one double-stream and two single-stream blocks at full shape,
                 extrapolated to the 5 + 20 blocks of a step
+
+--workload vae_c2 | vae_c3 | vae_c4 measures the step after the sampling loop instead: one "step" is
+one VAE decode of a 16/32/64-wide latent to a 256/512/1024-pixel image.
 """
 import argparse
 import json
@@ -110,12 +113,87 @@ def cpu_baseline(cfg, n_img, n_txt):
     }
 
 
+VAE_WORKLOADS = {"vae_c2": 16, "vae_c3": 32, "vae_c4": 64}   # latent side: 256^2, 512^2, 1024^2 images
+
+
+def vae_cpu_baseline(flops_decode):
+    """The CPU oracle's decoder (OpenMP loops) on a 128x128 image; its FLOP rate carried to the
+    benchmarked size."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import oracle as O
+    from model_spec import make_vae_weights, vae_decode_flops
+    o = O.VaeOracle(make_vae_weights())
+    lat = normal_f32((128, 8, 8), 9, 1)
+    o.decode(normal_f32((128, 2, 2), 9, 2), 2, 2)
+    t0 = time.perf_counter()
+    o.decode(lat, 8, 8)
+    dt = time.perf_counter() - t0
+    o.close()
+    rate = vae_decode_flops(8, 8) / dt
+    return {"value": rate / flops_decode, "unit": "decodes/s", "cores": O.lib().fo_num_threads(), "kind": "port",
+            "sample": f"one 128x128 decode ({dt:.1f} s, {rate / 1e9:.1f} GFLOP/s, OpenMP loops of the CPU oracle), "
+                      f"carried to this size by FLOP count"}
+
+
+def bench_vae(args):
+    """One step = one decode of a latent to an 8-bit image through flux_hip_vae_decode (host latent in,
+    host image out: 0.5 + 3 MB over PCIe at 1024^2, inside the timed region)."""
+    import ctypes
+    from model_spec import make_vae_weights, vae_decode_convs, vae_decode_flops
+    side = VAE_WORKLOADS[args.workload]
+    K, Wm = args.steps, args.warmup
+    fluxhip.init()
+    if args.tile_mask:
+        fluxhip.lib().flux_hip_linear_tile_mask(args.tile_mask)
+    v = fluxhip.Vae(make_vae_weights())
+    lat = normal_f32((128, side, side), 321, 1)
+    for _ in range(max(Wm, 1)):
+        f, u = v.decode(lat, side, side)
+    assert np.isfinite(f).all() and u.std() > 5.0
+    L = fluxhip.lib()
+    if not args.no_kernel_timing:
+        L.flux_hip_linear_probe(fluxhip.EPI_CONV_F32)
+    t0 = time.perf_counter()
+    for _ in range(K):
+        v.decode(lat, side, side)
+    wall = time.perf_counter() - t0
+    flops = vae_decode_flops(side, side)
+    roof = None
+    if not args.no_kernel_timing:
+        # dominant kernel: the 4-wave 256x256-tile GEMM with the convolution epilogue, which runs every
+        # convolution of 256 or more output channels; its launches differ in shape, so the figure is
+        # (sum of their algorithmic FLOPs) / (sum of their durations)
+        n_t, ms_t = ctypes.c_int(0), ctypes.c_float(0.0)
+        L.flux_hip_linear_probe_read_tile(2, ctypes.byref(n_t), ctypes.byref(ms_t))
+        L.flux_hip_linear_probe(-1)
+        big = [c for c in vae_decode_convs(side, side)
+               if c[4] >= 256 and c[0] not in ("mid.attn.to_q", "mid.attn.to_k", "mid.attn.to_v")]
+        if n_t.value == K * len(big):
+            k_flops = sum(2.0 * H * W * ci * co * t for _, H, W, ci, co, t in big)
+            per_ms = ms_t.value / n_t.value
+            ach = k_flops * K / (ms_t.value * 1e-3) / 1e12
+            roof = {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                    "kernel": "gemm4w_kernel<8,8,CONV_F32> (256x256 tile): 3x3 and 1x1 convolutions with 256 or 512 output channels",
+                    "launches_timed": n_t.value, "ms_per_launch": round(per_ms, 4),
+                    "flops_per_launch": k_flops / len(big), "launches_per_decode": len(big)}
+    v.close()
+    cpu = None if args.no_cpu_baseline else vae_cpu_baseline(flops)
+    print(json.dumps({
+        "metric": f"VAE decodes/s ({16 * side}x{16 * side} image, 1 GPU)", "value": round(K / wall, 3), "unit": "decodes/s",
+        "n_gpus": 1, "steps": K, "warmup": Wm, "ms_per_step": round(wall * 1000.0 / K, 3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: FLUX.2 VAE decoder (84 M parameters, random-init bf16), latent "
+                               f"[128,{side},{side}] -> {16 * side}x{16 * side} RGB, batch 1, host buffers in and out"},
+        "tflops": round(flops * K / wall / 1e12, 1), "flops_per_step": flops, "roofline": roof, "cpu_baseline": cpu}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=8)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + sorted(VAE_WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     ap.add_argument("--tile-mask", type=lambda v: int(v, 0), default=0,
@@ -129,6 +207,8 @@ def main():
               "run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    if args.workload in VAE_WORKLOADS:
+        return bench_vae(args)
     cfg = KLEIN_4B
     wl = WORKLOADS[args.workload]
     if args.calibrate:

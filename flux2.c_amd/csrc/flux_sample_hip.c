@@ -321,22 +321,23 @@ int flux_hip_session_read_latent(flux_hip_session *s, float *z_out) {
 /* Intermediate-image hook of the reference (flux_sample.c:258-266): when the application has set
  * flux_step_image_callback and flux_step_image_vae (flux.c:161-164), every step but the last
  * hands the current latent to the application's own VAE decoder and the image to the callback.
- * All four symbols belong to the application (flux_kernels.c:35-36, flux_vae.c, flux_image.c);
- * they are weak here, and without them the hook does nothing. Each use waits for the device. */
+ * The two globals and flux_image_free belong to the application (flux_kernels.c:35-36,
+ * flux_image.c); they are weak here, and without them the hook does nothing. flux_vae_decode is
+ * the application's own when it links one, else the device decoder's entry point of that name.
+ * Each use waits for the device. */
 struct flux_image;
 typedef void (*fh_step_image_cb)(int step, int total, const struct flux_image *img);
 extern fh_step_image_cb flux_step_image_callback __attribute__((weak));
 extern void *flux_step_image_vae __attribute__((weak));
-extern struct flux_image *flux_vae_decode(void *vae, const float *latent, int batch, int latent_h, int latent_w) __attribute__((weak));
 extern void flux_image_free(struct flux_image *img) __attribute__((weak));
 
 static void step_image_hook(flux_hip_session *s, int step) {
-    if (!&flux_step_image_callback || !&flux_step_image_vae || !flux_vae_decode || !flux_image_free) return;
+    if (!&flux_step_image_callback || !&flux_step_image_vae || !flux_image_free) return;
     if (!flux_step_image_callback || !flux_step_image_vae || step + 1 >= s->num_steps) return;
     float *z = (float *)malloc(s->n_lat * 4);
     if (!z) return;
     if (flux_hip_download(z, s->z_dev, s->n_lat * 4)) {
-        struct flux_image *img = flux_vae_decode(flux_step_image_vae, z, 1, s->h, s->w);
+        struct flux_image *img = (struct flux_image *)flux_vae_decode(flux_step_image_vae, z, 1, s->h, s->w);
         if (img) {
             flux_step_image_callback(step + 1, s->num_steps, img);
             flux_image_free(img);

@@ -321,6 +321,10 @@ static int ensure_work(flux_hip_vae *v, int h, int w) {
     return 1;
 }
 
+/* Called (when set) after each of the 15 blocks has been queued: 3 mid + 12 up, the reference's
+ * count (flux_vae.c:757-758). */
+void (*flux_hip_vae_progress)(int block, int total) = NULL;
+
 typedef struct {
     flux_hip_vae *v;
     float *x, *y; /* residual stream and the spare fp32 image */
@@ -380,11 +384,20 @@ int flux_hip_vae_decode(flux_hip_vae *v, const float *latent, int h, int w, uint
     if (!flux_hip_upload(v->lat, latent, (size_t)128 * h * w * 4)) return 0;
     if (!flux_hip_vae_latent_in(s.A, v->lat, v->bn_mean, v->bn_var, v->pq_w, v->pq_b, h, w, v->eps)) return 0;
     if (!run_conv(&s, &v->conv_in, FLUX_HIP_EPI_CONV_F32, s.A, NULL, s.x, 1)) return 0;
-    if (!run_res(&s, &v->mid[0]) || !run_attn(&s) || !run_res(&s, &v->mid[1])) return 0;
+    int done = 0;
+    const int total = 15;
+    if (!run_res(&s, &v->mid[0])) return 0;
+    if (flux_hip_vae_progress) flux_hip_vae_progress(done++, total);
+    if (!run_attn(&s)) return 0;
+    if (flux_hip_vae_progress) flux_hip_vae_progress(done++, total);
+    if (!run_res(&s, &v->mid[1])) return 0;
+    if (flux_hip_vae_progress) flux_hip_vae_progress(done++, total);
     int bi = 0;
     for (int level = 3; level >= 0; level--) {
-        for (int r = 0; r < 3; r++)
+        for (int r = 0; r < 3; r++) {
             if (!run_res(&s, &v->up[bi++])) return 0;
+            if (flux_hip_vae_progress) flux_hip_vae_progress(done++, total);
+        }
         if (level > 0) {
             const vconv *c = &v->up_conv[3 - level];
             if (!flux_hip_upsample2x(s.A, s.x, s.hp, s.wp, c->cin)) return 0;

@@ -240,6 +240,44 @@ def make_vae_weights(seed=77):
     return out
 
 
+def vae_decode_convs(h, w):
+    """The decoder's convolutions for an h x w latent, in execution order (flux_vae_decode,
+    flux_vae.c:690-837): (name, H, W, cin, cout, taps)."""
+    mult = [1, 2, 4, 4]
+    H, W = 2 * h, 2 * w
+    out = [("post_quant_conv", H, W, 32, 32, 1), ("conv_in", H, W, 32, 512, 9)]
+
+    def res(name, i, o):
+        out.append((name + ".conv1", H, W, i, o, 9))
+        out.append((name + ".conv2", H, W, o, o, 9))
+        if i != o:
+            out.append((name + ".conv_shortcut", H, W, i, o, 1))
+
+    res("mid.0", 512, 512)
+    for n in ("to_q", "to_k", "to_v", "to_out"):
+        out.append(("mid.attn." + n, H, W, 512, 512, 1))
+    res("mid.1", 512, 512)
+    prev = 512
+    for up in range(4):
+        ch = 128 * mult[3 - up]
+        for r in range(3):
+            res(f"up.{up}.{r}", prev if r == 0 else ch, ch)
+        if up < 3:
+            H, W = 2 * H, 2 * W
+            out.append((f"up.{up}.upsample", H, W, ch, ch, 9))
+        prev = ch
+    out.append(("conv_out", H, W, 128, 3, 9))
+    return out
+
+
+def vae_decode_flops(h, w):
+    """Algorithmic FLOPs of one decode (1 MAC = 2 FLOP): convolutions over the real image and channel
+    counts, plus the mid-block attention's two products over (2h * 2w) positions at width 512."""
+    conv = sum(2.0 * H * W * ci * co * t for _, H, W, ci, co, t in vae_decode_convs(h, w))
+    n = 4.0 * h * w
+    return conv + 4.0 * n * n * 512
+
+
 def flops_per_forward(cfg: FluxConfig, n_img, n_txt, n_img_out=None):
     """Algorithmic FLOPs of one forward (1 MAC = 2 FLOP)."""
     H, C, T = cfg.hidden, cfg.channels, cfg.text_dim

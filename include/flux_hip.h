@@ -333,6 +333,16 @@ void flux_hip_vae_free(flux_hip_vae *v);
 /* latent f32 [128, h, w] (host) -> rgb u8 [16h, 16w, 3] and/or rgb_f32 [3, 16h, 16w] (decoder output
  * before the conversion to 8 bits); either may be NULL. h, w <= 128. 1 = ok, 0 = failed. */
 int flux_hip_vae_decode(flux_hip_vae *v, const float *latent, int h, int w, uint8_t *rgb, float *rgb_f32);
+/* When set, called after each of the decoder's 15 blocks has been queued (role of
+ * flux_vae_progress_callback, flux_kernels.h:292-293). */
+extern void (*flux_hip_vae_progress)(int block, int total);
+
+/* The reference's own VAE entry points (flux.c:36-43) over the device decoder; see
+ * flux_vae_dropin.c for how an application keeps its CPU encoder beside them. The handles are
+ * flux_vae_t * / flux_image * / safetensors_file_t * in the reference's headers. */
+void *flux_vae_load_safetensors(void *safetensors_file);
+void *flux_vae_decode(void *vae, const float *latent, int batch, int latent_h, int latent_w);
+void flux_vae_free(void *vae);
 
 /*
  * The sampling loop in pieces, for callers that drive or time the steps themselves. begin()

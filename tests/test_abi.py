@@ -120,3 +120,12 @@ def test_reference_cli_links_against_the_library():
         assert re.search(rf"\bU {name}\b", syms), name
     for name in ("flux_load_dir", "flux_generate_with_embeddings", "flux_denoise_step"):
         assert re.search(rf"\bT {name}\b", syms), name
+    # the same with the VAE decoder taken from the backend: flux.c's three decoder-side calls are imports,
+    # the reference's CPU decoder and encoder are still there under the renamed/original names
+    r = subprocess.run(["make", "-C", os.path.join(ROOT, "oracle"), "pipeline_gpuvae"], capture_output=True, text=True)
+    assert r.returncode == 0 and "linked _ref/libfluxpipe_gpuvae.so" in r.stdout, r.stdout + r.stderr
+    syms = subprocess.run(["nm", "-D", os.path.join(ROOT, "oracle", "_ref", "libfluxpipe_gpuvae.so")], capture_output=True, text=True).stdout
+    for name in ("flux_vae_decode", "flux_vae_load_safetensors", "flux_vae_free", "flux_sample_euler"):
+        assert re.search(rf"\bU {name}\b", syms), name
+    for name in ("flux_vae_decode_cpu", "flux_vae_encode", "flux_generate_with_embeddings"):
+        assert re.search(rf"\bT {name}\b", syms), name

@@ -118,3 +118,85 @@ def test_reference_pipeline_runs_on_the_backend(oracle_mod, tmp_path):
     assert r <= 2e-2 and c >= 0.999
     o.close()
     P.flux_free(ctx)
+
+
+PIPE_GPUVAE = os.path.join(ROOT, "oracle", "_ref", "libfluxpipe_gpuvae.so")
+
+# Runs in a fresh process so that the pipeline library is the first thing loaded: the backend's
+# weak references to the application's CPU VAE (flux_vae_load_safetensors_cpu, ...) bind when
+# libflux_hip.so is loaded, as they would in an executable linked against both.
+_CHILD = r"""
+import ctypes, sys, os
+import numpy as np
+lib, model_dir, out, root = sys.argv[1:5]
+sys.path.insert(0, os.path.join(root, "flux2.c_amd"))
+from model_spec import normal_f32
+vp, c_i, c_f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+class FluxParams(ctypes.Structure):
+    _fields_ = [("width", c_i), ("height", c_i), ("num_steps", c_i), ("seed", ctypes.c_int64), ("guidance", c_f),
+                ("linear_schedule", c_i), ("power_schedule", c_i), ("power_alpha", c_f)]
+class FluxImage(ctypes.Structure):
+    _fields_ = [("width", c_i), ("height", c_i), ("channels", c_i), ("data", ctypes.POINTER(ctypes.c_uint8))]
+P = ctypes.CDLL(lib, mode=ctypes.RTLD_GLOBAL)
+P.flux_load_dir.restype = vp
+P.flux_load_dir.argtypes = [ctypes.c_char_p]
+P.flux_get_error.restype = ctypes.c_char_p
+P.flux_generate_with_embeddings.restype = vp
+P.flux_generate_with_embeddings.argtypes = [vp, vp, c_i, ctypes.POINTER(FluxParams)]
+P.flux_image_free.argtypes = [vp]
+P.flux_free.argtypes = [vp]
+progress = []
+CB = ctypes.CFUNCTYPE(None, c_i, c_i)
+cb = CB(lambda b, t: progress.append((b, t)))
+ctypes.c_void_p.in_dll(P, "flux_vae_progress_callback").value = ctypes.cast(cb, vp).value
+ctx = P.flux_load_dir(model_dir.encode())
+assert ctx, P.flux_get_error()
+width, height, steps, seed, seq, text_dim = [int(a) for a in sys.argv[5:11]]
+emb = normal_f32((seq, text_dim), 40, 1)
+prm = FluxParams(width, height, steps, seed, 0.0, 0, 0, 2.0)
+img_p = P.flux_generate_with_embeddings(ctx, emb.ctypes.data, seq, ctypes.byref(prm))
+assert img_p, P.flux_get_error()
+im = ctypes.cast(img_p, ctypes.POINTER(FluxImage)).contents
+np.save(out, np.ctypeslib.as_array(im.data, shape=(im.height, im.width, im.channels)).copy())
+P.flux_image_free(img_p)
+P.flux_free(ctx)
+assert progress == [(i, 15) for i in range(15)], progress
+print("child ok")
+"""
+
+
+@pytest.mark.skipif(not os.path.exists(PIPE_GPUVAE), reason="reference-built library not present")
+def test_reference_pipeline_with_the_device_vae(oracle_mod, tmp_path):
+    """flux_generate_with_embeddings through the reference's flux.c with both the transformer and the
+    VAE decoder on the device (flux_vae_dropin.c); expected image: CPU oracle sampler + CPU oracle decoder."""
+    import subprocess
+    import sys
+    cfg = SMALL
+    W = make_weights(cfg, 42, 0.05, "sharp")
+    VW = make_vae_weights()
+    os.makedirs(tmp_path / "transformer")
+    os.makedirs(tmp_path / "vae")
+    write_safetensors(str(tmp_path / "transformer" / "diffusion_pytorch_model.safetensors"), W)
+    write_safetensors(str(tmp_path / "vae" / "diffusion_pytorch_model.safetensors"), VW)
+    width, height, steps, seed, seq = 96, 64, 3, 12, 24
+    out = str(tmp_path / "img.npy")
+    r = subprocess.run([sys.executable, "-c", _CHILD, PIPE_GPUVAE, str(tmp_path), out, ROOT,
+                        str(width), str(height), str(steps), str(seed), str(seq), str(cfg.text_dim)],
+                       capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout + r.stderr
+    got = np.load(out)
+    lh, lw = height // 16, width // 16
+    assert got.shape == (height, width, 3)
+    o = oracle_mod.Oracle(cfg, W)
+    emb = normal_f32((seq, cfg.text_dim), 40, 1)
+    z0 = oracle_mod.init_noise(cfg.channels, lh, lw, seed)
+    latent = o.sample_euler(z0, lh, lw, emb, oracle_mod.official_schedule(steps, lh * lw))
+    o.close()
+    vo = oracle_mod.VaeOracle(VW)
+    _, want = vo.decode(latent, lh, lw)
+    vo.close()
+    diff = np.abs(got.astype(np.int32) - want.astype(np.int32))
+    print(f"pipeline image, device VAE: mean abs diff {diff.mean():.3f}, max {diff.max()}, image std {want.std():.1f}", flush=True)
+    assert want.std() > 5.0
+    assert diff.mean() <= 20.0                   # the reference's own acceptance threshold
+    assert diff.mean() <= 1.5 and diff.max() <= 12
