@@ -152,7 +152,7 @@ def bench_vae(args):
     assert np.isfinite(f).all() and u.std() > 5.0
     L = fluxhip.lib()
     if not args.no_kernel_timing:
-        L.flux_hip_linear_probe(fluxhip.EPI_CONV_F32)
+        L.flux_hip_linear_probe(-2)          # events around every convolution launch
     t0 = time.perf_counter()
     for _ in range(K):
         v.decode(lat, side, side)
@@ -160,23 +160,30 @@ def bench_vae(args):
     flops = vae_decode_flops(side, side)
     roof = None
     if not args.no_kernel_timing:
-        # dominant kernel: the 4-wave 256x256-tile GEMM with the convolution epilogue, which runs every
-        # convolution of 256 or more output channels; its launches differ in shape, so the figure is
-        # (sum of their algorithmic FLOPs) / (sum of their durations)
-        n_t, ms_t = ctypes.c_int(0), ctypes.c_float(0.0)
-        L.flux_hip_linear_probe_read_tile(2, ctypes.byref(n_t), ctypes.byref(ms_t))
+        # launch i of a decode is convolution i of vae_decode_convs (after the post-quant one, which the
+        # input kernel does); a kernel (= tile shape) runs layers of several shapes, so its figure is
+        # (sum of its launches' algorithmic FLOPs) / (sum of their durations). Dominant = most time.
+        convs = vae_decode_convs(side, side)[1:]
+        cap = K * len(convs)
+        tiles = np.zeros(cap, np.int32)
+        ms = np.zeros(cap, np.float32)
+        n = L.flux_hip_linear_probe_read_launches(cap, tiles.ctypes.data, ms.ctypes.data)
         L.flux_hip_linear_probe(-1)
-        big = [c for c in vae_decode_convs(side, side)
-               if c[4] >= 256 and c[0] not in ("mid.attn.to_q", "mid.attn.to_k", "mid.attn.to_v")]
-        if n_t.value == K * len(big):
-            k_flops = sum(2.0 * H * W * ci * co * t for _, H, W, ci, co, t in big)
-            per_ms = ms_t.value / n_t.value
-            ach = k_flops * K / (ms_t.value * 1e-3) / 1e12
+        if n == cap:
+            fl = np.array([2.0 * H * W * ci * co * t for _, H, W, ci, co, t in convs] * K)
+            names = {0: "gemm_kernel<64,128,2,2,CONV>", 1: "gemm_kernel<128,128,2,2,CONV>", 2: "gemm4w_kernel<8,8,CONV> (256x256 tile)",
+                     3: "gemm_kernel<64,64,2,2,CONV>"}
+            per_tile = {int(t): (float(ms[tiles == t].sum()), float(fl[tiles == t].sum()), int((tiles == t).sum())) for t in np.unique(tiles)}
+            dom = max(per_tile, key=lambda t: per_tile[t][0])
+            t_ms, t_fl, t_n = per_tile[dom]
+            ach = t_fl / (t_ms * 1e-3) / 1e12
             roof = {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
-                    "kernel": "gemm4w_kernel<8,8,CONV_F32> (256x256 tile): 3x3 and 1x1 convolutions with 256 or 512 output channels",
-                    "launches_timed": n_t.value, "ms_per_launch": round(per_ms, 4),
-                    "flops_per_launch": k_flops / len(big), "launches_per_decode": len(big)}
+                    "kernel": names.get(dom, f"tile {dom}") + ": 3x3 / 1x1 convolutions as GEMMs with bias, residual and border epilogue",
+                    "launches_timed": t_n, "ms_per_launch": round(t_ms / t_n, 4), "flops_per_launch": t_fl / t_n,
+                    "launches_per_decode": t_n // K,
+                    "all_conv_kernels": {names.get(t, str(t)): {"launches_per_decode": c // K, "ms_per_decode": round(m / K, 3),
+                                                                "tflops": round(f / (m * 1e-3) / 1e12, 1)} for t, (m, f, c) in per_tile.items()}}
     v.close()
     cpu = None if args.no_cpu_baseline else vae_cpu_baseline(flops)
     print(json.dumps({

@@ -340,9 +340,9 @@ static int run_conv(vstate *s, const vconv *c, int epi, const void *in, const fl
 static int run_res(vstate *s, const vres *r) {
     flux_hip_vae *v = s->v;
     const int differ = r->cin != r->cout;
-    if (!flux_hip_group_norm(s->A, differ ? v->R : NULL, s->x, r->n1g, r->n1b, v->gn, s->hp, s->wp, r->cin, v->eps, 1)) return 0;
-    if (!run_conv(s, &r->c1, FLUX_HIP_EPI_CONV_F32, s->A, NULL, v->Hb, 1)) return 0;
-    if (!flux_hip_group_norm(s->A, NULL, v->Hb, r->n2g, r->n2b, v->gn, s->hp, s->wp, r->cout, v->eps, 1)) return 0;
+    if (!flux_hip_group_norm(s->A, differ ? v->R : NULL, s->x, 0, r->n1g, r->n1b, v->gn, s->hp, s->wp, r->cin, v->eps, 1)) return 0;
+    if (!run_conv(s, &r->c1, FLUX_HIP_EPI_CONV_BF16, s->A, NULL, v->Hb, 1)) return 0; /* only the next norm reads it */
+    if (!flux_hip_group_norm(s->A, NULL, v->Hb, 1, r->n2g, r->n2b, v->gn, s->hp, s->wp, r->cout, v->eps, 1)) return 0;
     if (differ) {
         if (!run_conv(s, &r->skip, FLUX_HIP_EPI_CONV_F32, v->R, NULL, s->y, 1)) return 0;
         if (!run_conv(s, &r->c2, FLUX_HIP_EPI_CONV_F32, s->A, s->y, s->y, 1)) return 0;
@@ -356,7 +356,7 @@ static int run_res(vstate *s, const vres *r) {
 static int run_attn(vstate *s) {
     flux_hip_vae *v = s->v;
     const int C = 512, rows = s->hp * s->wp, ld = (rows + 127) & ~127;
-    if (!flux_hip_group_norm(s->A, NULL, s->x, v->attn_g, v->attn_b, v->gn, s->hp, s->wp, C, v->eps, 0)) return 0;
+    if (!flux_hip_group_norm(s->A, NULL, s->x, 0, v->attn_g, v->attn_b, v->gn, s->hp, s->wp, C, v->eps, 0)) return 0;
     /* key rows between the image and the padded width are read by the score GEMM: zero them */
     if (ld > rows && !flux_hip_memset((char *)v->R + (size_t)rows * 3 * C * 2, 0, (size_t)(ld - rows) * 3 * C * 2)) return 0;
     if (!run_conv(s, &v->qkv, FLUX_HIP_EPI_CONV_BF16, s->A, NULL, v->R, 0)) return 0;
@@ -378,7 +378,8 @@ static int run_attn(vstate *s) {
  * output [3, 16h, 16w], both optional, on the host. */
 int flux_hip_vae_decode(flux_hip_vae *v, const float *latent, int h, int w, uint8_t *rgb, float *rgb_f32) {
     if (!v || !latent) return flux_hip_fail("flux_hip_vae_decode: NULL argument");
-    if (h <= 0 || w <= 0 || h > 128 || w > 128) return flux_hip_fail("flux_hip_vae_decode: latent %d x %d out of range (1..128)", h, w);
+    if (h <= 0 || w <= 0 || h > 112 || w > 112) /* the reference's limit: 1792 pixels, flux.h:52 */
+        return flux_hip_fail("flux_hip_vae_decode: latent %d x %d out of range (1..112)", h, w);
     if (!vae_complete(v) || !ensure_work(v, h, w)) return 0;
     vstate s = {v, v->X, v->Y, (char *)v->A_base + v->guard * 2, 2 * h + 2, 2 * w + 2};
     if (!flux_hip_upload(v->lat, latent, (size_t)128 * h * w * 4)) return 0;
@@ -406,7 +407,7 @@ int flux_hip_vae_decode(flux_hip_vae *v, const float *latent, int h, int w, uint
             if (!run_conv(&s, c, FLUX_HIP_EPI_CONV_F32, s.A, NULL, s.x, 1)) return 0;
         }
     }
-    if (!flux_hip_group_norm(s.A, NULL, s.x, v->out_g, v->out_b, v->gn, s.hp, s.wp, 128, v->eps, 1)) return 0;
+    if (!flux_hip_group_norm(s.A, NULL, s.x, 0, v->out_g, v->out_b, v->gn, s.hp, s.wp, 128, v->eps, 1)) return 0;
     if (!run_conv(&s, &v->conv_out, FLUX_HIP_EPI_CONV_F32, s.A, NULL, v->Hb, 1)) return 0;
     const int H = 16 * h, W = 16 * w;
     if (!flux_hip_vae_image_out(rgb ? v->img_u8 : NULL, rgb_f32 ? v->img_f32 : NULL, v->Hb, v->conv_out.cout_pad, H, W)) return 0;

@@ -299,15 +299,17 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
  * Idle cycles for the hazards are placed explicitly next to it. */
 template <int TM, int TN>
 __device__ __forceinline__ void acc_fence(f32x4 (&acc)[TN][TM]) {
-    static_assert(TN == 8 || TN == 6, "one asm statement per accumulator column");
+    static_assert(TN == 8 || TN == 6 || TN == 4, "one asm statement per accumulator column");
 #pragma unroll
     for (int j = 0; j < TM; j++) {
         if constexpr (TN == 8)
             asm volatile("" : "+a"(acc[0][j]), "+a"(acc[1][j]), "+a"(acc[2][j]), "+a"(acc[3][j]),
                               "+a"(acc[4][j]), "+a"(acc[5][j]), "+a"(acc[6][j]), "+a"(acc[7][j]));
-        else
+        else if constexpr (TN == 6)
             asm volatile("" : "+a"(acc[0][j]), "+a"(acc[1][j]), "+a"(acc[2][j]), "+a"(acc[3][j]),
                               "+a"(acc[4][j]), "+a"(acc[5][j]));
+        else
+            asm volatile("" : "+a"(acc[0][j]), "+a"(acc[1][j]), "+a"(acc[2][j]), "+a"(acc[3][j]));
     }
 }
 
@@ -610,8 +612,21 @@ extern "C" int flux_hip_linear_probe_read(int *launches, float *total_ms) {
     return flux_hip_linear_probe_read_tile(-1, launches, total_ms);
 }
 
+/* Duration and tile id of each recorded launch, in launch order; returns how many were written. */
+extern "C" int flux_hip_linear_probe_read_launches(int max, int *tiles, float *ms) {
+    int n = 0;
+    for (int i = 0; i < g_probe_n && n < max; i++, n++) {
+        float t = 0.0f;
+        if (hipEventSynchronize(g_probe_ev[i][1]) != hipSuccess || hipEventElapsedTime(&t, g_probe_ev[i][0], g_probe_ev[i][1]) != hipSuccess) return -1;
+        if (tiles) tiles[n] = g_probe_tile[i];
+        if (ms) ms[n] = t;
+    }
+    return n;
+}
+
 static int probe_slot(int epilogue) {
-    if (epilogue != g_probe_epi || g_probe_n >= PROBE_MAX) return -1;
+    const bool conv = epilogue == FLUX_HIP_EPI_CONV_BF16 || epilogue == FLUX_HIP_EPI_CONV_F32;
+    if ((g_probe_epi == -2 ? !conv : epilogue != g_probe_epi) || g_probe_n >= PROBE_MAX) return -1;
     while (g_probe_created <= g_probe_n) {
         if (hipEventCreate(&g_probe_ev[g_probe_created][0]) != hipSuccess) return -1;
         if (hipEventCreate(&g_probe_ev[g_probe_created][1]) != hipSuccess) return -1;
@@ -737,7 +752,7 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
     }
     if (np == 0) return 1;
     g.N = N; g.K = K; g.lda = lda; g.ldw = ldw; g.ldc = ldc; g.w_row0 = w_row0; g.w_row1 = w_row1;
-    return gemm_dispatch(g, np, epilogue, g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask);
+    return gemm_dispatch(g, np, epilogue, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0xFFu);
 }
 
 /* Convolution over a zero-bordered channels-last image as one GEMM, see the header. */
@@ -766,7 +781,17 @@ extern "C" int flux_hip_conv(int epilogue, const void *in, const void *w, const 
     g.conv_taps = taps; g.conv_kshift = kshift; g.conv_wp = wp; g.conv_hp = wp > 0 ? rows / wp : 0;
     g.bias = bias; g.res = res;
     const unsigned conv_tiles = 0x0F; /* 64x128, 128x128, 256x256 (4 waves), 64x64 */
-    unsigned allowed = g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask;
-    if (!(allowed & conv_tiles)) allowed = conv_tiles;
+    static const int width[4] = {128, 128, 256, 64};
+    unsigned allowed;
+    if (g_force_tile >= 0 && g_force_tile < 4 && cout % width[g_force_tile] == 0) {
+        allowed = 1u << g_force_tile; /* a forced tile that this layer cannot use is ignored */
+    } else {
+        /* These layers move many bytes per FLOP (fp32 image in and out of the epilogue), which a
+         * second resident workgroup hides and the one-workgroup-per-CU 256 x 256 tile does not:
+         * measured over the decoder's layers, 128 x 128 wins (3-15 %) until the launch is at least
+         * eight full rounds of 256 x 256 tiles, where the big tile's higher MFMA rate takes over. */
+        const long big_tiles = cout % 256 ? 0 : (long)((rows + 255) / 256) * (cout / 256);
+        allowed = big_tiles >= 2048 ? 1u << 2 : cout % 128 == 0 ? 1u << 1 : 1u << 3;
+    }
     return gemm_dispatch(g, 1, epilogue, allowed & conv_tiles);
 }

@@ -52,16 +52,43 @@ __global__ __launch_bounds__(64) void vae_latent_kernel(bf16 *__restrict__ out, 
  * statistics over the whole image. Three kernels: per-block partial sums, their combination in
  * double precision, and the normalisation itself. Border positions hold zeros and add nothing
  * to the sums; the element count is the interior's. ---- */
-#define GN_ROWS 256 /* positions per workgroup of the partial-sum pass */
+#define GN_ROWS 256 /* positions per workgroup */
 
-__global__ __launch_bounds__(256) void gn_partial_kernel(float *__restrict__ partial, const float *__restrict__ x, int rows, int C) {
+/* p / wp for p < 2^22, wp < 2^12 through a multiplication: magic = ceil(2^40 / wp) */
+__device__ __forceinline__ int div_wp(int p, unsigned long long magic) { return (int)(((unsigned long long)p * magic) >> 40); }
+
+__device__ __forceinline__ f32x4 load_quad(const float *p) { return *(const f32x4 *)p; }
+__device__ __forceinline__ f32x4 load_quad(const bf16 *p) {
+    const bf16x4 v = *(const bf16x4 *)p;
+    f32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; e++) o[e] = (float)v[e];
+    return o;
+}
+
+/* A workgroup covers GN_ROWS positions: thread (r0, q) walks rows r0, r0 + rpi, ... of quad q
+ * (4 adjacent channels, always inside one group), four rows per trip so that four loads are in
+ * flight. */
+template <typename T>
+__global__ __launch_bounds__(256) void gn_partial_kernel(float *__restrict__ partial, const T *__restrict__ x, int rows, int C) {
     __shared__ float sh[256][2];
     const int quads = C >> 2, rpi = 256 / quads; /* C is 128, 256 or 512: 32, 64 or 128 quads */
     const int q = threadIdx.x % quads, r0 = threadIdx.x / quads;
     const int row_begin = blockIdx.x * GN_ROWS, row_end = min(rows, row_begin + GN_ROWS);
     float s = 0.0f, ss = 0.0f;
-    for (int r = row_begin + r0; r < row_end; r += rpi) {
-        const f32x4 v = *(const f32x4 *)(x + (size_t)r * C + q * 4);
+    const T *src = x + q * 4;
+    int r = row_begin + r0;
+    for (; r + 3 * rpi < row_end; r += 4 * rpi) {
+        f32x4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] = load_quad(src + (size_t)(r + k * rpi) * C);
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) { s += v[k][e]; ss += v[k][e] * v[k][e]; }
+    }
+    for (; r < row_end; r += rpi) {
+        const f32x4 v = load_quad(src + (size_t)r * C);
 #pragma unroll
         for (int e = 0; e < 4; e++) { s += v[e]; ss += v[e] * v[e]; }
     }
@@ -72,10 +99,10 @@ __global__ __launch_bounds__(256) void gn_partial_kernel(float *__restrict__ par
         /* group g owns quads [g * qpg, (g+1) * qpg) of every thread row; fixed summation order */
         const int g = threadIdx.x, qpg = quads >> 5;
         float a = 0.0f, b = 0.0f;
-        for (int r = 0; r < rpi; r++)
+        for (int rr = 0; rr < rpi; rr++)
             for (int k = 0; k < qpg; k++) {
-                a += sh[r * quads + g * qpg + k][0];
-                b += sh[r * quads + g * qpg + k][1];
+                a += sh[rr * quads + g * qpg + k][0];
+                b += sh[rr * quads + g * qpg + k][1];
             }
         partial[((size_t)blockIdx.x * 32 + g) * 2 + 0] = a;
         partial[((size_t)blockIdx.x * 32 + g) * 2 + 1] = b;
@@ -112,29 +139,50 @@ __global__ __launch_bounds__(256) void gn_finalize_kernel(float *__restrict__ st
 }
 
 /* out bf16 = [swish](gamma * (x - mean) * rstd + beta), zeros on the border; raw (optional)
- * receives x itself as bf16, the input of a residual block's 1x1 shortcut convolution */
-__global__ __launch_bounds__(256) void gn_apply_kernel(bf16 *__restrict__ out, bf16 *__restrict__ raw, const float *__restrict__ x,
+ * receives x itself as bf16, the input of a residual block's 1x1 shortcut convolution. Same
+ * thread-to-data map as the partial-sum pass. */
+template <typename T>
+__global__ __launch_bounds__(256) void gn_apply_kernel(bf16 *__restrict__ out, bf16 *__restrict__ raw, const T *__restrict__ x,
                                                        const float *__restrict__ stats, const float *__restrict__ gamma,
-                                                       const float *__restrict__ beta, int rows, int C, int hp, int wp, int swish) {
-    const int quads = C >> 2;
-    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (idx >= (size_t)rows * quads) return;
-    const int r = (int)(idx / quads), q = (int)(idx - (size_t)r * quads);
+                                                       const float *__restrict__ beta, int rows, int C, int hp, int wp,
+                                                       unsigned long long magic, int swish) {
+    const int quads = C >> 2, rpi = 256 / quads;
+    const int q = threadIdx.x % quads, r0 = threadIdx.x / quads;
+    const int row_begin = blockIdx.x * GN_ROWS, row_end = min(rows, row_begin + GN_ROWS);
     const int g = (q * 4) / (C >> 5);
-    const f32x4 v = *(const f32x4 *)(x + (size_t)r * C + q * 4);
-    const bool in = interior(r, hp, wp);
     const float mean = stats[g * 2], rstd = stats[g * 2 + 1];
     const f32x4 gm = *(const f32x4 *)(gamma + q * 4), bt = *(const f32x4 *)(beta + q * 4);
-    bf16x4 o, rw;
+    f32x4 sc, sh;
 #pragma unroll
-    for (int e = 0; e < 4; e++) {
-        float y = gm[e] * ((v[e] - mean) * rstd) + bt[e];
-        if (swish) y = silu_f(y);
-        o[e] = (bf16)(in ? y : 0.0f);
-        rw[e] = (bf16)v[e];
+    for (int e = 0; e < 4; e++) { sc[e] = gm[e] * rstd; sh[e] = bt[e] - mean * sc[e]; }
+    auto one = [&](int r, const f32x4 &v) {
+        const int y = div_wp(r, magic), xx = r - y * wp;
+        const bool in = y >= 1 && y < hp - 1 && xx >= 1 && xx < wp - 1;
+        bf16x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float t = v[e] * sc[e] + sh[e];
+            if (swish) t = silu_f(t);
+            o[e] = (bf16)(in ? t : 0.0f);
+        }
+        *(bf16x4 *)(out + (size_t)r * C + q * 4) = o;
+        if (raw) {
+            bf16x4 rw;
+#pragma unroll
+            for (int e = 0; e < 4; e++) rw[e] = (bf16)v[e];
+            *(bf16x4 *)(raw + (size_t)r * C + q * 4) = rw;
+        }
+    };
+    const T *src = x + q * 4;
+    int r = row_begin + r0;
+    for (; r + 3 * rpi < row_end; r += 4 * rpi) {
+        f32x4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] = load_quad(src + (size_t)(r + k * rpi) * C);
+#pragma unroll
+        for (int k = 0; k < 4; k++) one(r + k * rpi, v[k]);
     }
-    *(bf16x4 *)(out + (size_t)r * C + q * 4) = o;
-    if (raw) *(bf16x4 *)(raw + (size_t)r * C + q * 4) = rw;
+    for (; r < row_end; r += rpi) one(r, load_quad(src + (size_t)r * C));
 }
 
 /* nearest-neighbour 2x upsample (flux_upsample_nearest, flux_kernels.c:1017-1036): fp32
@@ -249,23 +297,30 @@ extern "C" int flux_hip_vae_latent_in(void *out_bf16, const float *latent, const
     return 1;
 }
 
-extern "C" int flux_hip_group_norm(void *out_bf16, void *raw_bf16, const float *x, const float *gamma, const float *beta,
-                                   float *scratch, int hp, int wp, int C, float eps, int swish) {
-    if (C != 128 && C != 256 && C != 512) return flux_hip_fail("flux_hip_group_norm: C=%d (128, 256 or 512)", C);
-    if (hp < 3 || wp < 3) return flux_hip_fail("flux_hip_group_norm: bad image %d x %d", hp, wp);
+template <typename T>
+static int group_norm_run(void *out_bf16, void *raw_bf16, const T *x, const float *gamma, const float *beta, float *scratch, int hp, int wp,
+                          int C, float eps, int swish) {
     const int rows = hp * wp, nblocks = (rows + GN_ROWS - 1) / GN_ROWS;
     float *partial = scratch + 64, *stats = scratch;
     hipStream_t st = flux_hip_stream_handle();
-    hipLaunchKernelGGL(gn_partial_kernel, dim3(nblocks), dim3(256), 0, st, partial, x, rows, C);
+    hipLaunchKernelGGL(gn_partial_kernel<T>, dim3(nblocks), dim3(256), 0, st, partial, x, rows, C);
     LAUNCH_OK("gn_partial_kernel");
     const double count = (double)(hp - 2) * (wp - 2) * (C / 32);
     hipLaunchKernelGGL(gn_finalize_kernel, dim3(32), dim3(256), 0, st, stats, partial, nblocks, count, eps);
     LAUNCH_OK("gn_finalize_kernel");
-    const size_t total = (size_t)rows * (C / 4);
-    hipLaunchKernelGGL(gn_apply_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, (bf16 *)out_bf16, (bf16 *)raw_bf16, x, stats,
-                       gamma, beta, rows, C, hp, wp, swish);
+    const unsigned long long magic = ((1ull << 40) + (unsigned)wp - 1) / (unsigned)wp;
+    hipLaunchKernelGGL(gn_apply_kernel<T>, dim3(nblocks), dim3(256), 0, st, (bf16 *)out_bf16, (bf16 *)raw_bf16, x, stats, gamma, beta, rows, C, hp,
+                       wp, magic, swish);
     LAUNCH_OK("gn_apply_kernel");
     return 1;
+}
+
+extern "C" int flux_hip_group_norm(void *out_bf16, void *raw_bf16, const void *x, int x_is_bf16, const float *gamma, const float *beta,
+                                   float *scratch, int hp, int wp, int C, float eps, int swish) {
+    if (C != 128 && C != 256 && C != 512) return flux_hip_fail("flux_hip_group_norm: C=%d (128, 256 or 512)", C);
+    if (hp < 3 || wp < 3 || wp >= 4096 || (long long)hp * wp >= (1 << 22)) return flux_hip_fail("flux_hip_group_norm: bad image %d x %d", hp, wp);
+    return x_is_bf16 ? group_norm_run(out_bf16, raw_bf16, (const bf16 *)x, gamma, beta, scratch, hp, wp, C, eps, swish)
+                     : group_norm_run(out_bf16, raw_bf16, (const float *)x, gamma, beta, scratch, hp, wp, C, eps, swish);
 }
 
 extern "C" size_t flux_hip_group_norm_scratch_floats(int hp, int wp) {

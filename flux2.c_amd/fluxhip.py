@@ -68,6 +68,7 @@ def lib():
     L.flux_hip_linear_probe.argtypes = [c_i]
     L.flux_hip_linear_probe_read.argtypes = [ctypes.POINTER(c_i), ctypes.POINTER(c_f)]
     L.flux_hip_linear_probe_read_tile.argtypes = [c_i, ctypes.POINTER(c_i), ctypes.POINTER(c_f)]
+    L.flux_hip_linear_probe_read_launches.argtypes = [c_i, vp, vp]
     L.flux_hip_adaln_norm.argtypes = [vp, c_i, vp, c_i, c_i, c_i, vp, vp, vp, vp, c_f]
     L.flux_hip_kv_prepare.argtypes = [vp, vp, c_i, vp, c_i, c_i, c_i, c_i, c_i, c_i, vp, vp, vp, vp, c_f]
     L.flux_hip_attention.argtypes = [vp, c_i, vp, c_i, vp, vp, c_i, c_i, c_i, c_i, c_i, vp, vp, vp, vp, c_f]
@@ -125,7 +126,7 @@ def lib():
     L.flux_power_schedule.argtypes = [c_i, c_f]
     L.flux_official_schedule.argtypes = [c_i, c_i]
     L.flux_hip_conv.argtypes = [c_i, vp, vp, vp, vp, vp, c_i, c_i, c_i, c_i, c_i]
-    L.flux_hip_group_norm.argtypes = [vp, vp, vp, vp, vp, vp, c_i, c_i, c_i, c_f, c_i]
+    L.flux_hip_group_norm.argtypes = [vp, vp, vp, c_i, vp, vp, vp, c_i, c_i, c_i, c_f, c_i]
     L.flux_hip_group_norm_scratch_floats.restype = c_sz
     L.flux_hip_group_norm_scratch_floats.argtypes = [c_i, c_i]
     L.flux_hip_upsample2x.argtypes = [vp, vp, c_i, c_i, c_i]

@@ -242,20 +242,21 @@ def make_vae_weights(seed=77):
 
 def vae_decode_convs(h, w):
     """The decoder's convolutions for an h x w latent, in execution order (flux_vae_decode,
-    flux_vae.c:690-837): (name, H, W, cin, cout, taps)."""
+    flux_vae.c:690-837): (name, H, W, cin, cout, taps). All but the first (which the device folds into
+    its input kernel) are one flux_hip_conv launch each, in this order."""
     mult = [1, 2, 4, 4]
     H, W = 2 * h, 2 * w
     out = [("post_quant_conv", H, W, 32, 32, 1), ("conv_in", H, W, 32, 512, 9)]
 
     def res(name, i, o):
         out.append((name + ".conv1", H, W, i, o, 9))
-        out.append((name + ".conv2", H, W, o, o, 9))
         if i != o:
             out.append((name + ".conv_shortcut", H, W, i, o, 1))
+        out.append((name + ".conv2", H, W, o, o, 9))
 
     res("mid.0", 512, 512)
-    for n in ("to_q", "to_k", "to_v", "to_out"):
-        out.append(("mid.attn." + n, H, W, 512, 512, 1))
+    out.append(("mid.attn.to_qkv", H, W, 512, 1536, 1))      # q, k and v projections, one launch on the device
+    out.append(("mid.attn.to_out", H, W, 512, 512, 1))
     res("mid.1", 512, 512)
     prev = 512
     for up in range(4):

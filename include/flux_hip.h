@@ -123,6 +123,9 @@ int flux_hip_linear_probe(int epilogue);
 int flux_hip_linear_probe_read(int *launches, float *total_ms);
 /* the same for the recorded launches that used one tile id (see force_tile) */
 int flux_hip_linear_probe_read_tile(int tile, int *launches, float *total_ms);
+/* probe(-2) records every flux_hip_conv launch. read_launches copies out, in launch order, the
+ * tile id and duration (ms) of up to `max` recorded launches and returns their number (-1 on error). */
+int flux_hip_linear_probe_read_launches(int max, int *tiles, float *ms);
 
 /*
  * out = (1 + scale) * LayerNorm(x) + shift per row, x f32 [rows, hidden], out bf16.
@@ -304,12 +307,13 @@ float *flux_hip_sample_ancestral_traced(void *transformer, const float *z, int c
  * the (H+2) x (W+2) grid: hp = H+2, wp = W+2 below. */
 
 /*
- * GroupNorm(32 groups, statistics over the whole image) with optional swish, x f32
+ * GroupNorm(32 groups, statistics over the whole image) with optional swish, x f32 or bf16
  * [hp*wp, C] -> out bf16, zeros on the border. raw (optional) receives x itself as bf16.
- * scratch: flux_hip_group_norm_scratch_floats(hp, wp) floats. C is 128, 256 or 512.
+ * scratch: flux_hip_group_norm_scratch_floats(hp, wp) floats. C is 128, 256 or 512;
+ * hp * wp < 2^22.
  * Replaces flux_group_norm (flux_kernels.c:511-553) + flux_silu (flux_kernels.c:581).
  */
-int flux_hip_group_norm(void *out_bf16, void *raw_bf16, const float *x, const float *gamma, const float *beta,
+int flux_hip_group_norm(void *out_bf16, void *raw_bf16, const void *x, int x_is_bf16, const float *gamma, const float *beta,
                         float *scratch, int hp, int wp, int C, float eps, int swish);
 size_t flux_hip_group_norm_scratch_floats(int hp, int wp);
 /* nearest-neighbour 2x: x f32 [hp*wp, C] -> out bf16 [(2H+2)*(2W+2), C] (flux_upsample_nearest, flux_kernels.c:1017) */
@@ -331,7 +335,7 @@ flux_hip_vae *flux_hip_vae_new(void);
 int flux_hip_vae_set_tensor(flux_hip_vae *v, const char *name, int dtype, const void *data, int64_t numel);
 void flux_hip_vae_free(flux_hip_vae *v);
 /* latent f32 [128, h, w] (host) -> rgb u8 [16h, 16w, 3] and/or rgb_f32 [3, 16h, 16w] (decoder output
- * before the conversion to 8 bits); either may be NULL. h, w <= 128. 1 = ok, 0 = failed. */
+ * before the conversion to 8 bits); either may be NULL. h, w <= 112. 1 = ok, 0 = failed. */
 int flux_hip_vae_decode(flux_hip_vae *v, const float *latent, int h, int w, uint8_t *rgb, float *rgb_f32);
 /* When set, called after each of the decoder's 15 blocks has been queued (role of
  * flux_vae_progress_callback, flux_kernels.h:292-293). */

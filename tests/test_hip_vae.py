@@ -152,19 +152,22 @@ def test_conv_rejects_bad_arguments(hip):
 
 @pytest.mark.parametrize("C", [128, 256, 512])
 @pytest.mark.parametrize("swish", [0, 1])
-def test_group_norm(hip, oracle_mod, C, swish):
+@pytest.mark.parametrize("in_bf16", [0, 1])
+def test_group_norm(hip, oracle_mod, C, swish, in_bf16):
     H, W = 19, 23                                    # 525 positions: more than one block of the partial-sum pass
     x = normal_f32((C, H, W), 54, 1, 0.4, 1.7)
+    if in_bf16:
+        x = q(x)
     gm, bt = normal_f32((C,), 54, 2, 1.0, 0.2), normal_f32((C,), 54, 3)
     want = oracle_mod.group_norm(x, gm, bt, 32, 1e-4)
     if swish:
         want = oracle_mod.silu(want)
     rows = (H + 2) * (W + 2)
-    dx = hip.DevBuf.from_array(to_padded(x))
+    dx = hip.DevBuf.from_array(f32_to_bf16(to_padded(x)) if in_bf16 else to_padded(x))
     dg, db = hip.DevBuf.from_array(gm), hip.DevBuf.from_array(bt)
     out, raw = hip.DevBuf(rows * C * 2), hip.DevBuf(rows * C * 2)
     scratch = hip.DevBuf(hip.lib().flux_hip_group_norm_scratch_floats(H + 2, W + 2) * 4)
-    hip.check(hip.lib().flux_hip_group_norm(out.ptr, raw.ptr, dx.ptr, dg.ptr, db.ptr, scratch.ptr, H + 2, W + 2, C, 1e-4, swish))
+    hip.check(hip.lib().flux_hip_group_norm(out.ptr, raw.ptr, dx.ptr, in_bf16, dg.ptr, db.ptr, scratch.ptr, H + 2, W + 2, C, 1e-4, swish))
     got = bf16_to_f32(out.to_array(np.uint16, (rows, C)))
     assert border_is_zero(got, H, W)
     assert rel_l2(from_padded(got, H, W), want) < 4e-3
