@@ -685,7 +685,7 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed) {
             }
         }
     }
-    if (tile < 0) return flux_hip_fail("flux_hip_linear: no permitted tile width divides N=%d", g.N);
+    if (tile < 0) tile = g.N % 128 == 0 ? 1 : 3; /* no permitted tile divides N (a forced tile that does not fit): 128 x 128, else 64 x 64 */
     g.ksplit = 1;
     g.kt_per = kt_total;
     if (best_split > 1) {

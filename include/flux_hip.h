@@ -110,7 +110,7 @@ int flux_hip_conv(int epilogue, const void *in, const void *w, const float *bias
 
 /* Measurement hooks. force_tile: 0/1/2/3/5/6/7 pins the GEMM tile (64x128, 128x128, 256x256, 64x64,
  * 288x192, 192x192, 256x192; 4 = 256x256 in its 8-wave form, never chosen automatically), -1 restores the automatic
- * choice (a tile whose width does not divide N is skipped; if none is left the call fails); enable_splitk(0) turns the split-K path off. probe(epilogue) records HIP events around every later
+ * choice (a tile whose width does not divide N is skipped; if none is left the 128x128 tile runs); enable_splitk(0) turns the split-K path off. probe(epilogue) records HIP events around every later
  * flux_hip_linear launch with that epilogue (-1 stops); probe_read waits for them and returns
  * their count and summed duration. */
 void flux_hip_linear_force_tile(int tile);
