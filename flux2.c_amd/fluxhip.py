@@ -22,6 +22,11 @@ class _Cfg(ctypes.Structure):
                                    "text_dim", "channels", "axis_dim", "sincos_dim")] + [("rope_theta", c_f)]
 
 
+class _QwenCfg(ctypes.Structure):
+    _fields_ = [(n, c_i) for n in ("hidden", "intermediate", "heads", "kv_heads", "head_dim", "layers", "vocab")] + \
+               [("out_layer", c_i * 3), ("rope_theta", c_f), ("eps", c_f)]
+
+
 class _Part(ctypes.Structure):
     _fields_ = [("A", vp), ("W", vp), ("C", vp), ("gate", vp), ("M", c_i)]
 
@@ -138,6 +143,16 @@ def lib():
     L.flux_hip_vae_set_tensor.argtypes = [vp, ctypes.c_char_p, c_i, vp, ctypes.c_int64]
     L.flux_hip_vae_free.argtypes = [vp]
     L.flux_hip_vae_decode.argtypes = [vp, vp, c_i, c_i, vp, vp]
+    L.flux_hip_rms_norm.argtypes = [vp, vp, vp, c_i, c_i, c_f]
+    L.flux_hip_causal_attention.argtypes = [vp, vp, vp, c_i, vp, c_i, c_i, c_i]
+    L.flux_hip_qwen3_new.restype = vp
+    L.flux_hip_qwen3_new.argtypes = [ctypes.POINTER(_QwenCfg)]
+    L.flux_hip_qwen3_load_dir.restype = vp
+    L.flux_hip_qwen3_load_dir.argtypes = [ctypes.c_char_p]
+    L.flux_hip_qwen3_set_tensor.argtypes = [vp, ctypes.c_char_p, c_i, vp, ctypes.c_int64]
+    L.flux_hip_qwen3_free.argtypes = [vp]
+    L.flux_hip_qwen3_forward.restype = vp
+    L.flux_hip_qwen3_forward.argtypes = [vp, vp, vp, c_i]
     _lib = L
     return L
 
@@ -450,3 +465,48 @@ class Vae:
         u = np.empty((16 * h, 16 * w, 3), np.uint8)
         check(lib().flux_hip_vae_decode(self.h, latent.ctypes.data, h, w, u.ctypes.data, f.ctypes.data), "flux_hip_vae_decode")
         return f, u
+
+
+class Qwen3:
+    """The Qwen3 text encoder on the GPU, from named tensors (uint16 = bf16 or float32) or a model directory."""
+
+    def __init__(self, cfg=None, weights=None, path=None):
+        init()
+        L = lib()
+        if path is not None:
+            self.h = L.flux_hip_qwen3_load_dir(os.fsencode(path))
+            if not self.h:
+                raise FluxHipError(f"qwen3 load_dir: {L.flux_hip_last_error().decode()}")
+            return
+        c = _QwenCfg(cfg.hidden, cfg.intermediate, cfg.heads, cfg.kv_heads, cfg.head_dim, cfg.layers, cfg.vocab,
+                     (c_i * 3)(*cfg.out_layers), cfg.rope_theta, cfg.eps)
+        self.hidden = cfg.hidden
+        self.h = L.flux_hip_qwen3_new(ctypes.byref(c))
+        if not self.h:
+            raise FluxHipError(f"qwen3_new: {L.flux_hip_last_error().decode()}")
+        for name, a in (weights or {}).items():
+            self.set_tensor(name, a)
+
+    def set_tensor(self, name, a):
+        a = np.ascontiguousarray(a)
+        dt = {np.dtype(np.float32): 0, np.dtype(np.float16): 1, np.dtype(np.uint16): 2}[a.dtype]
+        check(lib().flux_hip_qwen3_set_tensor(self.h, name.encode(), dt, a.ctypes.data, a.size), f"qwen3 set_tensor({name})")
+
+    def close(self):
+        if getattr(self, "h", None):
+            lib().flux_hip_qwen3_free(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def forward(self, ids, mask=None, hidden=None):
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        m = None if mask is None else np.ascontiguousarray(mask, dtype=np.int32)
+        p = lib().flux_hip_qwen3_forward(self.h, ids.ctypes.data, None if m is None else m.ctypes.data, ids.size)
+        if not p:
+            raise FluxHipError(f"flux_hip_qwen3_forward: {lib().flux_hip_last_error().decode()}")
+        return _take_host(p, (ids.size, 3 * (hidden or self.hidden)))

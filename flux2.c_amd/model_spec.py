@@ -279,6 +279,74 @@ def vae_decode_flops(h, w):
     return conv + 4.0 * n * n * 512
 
 
+@dataclass(frozen=True)
+class QwenConfig:
+    """Qwen3 text encoder (flux_qwen3.h:22-39): the hidden states after three layers, side by side,
+    are the transformer's text input."""
+    hidden: int = 2560
+    intermediate: int = 9728
+    heads: int = 32
+    kv_heads: int = 8
+    head_dim: int = 128
+    layers: int = 36
+    vocab: int = 151936
+    out_layers: tuple = (8, 17, 26)
+    rope_theta: float = 1000000.0
+    eps: float = 1e-6
+
+
+QWEN3_4B = QwenConfig()
+# structurally identical, small enough for the CPU oracle to run in milliseconds
+QWEN3_TINY = QwenConfig(hidden=256, intermediate=384, heads=4, kv_heads=2, layers=5, vocab=300, out_layers=(1, 2, 4))
+
+
+def qwen3_tensor_shapes(cfg: QwenConfig) -> "OrderedDict[str, tuple]":
+    """Tensor names and shapes as the reference loader reads them (flux_qwen3.c:1211-1253, 1361, 1376)."""
+    t = OrderedDict()
+    H, I, QD, KD = cfg.hidden, cfg.intermediate, cfg.heads * cfg.head_dim, cfg.kv_heads * cfg.head_dim
+    t["model.embed_tokens.weight"] = (cfg.vocab, H)
+    for i in range(cfg.layers):
+        p = f"model.layers.{i}."
+        t[p + "input_layernorm.weight"] = (H,)
+        t[p + "post_attention_layernorm.weight"] = (H,)
+        t[p + "self_attn.q_proj.weight"] = (QD, H)
+        t[p + "self_attn.k_proj.weight"] = (KD, H)
+        t[p + "self_attn.v_proj.weight"] = (KD, H)
+        t[p + "self_attn.o_proj.weight"] = (H, QD)
+        t[p + "self_attn.q_norm.weight"] = (cfg.head_dim,)
+        t[p + "self_attn.k_norm.weight"] = (cfg.head_dim,)
+        t[p + "mlp.gate_proj.weight"] = (I, H)
+        t[p + "mlp.up_proj.weight"] = (I, H)
+        t[p + "mlp.down_proj.weight"] = (H, I)
+    t["model.norm.weight"] = (H,)
+    return t
+
+
+def make_qwen3_weights(cfg: QwenConfig, seed=61, only=None):
+    """Synthetic bf16 encoder: projections ~N(0, 1/sqrt(fan_in)) (activations stay of order one through the
+    layers), norm weights ~N(1, 0.1), embeddings ~N(0, 1)."""
+    out = OrderedDict()
+    for idx, (name, shape) in enumerate(qwen3_tensor_shapes(cfg).items()):
+        if only is not None and name not in only:
+            continue
+        if len(shape) == 1:
+            out[name] = normal_bf16(shape, seed, 9000 + idx, 1.0, 0.1)
+        elif name == "model.embed_tokens.weight":
+            out[name] = normal_bf16(shape, seed, 9000 + idx, 0.0, 1.0)
+        else:
+            out[name] = normal_bf16(shape, seed, 9000 + idx, 0.0, 1.0 / np.sqrt(shape[1]))
+    return out
+
+
+def qwen3_flops(cfg: QwenConfig, seq):
+    """Algorithmic FLOPs of one encoder forward over seq tokens: the layers up to the last captured one;
+    attention counted over the full seq x seq score matrix, as the reference computes it."""
+    H, I, QD, KD = cfg.hidden, cfg.intermediate, cfg.heads * cfg.head_dim, cfg.kv_heads * cfg.head_dim
+    n_layers = max(cfg.out_layers) + 1
+    per_tok = 2.0 * (H * (QD + 2 * KD) + QD * H + 3 * H * I)
+    return n_layers * (seq * per_tok + 4.0 * seq * seq * QD)
+
+
 def flops_per_forward(cfg: FluxConfig, n_img, n_txt, n_img_out=None):
     """Algorithmic FLOPs of one forward (1 MAC = 2 FLOP)."""
     H, C, T = cfg.hidden, cfg.channels, cfg.text_dim

@@ -348,6 +348,57 @@ void *flux_vae_load_safetensors(void *safetensors_file);
 void *flux_vae_decode(void *vae, const float *latent, int batch, int latent_h, int latent_w);
 void flux_vae_free(void *vae);
 
+/* ---------------------------------------------------------------- Qwen3 text encoder
+ * The step before the sampling loop: token ids -> the transformer's text input
+ * (qwen3_forward, flux_qwen3.c:1041-1156). */
+
+/* out bf16 [rows, hidden] = x / sqrt(mean(x^2) + eps) * w per row, x f32 (qwen3_rms_norm, flux_qwen3.c:177-197) */
+int flux_hip_rms_norm(void *out_bf16, const float *x, const float *w, int rows, int hidden, float eps);
+/*
+ * Causal grouped-query attention with a padding mask, head_dim 128, seq <= 512
+ * (qwen3_attention_forward, flux_qwen3.c:352-437, and flux_metal_causal_attention there).
+ * qkv bf16 [seq, (heads + 2 kv_heads) * 128]: q heads, then k heads (both already normed and
+ * rotated); vt bf16 [kv_heads * 128, ldv]: v transposed, ldv >= seq rounded up to 32, columns
+ * beyond seq finite; mask int [seq] on the device or NULL. out bf16 [seq, heads * 128].
+ * A masked or future key scores -1e9 before the softmax over all seq columns, as in the reference.
+ */
+int flux_hip_causal_attention(void *out_bf16, const void *qkv_bf16, const void *vt_bf16, int ldv, const int *mask_dev, int seq,
+                              int heads, int kv_heads);
+
+typedef struct {
+    int hidden, intermediate, heads, kv_heads, head_dim, layers, vocab;
+    int out_layer[3];          /* hidden states after these layers (0-based) form the output, side by side */
+    float rope_theta, eps;
+} flux_hip_qwen3_config;
+void flux_hip_qwen3_default_config(flux_hip_qwen3_config *c);   /* flux_qwen3.h:22-39 */
+
+typedef struct flux_hip_qwen3 flux_hip_qwen3;
+/* From a directory with model-00001-of-00002.safetensors + model-00002-of-00002.safetensors
+ * (flux_qwen3.c:1341-1343) or one model.safetensors; sizes are read from the tensors. */
+flux_hip_qwen3 *flux_hip_qwen3_load_dir(const char *model_dir);
+/* Piecewise: new (NULL = the reference's sizes), one set_tensor per tensor (dtype 0 f32, 1 f16, 2 bf16). */
+flux_hip_qwen3 *flux_hip_qwen3_new(const flux_hip_qwen3_config *cfg);
+int flux_hip_qwen3_set_tensor(flux_hip_qwen3 *q, const char *name, int dtype, const void *data, int64_t numel);
+void flux_hip_qwen3_free(flux_hip_qwen3 *q);
+/* ids / mask: host int [seq_len], mask may be NULL; returns a malloc'd host array [seq_len, 3 * hidden]
+ * (caller frees) or NULL. seq_len <= 512. */
+float *flux_hip_qwen3_forward(flux_hip_qwen3 *q, const int *input_ids, const int *attention_mask, int seq_len);
+/* When set, called after each layer has been queued (role of flux_text_progress_callback). */
+extern void (*flux_hip_qwen3_progress)(int layer, int total);
+
+/* The reference's own entry points (flux_qwen3.h:93-141) over the device encoder: an application
+ * keeps flux_qwen3_tokenizer.c and leaves flux_qwen3.c out of its link. Declared here only when the
+ * reference's header has not been included (its declarations use its own opaque types). */
+#ifndef FLUX_QWEN3_H
+void *qwen3_model_load(const char *model_dir);
+void *qwen3_model_load_mmap(const char *model_dir);
+void qwen3_model_free(void *model);
+float *qwen3_forward(void *model, const int *input_ids, const int *attention_mask, int seq_len);
+void *qwen3_encoder_load(const char *model_dir, int use_mmap);
+void qwen3_encoder_free(void *enc);
+float *qwen3_encode_text(void *enc, const char *prompt);
+#endif
+
 /*
  * The sampling loop in pieces, for callers that drive or time the steps themselves. begin()
  * uploads latent, text and reference tokens and computes every step's modulation vectors;

@@ -27,6 +27,11 @@ class _Ref(ctypes.Structure):
     _fields_ = [("latent", vp), ("h", c_i), ("w", c_i), ("t_offset", c_i)]
 
 
+class _QwenCfg(ctypes.Structure):
+    _fields_ = [(n, c_i) for n in ("hidden", "intermediate", "heads", "kv_heads", "head_dim", "layers", "vocab")] + \
+               [("out_layer", c_i * 3), ("rope_theta", c_f), ("eps", c_f)]
+
+
 _lib = None
 
 
@@ -92,6 +97,17 @@ def lib():
     L.fo_vae_set.restype = c_i
     L.fo_vae_decode.argtypes = [vp, vp, c_i, c_i, vp, vp]
     L.fo_vae_decode.restype = c_i
+    L.fo_qwen3_new.argtypes = [ctypes.POINTER(_QwenCfg)]
+    L.fo_qwen3_new.restype = vp
+    L.fo_qwen3_free.argtypes = [vp]
+    L.fo_qwen3_set_bf16.argtypes = [vp, ctypes.c_char_p, vp, ctypes.c_int64]
+    L.fo_qwen3_set_bf16.restype = c_i
+    L.fo_qwen3_forward.argtypes = [vp, vp, vp, c_i]
+    L.fo_qwen3_forward.restype = vp
+    L.fo_qwen3_layer_forward.argtypes = [vp, c_i, vp, vp, c_i]
+    L.fo_qwen3_rms_norm.argtypes = [vp, vp, vp, c_i, c_i, c_f]
+    L.fo_qwen3_rope.argtypes = [vp, c_i, c_i, c_i, c_f]
+    L.fo_qwen3_attention.argtypes = [vp, vp, vp, vp, vp, c_i, c_i, c_i, c_i]
     _lib = L
     return L
 
@@ -422,3 +438,71 @@ class VaeOracle:
         if self._L.fo_vae_decode(self._v, latent.ctypes.data, h, w, f.ctypes.data, u.ctypes.data) != 0:
             raise RuntimeError("vae oracle: decode failed (missing tensor)")
         return f, u
+
+
+# ---- Qwen3 text encoder (oracle/qwen3_oracle.c) ----
+
+def qwen3_rms_norm(x, w, eps=1e-6):
+    x, w = _f32(x), _f32(w)
+    out = np.empty_like(x)
+    lib().fo_qwen3_rms_norm(out.ctypes.data, x.ctypes.data, w.ctypes.data, x.shape[0], x.shape[1], eps)
+    return out
+
+
+def qwen3_rope(x, heads, head_dim, theta=1000000.0):
+    """x [seq, heads*head_dim] -> rotated copy."""
+    x = _f32(x).copy()
+    lib().fo_qwen3_rope(x.ctypes.data, x.shape[0], heads, head_dim, theta)
+    return x
+
+
+def qwen3_attention(q, k, v, mask, heads, kv_heads, head_dim=128):
+    """q [seq, heads*hd], k, v [seq, kv_heads*hd], mask int [seq] or None -> [seq, heads*hd]."""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    m = None if mask is None else np.ascontiguousarray(mask, dtype=np.int32)
+    out = np.empty_like(q)
+    lib().fo_qwen3_attention(out.ctypes.data, q.ctypes.data, k.ctypes.data, v.ctypes.data, None if m is None else m.ctypes.data,
+                             q.shape[0], heads, kv_heads, head_dim)
+    return out
+
+
+class Qwen3Oracle:
+    """`weights` maps tensor name -> uint16 (bf16) array; cfg is a model_spec.QwenConfig."""
+
+    def __init__(self, cfg, weights):
+        self.cfg = cfg
+        self._L = lib()
+        c = _QwenCfg(cfg.hidden, cfg.intermediate, cfg.heads, cfg.kv_heads, cfg.head_dim, cfg.layers, cfg.vocab,
+                     (c_i * 3)(*cfg.out_layers), cfg.rope_theta, cfg.eps)
+        self._m = self._L.fo_qwen3_new(ctypes.byref(c))
+        for name, a in weights.items():
+            a = np.ascontiguousarray(a, dtype=np.uint16)
+            rc = self._L.fo_qwen3_set_bf16(self._m, name.encode(), a.ctypes.data, a.size)
+            if rc < 0:
+                raise ValueError(f"qwen3 oracle rejected tensor {name}: {rc}")
+
+    def close(self):
+        if self._m:
+            self._L.fo_qwen3_free(self._m)
+            self._m = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def forward(self, ids, mask=None):
+        ids = np.ascontiguousarray(ids, dtype=np.int32)
+        m = None if mask is None else np.ascontiguousarray(mask, dtype=np.int32)
+        p = self._L.fo_qwen3_forward(self._m, ids.ctypes.data, None if m is None else m.ctypes.data, ids.size)
+        n = ids.size * 3 * self.cfg.hidden
+        out = np.ctypeslib.as_array(ctypes.cast(p, ctypes.POINTER(c_f)), shape=(n,)).copy().reshape(ids.size, 3 * self.cfg.hidden)
+        self._L.fo_free(p)
+        return out
+
+    def layer(self, idx, h, mask=None):
+        h = _f32(h).copy()
+        m = None if mask is None else np.ascontiguousarray(mask, dtype=np.int32)
+        self._L.fo_qwen3_layer_forward(self._m, idx, h.ctypes.data, None if m is None else m.ctypes.data, h.shape[0])
+        return h

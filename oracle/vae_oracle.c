@@ -208,7 +208,7 @@ static int attnblock(const fo_vae *v, const char *prefix, float *out, const floa
         float *row = (float *)malloc(sizeof(float) * (size_t)sp);
         #pragma omp for schedule(static)
         for (int i = 0; i < sp; i++) {
-            float mx = -INFINITY;
+            float mx = -3.0e38f;
             for (int j = 0; j < sp; j++) {
                 float s = 0.0f;
                 for (int c = 0; c < ch; c++) s += q[(size_t)c * sp + i] * scale * k[(size_t)c * sp + j];

@@ -20,8 +20,8 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 sys.path.insert(0, os.path.join(ROOT, "flux2.c_amd"))
-from model_spec import (TINY, KLEIN_4B, make_weights, make_vae_weights, write_safetensors, normal_f32,  # noqa: E402
-                        bf16_to_f32)
+from model_spec import (TINY, KLEIN_4B, QWEN3_4B, make_weights, make_vae_weights, make_qwen3_weights,  # noqa: E402
+                        write_safetensors, normal_f32, bf16_to_f32)
 
 c_f, c_i, vp = ctypes.c_float, ctypes.c_int, ctypes.c_void_p
 
@@ -355,6 +355,45 @@ def vae_golden():
     return g
 
 
+# shared with tests/test_oracle_golden.py: token ids and masks of the two encoder cases
+QWEN3_CASES = {"masked8": ([151644, 872, 198, 64, 8251, 151645, 151643, 151643], [1, 1, 1, 1, 1, 1, 0, 0]),
+               "plain5": ([11, 4999, 151935, 0, 77777], None)}
+
+
+def qwen3_golden():
+    """The reference's qwen3_forward (flux_qwen3.c:1041, CPU arm, weights streamed layer by layer through
+    qwen3_model_load_mmap) on the synthetic full-size encoder of model_spec.make_qwen3_weights.
+    Writes an 8 GB model directory under a temporary directory while it runs."""
+    import tempfile
+    g = {}
+    L.qwen3_model_load_mmap.restype = vp
+    L.qwen3_model_load_mmap.argtypes = [ctypes.c_char_p]
+    L.qwen3_forward.restype = vp
+    L.qwen3_forward.argtypes = [vp, vp, vp, c_i]
+    L.qwen3_model_free.argtypes = [vp]
+    cfg = QWEN3_4B
+    with tempfile.TemporaryDirectory() as d:
+        W = make_qwen3_weights(cfg)
+        names = list(W)
+        half = names.index("model.layers.18.input_layernorm.weight")
+        write_safetensors(os.path.join(d, "model-00001-of-00002.safetensors"), {n: W[n] for n in names[:half]})
+        write_safetensors(os.path.join(d, "model-00002-of-00002.safetensors"), {n: W[n] for n in names[half:]})
+        del W
+        m = L.qwen3_model_load_mmap(d.encode())
+        assert m
+        for key, (ids, mask) in QWEN3_CASES.items():
+            ids = np.array(ids, np.int32)
+            mk = None if mask is None else np.array(mask, np.int32)
+            p = L.qwen3_forward(m, P(ids), None if mk is None else P(mk), ids.size)
+            assert p
+            out = np.ctypeslib.as_array(ctypes.cast(p, ctypes.POINTER(c_f)), shape=(ids.size * 3 * cfg.hidden,)).copy()
+            ctypes.CDLL(None).free(ctypes.c_void_p(p))
+            g[key] = out.reshape(ids.size, 3 * cfg.hidden)
+            print("qwen3", key, "std", g[key].std(), flush=True)
+        L.qwen3_model_free(m)
+    return g
+
+
 def full_c1(qk):
     """Config c1 of the benchmark at the real 4B architecture: 4x4 latent, 64 text tokens, t=1."""
     cfg = KLEIN_4B
@@ -372,8 +411,12 @@ if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--full", action="store_true")
     ap.add_argument("--only-vae", action="store_true", help="rewrite vae.npz only")
+    ap.add_argument("--qwen3", action="store_true", help="rewrite qwen3_4b.npz only (8 GB of temporary files, minutes)")
     args = ap.parse_args()
     L = load()
+    if args.qwen3:
+        np.savez_compressed(os.path.join(HERE, "qwen3_4b.npz"), **qwen3_golden())
+        sys.exit(0)
     np.savez_compressed(os.path.join(HERE, "vae.npz"), **vae_golden())
     if args.only_vae:
         sys.exit(0)

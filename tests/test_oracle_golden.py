@@ -257,3 +257,31 @@ def test_vae_decode_images(oracle_mod, vae_gold):
         q = np.clip((f.transpose(1, 2, 0) + 1.0) * 127.5, 0, 255).astype(np.uint8)
         np.testing.assert_array_equal(q, u)
     o.close()
+
+
+# ---- Qwen3 text encoder (oracle/qwen3_oracle.c) against the reference's qwen3_forward ----
+QWEN3_CASES = {"masked8": ([151644, 872, 198, 64, 8251, 151645, 151643, 151643], [1, 1, 1, 1, 1, 1, 0, 0]),
+               "plain5": ([11, 4999, 151935, 0, 77777], None)}
+
+
+@pytest.mark.slow
+@pytest.mark.skipif(not os.environ.get("FLUX_SLOW"), reason="full-size text encoder: ~20 GB of RAM and a minute; set FLUX_SLOW=1")
+def test_qwen3_full_size_forward(oracle_mod, golden_dir):
+    """The oracle at the reference's sizes on the synthetic encoder the fixture was made with
+    (tests/golden/make_golden.py --qwen3 ran the reference's qwen3_forward on the same tensors)."""
+    from dataclasses import replace
+    from model_spec import QWEN3_4B, qwen3_tensor_shapes, make_qwen3_weights
+    gold = np.load(os.path.join(golden_dir, "qwen3_4b.npz"))
+    cfg = replace(QWEN3_4B, layers=27)                    # layers after the last captured one do not matter
+    o = oracle_mod.Qwen3Oracle(cfg, {})
+    for name in qwen3_tensor_shapes(QWEN3_4B):
+        a = make_qwen3_weights(QWEN3_4B, only=[name])[name]
+        rc = o._L.fo_qwen3_set_bf16(o._m, name.encode(), a.ctypes.data, a.size)
+        assert rc >= 0, (name, rc)
+    for key, (ids, mask) in QWEN3_CASES.items():
+        got = o.forward(ids, mask)
+        assert got.shape == gold[key].shape
+        r = rel_l2(got, gold[key])
+        print(key, "rel_l2 vs reference", r)
+        assert r <= 2e-5, (key, r)
+    o.close()

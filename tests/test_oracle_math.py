@@ -158,3 +158,69 @@ def test_group_norm_statistics(oracle_mod):
     assert np.abs(g.mean(axis=1)).max() < 1e-5 and np.abs(g.var(axis=1) - 1.0).max() < 1e-4
     gm, bt = normal_f32((64,), 2, 4), normal_f32((64,), 2, 5)
     assert rel_l2(oracle_mod.group_norm(x, gm, bt, 32, 1e-6), y * gm[:, None, None] + bt[:, None, None]) < 1e-6
+
+
+# ---- Qwen3 text encoder ----
+
+def test_qwen3_layer_matches_numpy(oracle_mod):
+    """One layer of the tiny encoder against a float64 numpy evaluation of the same formulas."""
+    from model_spec import QWEN3_TINY as cfg, make_qwen3_weights, bf16_to_f32
+    W = make_qwen3_weights(cfg)
+    o = oracle_mod.Qwen3Oracle(cfg, W)
+    w = {k: bf16_to_f32(v).astype(np.float64) for k, v in W.items() if k.startswith("model.layers.1.")}
+    g = lambda n: w["model.layers.1." + n]
+    seq, H, hd, nh, nk = 7, cfg.hidden, cfg.head_dim, cfg.heads, cfg.kv_heads
+    h = normal_f32((seq, H), 3, 1).astype(np.float64)
+    mask = np.array([1, 1, 1, 1, 1, 0, 0])
+
+    def rms(x, wt):
+        return x / np.sqrt((x * x).mean(axis=-1, keepdims=True) + cfg.eps) * wt
+
+    def rope(x, heads):
+        x = x.reshape(seq, heads, hd).copy()
+        i = np.arange(hd // 2)
+        ang = np.arange(seq)[:, None] / cfg.rope_theta ** (2 * i / hd)[None, :]
+        c, s = np.cos(ang)[:, None, :], np.sin(ang)[:, None, :]
+        x0, x1 = x[..., :hd // 2].copy(), x[..., hd // 2:].copy()
+        x[..., :hd // 2] = x0 * c - x1 * s
+        x[..., hd // 2:] = x0 * s + x1 * c
+        return x
+
+    n = rms(h, g("input_layernorm.weight"))
+    q = rope(rms((n @ g("self_attn.q_proj.weight").T).reshape(seq, nh, hd), g("self_attn.q_norm.weight")).reshape(seq, -1), nh)
+    k = rope(rms((n @ g("self_attn.k_proj.weight").T).reshape(seq, nk, hd), g("self_attn.k_norm.weight")).reshape(seq, -1), nk)
+    v = (n @ g("self_attn.v_proj.weight").T).reshape(seq, nk, hd)
+    att = np.zeros((seq, nh, hd))
+    for hh in range(nh):
+        sc = q[:, hh] @ k[:, hh // (nh // nk)].T / np.sqrt(hd)
+        sc[np.triu_indices(seq, 1)] = -1e9
+        sc[:, mask == 0] = -1e9
+        p = np.exp(sc - sc.max(axis=1, keepdims=True))
+        att[:, hh] = (p / p.sum(axis=1, keepdims=True)) @ v[:, hh // (nh // nk)]
+    h1 = h + att.reshape(seq, -1) @ g("self_attn.o_proj.weight").T
+    n2 = rms(h1, g("post_attention_layernorm.weight"))
+    gate, up = n2 @ g("mlp.gate_proj.weight").T, n2 @ g("mlp.up_proj.weight").T
+    want = h1 + (gate / (1 + np.exp(-gate)) * up) @ g("mlp.down_proj.weight").T
+    assert rel_l2(o.layer(1, h.astype(np.float32), mask), want) < 2e-6
+    o.close()
+
+
+def test_qwen3_causality_and_padding(oracle_mod):
+    from model_spec import QWEN3_TINY as cfg, make_qwen3_weights
+    o = oracle_mod.Qwen3Oracle(cfg, make_qwen3_weights(cfg))
+    ids = np.array([3, 7, 299, 12, 5, 0, 0], np.int32)
+    mask = np.array([1, 1, 1, 1, 1, 0, 0], np.int32)
+    y = o.forward(ids, mask)
+    assert y.shape == (7, 3 * cfg.hidden)
+    ids2 = ids.copy()
+    ids2[3] = 100                                        # a later token cannot change earlier positions
+    y2 = o.forward(ids2, mask)
+    np.testing.assert_array_equal(y[:3], y2[:3])
+    assert np.abs(y[3:] - y2[3:]).max() > 1e-3
+    ids3 = ids.copy()
+    ids3[5:] = (44, 45)                                  # what sits in masked positions cannot change real positions
+    np.testing.assert_array_equal(o.forward(ids3, mask)[:5], y[:5])
+    # an id outside the vocabulary embeds as zeros (flux_qwen3.c:1053-1056): position 0 then stays zero in every captured layer
+    y4 = o.forward(np.array([cfg.vocab, 4], np.int32), None)
+    assert not y4[0].any() and np.abs(y4[1]).max() > 0
+    o.close()
