@@ -16,7 +16,8 @@ Also measured in the same run:
                 extrapolated to the 5 + 20 blocks of a step
 
 --workload vae_c2 | vae_c3 | vae_c4 measures the step after the sampling loop instead: one "step" is
-one VAE decode of a 16/32/64-wide latent to a 256/512/1024-pixel image.
+one VAE decode of a 16/32/64-wide latent to a 256/512/1024-pixel image. --workload qwen3 measures the
+step before it: one forward of the text encoder over 512 tokens.
 """
 import argparse
 import json
@@ -195,12 +196,87 @@ def bench_vae(args):
         "tflops": round(flops * K / wall / 1e12, 1), "flops_per_step": flops, "roofline": roof, "cpu_baseline": cpu}))
 
 
+def bench_qwen3(args):
+    """One step = one text-encoder forward over 512 tokens (the padded length the pipeline always uses,
+    flux_qwen3.c:1627-1652) through flux_hip_qwen3_forward: host token ids in, host embeddings
+    [512, 7680] fp32 out (15.7 MB over PCIe inside the timed region)."""
+    import ctypes
+    from model_spec import QWEN3_4B, qwen3_tensor_shapes, make_qwen3_weights, qwen3_flops
+    cfg = QWEN3_4B
+    K, Wm = args.steps, args.warmup
+    seq, real = 512, 40
+    fluxhip.init()
+    if args.tile_mask:
+        fluxhip.lib().flux_hip_linear_tile_mask(args.tile_mask)
+    m = fluxhip.Qwen3(cfg)
+    last = max(cfg.out_layers)
+    for name in qwen3_tensor_shapes(cfg):
+        if name.startswith("model.layers.") and int(name.split(".")[2]) > last:
+            continue
+        m.set_tensor(name, make_qwen3_weights(cfg, only=[name])[name])
+    rng = np.random.default_rng(5)
+    ids = rng.integers(0, cfg.vocab, seq).astype(np.int32)
+    mask = np.zeros(seq, np.int32)
+    mask[:real] = 1
+    ids[real:] = 151643
+    for _ in range(max(Wm, 1)):
+        out = m.forward(ids, mask)
+    assert np.isfinite(out).all()
+    L = fluxhip.lib()
+    if not args.no_kernel_timing:
+        L.flux_hip_linear_probe(fluxhip.EPI_SWIGLU)
+    t0 = time.perf_counter()
+    for _ in range(K):
+        m.forward(ids, mask)
+    wall = time.perf_counter() - t0
+    flops = qwen3_flops(cfg, seq)
+    roof = None
+    if not args.no_kernel_timing:
+        n_t, ms_t = ctypes.c_int(0), ctypes.c_float(0.0)
+        L.flux_hip_linear_probe_read(ctypes.byref(n_t), ctypes.byref(ms_t))
+        L.flux_hip_linear_probe(-1)
+        if n_t.value:
+            k_flops = 2.0 * seq * cfg.hidden * 2 * cfg.intermediate
+            per_ms = ms_t.value / n_t.value
+            ach = k_flops / (per_ms * 1e-3) / 1e12
+            roof = {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
+                    "kernel": "gate/up projection + SiLU*up GEMM at [512, 2560] x [19456, 2560]^T (the largest of a layer's four GEMMs)",
+                    "launches_timed": n_t.value, "ms_per_launch": round(per_ms, 4), "flops_per_launch": k_flops}
+    m.close()
+    cpu = None
+    if not args.no_cpu_baseline:
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        import oracle as O
+        from dataclasses import replace
+        # two full-size layers over 64 tokens on the CPU oracle, carried to the benchmarked size by FLOP count
+        c2 = replace(cfg, layers=2, out_layers=(0, 1, 1), vocab=1024)
+        o = O.Qwen3Oracle(c2, make_qwen3_weights(c2))
+        ids_c = rng.integers(0, 1024, 64).astype(np.int32)
+        o.forward(ids_c[:4])
+        t1 = time.perf_counter()
+        o.forward(ids_c)
+        dt = time.perf_counter() - t1
+        o.close()
+        rate = qwen3_flops(c2, 64) / dt
+        cpu = {"value": rate / flops, "unit": "encodes/s", "cores": O.lib().fo_num_threads(), "kind": "port",
+               "sample": f"two full-size layers over 64 tokens ({dt:.1f} s, {rate / 1e9:.1f} GFLOP/s, OpenMP loops of the CPU oracle), "
+                         f"carried to 27 layers x 512 tokens by FLOP count"}
+    print(json.dumps({
+        "metric": "text encodes/s (Qwen3-4B encoder, 512 tokens, 1 GPU)", "value": round(K / wall, 3), "unit": "encodes/s",
+        "n_gpus": 1, "steps": K, "warmup": Wm, "ms_per_step": round(wall * 1000.0 / K, 3), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "qwen3: Qwen3-4B text encoder (layers 0-26 of 36, random-init bf16), 512 token ids "
+                               "(40 real + padding) -> [512, 7680] embeddings, host buffers in and out"},
+        "tflops": round(flops * K / wall / 1e12, 1), "flops_per_step": flops, "roofline": roof, "cpu_baseline": cpu}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=8)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + sorted(VAE_WORKLOADS))
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + sorted(VAE_WORKLOADS) + ["qwen3"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     ap.add_argument("--tile-mask", type=lambda v: int(v, 0), default=0,
@@ -216,6 +292,8 @@ def main():
 
     if args.workload in VAE_WORKLOADS:
         return bench_vae(args)
+    if args.workload == "qwen3":
+        return bench_qwen3(args)
     cfg = KLEIN_4B
     wl = WORKLOADS[args.workload]
     if args.calibrate:

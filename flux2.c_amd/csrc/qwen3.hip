@@ -86,16 +86,24 @@ __global__ __launch_bounds__(64) void qwen3_qk_rope_kernel(bf16 *__restrict__ qk
  * plain three-step one. Inside each group of 32 keys the K rows are assigned to MFMA rows so that
  * a lane ends up with 8 consecutive keys of one query: that is the B-operand layout of the second
  * product O^T = V^T P^T. K, Q and V^T fragments are read straight from global memory (the whole
- * K and V of a layer are 2 MB and sit in L2).
+ * K and V of a layer are 2 MB and sit in L2), three steps ahead of their use. Every wave streams
+ * the K and V of its kv head on its own, which makes L2 traffic the bound (about 300 MB per call at
+ * 512 tokens); sharing the tiles between the four heads of a group through LDS would cut it by 4.
  */
 #define QW_MAXT 16 /* 32-key steps: 512 keys */
-__global__ __launch_bounds__(64) void qwen3_attention_kernel(bf16 *__restrict__ out, const bf16 *__restrict__ qkv, const bf16 *__restrict__ vt,
-                                                             int ldv, const int *__restrict__ mask, int seq, int heads, int kv_heads) {
+
+/* The body for NT 32-key steps, NT a compile-time constant: straight-line code, so that fragment
+ * loads can be kept three steps ahead of the MFMAs that use them (scheduling barriers stop the
+ * compiler from sinking them back next to their uses, where each would be waited for alone).
+ * Steps beyond the sequence read clamped rows and are masked like the padding of the last step. */
+template <int NT>
+__device__ __forceinline__ void qwen3_attend(bf16 *__restrict__ out, const bf16 *__restrict__ qkv, const bf16 *__restrict__ vt, int ldv,
+                                             const int *__restrict__ mask, int seq, int heads, int kv_heads) {
     const int lane = threadIdx.x, l15 = lane & 15, lq = lane >> 4;
     const int q0 = blockIdx.x * 16, h = blockIdx.y, kh = h / (heads / kv_heads);
     const int width = (heads + 2 * kv_heads) * 128;
-    const int nt = (seq + 31) >> 5;
     const float scale = 0.08838834764831845f; /* 1 / sqrt(128) */
+    constexpr int PD = NT >= 4 ? 3 : 1;       /* steps of fragment loads in flight */
 
     /* Q^T fragments (MFMA B operand): lane (query l15, lq) holds dims [32 ks + 8 lq, +8) */
     const int qrow = min(q0 + l15, seq - 1);
@@ -103,82 +111,100 @@ __global__ __launch_bounds__(64) void qwen3_attention_kernel(bf16 *__restrict__ 
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) qf[ks] = *(const bf16x8 *)(qkv + (size_t)qrow * width + h * 128 + ks * 32 + lq * 8);
 
-    f32x4 sc[2 * QW_MAXT];
+    auto load_k = [&](bf16x8 (&kf)[8], int t) {
 #pragma unroll
-    for (int t = 0; t < QW_MAXT; t++) {
-        if (t < nt) {
+        for (int half = 0; half < 2; half++) {
+            /* MFMA row m = l15 of this block is key 32 t + 8 (m / 4) + 4 half + (m % 4) */
+            const int key = min(32 * t + 8 * (l15 >> 2) + 4 * half + (l15 & 3), seq - 1);
+            const bf16 *kp = qkv + (size_t)key * width + (heads + kh) * 128 + lq * 8;
 #pragma unroll
-            for (int half = 0; half < 2; half++) {
-                /* MFMA row m = l15 of this block is key 32 t + 8 (m / 4) + 4 half + (m % 4) */
-                const int key = min(32 * t + 8 * (l15 >> 2) + 4 * half + (l15 & 3), seq - 1);
-                const bf16 *kp = qkv + (size_t)key * width + (heads + kh) * 128 + lq * 8;
-                f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-                for (int ks = 0; ks < 4; ks++)
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8 *)(kp + ks * 32), qf[ks], acc, 0, 0, 0);
-                sc[2 * t + half] = acc;
-            }
+            for (int ks = 0; ks < 4; ks++) kf[half * 4 + ks] = *(const bf16x8 *)(kp + ks * 32);
         }
+    };
+    f32x4 sc[2 * NT];
+    bf16x8 kbuf[PD + 1][8];
+#pragma unroll
+    for (int t = 0; t < PD && t < NT; t++) load_k(kbuf[t], t);
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        if (t + PD < NT) load_k(kbuf[(t + PD) % (PD + 1)], t + PD);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kbuf[t % (PD + 1)][half * 4 + ks], qf[ks], acc, 0, 0, 0);
+            sc[2 * t + half] = acc;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    /* padding mask as bits: word w covers keys [64 w, 64 w + 64), one ballot per word */
+    unsigned long long keep[(NT + 1) / 2];
+#pragma unroll
+    for (int w = 0; w < (NT + 1) / 2; w++) {
+        const int key = 64 * w + lane;
+        keep[w] = __ballot(key < seq && (!mask || mask[key] != 0));
     }
     /* accumulator element e of block (t, half): query l15, key 32 t + 8 lq + 4 half + e */
     const int qi = q0 + l15;
     float mx = -3.0e38f;
 #pragma unroll
-    for (int t = 0; t < QW_MAXT; t++) {
-        if (t < nt) {
+    for (int t = 0; t < NT; t++) {
+        const unsigned bits = (unsigned)(keep[t >> 1] >> (32 * (t & 1))) >> (8 * lq); /* this lane's 8 keys of step t */
 #pragma unroll
-            for (int half = 0; half < 2; half++)
+        for (int half = 0; half < 2; half++)
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int key = 32 * t + 8 * lq + 4 * half + e;
-                    float v = sc[2 * t + half][e] * scale;
-                    if (key >= seq) v = -INFINITY; /* padding of the last 32-key step: no column of the reference's matrix */
-                    else if (key > qi || (mask && mask[key] == 0)) v = -1e9f;
-                    sc[2 * t + half][e] = v;
-                    mx = fmaxf(mx, v);
-                }
-        }
+            for (int e = 0; e < 4; e++) {
+                const int key = 32 * t + 8 * lq + 4 * half + e;
+                float v = sc[2 * t + half][e] * scale;
+                if (key > qi || !((bits >> (4 * half + e)) & 1)) v = -1e9f;
+                if (key >= seq) v = -INFINITY; /* padding of the last 32-key step: no column of the reference's matrix */
+                sc[2 * t + half][e] = v;
+                mx = fmaxf(mx, v);
+            }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16));
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     float sum = 0.0f;
 #pragma unroll
-    for (int t = 0; t < QW_MAXT; t++) {
-        if (t < nt) {
+    for (int t = 0; t < NT; t++)
 #pragma unroll
-            for (int half = 0; half < 2; half++)
+        for (int half = 0; half < 2; half++)
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const float p = __expf(sc[2 * t + half][e] - mx);
-                    sc[2 * t + half][e] = p;
-                    sum += p;
-                }
-        }
-    }
+            for (int e = 0; e < 4; e++) {
+                const float p = __expf(sc[2 * t + half][e] - mx);
+                sc[2 * t + half][e] = p;
+                sum += p;
+            }
     sum += __shfl_xor(sum, 16);
     sum += __shfl_xor(sum, 32);
     const float inv = 1.0f / sum;
 
     /* O^T[d][q] = sum_key V^T[d][key] P^T[key][q]: A operand = V^T rows (lane: dim l15, keys
      * [32 t + 8 lq, +8)), B operand = this lane's 8 probabilities of step t */
+    auto load_v = [&](bf16x8 (&vf)[8], int t) {
+#pragma unroll
+        for (int d = 0; d < 8; d++) vf[d] = *(const bf16x8 *)(vt + (size_t)(kh * 128 + d * 16 + l15) * ldv + min(32 * t, ldv - 32) + 8 * lq);
+    };
     f32x4 o[8];
 #pragma unroll
     for (int d = 0; d < 8; d++) o[d] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+    bf16x8 vbuf[PD + 1][8];
 #pragma unroll
-    for (int t = 0; t < QW_MAXT; t++) {
-        if (t < nt) {
-            bf16x8 pf;
+    for (int t = 0; t < PD && t < NT; t++) load_v(vbuf[t], t);
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                pf[e] = (bf16)(sc[2 * t][e] * inv);
-                pf[4 + e] = (bf16)(sc[2 * t + 1][e] * inv);
-            }
+    for (int t = 0; t < NT; t++) {
+        if (t + PD < NT) load_v(vbuf[(t + PD) % (PD + 1)], t + PD);
+        bf16x8 pf;
 #pragma unroll
-            for (int d = 0; d < 8; d++) {
-                const bf16x8 vf = *(const bf16x8 *)(vt + (size_t)(kh * 128 + d * 16 + l15) * ldv + 32 * t + 8 * lq);
-                o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[d], 0, 0, 0);
-            }
+        for (int e = 0; e < 4; e++) {
+            pf[e] = (bf16)(sc[2 * t][e] * inv);
+            pf[4 + e] = (bf16)(sc[2 * t + 1][e] * inv);
         }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int d = 0; d < 8; d++) o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vbuf[t % (PD + 1)][d], pf, o[d], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
     }
     /* accumulator element e of block d: query l15, dim 16 d + 4 lq + e */
     if (qi < seq) {
@@ -191,6 +217,22 @@ __global__ __launch_bounds__(64) void qwen3_attention_kernel(bf16 *__restrict__ 
             *(bf16x4 *)(op + d * 16) = ov;
         }
     }
+}
+
+/* Steps whose 32 keys all lie after the block's last query hold no admissible key and are left
+ * out - unless the first key is masked: only then can a row have no admissible key at all, and such
+ * a row is uniform over every column (see above), so every step is computed. The step count is
+ * rounded up to one of four compiled bodies. */
+__global__ __launch_bounds__(64) void qwen3_attention_kernel(bf16 *__restrict__ out, const bf16 *__restrict__ qkv, const bf16 *__restrict__ vt,
+                                                             int ldv, const int *__restrict__ mask, int seq, int heads, int kv_heads) {
+    const int all = (seq + 31) >> 5;
+    const bool first_masked = mask && mask[0] == 0;
+    const int need = first_masked ? all : min(all, ((blockIdx.x * 16 + 15) >> 5) + 1);
+    if (need <= 2) qwen3_attend<2>(out, qkv, vt, ldv, mask, seq, heads, kv_heads);
+    else if (need <= 4) qwen3_attend<4>(out, qkv, vt, ldv, mask, seq, heads, kv_heads);
+    else if (need <= 8) qwen3_attend<8>(out, qkv, vt, ldv, mask, seq, heads, kv_heads);
+    else if (need <= 12) qwen3_attend<12>(out, qkv, vt, ldv, mask, seq, heads, kv_heads);
+    else qwen3_attend<16>(out, qkv, vt, ldv, mask, seq, heads, kv_heads);
 }
 
 /* dst[s, col0 + i] = src[s, i]: one layer's hidden state into its third of the output rows */
