@@ -200,3 +200,135 @@ def test_reference_pipeline_with_the_device_vae(oracle_mod, tmp_path):
     assert want.std() > 5.0
     assert diff.mean() <= 20.0                   # the reference's own acceptance threshold
     assert diff.mean() <= 1.5 and diff.max() <= 12
+
+
+PIPE_GPUALL = os.path.join(ROOT, "oracle", "_ref", "libfluxpipe_gpuall.so")
+
+_CHILD_PROMPT = r"""
+import ctypes, sys, os
+import numpy as np
+lib, model_dir, out = sys.argv[1:4]
+width, height, steps, seed = [int(a) for a in sys.argv[4:8]]
+prompt = sys.argv[8]
+vp, c_i, c_f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+class FluxParams(ctypes.Structure):
+    _fields_ = [("width", c_i), ("height", c_i), ("num_steps", c_i), ("seed", ctypes.c_int64), ("guidance", c_f),
+                ("linear_schedule", c_i), ("power_schedule", c_i), ("power_alpha", c_f)]
+class FluxImage(ctypes.Structure):
+    _fields_ = [("width", c_i), ("height", c_i), ("channels", c_i), ("data", ctypes.POINTER(ctypes.c_uint8))]
+P = ctypes.CDLL(lib, mode=ctypes.RTLD_GLOBAL)
+P.flux_load_dir.restype = vp
+P.flux_load_dir.argtypes = [ctypes.c_char_p]
+P.flux_get_error.restype = ctypes.c_char_p
+P.flux_generate.restype = vp
+P.flux_generate.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(FluxParams)]
+P.flux_image_free.argtypes = [vp]
+P.flux_free.argtypes = [vp]
+layers = []
+CB = ctypes.CFUNCTYPE(None, c_i, c_i)
+cb = CB(lambda l, t: layers.append((l, t)))
+ctypes.c_void_p.in_dll(P, "flux_text_progress_callback").value = ctypes.cast(cb, vp).value
+ctx = P.flux_load_dir(model_dir.encode())
+assert ctx, P.flux_get_error()
+prm = FluxParams(width, height, steps, seed, 0.0, 0, 0, 2.0)
+img_p = P.flux_generate(ctx, prompt.encode(), ctypes.byref(prm))
+assert img_p, P.flux_get_error()
+im = ctypes.cast(img_p, ctypes.POINTER(FluxImage)).contents
+np.save(out, np.ctypeslib.as_array(im.data, shape=(im.height, im.width, im.channels)).copy())
+P.flux_image_free(img_p)
+P.flux_free(ctx)
+assert layers and layers[0] == (0, 27) and layers[-1] == (26, 27), layers[:3]
+print("child ok", len(layers))
+"""
+
+
+def _byte_level_tokenizer_json():
+    """A tokenizer.json the reference's loader accepts (flux_qwen3_tokenizer.c:317-560): the 256 byte-level
+    symbols of the GPT-2 alphabet as the vocabulary, no merges, no added tokens - every byte is one token."""
+    import json
+    bs = list(range(33, 127)) + list(range(161, 173)) + list(range(174, 256))
+    cs = bs[:]
+    n = 0
+    for b in range(256):
+        if b not in bs:
+            bs.append(b)
+            cs.append(256 + n)
+            n += 1
+    vocab = {chr(c): b for b, c in zip(bs, cs)}
+    return json.dumps({"model": {"vocab": vocab, "merges": []}, "added_tokens": []}, ensure_ascii=False)
+
+
+@pytest.mark.skipif(not (os.path.exists(PIPE_GPUALL) and os.path.exists(REF)), reason="reference-built libraries not present")
+@pytest.mark.parametrize("distilled", [True, False])
+def test_prompt_to_image_with_all_stages_on_the_device(oracle_mod, tmp_path, distilled):
+    """flux_generate(ctx, prompt) through the reference's flux.c: its tokenizer on the CPU, then text encoder,
+    denoising loop (Euler, or CFG with the empty prompt for a non-distilled model) and VAE decoder on the
+    device. Expected image: the reference's tokenizer, then the CPU oracles of the three stages."""
+    import subprocess
+    import sys
+    from dataclasses import replace
+    from model_spec import QwenConfig, make_qwen3_weights
+    cfg = SMALL
+    qcfg = QwenConfig(hidden=cfg.text_dim // 3, intermediate=384, heads=4, kv_heads=2, layers=27, vocab=151936)
+    W, VW, QW = make_weights(cfg, 42, 0.05, "sharp"), make_vae_weights(), make_qwen3_weights(qcfg)
+    for d in ("transformer", "vae", "text_encoder", "tokenizer"):
+        os.makedirs(tmp_path / d)
+    write_safetensors(str(tmp_path / "transformer" / "diffusion_pytorch_model.safetensors"), W)
+    write_safetensors(str(tmp_path / "vae" / "diffusion_pytorch_model.safetensors"), VW)
+    names = list(QW)
+    half = len(names) // 2
+    write_safetensors(str(tmp_path / "text_encoder" / "model-00001-of-00002.safetensors"), {n: QW[n] for n in names[:half]})
+    write_safetensors(str(tmp_path / "text_encoder" / "model-00002-of-00002.safetensors"), {n: QW[n] for n in names[half:]})
+    (tmp_path / "tokenizer" / "tokenizer.json").write_text(_byte_level_tokenizer_json(), encoding="utf-8")
+    (tmp_path / "model_index.json").write_text('{"is_distilled": true}' if distilled else '{"_class_name": "Flux2Pipeline"}')
+    width, height, steps, seed, prompt = 64, 64, 3, 21, "a small red fox"
+    out = str(tmp_path / "img.npy")
+    r = subprocess.run([sys.executable, "-c", _CHILD_PROMPT, PIPE_GPUALL, str(tmp_path), out,
+                        str(width), str(height), str(steps), str(seed), prompt], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0, r.stdout + r.stderr
+    got = np.load(out)
+
+    # expected, on the CPU: the reference's tokenizer ...
+    R = ctypes.CDLL(REF)
+    R.qwen3_tokenizer_load.restype = vp
+    R.qwen3_tokenizer_load.argtypes = [ctypes.c_char_p]
+    R.qwen3_tokenize_chat.restype = ctypes.POINTER(c_i)
+    R.qwen3_tokenize_chat.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(c_i), c_i]
+    R.qwen3_tokenizer_free.argtypes = [vp]
+    tok = R.qwen3_tokenizer_load(str(tmp_path / "tokenizer" / "tokenizer.json").encode())
+    assert tok
+
+    def encode(text, q):
+        n = c_i(0)
+        p = R.qwen3_tokenize_chat(tok, text.encode(), ctypes.byref(n), 512)
+        ids = np.full(512, 151643, np.int32)                 # padded with <|endoftext|> (flux_qwen3_tokenizer.c:1059-1075)
+        ids[:n.value] = np.ctypeslib.as_array(p, shape=(n.value,))
+        mask = np.zeros(512, np.int32)
+        mask[:n.value] = 1
+        assert 10 < n.value < 64
+        return q.forward(ids, mask)
+
+    # ... then the three oracles
+    q = oracle_mod.Qwen3Oracle(qcfg, QW)
+    emb = encode(prompt, q)
+    emb_u = None if distilled else encode("", q)
+    q.close()
+    R.qwen3_tokenizer_free(tok)
+    lh, lw = height // 16, width // 16
+    o = oracle_mod.Oracle(cfg, W)
+    z0 = oracle_mod.init_noise(cfg.channels, lh, lw, seed)
+    sched = oracle_mod.official_schedule(steps, lh * lw)
+    if distilled:
+        latent = o.sample_euler(z0, lh, lw, emb, sched)
+    else:
+        latent = o.sample_euler_cfg(z0, lh, lw, emb, emb_u, 4.0, sched)    # default guidance of a base model, flux.c:222
+    o.close()
+    vo = oracle_mod.VaeOracle(VW)
+    _, want = vo.decode(latent, lh, lw)
+    vo.close()
+    diff = np.abs(got.astype(np.int32) - want.astype(np.int32))
+    print(f"prompt -> image, all stages on the device (distilled={distilled}): mean abs diff {diff.mean():.3f}, max {diff.max()}, "
+          f"image std {want.std():.1f}", flush=True)
+    assert got.shape == (height, width, 3) and want.std() > 5.0
+    assert diff.mean() <= 20.0                   # the reference's own acceptance threshold
+    assert diff.mean() <= 2.0
