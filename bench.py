@@ -281,6 +281,8 @@ def main():
     ap.add_argument("--no-kernel-timing", action="store_true")
     ap.add_argument("--tile-mask", type=lambda v: int(v, 0), default=0,
                     help="restrict the GEMM tiles the backend may choose (bit t = tile id t), for A/B runs")
+    ap.add_argument("--sequential-cfg", action="store_true",
+                    help="run the two forwards of a CFG step one after the other instead of as one batch (A/B runs)")
     ap.add_argument("--calibrate", action="store_true",
                     help="launch only a streaming kernel of known size (f32->bf16 over 64 Mi elements: reads 256 MiB, "
                          "writes 128 MiB) and the dominant GEMM, for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
@@ -319,6 +321,8 @@ def main():
     fluxhip.init()
     if args.tile_mask:
         fluxhip.lib().flux_hip_linear_tile_mask(args.tile_mask)
+    if args.sequential_cfg:
+        fluxhip.lib().flux_hip_set_batched_cfg(0)
     model = load_model(cfg)
     z = normal_f32((cfg.channels, h, w), 123, 1)
     txt = normal_f32((nt, cfg.text_dim), 123, 2)

@@ -206,11 +206,16 @@ static int upload_ref_tokens(flux_transformer_t *tf, int n_target, const flux_re
     return 1;
 }
 
+/* CFG steps run their two forwards as one batch of two sequences unless this is switched off
+ * (comparison runs). */
+static int g_batched_cfg = 1;
+void flux_hip_set_batched_cfg(int on) { g_batched_cfg = on != 0; }
+
 /* Device-resident state of one sampling run. */
 struct flux_hip_session {
     flux_transformer_t *tf;
     fh_rope *rp_c, *rp_u;
-    int cfg, n_target, num_steps, next_forward, h, w;
+    int cfg, batched, n_target, num_steps, next_forward, h, w;
     size_t n_lat;
     float guidance;
     float *schedule;
@@ -249,7 +254,7 @@ flux_hip_session *flux_hip_session_begin(void *transformer, const float *z, int 
     if (!s) { flux_hip_fail("out of host memory"); return NULL; }
     tf->session_active = 1;
     s->owns_tf = 1;
-    s->tf = tf; s->cfg = cfg; s->n_target = h * w; s->num_steps = num_steps; s->guidance = guidance_scale;
+    s->tf = tf; s->cfg = cfg; s->batched = cfg && g_batched_cfg; s->n_target = h * w; s->num_steps = num_steps; s->guidance = guidance_scale;
     s->h = h; s->w = w;
     s->n_lat = (size_t)channels * s->n_target;
     s->schedule = (float *)malloc((num_steps + 1) * sizeof(float));
@@ -265,7 +270,7 @@ flux_hip_session *flux_hip_session_begin(void *transformer, const float *z, int 
         /* the table cache may have recycled the first slot */
         s->rp_c = fh_get_rope(tf, text_seq_cond, h, w, refs, num_refs);
         if (!s->rp_c) goto fail;
-        if (s->rp_u->n > max_tokens) max_tokens = s->rp_u->n;
+        max_tokens = s->batched ? max_tokens + s->rp_u->n : (s->rp_u->n > max_tokens ? s->rp_u->n : max_tokens);
     }
     if (!fh_ensure_workspace(tf, max_tokens)) goto fail;
     if (num_steps > 0 && !fh_compute_modulation(tf, schedule, num_steps)) goto fail;
@@ -292,12 +297,21 @@ int flux_hip_session_step(flux_hip_session *s, int step, float *v_trace) {
     const float dt = s->schedule[step + 1] - s->schedule[step];
     const size_t n = s->n_lat;
     if (flux_step_callback) flux_step_callback(step + 1, s->num_steps);
-    if (s->cfg) {
+    if (s->batched) {
+        /* the unconditional and the conditional pass (flux_sample.c:485-493) as one batch of two sequences */
+        const fh_rope *rp[2] = {s->rp_u, s->rp_c};
+        const void *txt[2] = {s->txt_u, s->txt_c};
+        float *v[2] = {s->v_u, s->v_c};
+        if (!fh_forward_device_n(tf, 2, rp, s->z_dev, s->n_target, txt, step, v, s->ev)) return 0;
+        if (s->ev) s->ev->used++;
+    } else if (s->cfg) {
         /* unconditional first, then conditional (flux_sample.c:485-493) */
         if (!fh_forward_device(tf, s->rp_u, s->z_dev, s->n_target, s->txt_u, step, s->v_u, s->ev)) return 0;
         if (s->ev) s->ev->used++;
         if (!fh_forward_device(tf, s->rp_c, s->z_dev, s->n_target, s->txt_c, step, s->v_c, s->ev)) return 0;
         if (s->ev) s->ev->used++;
+    }
+    if (s->cfg) {
         if (v_trace) {
             if (!flux_hip_download(v_trace, s->v_u, n * 4)) return 0;
             if (!flux_hip_download(v_trace + n, s->v_c, n * 4)) return 0;

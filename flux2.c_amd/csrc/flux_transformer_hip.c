@@ -200,7 +200,7 @@ int fh_ensure_workspace(flux_transformer_t *tf, int tokens) {
     tf->xn = flux_hip_malloc(n * H * 2);
     tf->qkv = flux_hip_malloc(n * 3 * H * 2);
     tf->kn = flux_hip_malloc(n * H * 2);
-    tf->vt = flux_hip_malloc(H * npad * 2);
+    tf->vt = flux_hip_malloc(H * (npad + 64) * 2); /* two sequences pad their key counts to 64 separately */
     tf->cat = flux_hip_malloc(n * (H + M) * 2);
     tf->tok = flux_hip_malloc(n * tf->c.channels * 2);
     if (!tf->x || !tf->xn || !tf->qkv || !tf->kn || !tf->vt || !tf->cat || !tf->tok) {
@@ -335,85 +335,120 @@ static int linear1(int epi, const void *A, const void *W, void *C, const float *
 }
 
 /*
- * One velocity prediction, entirely on the device.
- *   z_dev   fp32 [channels, img_h*img_w] target latent
- *   txt_dev bf16 [txt_seq, text_dim]
+ * One velocity prediction per sequence, entirely on the device, for nb = 1 or 2 sequences that
+ * share the target latent, the reference tokens and the timestep (the unconditional and the
+ * conditional pass of a CFG step; the reference runs them one after the other,
+ * flux_sample.c:485-493). Rows are laid out sequence after sequence, each as
+ * [text ; target ; refs], so every GEMM of the single-stream blocks sees all rows of both
+ * sequences as one matrix (each weight matrix is streamed once per step instead of twice, and the
+ * launch has twice the tiles), the double-stream GEMMs run as 2 nb row ranges, and only attention
+ * and its K/V preparation run per sequence.
+ *   z_dev      fp32 [channels, img_h*img_w] target latent
+ *   txt_dev[b] bf16 [txt_seq_b, text_dim]
  *   tf->tok rows [n_target, n_img) must already hold the reference tokens (bf16)
- *   v_dev   fp32 [channels, img_h*img_w] output
+ *   v_dev[b]   fp32 [channels, img_h*img_w] outputs
  * Mirrors flux_transformer_forward (flux_transformer.c:3115-3577) and the refs variants.
  */
-int fh_forward_device(flux_transformer_t *tf, const fh_rope *rp, const float *z_dev, int n_target,
-                      const void *txt_dev, int step, float *v_dev, fh_events *ev) {
+int fh_forward_device_n(flux_transformer_t *tf, int nb, const fh_rope *const *rp, const float *z_dev, int n_target,
+                        const void *const *txt_dev, int step, float *const *v_dev, fh_events *ev) {
     const flux_hip_config *c = &tf->c;
     const int H = c->hidden, M = c->mlp, C = c->channels, heads = c->heads;
-    const int Nt = rp->txt_seq, Ni = rp->n_img, N = rp->n;
-    const int ldcat = H + M, ldvt = (N + 63) / 64 * 64;
+    const int ldcat = H + M;
     const float eps = 1e-6f;
-    char *xn = (char *)tf->xn, *qkv = (char *)tf->qkv, *cat = (char *)tf->cat;
+    if (nb < 1 || nb > 2) return flux_hip_fail("forward: %d sequences (1 or 2)", nb);
+    int R[2] = {0, 0}, Nt[2] = {0, 0}, N[2] = {0, 0}, ldvt[2] = {0, 0}, Ntot = 0;
+    size_t vt_off[2] = {0, 0};
+    const int Ni = rp[0]->n_img;
+    for (int b = 0; b < nb; b++) {
+        if (rp[b]->n_img != Ni) return flux_hip_fail("forward: sequences differ in image tokens");
+        R[b] = Ntot; Nt[b] = rp[b]->txt_seq; N[b] = rp[b]->n;
+        ldvt[b] = (N[b] + 63) / 64 * 64;
+        vt_off[b] = b ? vt_off[b - 1] + (size_t)H * ldvt[b - 1] * 2 : 0;
+        Ntot += N[b];
+    }
+    if (Ntot > tf->cap_tokens) return flux_hip_fail("forward: work buffers hold %d tokens, %d needed", tf->cap_tokens, Ntot);
+    char *xn = (char *)tf->xn, *qkv = (char *)tf->qkv, *cat = (char *)tf->cat, *kn = (char *)tf->kn, *vt = (char *)tf->vt;
     float *x = tf->x;
     const float *mt = mod_ptr(tf, 0, step), *mi = mod_ptr(tf, 1, step), *ms = mod_ptr(tf, 2, step), *mf = mod_ptr(tf, 3, step);
+    flux_hip_linear_part p[4];
 
     if (ev) fh_event_record(ev, 0);
     /* inputs -> hidden (flux_transformer.c:3156-3196) */
     if (!flux_hip_latent_to_tokens(tf->tok, z_dev, C, n_target)) return 0;
-    if (!linear1(FLUX_HIP_EPI_F32, tf->tok, tf->img_in, x + (size_t)Nt * H, NULL, Ni, H, C, C, C, H, 0, 0)) return 0;
-    if (!linear1(FLUX_HIP_EPI_F32, txt_dev, tf->txt_in, x, NULL, Nt, H, c->text_dim, c->text_dim, c->text_dim, H, 0, 0)) return 0;
+    for (int b = 0; b < nb; b++) p[b] = (flux_hip_linear_part){tf->tok, tf->img_in, x + (size_t)(R[b] + Nt[b]) * H, NULL, Ni};
+    if (!flux_hip_linear(FLUX_HIP_EPI_F32, nb, p, H, C, C, C, H, 0, 0)) return 0;
+    for (int b = 0; b < nb; b++) p[b] = (flux_hip_linear_part){txt_dev[b], tf->txt_in, x + (size_t)R[b] * H, NULL, Nt[b]};
+    if (!flux_hip_linear(FLUX_HIP_EPI_F32, nb, p, H, c->text_dim, c->text_dim, c->text_dim, H, 0, 0)) return 0;
 
-    /* double-stream blocks (flux_transformer.c:1774-1986); part 0 = text rows, part 1 = image rows */
+    /* double-stream blocks (flux_transformer.c:1774-1986); per sequence: text rows, then image rows */
     for (int i = 0; i < c->n_double; i++) {
-        const fh_double *b = &tf->dbl[i];
-        if (!flux_hip_adaln_norm(xn, H, x, N, H, Nt, mt, mt + H, mi, mi + H, eps)) return 0;
-        {
-            flux_hip_linear_part p[2] = {
-                {xn, b->qkv[0], qkv, NULL, Nt},
-                {xn + (size_t)Nt * H * 2, b->qkv[1], qkv + (size_t)Nt * 3 * H * 2, NULL, Ni}};
-            if (!flux_hip_linear(FLUX_HIP_EPI_BF16, 2, p, 3 * H, H, H, H, 3 * H, 0, 0)) return 0;
+        const fh_double *blk = &tf->dbl[i];
+        for (int b = 0; b < nb; b++)
+            if (!flux_hip_adaln_norm(xn + (size_t)R[b] * H * 2, H, x + (size_t)R[b] * H, N[b], H, Nt[b], mt, mt + H, mi, mi + H, eps)) return 0;
+        for (int b = 0; b < nb; b++) {
+            p[2 * b] = (flux_hip_linear_part){xn + (size_t)R[b] * H * 2, blk->qkv[0], qkv + (size_t)R[b] * 3 * H * 2, NULL, Nt[b]};
+            p[2 * b + 1] = (flux_hip_linear_part){xn + (size_t)(R[b] + Nt[b]) * H * 2, blk->qkv[1], qkv + (size_t)(R[b] + Nt[b]) * 3 * H * 2, NULL, Ni};
         }
-        if (!flux_hip_kv_prepare(tf->kn, tf->vt, ldvt, qkv, 3 * H, H, 2 * H, N, heads, Nt, b->norm_k[0], b->norm_k[1],
-                                 rp->cos, rp->sin, eps)) return 0;
-        if (!flux_hip_attention(cat, ldcat, qkv, 3 * H, tf->kn, tf->vt, ldvt, N, N, heads, Nt, b->norm_q[0], b->norm_q[1],
-                                rp->cos, rp->sin, eps)) return 0;
-        {
-            flux_hip_linear_part p[2] = {
-                {cat, b->proj[0], x, mt + 2 * H, Nt},
-                {cat + (size_t)Nt * ldcat * 2, b->proj[1], x + (size_t)Nt * H, mi + 2 * H, Ni}};
-            if (!flux_hip_linear(FLUX_HIP_EPI_RESID, 2, p, H, H, ldcat, H, H, 0, 0)) return 0;
+        if (!flux_hip_linear(FLUX_HIP_EPI_BF16, 2 * nb, p, 3 * H, H, H, H, 3 * H, 0, 0)) return 0;
+        for (int b = 0; b < nb; b++) {
+            const char *q_b = qkv + (size_t)R[b] * 3 * H * 2;
+            if (!flux_hip_kv_prepare(kn + (size_t)R[b] * H * 2, vt + vt_off[b], ldvt[b], q_b, 3 * H, H, 2 * H, N[b], heads, Nt[b], blk->norm_k[0],
+                                     blk->norm_k[1], rp[b]->cos, rp[b]->sin, eps)) return 0;
+            if (!flux_hip_attention(cat + (size_t)R[b] * ldcat * 2, ldcat, q_b, 3 * H, kn + (size_t)R[b] * H * 2, vt + vt_off[b], ldvt[b], N[b], N[b],
+                                    heads, Nt[b], blk->norm_q[0], blk->norm_q[1], rp[b]->cos, rp[b]->sin, eps)) return 0;
         }
-        if (!flux_hip_adaln_norm(xn, H, x, N, H, Nt, mt + 3 * H, mt + 4 * H, mi + 3 * H, mi + 4 * H, eps)) return 0;
-        {
-            /* linear_in rows are [gate ; up] (flux_transformer.c:4503-4523) */
-            flux_hip_linear_part p[2] = {
-                {xn, b->ff_in[0], cat + (size_t)H * 2, NULL, Nt},
-                {xn + (size_t)Nt * H * 2, b->ff_in[1], cat + ((size_t)Nt * ldcat + H) * 2, NULL, Ni}};
-            if (!flux_hip_linear(FLUX_HIP_EPI_SWIGLU, 2, p, 2 * M, H, H, H, ldcat, 0, M)) return 0;
+        for (int b = 0; b < nb; b++) {
+            p[2 * b] = (flux_hip_linear_part){cat + (size_t)R[b] * ldcat * 2, blk->proj[0], x + (size_t)R[b] * H, mt + 2 * H, Nt[b]};
+            p[2 * b + 1] = (flux_hip_linear_part){cat + (size_t)(R[b] + Nt[b]) * ldcat * 2, blk->proj[1], x + (size_t)(R[b] + Nt[b]) * H, mi + 2 * H, Ni};
         }
-        {
-            flux_hip_linear_part p[2] = {
-                {cat + (size_t)H * 2, b->ff_out[0], x, mt + 5 * H, Nt},
-                {cat + ((size_t)Nt * ldcat + H) * 2, b->ff_out[1], x + (size_t)Nt * H, mi + 5 * H, Ni}};
-            if (!flux_hip_linear(FLUX_HIP_EPI_RESID, 2, p, H, M, ldcat, M, H, 0, 0)) return 0;
+        if (!flux_hip_linear(FLUX_HIP_EPI_RESID, 2 * nb, p, H, H, ldcat, H, H, 0, 0)) return 0;
+        for (int b = 0; b < nb; b++)
+            if (!flux_hip_adaln_norm(xn + (size_t)R[b] * H * 2, H, x + (size_t)R[b] * H, N[b], H, Nt[b], mt + 3 * H, mt + 4 * H, mi + 3 * H, mi + 4 * H, eps)) return 0;
+        /* linear_in rows are [gate ; up] (flux_transformer.c:4503-4523) */
+        for (int b = 0; b < nb; b++) {
+            p[2 * b] = (flux_hip_linear_part){xn + (size_t)R[b] * H * 2, blk->ff_in[0], cat + ((size_t)R[b] * ldcat + H) * 2, NULL, Nt[b]};
+            p[2 * b + 1] = (flux_hip_linear_part){xn + (size_t)(R[b] + Nt[b]) * H * 2, blk->ff_in[1], cat + ((size_t)(R[b] + Nt[b]) * ldcat + H) * 2, NULL, Ni};
         }
+        if (!flux_hip_linear(FLUX_HIP_EPI_SWIGLU, 2 * nb, p, 2 * M, H, H, H, ldcat, 0, M)) return 0;
+        for (int b = 0; b < nb; b++) {
+            p[2 * b] = (flux_hip_linear_part){cat + ((size_t)R[b] * ldcat + H) * 2, blk->ff_out[0], x + (size_t)R[b] * H, mt + 5 * H, Nt[b]};
+            p[2 * b + 1] = (flux_hip_linear_part){cat + ((size_t)(R[b] + Nt[b]) * ldcat + H) * 2, blk->ff_out[1], x + (size_t)(R[b] + Nt[b]) * H, mi + 5 * H, Ni};
+        }
+        if (!flux_hip_linear(FLUX_HIP_EPI_RESID, 2 * nb, p, H, M, ldcat, M, H, 0, 0)) return 0;
         if (flux_substep_callback) flux_substep_callback(FLUX_SUBSTEP_DOUBLE_BLOCK, i, c->n_double);
     }
     if (ev) fh_event_record(ev, 1);
 
-    /* single-stream blocks (flux_transformer.c:2992-3109): fused rows [Q | K | V | gate | up] */
+    /* single-stream blocks (flux_transformer.c:2992-3109): fused rows [Q | K | V | gate | up]; all rows of all sequences at once */
     for (int i = 0; i < c->n_single; i++) {
-        const fh_single *b = &tf->sgl[i];
-        if (!flux_hip_adaln_norm(xn, H, x, N, H, N, ms, ms + H, NULL, NULL, eps)) return 0;
-        if (!linear1(FLUX_HIP_EPI_BF16, xn, b->qkv_mlp, qkv, NULL, N, 3 * H, H, H, H, 3 * H, 0, 0)) return 0;
-        if (!linear1(FLUX_HIP_EPI_SWIGLU, xn, b->qkv_mlp, cat + (size_t)H * 2, NULL, N, 2 * M, H, H, H, ldcat, 3 * H, 3 * H + M)) return 0;
-        if (!flux_hip_kv_prepare(tf->kn, tf->vt, ldvt, qkv, 3 * H, H, 2 * H, N, heads, N, b->norm_k, NULL, rp->cos, rp->sin, eps)) return 0;
-        if (!flux_hip_attention(cat, ldcat, qkv, 3 * H, tf->kn, tf->vt, ldvt, N, N, heads, N, b->norm_q, NULL, rp->cos, rp->sin, eps)) return 0;
-        if (!linear1(FLUX_HIP_EPI_RESID, cat, b->out, x, ms + 2 * H, N, H, H + M, ldcat, H + M, H, 0, 0)) return 0;
+        const fh_single *blk = &tf->sgl[i];
+        if (!flux_hip_adaln_norm(xn, H, x, Ntot, H, Ntot, ms, ms + H, NULL, NULL, eps)) return 0;
+        if (!linear1(FLUX_HIP_EPI_BF16, xn, blk->qkv_mlp, qkv, NULL, Ntot, 3 * H, H, H, H, 3 * H, 0, 0)) return 0;
+        if (!linear1(FLUX_HIP_EPI_SWIGLU, xn, blk->qkv_mlp, cat + (size_t)H * 2, NULL, Ntot, 2 * M, H, H, H, ldcat, 3 * H, 3 * H + M)) return 0;
+        for (int b = 0; b < nb; b++) {
+            const char *q_b = qkv + (size_t)R[b] * 3 * H * 2;
+            if (!flux_hip_kv_prepare(kn + (size_t)R[b] * H * 2, vt + vt_off[b], ldvt[b], q_b, 3 * H, H, 2 * H, N[b], heads, N[b], blk->norm_k, NULL,
+                                     rp[b]->cos, rp[b]->sin, eps)) return 0;
+            if (!flux_hip_attention(cat + (size_t)R[b] * ldcat * 2, ldcat, q_b, 3 * H, kn + (size_t)R[b] * H * 2, vt + vt_off[b], ldvt[b], N[b], N[b],
+                                    heads, N[b], blk->norm_q, NULL, rp[b]->cos, rp[b]->sin, eps)) return 0;
+        }
+        if (!linear1(FLUX_HIP_EPI_RESID, cat, blk->out, x, ms + 2 * H, Ntot, H, H + M, ldcat, H + M, H, 0, 0)) return 0;
         if (flux_substep_callback) flux_substep_callback(FLUX_SUBSTEP_SINGLE_BLOCK, i, c->n_single);
     }
     if (ev) fh_event_record(ev, 2);
 
     /* final layer on the target rows; modulation chunks are (scale, shift) (flux_transformer.c:3532-3534) */
-    if (!flux_hip_adaln_norm(xn, H, x + (size_t)Nt * H, n_target, H, n_target, mf + H, mf, NULL, NULL, eps)) return 0;
-    if (!linear1(FLUX_HIP_EPI_F32_T, xn, tf->proj_out, v_dev, NULL, n_target, C, H, H, H, n_target, 0, 0)) return 0;
+    for (int b = 0; b < nb; b++) {
+        if (!flux_hip_adaln_norm(xn + (size_t)R[b] * H * 2, H, x + (size_t)(R[b] + Nt[b]) * H, n_target, H, n_target, mf + H, mf, NULL, NULL, eps)) return 0;
+        p[b] = (flux_hip_linear_part){xn + (size_t)R[b] * H * 2, tf->proj_out, v_dev[b], NULL, n_target};
+    }
+    if (!flux_hip_linear(FLUX_HIP_EPI_F32_T, nb, p, C, H, H, H, n_target, 0, 0)) return 0;
     if (flux_substep_callback) flux_substep_callback(FLUX_SUBSTEP_FINAL_LAYER, 0, 1);
     if (ev) fh_event_record(ev, 3);
     return 1;
+}
+
+int fh_forward_device(flux_transformer_t *tf, const fh_rope *rp, const float *z_dev, int n_target,
+                      const void *txt_dev, int step, float *v_dev, fh_events *ev) {
+    return fh_forward_device_n(tf, 1, &rp, z_dev, n_target, &txt_dev, step, &v_dev, ev);
 }

@@ -38,19 +38,21 @@
 #include "common.h"
 #include "../../include/flux_hip.h"
 
+#define GEMM_MAX_PARTS 4
 struct GemmArgs {
-    const bf16 *A[2];
-    const bf16 *W[2];
-    void *C[2];
-    const float *gate[2];
-    int M[2];
-    int mtiles0, mtiles, ntiles, total_tiles;
+    const bf16 *A[GEMM_MAX_PARTS];
+    const bf16 *W[GEMM_MAX_PARTS];
+    void *C[GEMM_MAX_PARTS];
+    const float *gate[GEMM_MAX_PARTS];
+    int M[GEMM_MAX_PARTS];
+    int mt_end[GEMM_MAX_PARTS]; /* row tiles of parts 0..i together; unused parts repeat the total */
+    int mtiles, ntiles, total_tiles;
     int N, K, lda, ldw, ldc, w_row0, w_row1;
     /* split-K: workgroup (tile, s) multiplies K-steps [s*kt_per, (s+1)*kt_per) and stores its
      * fp32 partial tile into ws[s][moff[part] + m][n]; a second kernel sums the slices */
     int ksplit, kt_per;
     float *ws;
-    int moff[2], ws_rows;
+    int moff[GEMM_MAX_PARTS], ws_rows;
     /* convolution epilogues (see flux_hip_conv): rows are the positions of a zero-bordered
      * conv_hp x conv_wp image with channels contiguous. With 9 taps K runs tap-major over
      * 9 x cin and K step kt reads the activation rows shifted by its tap's (dy, dx);
@@ -105,8 +107,8 @@ __device__ __forceinline__ bool decode_tile(const GemmArgs &g, TileId &t) {
     int in_grp = logical - grp * per_group;
     t.tm = first_m + in_grp % gsz;
     t.tn = in_grp / gsz;
-    t.prob = t.tm >= g.mtiles0 ? 1 : 0;
-    t.tml = t.prob ? t.tm - g.mtiles0 : t.tm;
+    t.prob = (t.tm >= g.mt_end[0]) + (t.tm >= g.mt_end[1]) + (t.tm >= g.mt_end[2]);
+    t.tml = t.prob ? t.tm - g.mt_end[t.prob - 1] : t.tm;
     return true;
 }
 
@@ -431,6 +433,15 @@ __global__ __launch_bounds__(256) void gemm4w_kernel(GemmArgs g) {
 
 /* ------------------------------------------------------------------ host side */
 
+static void set_row_tiles(GemmArgs &g, int BM) {
+    int end = 0;
+    for (int i = 0; i < GEMM_MAX_PARTS; i++) {
+        end += (g.M[i] + BM - 1) / BM; /* empty parts (M = 0) add nothing */
+        g.mt_end[i] = end;
+    }
+    g.mtiles = end;
+}
+
 template <int BM, int BN, int WGM, int WGN, int EPI>
 static int launch_cfg(GemmArgs &g) {
     constexpr int T = WGM * WGN * 64;
@@ -441,9 +452,7 @@ static int launch_cfg(GemmArgs &g) {
         HIP_OK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
         attr_done = true;
     }
-    g.mtiles0 = (g.M[0] + BM - 1) / BM;
-    int mt1 = g.M[1] > 0 ? (g.M[1] + BM - 1) / BM : 0;
-    g.mtiles = g.mtiles0 + mt1;
+    set_row_tiles(g, BM);
     g.ntiles = g.N / BN;
     g.total_tiles = g.mtiles * g.ntiles;
     int grid = (g.total_tiles * g.ksplit + 7) & ~7;
@@ -461,9 +470,7 @@ static int launch_4w(GemmArgs &g) {
         HIP_OK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
         attr_done = true;
     }
-    g.mtiles0 = (g.M[0] + BM - 1) / BM;
-    int mt1 = g.M[1] > 0 ? (g.M[1] + BM - 1) / BM : 0;
-    g.mtiles = g.mtiles0 + mt1;
+    set_row_tiles(g, BM);
     g.ntiles = g.N / BN;
     g.total_tiles = g.mtiles * g.ntiles;
     int grid = (g.total_tiles * g.ksplit + 7) & ~7;
@@ -506,12 +513,13 @@ template <int EPI>
 __global__ __launch_bounds__(256) void splitk_finish_kernel(GemmArgs g) {
     const int ncols = EPI == FLUX_HIP_EPI_SWIGLU ? g.N >> 1 : g.N;
     const int n4 = ncols >> 2;
-    const size_t total = (size_t)(g.M[0] + g.M[1]) * n4;
+    const size_t total = (size_t)g.ws_rows * n4;
     size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= total) return;
     int row = (int)(idx / n4), n = (int)(idx - (size_t)row * n4) << 2;
-    int prob = row >= g.M[0] ? 1 : 0;
-    int m = prob ? row - g.M[0] : row;
+    /* moff[i] = first workspace row of part i; unused parts start at ws_rows */
+    int prob = (row >= g.moff[1]) + (row >= g.moff[2]) + (row >= g.moff[3]);
+    int m = row - g.moff[prob];
     f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f}, sum2 = {0.0f, 0.0f, 0.0f, 0.0f};
     for (int s = 0; s < g.ksplit; s++) {
         const float *w = g.ws + ((size_t)s * g.ws_rows + g.moff[prob] + m) * g.N + n;
@@ -544,7 +552,7 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(GemmArgs g) {
 template <int EPI>
 static int launch_split(GemmArgs &g, int tile) {
     if (!launch_epi<EPI_PARTIAL>(g, tile)) return 0;
-    const size_t total = (size_t)(g.M[0] + g.M[1]) * ((EPI == FLUX_HIP_EPI_SWIGLU ? g.N >> 1 : g.N) >> 2);
+    const size_t total = (size_t)g.ws_rows * ((EPI == FLUX_HIP_EPI_SWIGLU ? g.N >> 1 : g.N) >> 2);
     hipLaunchKernelGGL(splitk_finish_kernel<EPI>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, flux_hip_stream_handle(), g);
     return hipGetLastError() == hipSuccess ? 1 : flux_hip_fail("split-K reduction launch failed");
 }
@@ -691,9 +699,11 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed) {
     if (best_split > 1) {
         g.kt_per = (kt_total + best_split - 1) / best_split;
         g.ksplit = (kt_total + g.kt_per - 1) / g.kt_per;
-        g.moff[0] = 0;
-        g.moff[1] = g.M[0];
-        g.ws_rows = g.M[0] + g.M[1];
+        g.ws_rows = 0;
+        for (int i = 0; i < GEMM_MAX_PARTS; i++) {
+            g.moff[i] = g.ws_rows;
+            g.ws_rows += g.M[i];
+        }
         if (!ensure_ws((size_t)g.ksplit * g.ws_rows * g.N * sizeof(float))) return 0;
         g.ws = g_ws;
     }
@@ -720,7 +730,7 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed) {
 extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
                                int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1) {
     if (epilogue < FLUX_HIP_EPI_BF16 || epilogue > FLUX_HIP_EPI_SWIGLU) return flux_hip_fail("flux_hip_linear: unknown epilogue %d", epilogue);
-    if (nparts < 1 || nparts > 2) return flux_hip_fail("flux_hip_linear: nparts=%d (1 or 2)", nparts);
+    if (nparts < 1 || nparts > GEMM_MAX_PARTS) return flux_hip_fail("flux_hip_linear: nparts=%d (1 to %d)", nparts, GEMM_MAX_PARTS);
     if (K <= 0 || (K & 63)) return flux_hip_fail("flux_hip_linear: K=%d must be a positive multiple of 64", K);
     if (N <= 0 || (N & 127)) return flux_hip_fail("flux_hip_linear: N=%d must be a positive multiple of 128", N);
     if (lda < K || ldw < K || (lda & 7) || (ldw & 7))

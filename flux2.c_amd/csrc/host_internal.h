@@ -65,6 +65,8 @@ fh_rope *fh_get_rope(flux_transformer_t *tf, int txt_seq, int img_h, int img_w, 
 int fh_compute_modulation(flux_transformer_t *tf, const float *timesteps, int steps);
 int fh_forward_device(flux_transformer_t *tf, const fh_rope *rp, const float *z_dev, int n_target,
                       const void *txt_dev, int step, float *v_dev, fh_events *ev);
+int fh_forward_device_n(flux_transformer_t *tf, int nb, const fh_rope *const *rp, const float *z_dev, int n_target,
+                        const void *const *txt_dev, int step, float *const *v_dev, fh_events *ev);
 int flux_hip_fail(const char *fmt, ...);
 
 /* safetensors access shared by the transformer and VAE loaders (flux_loader_hip.c) */

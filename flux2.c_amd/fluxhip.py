@@ -68,6 +68,7 @@ def lib():
     L.flux_hip_timer_stop.restype = c_f
     L.flux_hip_linear.argtypes = [c_i, c_i, ctypes.POINTER(_Part), c_i, c_i, c_i, c_i, c_i, c_i, c_i]
     L.flux_hip_linear_force_tile.argtypes = [c_i]
+    L.flux_hip_set_batched_cfg.argtypes = [c_i]
     L.flux_hip_linear_enable_splitk.argtypes = [c_i]
     L.flux_hip_attention_force_variant.argtypes = [c_i]
     L.flux_hip_linear_probe.argtypes = [c_i]

@@ -83,8 +83,8 @@ typedef struct {
  * flux_linear_nobias_bf16 (flux_kernels.h:59,66; flux_kernels.c:210-320) and, through the
  * epilogues, gated_add (flux_transformer.c:90), flux_silu + flux_mul_inplace
  * (flux_kernels.c:120,581) and the output transposes (flux_transformer.c:3547-3552).
- * Up to two row ranges with different weights run in one launch (the image and text streams
- * of a double block). K % 64 == 0 and N % 128 == 0 are required.
+ * Up to four row ranges with their own weights run in one launch (the image and text streams
+ * of a double block, for one sequence or for the two sequences of a batched CFG step). K % 64 == 0 and N % 128 == 0 are required.
  * For FLUX_HIP_EPI_SWIGLU, N counts gate+up columns (2*mlp); gate rows start at W row w_row0,
  * up rows at w_row1; the output has N/2 columns. Otherwise W rows [w_row0, w_row0+N) are used.
  */
@@ -406,6 +406,11 @@ float *qwen3_encode_text(void *enc, const char *prompt);
  * step's velocity or, under CFG, the unconditional then the conditional one); read_latent()
  * waits and copies the current latent out. The samplers above are built from these.
  */
+/* A CFG step's unconditional and conditional forwards run as one batch of two sequences (each weight
+ * matrix streamed once, twice the rows per GEMM); 0 switches back to two separate forwards, the
+ * reference's order (flux_sample.c:485-493). Takes effect at the next session_begin. */
+void flux_hip_set_batched_cfg(int on);
+
 typedef struct flux_hip_session flux_hip_session;
 flux_hip_session *flux_hip_session_begin(void *transformer, const float *z, int channels, int h, int w,
                                          const flux_ref_t *refs, int num_refs,

@@ -102,6 +102,35 @@ def test_sampler_trace_and_latent(hip, oracle_mod):
     m.close(); o.close()
 
 
+def test_batched_cfg_equals_two_forwards(hip, oracle_mod):
+    """A CFG step runs its unconditional and conditional forwards as one batch of two sequences (the default)
+    or one after the other: same velocities up to GEMM tile/summation-order noise, and both within the gate
+    of the oracle. Text lengths differ, and there are reference images, so every row offset is exercised."""
+    cfg = SMALL
+    W = make_weights(cfg, 42, 0.02, "sharp")
+    o = oracle_mod.Oracle(cfg, W)
+    m = hip.Transformer(cfg, W)
+    h, w = 5, 7
+    z = normal_f32((cfg.channels, h, w), 14, 1)
+    txt = normal_f32((40, cfg.text_dim), 14, 2)
+    txt_u = normal_f32((23, cfg.text_dim), 14, 3)
+    refs = [(normal_f32((cfg.channels, 3, 4), 14, 4), 3, 4, 10), (normal_f32((cfg.channels, 2, 5), 14, 5), 2, 5, 20)]
+    s = hip.schedule("official", 3, h * w)
+    zo, vo = o.sample_euler_cfg(z, h, w, txt, txt_u, 3.5, s, refs=refs, trace=True)
+    out = {}
+    for on in (1, 0):
+        hip.lib().flux_hip_set_batched_cfg(on)
+        out[on] = m.sample(z, h, w, txt, s, refs=refs, txt_uncond=txt_u, guidance=3.5, trace=True)
+    hip.lib().flux_hip_set_batched_cfg(1)
+    for on in (1, 0):
+        zg, vg = out[on]
+        for i in range(6):
+            gate(vg[i], vo[i], f"cfg forward {i} (batched={on})")
+        assert psnr(zg, zo) >= PSNR_MIN
+    assert rel_l2(out[1][1], out[0][1]) < 2e-3
+    m.close(); o.close()
+
+
 def test_broken_rope_would_be_caught(hip, oracle_mod):
     """Sensitivity check: against an oracle whose image RoPE is mirrored the gate must fail,
     otherwise the sharp fixture would say nothing about RoPE in the HIP kernels."""
