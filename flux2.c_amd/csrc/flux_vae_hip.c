@@ -56,8 +56,8 @@ struct flux_hip_vae {
     vslot *slots;
     int nslots, cap_slots;
     /* work buffers, grown on demand */
-    size_t f32_elems, bf16_elems, guard, att_ld, att_chunk, gn_floats, lat_elems, img_pixels;
-    float *X, *Y, *Hb, *S, *kbias, *gn, *lat, *img_f32;
+    size_t f32_elems, bf16_elems, guard, att_ld, att_chunk, gn_floats, lat_elems, img_pixels, st_floats;
+    float *X, *Y, *Hb, *S, *kbias, *gn, *lat, *img_f32, *st_x, *st_h;
     void *A_base, *R, *P, *VT;
     uint8_t *img_u8;
 };
@@ -256,11 +256,11 @@ static void free_res(vres *r) {
 static void free_work(flux_hip_vae *v) {
     flux_hip_free(v->X); flux_hip_free(v->Y); flux_hip_free(v->Hb); flux_hip_free(v->S); flux_hip_free(v->kbias);
     flux_hip_free(v->gn); flux_hip_free(v->lat); flux_hip_free(v->img_f32); flux_hip_free(v->A_base); flux_hip_free(v->R);
-    flux_hip_free(v->P); flux_hip_free(v->VT); flux_hip_free(v->img_u8);
-    v->X = v->Y = v->Hb = v->S = v->kbias = v->gn = v->lat = v->img_f32 = NULL;
+    flux_hip_free(v->P); flux_hip_free(v->VT); flux_hip_free(v->img_u8); flux_hip_free(v->st_x); flux_hip_free(v->st_h);
+    v->X = v->Y = v->Hb = v->S = v->kbias = v->gn = v->lat = v->img_f32 = v->st_x = v->st_h = NULL;
     v->A_base = v->R = v->P = v->VT = NULL;
     v->img_u8 = NULL;
-    v->f32_elems = v->bf16_elems = v->guard = v->att_ld = v->att_chunk = v->gn_floats = v->lat_elems = v->img_pixels = 0;
+    v->f32_elems = v->bf16_elems = v->guard = v->att_ld = v->att_chunk = v->gn_floats = v->lat_elems = v->img_pixels = v->st_floats = 0;
 }
 
 void flux_hip_vae_free(flux_hip_vae *v) {
@@ -291,8 +291,9 @@ static int ensure_work(flux_hip_vae *v, int h, int w) {
     if (chunk < 128) chunk = 128;
     if (chunk > mpm) chunk = mpm;
     const size_t gn_floats = flux_hip_group_norm_scratch_floats((int)hp0, (int)wp0);
+    const size_t st_floats = (mp0 / 32 + 2) * (256 / 4) * 2; /* convolution statistics: at most rows/32 + 2 partial rows of cout/4 quads */
     if (f32_elems <= v->f32_elems && bf16_elems <= v->bf16_elems && guard <= v->guard && ld <= v->att_ld && chunk <= v->att_chunk &&
-        gn_floats <= v->gn_floats && (size_t)128 * h * w <= v->lat_elems && (size_t)256 * h * w <= v->img_pixels)
+        gn_floats <= v->gn_floats && st_floats <= v->st_floats && (size_t)128 * h * w <= v->lat_elems && (size_t)256 * h * w <= v->img_pixels)
         return 1;
     flux_hip_sync();
     free_work(v);
@@ -306,18 +307,20 @@ static int ensure_work(flux_hip_vae *v, int h, int w) {
     v->VT = flux_hip_malloc(512 * ld * 2);
     v->kbias = (float *)flux_hip_malloc(ld * 4);
     v->gn = (float *)flux_hip_malloc(gn_floats * 4);
+    v->st_x = (float *)flux_hip_malloc(st_floats * 4);
+    v->st_h = (float *)flux_hip_malloc(st_floats * 4);
     v->lat = (float *)flux_hip_malloc((size_t)128 * h * w * 4);
     v->img_f32 = (float *)flux_hip_malloc((size_t)256 * h * w * 3 * 4);
     v->img_u8 = (uint8_t *)flux_hip_malloc((size_t)256 * h * w * 3);
     if (!v->X || !v->Y || !v->Hb || !v->A_base || !v->R || !v->S || !v->P || !v->VT || !v->kbias || !v->gn || !v->lat || !v->img_f32 ||
-        !v->img_u8) {
+        !v->img_u8 || !v->st_x || !v->st_h) {
         free_work(v);
         return flux_hip_fail("VAE work buffers for a %d x %d latent could not be allocated", h, w);
     }
     /* guards are read (their contents never reach an output that is kept), so give them defined values */
     if (!flux_hip_memset(v->A_base, 0, (bf16_elems + 2 * guard) * 2)) return 0;
     v->f32_elems = f32_elems; v->bf16_elems = bf16_elems; v->guard = guard; v->att_ld = ld; v->att_chunk = chunk;
-    v->gn_floats = gn_floats; v->lat_elems = (size_t)128 * h * w; v->img_pixels = (size_t)256 * h * w;
+    v->gn_floats = gn_floats; v->st_floats = st_floats; v->lat_elems = (size_t)128 * h * w; v->img_pixels = (size_t)256 * h * w;
     return 1;
 }
 
@@ -330,36 +333,40 @@ typedef struct {
     float *x, *y; /* residual stream and the spare fp32 image */
     void *A;      /* bf16 convolution input (inside its guards) */
     int hp, wp;
+    int x_rows, h_rows; /* partial rows of the statistics the last convolution into x / into Hb left in st_x / st_h */
 } vstate;
 
-static int run_conv(vstate *s, const vconv *c, int epi, const void *in, const float *res, void *out, int masked) {
-    return flux_hip_conv(epi, in, c->w, c->b, res, out, s->hp * s->wp, masked ? s->wp : 0, c->cin_pad, c->cout_pad, c->taps);
+/* stats: NULL, or the buffer that receives the sums for the next group norm over `out` (its row count goes to *stats_rows) */
+static int run_conv(vstate *s, const vconv *c, int epi, const void *in, const float *res, void *out, int masked, float *stats, int *stats_rows) {
+    return flux_hip_conv_stats(epi, in, c->w, c->b, res, out, s->hp * s->wp, masked ? s->wp : 0, c->cin_pad, c->cout_pad, c->taps, stats,
+                               stats_rows);
 }
 
-/* resblock_forward, flux_vae.c:179-219 */
+/* resblock_forward, flux_vae.c:179-219. Every group norm takes its statistics from the epilogue of
+ * the convolution that produced its input. */
 static int run_res(vstate *s, const vres *r) {
     flux_hip_vae *v = s->v;
     const int differ = r->cin != r->cout;
-    if (!flux_hip_group_norm(s->A, differ ? v->R : NULL, s->x, 0, r->n1g, r->n1b, v->gn, s->hp, s->wp, r->cin, v->eps, 1)) return 0;
-    if (!run_conv(s, &r->c1, FLUX_HIP_EPI_CONV_BF16, s->A, NULL, v->Hb, 1)) return 0; /* only the next norm reads it */
-    if (!flux_hip_group_norm(s->A, NULL, v->Hb, 1, r->n2g, r->n2b, v->gn, s->hp, s->wp, r->cout, v->eps, 1)) return 0;
+    if (!flux_hip_group_norm_stats(s->A, differ ? v->R : NULL, s->x, 0, r->n1g, r->n1b, v->gn, s->hp, s->wp, r->cin, v->eps, 1, v->st_x, s->x_rows)) return 0;
+    if (!run_conv(s, &r->c1, FLUX_HIP_EPI_CONV_BF16, s->A, NULL, v->Hb, 1, v->st_h, &s->h_rows)) return 0; /* only the next norm reads it */
+    if (!flux_hip_group_norm_stats(s->A, NULL, v->Hb, 1, r->n2g, r->n2b, v->gn, s->hp, s->wp, r->cout, v->eps, 1, v->st_h, s->h_rows)) return 0;
     if (differ) {
-        if (!run_conv(s, &r->skip, FLUX_HIP_EPI_CONV_F32, v->R, NULL, s->y, 1)) return 0;
-        if (!run_conv(s, &r->c2, FLUX_HIP_EPI_CONV_F32, s->A, s->y, s->y, 1)) return 0;
+        if (!run_conv(s, &r->skip, FLUX_HIP_EPI_CONV_F32, v->R, NULL, s->y, 1, NULL, NULL)) return 0;
+        if (!run_conv(s, &r->c2, FLUX_HIP_EPI_CONV_F32, s->A, s->y, s->y, 1, v->st_x, &s->x_rows)) return 0;
         float *t = s->x; s->x = s->y; s->y = t;
         return 1;
     }
-    return run_conv(s, &r->c2, FLUX_HIP_EPI_CONV_F32, s->A, s->x, s->x, 1);
+    return run_conv(s, &r->c2, FLUX_HIP_EPI_CONV_F32, s->A, s->x, s->x, 1, v->st_x, &s->x_rows);
 }
 
 /* attnblock_forward, flux_vae.c:223-313 */
 static int run_attn(vstate *s) {
     flux_hip_vae *v = s->v;
     const int C = 512, rows = s->hp * s->wp, ld = (rows + 127) & ~127;
-    if (!flux_hip_group_norm(s->A, NULL, s->x, 0, v->attn_g, v->attn_b, v->gn, s->hp, s->wp, C, v->eps, 0)) return 0;
+    if (!flux_hip_group_norm_stats(s->A, NULL, s->x, 0, v->attn_g, v->attn_b, v->gn, s->hp, s->wp, C, v->eps, 0, v->st_x, s->x_rows)) return 0;
     /* key rows between the image and the padded width are read by the score GEMM: zero them */
     if (ld > rows && !flux_hip_memset((char *)v->R + (size_t)rows * 3 * C * 2, 0, (size_t)(ld - rows) * 3 * C * 2)) return 0;
-    if (!run_conv(s, &v->qkv, FLUX_HIP_EPI_CONV_BF16, s->A, NULL, v->R, 0)) return 0;
+    if (!run_conv(s, &v->qkv, FLUX_HIP_EPI_CONV_BF16, s->A, NULL, v->R, 0, NULL, NULL)) return 0;
     if (!flux_hip_vae_key_bias(v->kbias, ld, s->hp, s->wp)) return 0;
     if (!flux_hip_transpose_bf16(v->VT, ld, (char *)v->R + 2 * C * 2, 3 * C, rows, C)) return 0;
     const float scale = 1.0f / sqrtf((float)C);
@@ -371,7 +378,7 @@ static int run_attn(vstate *s) {
         flux_hip_linear_part pv = {v->P, v->VT, (char *)s->A + (size_t)r0 * C * 2, NULL, n};
         if (!flux_hip_linear(FLUX_HIP_EPI_BF16, 1, &pv, C, ld, ld, ld, C, 0, 0)) return 0;
     }
-    return run_conv(s, &v->attn_out, FLUX_HIP_EPI_CONV_F32, s->A, s->x, s->x, 1);
+    return run_conv(s, &v->attn_out, FLUX_HIP_EPI_CONV_F32, s->A, s->x, s->x, 1, v->st_x, &s->x_rows);
 }
 
 /* latent [128, h, w] on the host -> 8-bit image [16h, 16w, 3] and/or the unquantised decoder
@@ -381,10 +388,10 @@ int flux_hip_vae_decode(flux_hip_vae *v, const float *latent, int h, int w, uint
     if (h <= 0 || w <= 0 || h > 112 || w > 112) /* the reference's limit: 1792 pixels, flux.h:52 */
         return flux_hip_fail("flux_hip_vae_decode: latent %d x %d out of range (1..112)", h, w);
     if (!vae_complete(v) || !ensure_work(v, h, w)) return 0;
-    vstate s = {v, v->X, v->Y, (char *)v->A_base + v->guard * 2, 2 * h + 2, 2 * w + 2};
+    vstate s = {v, v->X, v->Y, (char *)v->A_base + v->guard * 2, 2 * h + 2, 2 * w + 2, 0, 0};
     if (!flux_hip_upload(v->lat, latent, (size_t)128 * h * w * 4)) return 0;
     if (!flux_hip_vae_latent_in(s.A, v->lat, v->bn_mean, v->bn_var, v->pq_w, v->pq_b, h, w, v->eps)) return 0;
-    if (!run_conv(&s, &v->conv_in, FLUX_HIP_EPI_CONV_F32, s.A, NULL, s.x, 1)) return 0;
+    if (!run_conv(&s, &v->conv_in, FLUX_HIP_EPI_CONV_F32, s.A, NULL, s.x, 1, v->st_x, &s.x_rows)) return 0;
     int done = 0;
     const int total = 15;
     if (!run_res(&s, &v->mid[0])) return 0;
@@ -404,11 +411,11 @@ int flux_hip_vae_decode(flux_hip_vae *v, const float *latent, int h, int w, uint
             if (!flux_hip_upsample2x(s.A, s.x, s.hp, s.wp, c->cin)) return 0;
             s.hp = 2 * (s.hp - 2) + 2;
             s.wp = 2 * (s.wp - 2) + 2;
-            if (!run_conv(&s, c, FLUX_HIP_EPI_CONV_F32, s.A, NULL, s.x, 1)) return 0;
+            if (!run_conv(&s, c, FLUX_HIP_EPI_CONV_F32, s.A, NULL, s.x, 1, v->st_x, &s.x_rows)) return 0;
         }
     }
-    if (!flux_hip_group_norm(s.A, NULL, s.x, 0, v->out_g, v->out_b, v->gn, s.hp, s.wp, 128, v->eps, 1)) return 0;
-    if (!run_conv(&s, &v->conv_out, FLUX_HIP_EPI_CONV_F32, s.A, NULL, v->Hb, 1)) return 0;
+    if (!flux_hip_group_norm_stats(s.A, NULL, s.x, 0, v->out_g, v->out_b, v->gn, s.hp, s.wp, 128, v->eps, 1, v->st_x, s.x_rows)) return 0;
+    if (!run_conv(&s, &v->conv_out, FLUX_HIP_EPI_CONV_F32, s.A, NULL, v->Hb, 1, NULL, NULL)) return 0;
     const int H = 16 * h, W = 16 * w;
     if (!flux_hip_vae_image_out(rgb ? v->img_u8 : NULL, rgb_f32 ? v->img_f32 : NULL, v->Hb, v->conv_out.cout_pad, H, W)) return 0;
     if (rgb && !flux_hip_download(rgb, v->img_u8, (size_t)H * W * 3)) return 0;

@@ -59,6 +59,9 @@ struct GemmArgs {
      * conv_kshift = log2(cin / 64) */
     int conv_taps, conv_kshift, conv_wp, conv_hp;
     const float *bias, *res;
+    /* optional: per (row-tile half, 4-channel group) sums and sums of squares of what a convolution
+     * epilogue writes, [prow][N/4][2], for the group norm that follows */
+    float *stats;
 };
 
 template <int EPI> struct IsConv { static constexpr bool value = EPI == FLUX_HIP_EPI_CONV_BF16 || EPI == FLUX_HIP_EPI_CONV_F32; };
@@ -128,9 +131,12 @@ __device__ __forceinline__ int weight_row(const GemmArgs &g, int tn, int v) {
  * token m = lane%16 of the 16-row block. */
 template <int BN, int WM, int WN, int EPI>
 __device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f32x4 (&acc)[WN / 16][WM / 16], int m0, int M,
-                                           int wm, int wn, int l15, int lq) {
+                                           int wm, int wn, int l15, int lq, int prow) {
     constexpr int TM = WM / 16, TN = WN / 16;
     const int ldc = g.ldc, prob = t.prob, tn = t.tn, n0 = tn * BN, ks = t.ks;
+    float st_s[TN], st_q[TN]; /* convolutions with statistics: this lane's sums per 16-column block */
+#pragma unroll
+    for (int i = 0; i < TN; i++) st_s[i] = st_q[i] = 0.0f;
 #pragma unroll
     for (int j = 0; j < TM; j++) {
         const int m = m0 + wm * WM + j * 16 + l15;
@@ -176,16 +182,41 @@ __device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f
                     const f32x4 bv = *(const f32x4 *)(g.bias + n);
                     bf16x4 o;
 #pragma unroll
-                    for (int e = 0; e < 4; e++) o[e] = (bf16)(inside ? acc[i][j][e] + bv[e] : 0.0f);
+                    for (int e = 0; e < 4; e++) {
+                        const float v = inside ? acc[i][j][e] + bv[e] : 0.0f;
+                        o[e] = (bf16)v;
+                        st_s[i] += v;
+                        st_q[i] += v * v;
+                    }
                     *(bf16x4 *)((bf16 *)g.C[prob] + (size_t)m * ldc + n) = o;
                 } else if (EPI == FLUX_HIP_EPI_CONV_F32) {
                     const f32x4 bv = *(const f32x4 *)(g.bias + n);
                     f32x4 r = {0.0f, 0.0f, 0.0f, 0.0f};
                     if (g.res) r = *(const f32x4 *)(g.res + (size_t)m * ldc + n);
 #pragma unroll
-                    for (int e = 0; e < 4; e++) r[e] = inside ? r[e] + acc[i][j][e] + bv[e] : 0.0f;
+                    for (int e = 0; e < 4; e++) {
+                        r[e] = inside ? r[e] + acc[i][j][e] + bv[e] : 0.0f;
+                        st_s[i] += r[e];
+                        st_q[i] += r[e] * r[e];
+                    }
                     *(f32x4 *)((float *)g.C[prob] + (size_t)m * ldc + n) = r;
                 }
+            }
+        }
+    }
+    if (IsConv<EPI>::value && g.stats) {
+        /* sum over the 16 rows held by lanes of equal lane/16, then one lane per column quad stores */
+#pragma unroll
+        for (int i = 0; i < TN; i++) {
+#pragma unroll
+            for (int o = 1; o < 16; o <<= 1) {
+                st_s[i] += __shfl_xor(st_s[i], o);
+                st_q[i] += __shfl_xor(st_q[i], o);
+            }
+            if (l15 == 0) {
+                const int n = n0 + wn * WN + i * 16 + lq * 4;
+                f32x2 v = {st_s[i], st_q[i]};
+                *(f32x2 *)(g.stats + ((size_t)prow * (g.N >> 2) + (n >> 2)) * 2) = v;
             }
         }
     }
@@ -284,7 +315,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
         }
     }
 
-    store_tile<BN, WM, WN, EPI>(g, t, acc, m0, M, wm, wn, l15, lq);
+    store_tile<BN, WM, WN, EPI>(g, t, acc, m0, M, wm, wn, l15, lq, t.tm * WGM + wm);
 }
 
 /* The large tiles: 4 waves (2 x 2), one per SIMD, each owning a (16 TM) x (16 TN) part of a
@@ -428,7 +459,7 @@ __global__ __launch_bounds__(256) void gemm4w_kernel(GemmArgs g) {
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); /* the last MFMA results retire before they are read */
     acc_fence<TM, TN>(acc);
 
-    store_tile<BN, WM, WN, EPI>(g, t, acc, m0, M, wm, wn, l15, lq);
+    store_tile<BN, WM, WN, EPI>(g, t, acc, m0, M, wm, wn, l15, lq, t.tm * 2 + wm);
 }
 
 /* ------------------------------------------------------------------ host side */
@@ -644,7 +675,7 @@ static int probe_slot(int epilogue) {
 }
 
 /* Tile and K-split choice, then the launch; `allowed` has bit t set for every tile id that may be used. */
-static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed) {
+static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, int *tile_out = nullptr) {
     /* Choose tile and K split with a small cost model: workgroups run in rounds over
      * 256 CUs x occupancy; a workgroup's time is its FLOPs at the tile's measured rate plus a
      * fixed prologue/epilogue cost; the launch cannot beat the time to stream its operands,
@@ -708,6 +739,7 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed) {
         g.ws = g_ws;
     }
 
+    if (tile_out) *tile_out = tile;
     const int slot = probe_slot(epilogue);
     if (slot >= 0) g_probe_tile[slot] = (unsigned char)tile;
     if (slot >= 0) (void)hipEventRecord(g_probe_ev[slot][0], flux_hip_stream_handle());
@@ -766,8 +798,17 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
 }
 
 /* Convolution over a zero-bordered channels-last image as one GEMM, see the header. */
+extern "C" int flux_hip_conv_stats(int epilogue, const void *in, const void *w, const float *bias, const float *res, void *out, int rows,
+                                   int wp, int cin, int cout, int taps, float *stats, int *stats_rows);
+
 extern "C" int flux_hip_conv(int epilogue, const void *in, const void *w, const float *bias, const float *res,
                              void *out, int rows, int wp, int cin, int cout, int taps) {
+    return flux_hip_conv_stats(epilogue, in, w, bias, res, out, rows, wp, cin, cout, taps, nullptr, nullptr);
+}
+
+/* The same, and (stats != NULL) the sums for the group norm that follows, see the header. */
+extern "C" int flux_hip_conv_stats(int epilogue, const void *in, const void *w, const float *bias, const float *res, void *out, int rows,
+                                   int wp, int cin, int cout, int taps, float *stats, int *stats_rows) {
     if (epilogue != FLUX_HIP_EPI_CONV_BF16 && epilogue != FLUX_HIP_EPI_CONV_F32)
         return flux_hip_fail("flux_hip_conv: epilogue %d is not a convolution epilogue", epilogue);
     if (taps != 1 && taps != 9) return flux_hip_fail("flux_hip_conv: taps=%d (1 or 9)", taps);
@@ -789,7 +830,8 @@ extern "C" int flux_hip_conv(int epilogue, const void *in, const void *w, const 
     g.M[0] = rows;
     g.N = cout; g.K = taps * cin; g.lda = cin; g.ldw = taps * cin; g.ldc = cout;
     g.conv_taps = taps; g.conv_kshift = kshift; g.conv_wp = wp; g.conv_hp = wp > 0 ? rows / wp : 0;
-    g.bias = bias; g.res = res;
+    g.bias = bias; g.res = res; g.stats = stats;
+    if (stats && (!stats_rows || ((uintptr_t)stats & 7))) return flux_hip_fail("flux_hip_conv_stats: stats needs stats_rows and 8-byte alignment");
     const unsigned conv_tiles = 0x0F; /* 64x128, 128x128, 256x256 (4 waves), 64x64 */
     static const int width[4] = {128, 128, 256, 64};
     unsigned allowed;
@@ -803,5 +845,9 @@ extern "C" int flux_hip_conv(int epilogue, const void *in, const void *w, const 
         const long big_tiles = cout % 256 ? 0 : (long)((rows + 255) / 256) * (cout / 256);
         allowed = big_tiles >= 2048 ? 1u << 2 : cout % 128 == 0 ? 1u << 1 : 1u << 3;
     }
-    return gemm_dispatch(g, 1, epilogue, allowed & conv_tiles);
+    int tile = -1;
+    if (!gemm_dispatch(g, 1, epilogue, allowed & conv_tiles, &tile)) return 0;
+    static const int tile_rows[4] = {64, 128, 256, 64}; /* every convolution tile is two waves high */
+    if (stats_rows) *stats_rows = 2 * ((rows + tile_rows[tile & 3] - 1) / tile_rows[tile & 3]);
+    return 1;
 }

@@ -138,6 +138,38 @@ __global__ __launch_bounds__(256) void gn_finalize_kernel(float *__restrict__ st
     }
 }
 
+/* The same from sums that convolution epilogues left behind (flux_hip_conv_stats): partial
+ * [prows][C/4][2], one (sum, sum of squares) per row-tile half and 4-channel quad. */
+__global__ __launch_bounds__(256) void gn_finalize_quads_kernel(float *__restrict__ stats, const float *__restrict__ partial, int prows, int C,
+                                                                double count, float eps) {
+    __shared__ double sh[256][2];
+    const int g = blockIdx.x, quads = C >> 2, qpg = quads >> 5;
+    double a = 0.0, b = 0.0;
+    for (int i = threadIdx.x; i < prows * qpg; i += 256) {
+        const int r = i / qpg, k = i - r * qpg;
+        const f32x2 v = *(const f32x2 *)(partial + ((size_t)r * quads + g * qpg + k) * 2);
+        a += (double)v[0];
+        b += (double)v[1];
+    }
+    sh[threadIdx.x][0] = a;
+    sh[threadIdx.x][1] = b;
+    __syncthreads();
+    for (int s = 128; s > 0; s >>= 1) {
+        if (threadIdx.x < s) {
+            sh[threadIdx.x][0] += sh[threadIdx.x + s][0];
+            sh[threadIdx.x][1] += sh[threadIdx.x + s][1];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const double mean = sh[0][0] / count;
+        double var = sh[0][1] / count - mean * mean;
+        if (var < 0.0) var = 0.0;
+        stats[g * 2 + 0] = (float)mean;
+        stats[g * 2 + 1] = (float)(1.0 / sqrt(var + (double)eps));
+    }
+}
+
 /* out bf16 = [swish](gamma * (x - mean) * rstd + beta), zeros on the border; raw (optional)
  * receives x itself as bf16, the input of a residual block's 1x1 shortcut convolution. Same
  * thread-to-data map as the partial-sum pass. */
@@ -299,15 +331,20 @@ extern "C" int flux_hip_vae_latent_in(void *out_bf16, const float *latent, const
 
 template <typename T>
 static int group_norm_run(void *out_bf16, void *raw_bf16, const T *x, const float *gamma, const float *beta, float *scratch, int hp, int wp,
-                          int C, float eps, int swish) {
+                          int C, float eps, int swish, const float *conv_stats, int conv_stats_rows) {
     const int rows = hp * wp, nblocks = (rows + GN_ROWS - 1) / GN_ROWS;
     float *partial = scratch + 64, *stats = scratch;
     hipStream_t st = flux_hip_stream_handle();
-    hipLaunchKernelGGL(gn_partial_kernel<T>, dim3(nblocks), dim3(256), 0, st, partial, x, rows, C);
-    LAUNCH_OK("gn_partial_kernel");
     const double count = (double)(hp - 2) * (wp - 2) * (C / 32);
-    hipLaunchKernelGGL(gn_finalize_kernel, dim3(32), dim3(256), 0, st, stats, partial, nblocks, count, eps);
-    LAUNCH_OK("gn_finalize_kernel");
+    if (conv_stats) {
+        hipLaunchKernelGGL(gn_finalize_quads_kernel, dim3(32), dim3(256), 0, st, stats, conv_stats, conv_stats_rows, C, count, eps);
+        LAUNCH_OK("gn_finalize_quads_kernel");
+    } else {
+        hipLaunchKernelGGL(gn_partial_kernel<T>, dim3(nblocks), dim3(256), 0, st, partial, x, rows, C);
+        LAUNCH_OK("gn_partial_kernel");
+        hipLaunchKernelGGL(gn_finalize_kernel, dim3(32), dim3(256), 0, st, stats, partial, nblocks, count, eps);
+        LAUNCH_OK("gn_finalize_kernel");
+    }
     const unsigned long long magic = ((1ull << 40) + (unsigned)wp - 1) / (unsigned)wp;
     hipLaunchKernelGGL(gn_apply_kernel<T>, dim3(nblocks), dim3(256), 0, st, (bf16 *)out_bf16, (bf16 *)raw_bf16, x, stats, gamma, beta, rows, C, hp,
                        wp, magic, swish);
@@ -315,12 +352,19 @@ static int group_norm_run(void *out_bf16, void *raw_bf16, const T *x, const floa
     return 1;
 }
 
-extern "C" int flux_hip_group_norm(void *out_bf16, void *raw_bf16, const void *x, int x_is_bf16, const float *gamma, const float *beta,
-                                   float *scratch, int hp, int wp, int C, float eps, int swish) {
+extern "C" int flux_hip_group_norm_stats(void *out_bf16, void *raw_bf16, const void *x, int x_is_bf16, const float *gamma, const float *beta,
+                                         float *scratch, int hp, int wp, int C, float eps, int swish, const float *conv_stats,
+                                         int conv_stats_rows) {
     if (C != 128 && C != 256 && C != 512) return flux_hip_fail("flux_hip_group_norm: C=%d (128, 256 or 512)", C);
     if (hp < 3 || wp < 3 || wp >= 4096 || (long long)hp * wp >= (1 << 22)) return flux_hip_fail("flux_hip_group_norm: bad image %d x %d", hp, wp);
-    return x_is_bf16 ? group_norm_run(out_bf16, raw_bf16, (const bf16 *)x, gamma, beta, scratch, hp, wp, C, eps, swish)
-                     : group_norm_run(out_bf16, raw_bf16, (const float *)x, gamma, beta, scratch, hp, wp, C, eps, swish);
+    if (conv_stats && conv_stats_rows <= 0) return flux_hip_fail("flux_hip_group_norm_stats: conv_stats_rows=%d", conv_stats_rows);
+    return x_is_bf16 ? group_norm_run(out_bf16, raw_bf16, (const bf16 *)x, gamma, beta, scratch, hp, wp, C, eps, swish, conv_stats, conv_stats_rows)
+                     : group_norm_run(out_bf16, raw_bf16, (const float *)x, gamma, beta, scratch, hp, wp, C, eps, swish, conv_stats, conv_stats_rows);
+}
+
+extern "C" int flux_hip_group_norm(void *out_bf16, void *raw_bf16, const void *x, int x_is_bf16, const float *gamma, const float *beta,
+                                   float *scratch, int hp, int wp, int C, float eps, int swish) {
+    return flux_hip_group_norm_stats(out_bf16, raw_bf16, x, x_is_bf16, gamma, beta, scratch, hp, wp, C, eps, swish, nullptr, 0);
 }
 
 extern "C" size_t flux_hip_group_norm_scratch_floats(int hp, int wp) {

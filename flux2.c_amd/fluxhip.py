@@ -133,6 +133,8 @@ def lib():
     L.flux_official_schedule.argtypes = [c_i, c_i]
     L.flux_hip_conv.argtypes = [c_i, vp, vp, vp, vp, vp, c_i, c_i, c_i, c_i, c_i]
     L.flux_hip_group_norm.argtypes = [vp, vp, vp, c_i, vp, vp, vp, c_i, c_i, c_i, c_f, c_i]
+    L.flux_hip_conv_stats.argtypes = [c_i, vp, vp, vp, vp, vp, c_i, c_i, c_i, c_i, c_i, vp, ctypes.POINTER(c_i)]
+    L.flux_hip_group_norm_stats.argtypes = [vp, vp, vp, c_i, vp, vp, vp, c_i, c_i, c_i, c_f, c_i, vp, c_i]
     L.flux_hip_group_norm_scratch_floats.restype = c_sz
     L.flux_hip_group_norm_scratch_floats.argtypes = [c_i, c_i]
     L.flux_hip_upsample2x.argtypes = [vp, vp, c_i, c_i, c_i]

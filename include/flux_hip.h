@@ -107,6 +107,12 @@ int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
  */
 int flux_hip_conv(int epilogue, const void *in, const void *w, const float *bias, const float *res,
                   void *out, int rows, int wp, int cin, int cout, int taps);
+/* The same; when stats is given, the epilogue also leaves there the sums the following group norm
+ * needs (sum and sum of squares of what it writes, per half row-tile and 4-channel quad:
+ * [*stats_rows][cout/4][2] floats, at most rows/32 + 2 rows), which saves that norm its pass over
+ * the image (flux_hip_group_norm_stats). */
+int flux_hip_conv_stats(int epilogue, const void *in, const void *w, const float *bias, const float *res, void *out, int rows,
+                        int wp, int cin, int cout, int taps, float *stats, int *stats_rows);
 
 /* Measurement hooks. force_tile: 0/1/2/3/5/6/7 pins the GEMM tile (64x128, 128x128, 256x256, 64x64,
  * 288x192, 192x192, 256x192; 4 = 256x256 in its 8-wave form, never chosen automatically), -1 restores the automatic
@@ -315,6 +321,9 @@ float *flux_hip_sample_ancestral_traced(void *transformer, const float *z, int c
  */
 int flux_hip_group_norm(void *out_bf16, void *raw_bf16, const void *x, int x_is_bf16, const float *gamma, const float *beta,
                         float *scratch, int hp, int wp, int C, float eps, int swish);
+/* conv_stats / conv_stats_rows: what flux_hip_conv_stats left behind for this x (NULL: sums are computed here) */
+int flux_hip_group_norm_stats(void *out_bf16, void *raw_bf16, const void *x, int x_is_bf16, const float *gamma, const float *beta,
+                              float *scratch, int hp, int wp, int C, float eps, int swish, const float *conv_stats, int conv_stats_rows);
 size_t flux_hip_group_norm_scratch_floats(int hp, int wp);
 /* nearest-neighbour 2x: x f32 [hp*wp, C] -> out bf16 [(2H+2)*(2W+2), C] (flux_upsample_nearest, flux_kernels.c:1017) */
 int flux_hip_upsample2x(void *out_bf16, const float *x, int hp, int wp, int C);

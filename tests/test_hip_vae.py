@@ -174,6 +174,46 @@ def test_group_norm(hip, oracle_mod, C, swish, in_bf16):
     np.testing.assert_array_equal(raw.to_array(np.uint16, (rows, C)), f32_to_bf16(to_padded(x)))
 
 
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3])
+@pytest.mark.parametrize("epi_bf16", [0, 1])
+def test_group_norm_from_convolution_statistics(hip, oracle_mod, tile, epi_bf16):
+    """The convolution epilogue leaves the sums of what it wrote; the group norm that takes them must give
+    what the group norm that computes its own sums gives, and what the oracle gives."""
+    import ctypes
+    H, W, cin, cout = 21, 18, 128, 256
+    hip.lib().flux_hip_linear_force_tile(tile)
+    x = q(normal_f32((cin, H, W), 57, 1))
+    w = q(normal_f32((cout, cin, 3, 3), 57, 2, 0.0, 0.05))
+    b = normal_f32((cout,), 57, 3)
+    res = None if epi_bf16 else normal_f32((cout, H, W), 57, 4)
+    gm, bt = normal_f32((cout,), 57, 5, 1.0, 0.2), normal_f32((cout,), 57, 6)
+    rows, wp = (H + 2) * (W + 2), W + 2
+    din = Guarded(hip, to_padded(x), wp)
+    dw, db = hip.DevBuf.from_array(conv_weight(w)), hip.DevBuf.from_array(b)
+    dg, dbt = hip.DevBuf.from_array(gm), hip.DevBuf.from_array(bt)
+    out = hip.DevBuf.from_array(to_padded(res)) if res is not None else hip.DevBuf(rows * cout * 2)
+    stats = hip.DevBuf.from_array(np.full(((rows // 32 + 2) * (cout // 4) * 2,), np.nan, np.float32))
+    nrows = ctypes.c_int(0)
+    hip.check(hip.lib().flux_hip_conv_stats(hip.EPI_CONV_BF16 if epi_bf16 else hip.EPI_CONV_F32, din.ptr, dw.ptr, db.ptr,
+                                            None if epi_bf16 else out.ptr, out.ptr, rows, wp, cin, cout, 9, stats.ptr, ctypes.byref(nrows)))
+    assert 0 < nrows.value <= rows // 32 + 2
+    st = stats.to_array(np.float32, (nrows.value, cout // 4, 2))
+    assert np.isfinite(st).all()                       # every slot was written
+    scratch = hip.DevBuf(hip.lib().flux_hip_group_norm_scratch_floats(H + 2, W + 2) * 4)
+    y1, y2 = hip.DevBuf(rows * cout * 2), hip.DevBuf(rows * cout * 2)
+    hip.check(hip.lib().flux_hip_group_norm_stats(y1.ptr, None, out.ptr, epi_bf16, dg.ptr, dbt.ptr, scratch.ptr, H + 2, W + 2, cout, 1e-4, 1,
+                                                  stats.ptr, nrows.value))
+    hip.check(hip.lib().flux_hip_group_norm(y2.ptr, None, out.ptr, epi_bf16, dg.ptr, dbt.ptr, scratch.ptr, H + 2, W + 2, cout, 1e-4, 1))
+    a1 = bf16_to_f32(y1.to_array(np.uint16, (rows, cout)))
+    a2 = bf16_to_f32(y2.to_array(np.uint16, (rows, cout)))
+    assert border_is_zero(a1, H, W)
+    assert rel_l2(a1, a2) < 2e-3                       # sums of unrounded vs rounded values when the output is bf16
+    conv = oracle_mod.conv2d(x, w, b, 1) + (0 if res is None else res)
+    want = oracle_mod.silu(oracle_mod.group_norm(conv, gm, bt, 32, 1e-4))
+    assert rel_l2(from_padded(a1, H, W), want) < 6e-3
+    hip.lib().flux_hip_linear_force_tile(-1)
+
+
 def test_upsample(hip, oracle_mod):
     C, H, W = 128, 5, 7
     x = normal_f32((C, H, W), 55, 1)
