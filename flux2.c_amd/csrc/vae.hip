@@ -138,35 +138,35 @@ __global__ __launch_bounds__(256) void gn_finalize_kernel(float *__restrict__ st
     }
 }
 
-/* The same from sums that convolution epilogues left behind (flux_hip_conv_stats): partial
- * [prows][C/4][2], one (sum, sum of squares) per row-tile half and 4-channel quad. */
-__global__ __launch_bounds__(256) void gn_finalize_quads_kernel(float *__restrict__ stats, const float *__restrict__ partial, int prows, int C,
-                                                                double count, float eps) {
-    __shared__ double sh[256][2];
-    const int g = blockIdx.x, quads = C >> 2, qpg = quads >> 5;
-    double a = 0.0, b = 0.0;
-    for (int i = threadIdx.x; i < prows * qpg; i += 256) {
-        const int r = i / qpg, k = i - r * qpg;
-        const f32x2 v = *(const f32x2 *)(partial + ((size_t)r * quads + g * qpg + k) * 2);
-        a += (double)v[0];
-        b += (double)v[1];
+/* First stage when the sums come from convolution epilogues (flux_hip_conv_stats): conv
+ * [prows][C/4][2] holds one (sum, sum of squares) per row-tile half and 4-channel quad. Each
+ * workgroup folds a contiguous range of those rows into per-group sums, in the layout the
+ * finalize kernel reads. Same thread-to-quad map as the partial-sum pass: coalesced reads. */
+__global__ __launch_bounds__(256) void gn_fold_quads_kernel(float *__restrict__ partial, const float *__restrict__ conv, int prows, int C) {
+    __shared__ float sh[256][2];
+    const int quads = C >> 2, rpi = 256 / quads;
+    const int q = threadIdx.x % quads, r0 = threadIdx.x / quads;
+    const int per = (prows + gridDim.x - 1) / gridDim.x;
+    const int row_begin = blockIdx.x * per, row_end = min(prows, row_begin + per);
+    float s = 0.0f, ss = 0.0f;
+    for (int r = row_begin + r0; r < row_end; r += rpi) {
+        const f32x2 v = *(const f32x2 *)(conv + ((size_t)r * quads + q) * 2);
+        s += v[0];
+        ss += v[1];
     }
-    sh[threadIdx.x][0] = a;
-    sh[threadIdx.x][1] = b;
+    sh[threadIdx.x][0] = s;
+    sh[threadIdx.x][1] = ss;
     __syncthreads();
-    for (int s = 128; s > 0; s >>= 1) {
-        if (threadIdx.x < s) {
-            sh[threadIdx.x][0] += sh[threadIdx.x + s][0];
-            sh[threadIdx.x][1] += sh[threadIdx.x + s][1];
-        }
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) {
-        const double mean = sh[0][0] / count;
-        double var = sh[0][1] / count - mean * mean;
-        if (var < 0.0) var = 0.0;
-        stats[g * 2 + 0] = (float)mean;
-        stats[g * 2 + 1] = (float)(1.0 / sqrt(var + (double)eps));
+    if (threadIdx.x < 32) {
+        const int g = threadIdx.x, qpg = quads >> 5;
+        float a = 0.0f, b = 0.0f;
+        for (int rr = 0; rr < rpi; rr++)
+            for (int k = 0; k < qpg; k++) {
+                a += sh[rr * quads + g * qpg + k][0];
+                b += sh[rr * quads + g * qpg + k][1];
+            }
+        partial[((size_t)blockIdx.x * 32 + g) * 2 + 0] = a;
+        partial[((size_t)blockIdx.x * 32 + g) * 2 + 1] = b;
     }
 }
 
@@ -337,8 +337,13 @@ static int group_norm_run(void *out_bf16, void *raw_bf16, const T *x, const floa
     hipStream_t st = flux_hip_stream_handle();
     const double count = (double)(hp - 2) * (wp - 2) * (C / 32);
     if (conv_stats) {
-        hipLaunchKernelGGL(gn_finalize_quads_kernel, dim3(32), dim3(256), 0, st, stats, conv_stats, conv_stats_rows, C, count, eps);
-        LAUNCH_OK("gn_finalize_quads_kernel");
+        const int rpi = 256 / (C / 4);
+        int nb = (conv_stats_rows + 8 * rpi - 1) / (8 * rpi); /* about eight trips per thread, at most as many workgroups as the scratch has rows */
+        nb = nb < 1 ? 1 : nb > nblocks ? nblocks : nb > 256 ? 256 : nb;
+        hipLaunchKernelGGL(gn_fold_quads_kernel, dim3(nb), dim3(256), 0, st, partial, conv_stats, conv_stats_rows, C);
+        LAUNCH_OK("gn_fold_quads_kernel");
+        hipLaunchKernelGGL(gn_finalize_kernel, dim3(32), dim3(256), 0, st, stats, partial, nb, count, eps);
+        LAUNCH_OK("gn_finalize_kernel");
     } else {
         hipLaunchKernelGGL(gn_partial_kernel<T>, dim3(nblocks), dim3(256), 0, st, partial, x, rows, C);
         LAUNCH_OK("gn_partial_kernel");
