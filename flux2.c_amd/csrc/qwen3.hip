@@ -81,29 +81,32 @@ __global__ __launch_bounds__(64) void qwen3_qk_rope_kernel(bf16 *__restrict__ qk
  * is 0, gets the score -1e9 (not -inf: a row with no admissible key then comes out uniform over all
  * seq columns, exactly as in the reference); softmax over all seq columns; out = P v.
  *
- * One wave per (16 queries, head). All scores of the 16 queries against all keys stay in registers
- * (S^T = K Q^T as 16 x 16 blocks, keys x queries: 32 blocks of 4 registers), so the softmax is the
- * plain three-step one. Inside each group of 32 keys the K rows are assigned to MFMA rows so that
- * a lane ends up with 8 consecutive keys of one query: that is the B-operand layout of the second
- * product O^T = V^T P^T. K, Q and V^T fragments are read straight from global memory (the whole
- * K and V of a layer are 2 MB and sit in L2), three steps ahead of their use. Every wave streams
- * the K and V of its kv head on its own, which makes L2 traffic the bound (about 300 MB per call at
- * 512 tokens); sharing the tiles between the four heads of a group through LDS would cut it by 4.
+ * One workgroup per (16 queries, kv head): its waves are the query heads that share that kv head,
+ * so each 32-key tile of K and of V^T is fetched once and shared through LDS (two slots; the next
+ * tile travels global -> registers while the current one is multiplied, then registers -> LDS,
+ * one barrier per tile). A wave keeps all scores of its 16 queries against all keys in registers
+ * (S^T = K Q^T as 16 x 16 blocks, keys x queries: 32 blocks of 4 registers), so the softmax is
+ * the plain three-step one. Inside each group of 32 keys the K rows are assigned to MFMA rows so
+ * that a lane ends up with 8 consecutive keys of one query: that is the B-operand layout of the
+ * second product O^T = V^T P^T. LDS rows are chunk-swizzled so that the 16 rows a fragment read
+ * touches fall into different banks.
  */
 #define QW_MAXT 16 /* 32-key steps: 512 keys */
+__device__ __forceinline__ int qw_kswz(int j) { return (j & 15) ^ ((j >> 4) << 2); } /* K tile: 32 rows of 16 chunks */
+__device__ __forceinline__ int qw_vswz(int d) { return (d >> 2) & 3; }               /* V^T tile: 128 rows of 4 chunks */
 
-/* The body for NT 32-key steps, NT a compile-time constant: straight-line code, so that fragment
- * loads can be kept three steps ahead of the MFMAs that use them (scheduling barriers stop the
- * compiler from sinking them back next to their uses, where each would be waited for alone).
- * Steps beyond the sequence read clamped rows and are masked like the padding of the last step. */
-template <int NT>
+/* The body for NT 32-key steps, NT a compile-time constant (straight-line code). Steps beyond the
+ * sequence read clamped rows and are masked like the padding of the last step. */
+template <int NT, int G>
 __device__ __forceinline__ void qwen3_attend(bf16 *__restrict__ out, const bf16 *__restrict__ qkv, const bf16 *__restrict__ vt, int ldv,
-                                             const int *__restrict__ mask, int seq, int heads, int kv_heads) {
-    const int lane = threadIdx.x, l15 = lane & 15, lq = lane >> 4;
-    const int q0 = blockIdx.x * 16, h = blockIdx.y, kh = h / (heads / kv_heads);
+                                             const int *__restrict__ mask, int seq, int heads, int kv_heads, char *smem) {
+    const int tid = threadIdx.x, lane = tid & 63, l15 = lane & 15, lq = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    constexpr int nthreads = 64 * G;
+    const int q0 = blockIdx.x * 16, kh = blockIdx.y, h = kh * (heads / kv_heads) + wave;
     const int width = (heads + 2 * kv_heads) * 128;
     const float scale = 0.08838834764831845f; /* 1 / sqrt(128) */
-    constexpr int PD = NT >= 4 ? 3 : 1;       /* steps of fragment loads in flight */
+    constexpr int per_lane = 512 / nthreads;  /* 16-byte chunks of a tile per lane: 8, 4, 2 or 1 */
 
     /* Q^T fragments (MFMA B operand): lane (query l15, lq) holds dims [32 ks + 8 lq, +8) */
     const int qrow = min(q0 + l15, seq - 1);
@@ -111,33 +114,69 @@ __device__ __forceinline__ void qwen3_attend(bf16 *__restrict__ out, const bf16 
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) qf[ks] = *(const bf16x8 *)(qkv + (size_t)qrow * width + h * 128 + ks * 32 + lq * 8);
 
-    auto load_k = [&](bf16x8 (&kf)[8], int t) {
+    bf16x8 stage[per_lane];
+    /* K tile t: LDS row j = key 32 t + j, 16 chunks of 8 dims, chunk c stored at c ^ kswz(j) */
+    auto fetch_k = [&](int t) {
 #pragma unroll
-        for (int half = 0; half < 2; half++) {
-            /* MFMA row m = l15 of this block is key 32 t + 8 (m / 4) + 4 half + (m % 4) */
-            const int key = min(32 * t + 8 * (l15 >> 2) + 4 * half + (l15 & 3), seq - 1);
-            const bf16 *kp = qkv + (size_t)key * width + (heads + kh) * 128 + lq * 8;
-#pragma unroll
-            for (int ks = 0; ks < 4; ks++) kf[half * 4 + ks] = *(const bf16x8 *)(kp + ks * 32);
-        }
+        for (int u = 0; u < per_lane; u++)
+            {
+                const int idx = tid + u * nthreads, j = idx >> 4, c = idx & 15;
+                stage[u] = *(const bf16x8 *)(qkv + (size_t)min(32 * t + j, seq - 1) * width + (heads + kh) * 128 + c * 8);
+            }
     };
-    f32x4 sc[2 * NT];
-    bf16x8 kbuf[PD + 1][8];
+    auto put_k = [&](int slot) {
 #pragma unroll
-    for (int t = 0; t < PD && t < NT; t++) load_k(kbuf[t], t);
+        for (int u = 0; u < per_lane; u++)
+            {
+                const int idx = tid + u * nthreads, j = idx >> 4, c = idx & 15;
+                *(bf16x8 *)(smem + slot * 8192 + j * 256 + ((c ^ qw_kswz(j)) << 4)) = stage[u];
+            }
+    };
+    /* V^T tile t: LDS row d = head dim, 4 chunks of 8 keys, chunk c stored at c ^ vswz(d) */
+    auto fetch_v = [&](int t) {
+#pragma unroll
+        for (int u = 0; u < per_lane; u++)
+            {
+                const int idx = tid + u * nthreads, d = idx >> 2, c = idx & 3;
+                stage[u] = *(const bf16x8 *)(vt + (size_t)(kh * 128 + d) * ldv + min(32 * t, ldv - 32) + c * 8);
+            }
+    };
+    auto put_v = [&](int slot) {
+#pragma unroll
+        for (int u = 0; u < per_lane; u++)
+            {
+                const int idx = tid + u * nthreads, d = idx >> 2, c = idx & 3;
+                *(bf16x8 *)(smem + 16384 + slot * 8192 + d * 64 + ((c ^ qw_vswz(d)) << 4)) = stage[u];
+            }
+    };
+
+    f32x4 sc[2 * NT];
+    fetch_k(0);
+    put_k(0);
+    __syncthreads();
 #pragma unroll
     for (int t = 0; t < NT; t++) {
-        if (t + PD < NT) load_k(kbuf[(t + PD) % (PD + 1)], t + PD);
-        __builtin_amdgcn_sched_barrier(0);
+        if (t + 1 < NT) fetch_k(t + 1);
+        const char *kt = smem + (t & 1) * 8192;
 #pragma unroll
         for (int half = 0; half < 2; half++) {
+            /* MFMA row m = l15 of this block is key 32 t + j with j = 8 (m / 4) + 4 half + (m % 4) */
+            const int j = 8 * (l15 >> 2) + 4 * half + (l15 & 3);
             f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kbuf[t % (PD + 1)][half * 4 + ks], qf[ks], acc, 0, 0, 0);
+            for (int ks = 0; ks < 4; ks++) {
+                const bf16x8 kf = *(const bf16x8 *)(kt + j * 256 + (((ks * 4 + lq) ^ qw_kswz(j)) << 4));
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], acc, 0, 0, 0);
+            }
             sc[2 * t + half] = acc;
         }
-        __builtin_amdgcn_sched_barrier(0);
+        if (t + 1 < NT) {
+            put_k((t + 1) & 1);
+            __syncthreads();
+        }
     }
+    fetch_v(0); /* in flight during the softmax */
+
     /* padding mask as bits: word w covers keys [64 w, 64 w + 64), one ballot per word */
     unsigned long long keep[(NT + 1) / 2];
 #pragma unroll
@@ -182,29 +221,31 @@ __device__ __forceinline__ void qwen3_attend(bf16 *__restrict__ out, const bf16 
 
     /* O^T[d][q] = sum_key V^T[d][key] P^T[key][q]: A operand = V^T rows (lane: dim l15, keys
      * [32 t + 8 lq, +8)), B operand = this lane's 8 probabilities of step t */
-    auto load_v = [&](bf16x8 (&vf)[8], int t) {
-#pragma unroll
-        for (int d = 0; d < 8; d++) vf[d] = *(const bf16x8 *)(vt + (size_t)(kh * 128 + d * 16 + l15) * ldv + min(32 * t, ldv - 32) + 8 * lq);
-    };
     f32x4 o[8];
 #pragma unroll
     for (int d = 0; d < 8; d++) o[d] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
-    bf16x8 vbuf[PD + 1][8];
-#pragma unroll
-    for (int t = 0; t < PD && t < NT; t++) load_v(vbuf[t], t);
+    put_v(0);
+    __syncthreads();
 #pragma unroll
     for (int t = 0; t < NT; t++) {
-        if (t + PD < NT) load_v(vbuf[(t + PD) % (PD + 1)], t + PD);
+        if (t + 1 < NT) fetch_v(t + 1);
+        const char *vtile = smem + 16384 + (t & 1) * 8192;
         bf16x8 pf;
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             pf[e] = (bf16)(sc[2 * t][e] * inv);
             pf[4 + e] = (bf16)(sc[2 * t + 1][e] * inv);
         }
-        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int d = 0; d < 8; d++) o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vbuf[t % (PD + 1)][d], pf, o[d], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
+        for (int d = 0; d < 8; d++) {
+            const int row = d * 16 + l15;
+            const bf16x8 vf = *(const bf16x8 *)(vtile + row * 64 + ((lq ^ qw_vswz(row)) << 4));
+            o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf, o[d], 0, 0, 0);
+        }
+        if (t + 1 < NT) {
+            put_v((t + 1) & 1);
+            __syncthreads();
+        }
     }
     /* accumulator element e of block d: query l15, dim 16 d + 4 lq + e */
     if (qi < seq) {
@@ -222,17 +263,19 @@ __device__ __forceinline__ void qwen3_attend(bf16 *__restrict__ out, const bf16 
 /* Steps whose 32 keys all lie after the block's last query hold no admissible key and are left
  * out - unless the first key is masked: only then can a row have no admissible key at all, and such
  * a row is uniform over every column (see above), so every step is computed. The step count is
- * rounded up to one of four compiled bodies. */
-__global__ __launch_bounds__(64) void qwen3_attention_kernel(bf16 *__restrict__ out, const bf16 *__restrict__ qkv, const bf16 *__restrict__ vt,
-                                                             int ldv, const int *__restrict__ mask, int seq, int heads, int kv_heads) {
+ * rounded up to one of five compiled bodies. Workgroup = heads / kv_heads waves. */
+template <int G>
+__global__ __launch_bounds__(64 * G) void qwen3_attention_kernel(bf16 *__restrict__ out, const bf16 *__restrict__ qkv, const bf16 *__restrict__ vt,
+                                                              int ldv, const int *__restrict__ mask, int seq, int heads, int kv_heads) {
+    __shared__ __attribute__((aligned(16))) char smem[32768]; /* K tiles: 2 x 8 KB, V^T tiles: 2 x 8 KB */
     const int all = (seq + 31) >> 5;
     const bool first_masked = mask && mask[0] == 0;
     const int need = first_masked ? all : min(all, ((blockIdx.x * 16 + 15) >> 5) + 1);
-    if (need <= 2) qwen3_attend<2>(out, qkv, vt, ldv, mask, seq, heads, kv_heads);
-    else if (need <= 4) qwen3_attend<4>(out, qkv, vt, ldv, mask, seq, heads, kv_heads);
-    else if (need <= 8) qwen3_attend<8>(out, qkv, vt, ldv, mask, seq, heads, kv_heads);
-    else if (need <= 12) qwen3_attend<12>(out, qkv, vt, ldv, mask, seq, heads, kv_heads);
-    else qwen3_attend<16>(out, qkv, vt, ldv, mask, seq, heads, kv_heads);
+    if (need <= 2) qwen3_attend<2, G>(out, qkv, vt, ldv, mask, seq, heads, kv_heads, smem);
+    else if (need <= 4) qwen3_attend<4, G>(out, qkv, vt, ldv, mask, seq, heads, kv_heads, smem);
+    else if (need <= 8) qwen3_attend<8, G>(out, qkv, vt, ldv, mask, seq, heads, kv_heads, smem);
+    else if (need <= 12) qwen3_attend<12, G>(out, qkv, vt, ldv, mask, seq, heads, kv_heads, smem);
+    else qwen3_attend<16, G>(out, qkv, vt, ldv, mask, seq, heads, kv_heads, smem);
 }
 
 /* dst[s, col0 + i] = src[s, i]: one layer's hidden state into its third of the output rows */
@@ -269,9 +312,19 @@ extern "C" int flux_hip_causal_attention(void *out_bf16, const void *qkv_bf16, c
                                          int heads, int kv_heads) {
     if (seq <= 0 || seq > 32 * QW_MAXT) return flux_hip_fail("flux_hip_causal_attention: seq=%d (1..%d)", seq, 32 * QW_MAXT);
     if (heads <= 0 || kv_heads <= 0 || heads % kv_heads) return flux_hip_fail("flux_hip_causal_attention: heads=%d kv_heads=%d", heads, kv_heads);
+    const int group = heads / kv_heads; /* waves per workgroup */
+    if (group != 1 && group != 2 && group != 4 && group != 8)
+        return flux_hip_fail("flux_hip_causal_attention: %d query heads per kv head (1, 2, 4 or 8)", group);
     if (ldv < ((seq + 31) & ~31) || (ldv & 7)) return flux_hip_fail("flux_hip_causal_attention: ldv=%d too small or not a multiple of 8", ldv);
-    hipLaunchKernelGGL(qwen3_attention_kernel, dim3((seq + 15) / 16, heads), dim3(64), 0, flux_hip_stream_handle(), (bf16 *)out_bf16,
-                       (const bf16 *)qkv_bf16, (const bf16 *)vt_bf16, ldv, mask_dev, seq, heads, kv_heads);
+    const dim3 grid((seq + 15) / 16, kv_heads);
+#define QW_LAUNCH(G)                                                                                                                   \
+    hipLaunchKernelGGL(qwen3_attention_kernel<G>, grid, dim3(64 * G), 0, flux_hip_stream_handle(), (bf16 *)out_bf16, (const bf16 *)qkv_bf16, \
+                       (const bf16 *)vt_bf16, ldv, mask_dev, seq, heads, kv_heads)
+    if (group == 1) QW_LAUNCH(1);
+    else if (group == 2) QW_LAUNCH(2);
+    else if (group == 4) QW_LAUNCH(4);
+    else QW_LAUNCH(8);
+#undef QW_LAUNCH
     LAUNCH_OK("qwen3_attention_kernel");
     return 1;
 }
