@@ -277,6 +277,11 @@ void flux_hip_vae_free(flux_hip_vae *v) {
     free(v);
 }
 
+/* Test hook: upper bound on the query rows per attention chunk (0 = the buffer's own bound,
+ * 1 GB of fp32 scores). */
+static int g_att_chunk_limit = 0;
+void flux_hip_vae_set_attention_chunk(int rows) { g_att_chunk_limit = rows > 0 ? rows : 0; }
+
 /* Work buffers for a latent of h x w. The largest image is the full-resolution one with 256
  * channels (output of the last upsample convolution). bf16 convolution inputs carry a guard of
  * one image row + 2 positions on both sides (flux_hip_conv reads that far beyond the image). */
@@ -370,8 +375,10 @@ static int run_attn(vstate *s) {
     if (!flux_hip_vae_key_bias(v->kbias, ld, s->hp, s->wp)) return 0;
     if (!flux_hip_transpose_bf16(v->VT, ld, (char *)v->R + 2 * C * 2, 3 * C, rows, C)) return 0;
     const float scale = 1.0f / sqrtf((float)C);
-    for (int r0 = 0; r0 < rows; r0 += (int)v->att_chunk) {
-        const int n = rows - r0 < (int)v->att_chunk ? rows - r0 : (int)v->att_chunk;
+    int chunk = (int)v->att_chunk;
+    if (g_att_chunk_limit && g_att_chunk_limit < chunk) chunk = g_att_chunk_limit;
+    for (int r0 = 0; r0 < rows; r0 += chunk) {
+        const int n = rows - r0 < chunk ? rows - r0 : chunk;
         flux_hip_linear_part sp = {(char *)v->R + (size_t)r0 * 3 * C * 2, (char *)v->R + C * 2, v->S, NULL, n};
         if (!flux_hip_linear(FLUX_HIP_EPI_F32, 1, &sp, ld, C, 3 * C, 3 * C, ld, 0, 0)) return 0;
         if (!flux_hip_softmax_rows(v->P, v->S, v->kbias, n, ld, scale)) return 0;

@@ -146,6 +146,7 @@ def lib():
     L.flux_hip_vae_set_tensor.argtypes = [vp, ctypes.c_char_p, c_i, vp, ctypes.c_int64]
     L.flux_hip_vae_free.argtypes = [vp]
     L.flux_hip_vae_decode.argtypes = [vp, vp, c_i, c_i, vp, vp]
+    L.flux_hip_vae_set_attention_chunk.argtypes = [c_i]
     L.flux_hip_rms_norm.argtypes = [vp, vp, vp, c_i, c_i, c_f]
     L.flux_hip_causal_attention.argtypes = [vp, vp, vp, c_i, vp, c_i, c_i, c_i]
     L.flux_hip_qwen3_new.restype = vp

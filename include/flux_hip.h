@@ -346,6 +346,8 @@ void flux_hip_vae_free(flux_hip_vae *v);
 /* latent f32 [128, h, w] (host) -> rgb u8 [16h, 16w, 3] and/or rgb_f32 [3, 16h, 16w] (decoder output
  * before the conversion to 8 bits); either may be NULL. h, w <= 112. 1 = ok, 0 = failed. */
 int flux_hip_vae_decode(flux_hip_vae *v, const float *latent, int h, int w, uint8_t *rgb, float *rgb_f32);
+/* Test hook: at most `rows` query rows per attention chunk (0 = default: 1 GB of fp32 scores per chunk). */
+void flux_hip_vae_set_attention_chunk(int rows);
 /* When set, called after each of the decoder's 15 blocks has been queued (role of
  * flux_vae_progress_callback, flux_kernels.h:292-293). */
 extern void (*flux_hip_vae_progress)(int block, int total);

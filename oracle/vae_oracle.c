@@ -203,30 +203,45 @@ static int attnblock(const fo_vae *v, const char *prefix, float *out, const floa
     fo_conv2d(k, xn, kw, kb, ch, ch, H, W, 1, 0);
     fo_conv2d(vv, xn, vw, vb, ch, ch, H, W, 1, 0);
     float scale = 1.0f / sqrtf((float)ch);
+    /* token-major copies, as the reference makes them (flux_vae.c:267-275), so that the inner
+     * loops run over contiguous memory */
+    float *qt = (float *)malloc(sizeof(float) * n), *kt = (float *)malloc(sizeof(float) * n), *vt = (float *)malloc(sizeof(float) * n);
+    #pragma omp parallel for schedule(static)
+    for (int i = 0; i < sp; i++)
+        for (int c = 0; c < ch; c++) {
+            qt[(size_t)i * ch + c] = q[(size_t)c * sp + i] * scale;
+            kt[(size_t)i * ch + c] = k[(size_t)c * sp + i];
+            vt[(size_t)i * ch + c] = vv[(size_t)c * sp + i];
+        }
     #pragma omp parallel
     {
         float *row = (float *)malloc(sizeof(float) * (size_t)sp);
+        float *acc = (float *)malloc(sizeof(float) * (size_t)ch);
         #pragma omp for schedule(static)
         for (int i = 0; i < sp; i++) {
+            const float *qi = qt + (size_t)i * ch;
             float mx = -3.0e38f;
             for (int j = 0; j < sp; j++) {
+                const float *kj = kt + (size_t)j * ch;
                 float s = 0.0f;
-                for (int c = 0; c < ch; c++) s += q[(size_t)c * sp + i] * scale * k[(size_t)c * sp + j];
+                for (int c = 0; c < ch; c++) s += qi[c] * kj[c];
                 row[j] = s;
                 if (s > mx) mx = s;
             }
             float sum = 0.0f;
             for (int j = 0; j < sp; j++) { row[j] = expf(row[j] - mx); sum += row[j]; }
             float inv = 1.0f / sum;
-            for (int c = 0; c < ch; c++) {
-                float acc = 0.0f;
-                const float *vc = vv + (size_t)c * sp;
-                for (int j = 0; j < sp; j++) acc += row[j] * vc[j];
-                o[(size_t)c * sp + i] = acc * inv;
+            for (int c = 0; c < ch; c++) acc[c] = 0.0f;
+            for (int j = 0; j < sp; j++) {
+                const float p = row[j];
+                const float *vj = vt + (size_t)j * ch;
+                for (int c = 0; c < ch; c++) acc[c] += p * vj[c];
             }
+            for (int c = 0; c < ch; c++) o[(size_t)c * sp + i] = acc[c] * inv;
         }
-        free(row);
+        free(row); free(acc);
     }
+    free(qt); free(kt); free(vt);
     fo_conv2d(xn, o, ow, ob, ch, ch, H, W, 1, 0);
     for (size_t i = 0; i < n; i++) out[i] = x[i] + xn[i];
     free(xn); free(q); free(k); free(vv); free(o);

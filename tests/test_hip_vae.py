@@ -295,6 +295,36 @@ def test_vae_decode_smaller_after_larger(vae_pair):
     assert rel_l2(f1, cpu.decode(lat, 2, 3)[0]) <= 2e-2
 
 
+def test_vae_attention_in_chunks(hip, vae_pair):
+    """The mid-block attention walks its queries in chunks when the score matrix would not fit its buffer
+    (1024x1024 and up); forced here at a small size: same image as in one piece."""
+    dev, cpu = vae_pair
+    lat = normal_f32((128, 6, 5), 307, 1)
+    f0, u0 = dev.decode(lat, 6, 5)
+    hip.lib().flux_hip_vae_set_attention_chunk(37)          # 12 * 14 = 168 positions -> 5 chunks, the last one ragged
+    try:
+        f1, u1 = dev.decode(lat, 6, 5)
+    finally:
+        hip.lib().flux_hip_vae_set_attention_chunk(0)
+    assert rel_l2(f1, f0) < 1e-3                             # chunk heights change GEMM tile choices: summation order only
+    assert np.abs(u1.astype(np.int32) - u0.astype(np.int32)).max() <= 1
+    assert rel_l2(f1, cpu.decode(lat, 6, 5)[0]) <= 2e-2
+
+
+@pytest.mark.parametrize("side", [32, 64])
+def test_vae_decode_large(vae_pair, side):
+    """Full-size decodes (512x512, 1024x1024: the 256x256 convolution tile and the chunked attention are
+    only chosen there) against the oracle (about half a minute of CPU work on 16 cores)."""
+    dev, cpu = vae_pair
+    lat = normal_f32((128, side, side), 308, 1)
+    f, u = dev.decode(lat, side, side)
+    fo, uo = cpu.decode(lat, side, side)
+    r = rel_l2(f, fo)
+    diff = np.abs(u.astype(np.int32) - uo.astype(np.int32))
+    print(f"vae decode {16 * side}^2: rel_l2={r:.3e} mean|d|={diff.mean():.3f} max|d|={diff.max()}", flush=True)
+    assert r <= 2e-2 and diff.mean() <= 1.5
+
+
 def test_vae_missing_tensor_fails(hip):
     W = make_vae_weights()
     del W["decoder.mid_block.attentions.0.to_k.bias"]
