@@ -240,6 +240,13 @@ def make_vae_weights(seed=77):
     return out
 
 
+def vae_test_image(H, W, seed):
+    """[3, H, W] in [-1, 1]: a smooth ramp plus noise, so that the VAE encoder sees structure and texture."""
+    yy, xx = np.meshgrid(np.linspace(-1, 1, H, dtype=np.float32), np.linspace(-1, 1, W, dtype=np.float32), indexing="ij")
+    base = np.stack([yy, xx, -0.5 * (yy + xx)]).astype(np.float32)
+    return np.clip(0.6 * base + normal_f32((3, H, W), seed, 1, 0.0, 0.3), -1.0, 1.0).astype(np.float32)
+
+
 def vae_decode_convs(h, w):
     """The decoder's convolutions for an h x w latent, in execution order (flux_vae_decode,
     flux_vae.c:690-837): (name, H, W, cin, cout, taps). All but the first (which the device folds into

@@ -90,6 +90,11 @@ def lib():
     L.fo_group_norm.argtypes = [vp, vp, vp, vp, c_i, c_i, c_i, c_i, c_f]
     L.fo_upsample_nearest.argtypes = [vp, vp, c_i, c_i, c_i]
     L.fo_unpatchify.argtypes = [vp, vp, c_i, c_i, c_i, c_i]
+    L.fo_patchify.argtypes = [vp, vp, c_i, c_i, c_i, c_i]
+    L.fo_conv2d_down.argtypes = [vp, vp, vp, vp, c_i, c_i, c_i, c_i]
+    L.fo_vae_encode.argtypes = [vp, vp, c_i, c_i, vp]
+    L.fo_vae_encode.restype = c_i
+    L.fo_vae_set_reference_aliasing.argtypes = [vp, c_i]
     L.fo_vae_new.argtypes = [c_i]
     L.fo_vae_new.restype = vp
     L.fo_vae_free.argtypes = [vp]
@@ -404,16 +409,34 @@ def unpatchify(x, p=2):
     return out
 
 
+def patchify(x, p=2):
+    """[C, H, W] -> [C*p*p, H/p, W/p]."""
+    x = _f32(x)
+    out = np.empty((x.shape[0] * p * p, x.shape[1] // p, x.shape[2] // p), np.float32)
+    lib().fo_patchify(out.ctypes.data, x.ctypes.data, x.shape[0], x.shape[1], x.shape[2], p)
+    return out
+
+
+def conv2d_down(x, w, bias=None):
+    """The encoder's downsampling convolution: x [cin, H, W] padded by one row below and one column on the
+    right, 3x3 kernel w [cout, cin, 3, 3], stride 2."""
+    x, w = _f32(x), _f32(w)
+    b = None if bias is None else _f32(bias)
+    H, W = x.shape[1], x.shape[2]
+    out = np.empty((w.shape[0], (H - 2) // 2 + 1, (W - 2) // 2 + 1), np.float32)
+    lib().fo_conv2d_down(out.ctypes.data, x.ctypes.data, w.ctypes.data, None if b is None else b.ctypes.data,
+                         x.shape[0], w.shape[0], H, W)
+    return out
+
+
 class VaeOracle:
-    """The decoder half of the VAE. `weights` maps tensor name -> uint16 (bf16) or float32 array."""
+    """The VAE. `weights` maps tensor name -> uint16 (bf16) or float32 array."""
 
     def __init__(self, weights, base_channels=128):
         from model_spec import bf16_to_f32
         self._L = lib()
         self._v = self._L.fo_vae_new(base_channels)
         for name, a in weights.items():
-            if not (name.startswith("decoder.") or name.startswith("bn.") or name.startswith("post_quant_conv")):
-                continue
             a = _f32(bf16_to_f32(a) if a.dtype == np.uint16 else a)
             rc = self._L.fo_vae_set(self._v, name.encode(), a.ctypes.data, a.size)
             if rc != 0:
@@ -438,6 +461,18 @@ class VaeOracle:
         if self._L.fo_vae_decode(self._v, latent.ctypes.data, h, w, f.ctypes.data, u.ctypes.data) != 0:
             raise RuntimeError("vae oracle: decode failed (missing tensor)")
         return f, u
+
+    def encode(self, img, reference_aliasing=False):
+        """img [3, H, W] in [-1, 1], H and W multiples of 16 -> normalised latent [128, H/16, W/16].
+        reference_aliasing: reproduce the buffer overlap of the reference's generic build in the two
+        widening residual blocks (see resblock() in vae_oracle.c); only for checks against that build."""
+        img = _f32(img)
+        self._L.fo_vae_set_reference_aliasing(self._v, int(reference_aliasing))
+        H, W = img.shape[1], img.shape[2]
+        lat = np.empty((128, H // 16, W // 16), np.float32)
+        if self._L.fo_vae_encode(self._v, img.ctypes.data, H, W, lat.ctypes.data) != 0:
+            raise RuntimeError("vae oracle: encode failed (missing tensor or size not a multiple of 16)")
+        return lat
 
 
 # ---- Qwen3 text encoder (oracle/qwen3_oracle.c) ----

@@ -20,7 +20,7 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 sys.path.insert(0, os.path.join(ROOT, "flux2.c_amd"))
-from model_spec import (TINY, KLEIN_4B, QWEN3_4B, make_weights, make_vae_weights, make_qwen3_weights,  # noqa: E402
+from model_spec import (TINY, KLEIN_4B, QWEN3_4B, make_weights, make_vae_weights, vae_test_image, make_qwen3_weights,  # noqa: E402
                         write_safetensors, normal_f32, bf16_to_f32)
 
 c_f, c_i, vp = ctypes.c_float, ctypes.c_int, ctypes.c_void_p
@@ -288,12 +288,13 @@ class FluxImage(ctypes.Structure):           # flux.h:73-78
 # shapes shared with tests/test_oracle_golden.py
 VAE_OP_SEED = 21
 VAE_DECODE_CASES = ((2, 2, 301), (3, 2, 302))     # latent h, w, seed
+VAE_ENCODE_CASES = ((32, 32, 311), (48, 32, 312))   # image H, W, seed
 
 
 def vae_golden():
-    """The reference's convolution, group norm, upsample and unpatchify (flux_kernels.c) on small
-    seeded tensors, and its VAE decoder (flux_vae_decode, flux_vae.c:690) on the synthetic
-    full-size VAE of model_spec.make_vae_weights."""
+    """The reference's convolution, group norm, upsample, patchify and unpatchify (flux_kernels.c) on
+    small seeded tensors, and its VAE decoder and encoder (flux_vae_decode, flux_vae.c:690;
+    flux_vae_encode, flux_vae.c:320) on the synthetic full-size VAE of model_spec.make_vae_weights."""
     import tempfile
     g = {}
     for fn in ("flux_conv2d", "flux_group_norm", "flux_upsample_nearest", "flux_unpatchify"):
@@ -326,6 +327,20 @@ def vae_golden():
     op = np.empty((3, 6, 4), np.float32)
     L.flux_unpatchify(P(op), P(xp), 1, 3, 3, 2, 2)
     g["unpatchify"] = op
+    L.flux_patchify.restype = None
+    L.flux_patchify.argtypes = [vp, vp] + [c_i] * 5
+    xq = normal_f32((3, 6, 4), VAE_OP_SEED, 10)
+    oq = np.empty((12, 3, 2), np.float32)
+    L.flux_patchify(P(oq), P(xq), 1, 3, 6, 4, 2)
+    g["patchify"] = oq
+    # the encoder's downsampling step (flux_vae.c:363-377): zeros below and on the right, then stride 2 without padding
+    for tag, (H, W) in (("even", (8, 6)), ("odd", (7, 9))):
+        xd = normal_f32((5, H, W), VAE_OP_SEED, 11)
+        xpad = np.zeros((5, H + 1, W + 1), np.float32)
+        xpad[:, :H, :W] = xd
+        od = np.empty((4, (H - 2) // 2 + 1, (W - 2) // 2 + 1), np.float32)
+        L.flux_conv2d(P(od), P(xpad), P(w3), P(b), 1, 5, 4, H + 1, W + 1, 3, 3, 2, 0)
+        g[f"conv_down_{tag}"] = od
 
     L.safetensors_open.restype = vp
     L.safetensors_open.argtypes = [ctypes.c_char_p]
@@ -351,6 +366,18 @@ def vae_golden():
             g[f"decode_{h}x{w}"] = np.ctypeslib.as_array(im.data, shape=(im.height, im.width, im.channels)).copy()
             L.flux_image_free(ip)
             print("vae decode", h, w, "std", g[f"decode_{h}x{w}"].std(), flush=True)
+        L.flux_vae_encode.restype = ctypes.POINTER(ctypes.c_float)
+        L.flux_vae_encode.argtypes = [vp, vp, c_i, c_i, c_i, ctypes.POINTER(c_i), ctypes.POINTER(c_i)]
+        libc = ctypes.CDLL(None)
+        libc.free.argtypes = [vp]
+        for H, W, seed in VAE_ENCODE_CASES:
+            img = vae_test_image(H, W, seed)
+            oh, ow = c_i(0), c_i(0)
+            lp = L.flux_vae_encode(vae, P(img), 1, H, W, ctypes.byref(oh), ctypes.byref(ow))
+            assert lp and oh.value == H // 16 and ow.value == W // 16
+            g[f"encode_{H}x{W}"] = np.ctypeslib.as_array(lp, shape=(128, oh.value, ow.value)).copy()
+            libc.free(ctypes.cast(lp, vp))
+            print("vae encode", H, W, "std", g[f"encode_{H}x{W}"].std(), flush=True)
         L.flux_vae_free(vae)
     return g
 

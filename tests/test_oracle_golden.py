@@ -219,6 +219,7 @@ def test_klein4b_c1(oracle_mod, golden_dir, qk):
 # ---- VAE decoder (oracle/vae_oracle.c) against the reference's flux_kernels.c / flux_vae.c ----
 VAE_OP_SEED = 21
 VAE_DECODE_CASES = ((2, 2, 301), (3, 2, 302))
+VAE_ENCODE_CASES = ((32, 32, 311), (48, 32, 312))
 
 
 @pytest.fixture(scope="module")
@@ -239,6 +240,9 @@ def test_vae_operators(oracle_mod, vae_gold):
     close(oracle_mod.group_norm(xg, gm, bt, 32, 1e-4), vae_gold["group_norm"], 2e-6)
     np.testing.assert_array_equal(oracle_mod.upsample_nearest(normal_f32((3, 4, 5), VAE_OP_SEED, 8)), vae_gold["upsample"])
     np.testing.assert_array_equal(oracle_mod.unpatchify(normal_f32((12, 3, 2), VAE_OP_SEED, 9)), vae_gold["unpatchify"])
+    np.testing.assert_array_equal(oracle_mod.patchify(normal_f32((3, 6, 4), VAE_OP_SEED, 10)), vae_gold["patchify"])
+    for tag, (H, W) in (("even", (8, 6)), ("odd", (7, 9))):
+        close(oracle_mod.conv2d_down(normal_f32((5, H, W), VAE_OP_SEED, 11), w3, b), vae_gold[f"conv_down_{tag}"], 2e-6)
 
 
 def test_vae_decode_images(oracle_mod, vae_gold):
@@ -256,6 +260,27 @@ def test_vae_decode_images(oracle_mod, vae_gold):
         # the float image is consistent with the 8-bit one
         q = np.clip((f.transpose(1, 2, 0) + 1.0) * 127.5, 0, 255).astype(np.uint8)
         np.testing.assert_array_equal(q, u)
+    o.close()
+
+
+def test_vae_encode_latents(oracle_mod, vae_gold):
+    """Whole encoder on the synthetic full-size VAE against the reference's flux_vae_encode. The
+    vectors come from the reference's generic (plain C) build, in which the second convolution of a
+    widening residual block overwrites its own input as it goes (flux_vae.c:203,
+    flux_kernels.c:441-470); the oracle reproduces that on request and must then agree to rounding.
+    Without it - the arithmetic the block is meant to do, what the reference's BLAS path computes at
+    these sizes, and what the device is compared with - the result differs visibly."""
+    from model_spec import make_vae_weights, vae_test_image
+    o = oracle_mod.VaeOracle(make_vae_weights())
+    for H, W, seed in VAE_ENCODE_CASES:
+        img = vae_test_image(H, W, seed)
+        got = o.encode(img, reference_aliasing=True)
+        want = vae_gold[f"encode_{H}x{W}"]
+        assert got.shape == want.shape == (128, H // 16, W // 16)
+        assert want.std() > 0.2
+        close(got, want, 2e-5)
+        clean = o.encode(img)
+        assert np.isfinite(clean).all() and 0.1 < rel_l2(clean, want) < 1.5
     o.close()
 
 

@@ -151,6 +151,32 @@ def test_conv2d_closed_forms(oracle_mod):
     assert rel_l2(oracle_mod.conv2d(x, w, None, 1), ref) < 1e-6
 
 
+def test_downsample_and_patchify(oracle_mod):
+    """The stride-2 step equals the plain 3x3 convolution of the image moved one pixel up and left
+    (so that 'pad 1' supplies the zero row below / column on the right), sampled at the odd pixels;
+    patchify and unpatchify are inverses, and patchify puts pixel (1, 0) of a 2x2 patch in channel 2."""
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((3, 8, 10)).astype(np.float32)
+    w = rng.standard_normal((4, 3, 3, 3)).astype(np.float32)
+    b = rng.standard_normal(4).astype(np.float32)
+    down = oracle_mod.conv2d_down(x, w, b)
+    assert down.shape == (4, 4, 5)
+    full = oracle_mod.conv2d(x, w, b, 1)                 # full[y, x] reads rows y-1..y+1
+    np.testing.assert_allclose(down, full[:, 1::2, 1::2], rtol=1e-5, atol=1e-5)
+    # a kernel with a single 1 at (ky, kx) picks in[2y+ky, 2x+kx]
+    for ky, kx in ((0, 0), (2, 1), (2, 2)):
+        w1 = np.zeros((1, 1, 3, 3), np.float32)
+        w1[0, 0, ky, kx] = 1.0
+        xp = np.zeros((9, 11), np.float32)
+        xp[:8, :10] = x[0]
+        np.testing.assert_array_equal(oracle_mod.conv2d_down(x[:1], w1)[0], xp[ky::2, kx::2][:4, :5])
+    p = oracle_mod.patchify(x)
+    assert p.shape == (12, 4, 5)
+    np.testing.assert_array_equal(oracle_mod.unpatchify(p), x)
+    np.testing.assert_array_equal(p[2], x[0, 1::2, 0::2])
+    np.testing.assert_array_equal(p[4 + 1], x[1, 0::2, 1::2])
+
+
 def test_group_norm_statistics(oracle_mod):
     x = normal_f32((64, 6, 7), 2, 3, 1.5, 3.0)
     y = oracle_mod.group_norm(x, np.ones(64, np.float32), np.zeros(64, np.float32), 32, 1e-6)
