@@ -1,15 +1,16 @@
 /*
- * flux_vae_dropin.c - the reference's VAE entry points as flux.c binds them (flux.c:36-43)
- * with the decoder on the device: flux_vae_load_safetensors, flux_vae_decode, flux_vae_free.
+ * flux_vae_dropin.c - the reference's VAE entry points as flux.c binds them (flux.c:36-43) over
+ * the device VAE: flux_vae_load_safetensors, flux_vae_decode, flux_vae_encode, flux_vae_free.
  *
- * The encoder (image-to-image input) stays the reference's CPU code. An application keeps its
- * flux_vae.c and compiles that one file with
+ * An application keeps its flux_vae.c (flux_image_to_tensor lives there) and compiles that one
+ * file with
  *     -Dflux_vae_load_safetensors=flux_vae_load_safetensors_cpu
  *     -Dflux_vae_decode=flux_vae_decode_cpu -Dflux_vae_free=flux_vae_free_cpu
- * so that the three names resolve here. The handle handed back to flux.c is still the reference's
- * own flux_vae_t (flux_vae_encode needs it); the device decoder is kept beside it. Without a CPU
- * VAE in the link the handle is the device decoder itself.
- * There is no fallback: when the device decoder fails, flux_vae_decode returns NULL.
+ *     -Dflux_vae_encode=flux_vae_encode_cpu
+ * so that the four names resolve here. Leaving the last one out keeps the reference's CPU encoder:
+ * the handle handed back to flux.c is then the reference's own flux_vae_t, which that encoder
+ * needs, and the device VAE is kept beside it. Otherwise the handle is the device VAE itself.
+ * There is no fallback: when the device fails, flux_vae_decode and flux_vae_encode return NULL.
  */
 #include "../../include/flux_hip.h"
 #include "host_internal.h"
@@ -20,6 +21,7 @@ typedef struct { int width, height, channels; uint8_t *data; } dropin_image; /* 
 
 extern void *flux_vae_load_safetensors_cpu(void *sf) __attribute__((weak));
 extern void flux_vae_free_cpu(void *vae) __attribute__((weak));
+extern float *flux_vae_encode_cpu(void *vae, const float *img, int batch, int H, int W, int *out_h, int *out_w) __attribute__((weak));
 typedef void (*vae_progress_fn)(int block, int total);
 extern vae_progress_fn flux_vae_progress_callback __attribute__((weak)); /* flux_kernels.h:292-293 */
 
@@ -34,7 +36,7 @@ void *flux_vae_load_safetensors(void *sf) {
     flux_hip_vae *dev = flux_hip_vae_load_safetensors(sf);
     if (!dev) return NULL;
     void *handle = dev;
-    if (flux_vae_load_safetensors_cpu) {
+    if (flux_vae_load_safetensors_cpu && !flux_vae_encode_cpu) { /* the application's CPU encoder is in use */
         handle = flux_vae_load_safetensors_cpu(sf);
         if (!handle) { flux_hip_vae_free(dev); return NULL; }
     }
@@ -67,6 +69,24 @@ void *flux_vae_decode(void *vae, const float *latent, int batch, int latent_h, i
     flux_hip_vae_progress = NULL;
     if (!ok) { free(img->data); free(img); return NULL; }
     return img;
+}
+
+/* flux_vae_encode, flux_vae.c:320: image [1, 3, H, W] in [-1, 1] -> normalised latent
+ * [128, H/16, W/16], caller frees. */
+float *flux_vae_encode(void *vae, const float *img, int batch, int H, int W, int *out_h, int *out_w) {
+    const int slot = find_vae(vae);
+    if (slot < 0) { flux_hip_fail("flux_vae_encode: unknown VAE handle"); return NULL; }
+    if (batch != 1 || !img || !out_h || !out_w) { flux_hip_fail("flux_vae_encode: bad arguments (one image at a time)"); return NULL; }
+    if (H <= 0 || W <= 0 || (H & 15) || (W & 15)) { flux_hip_fail("flux_vae_encode: image %d x %d, sides must be multiples of 16", H, W); return NULL; }
+    float *latent = (float *)malloc(sizeof(float) * 128 * (size_t)(H / 16) * (W / 16));
+    if (!latent) return NULL;
+    flux_hip_vae_progress = &flux_vae_progress_callback ? flux_vae_progress_callback : NULL;
+    const int ok = flux_hip_vae_encode(g_vaes[slot].dev, img, H, W, latent);
+    flux_hip_vae_progress = NULL;
+    if (!ok) { free(latent); return NULL; }
+    *out_h = H / 16;
+    *out_w = W / 16;
+    return latent;
 }
 
 void flux_vae_free(void *vae) {

@@ -1,6 +1,7 @@
 /*
- * vae.hip - the memory-bound kernels of the VAE decoder (reference: flux_vae_decode,
- * flux_vae.c:690-837); its convolutions and attention products run as MFMA GEMMs (gemm.hip).
+ * vae.hip - the memory-bound kernels of the VAE decoder and encoder (reference: flux_vae_decode,
+ * flux_vae.c:690-837; flux_vae_encode, flux_vae.c:320-443); their convolutions and attention
+ * products run as MFMA GEMMs (gemm.hip).
  *
  * Images are channels-last with a one-pixel zero border: position p = y * Wp + x over the
  * (H+2) x (W+2) grid, channels contiguous. That makes a 3x3 convolution one GEMM whose K steps
@@ -236,6 +237,66 @@ __global__ __launch_bounds__(256) void vae_upsample_kernel(bf16 *__restrict__ ou
     *(bf16x4 *)(out + (size_t)p * C + q * 4) = o;
 }
 
+/* ---- encoder side (flux_vae_encode, flux_vae.c:320-443) ---- */
+
+/* image [3, H, W] fp32 -> the 3x3 neighbourhood of every position as one row of 64 bf16:
+ * element (ky*3 + kx)*3 + c = img[c, y-1+ky, x-1+kx] (zero outside the image), elements 27..63
+ * zero. The first convolution (3 -> 128 channels, flux_vae.c:336-338) is then a GEMM with K = 64
+ * over these rows. Four positions per workgroup of 256 threads. */
+__global__ __launch_bounds__(256) void vae_image_in_kernel(bf16 *__restrict__ out, const float *__restrict__ img, int H, int W) {
+    const int wp = W + 2, rows = (H + 2) * wp;
+    const int p = blockIdx.x * 4 + (threadIdx.x >> 6), k = threadIdx.x & 63;
+    if (p >= rows) return;
+    float v = 0.0f;
+    if (k < 27) {
+        const int tap = k / 3, c = k - tap * 3, ky = tap / 3, kx = tap - ky * 3;
+        const int py = p / wp, px = p - py * wp;
+        const int y = py - 2 + ky, x = px - 2 + kx; /* image coordinates: bordered position minus 1, tap offset minus 1 */
+        if (y >= 0 && y < H && x >= 0 && x < W) v = img[((size_t)c * H + y) * W + x];
+    }
+    out[(size_t)p * 64 + k] = (bf16)v;
+}
+
+/* The downsampling step (flux_vae.c:363-377: one row of zeros below and one column on the right,
+ * then a 3x3 convolution with stride 2): fp32 [hp*wp, C] -> bf16 [hp2*wp2, 9*C] over the bordered
+ * half-size grid, row (y', x') holding in[2(y'-1)+ky, 2(x'-1)+kx] for the nine taps, tap-major,
+ * so that the convolution is a GEMM with K = 9*C over these rows. The input's own zero border
+ * supplies the padding: the furthest row read is its bottom border. Border rows of the output
+ * are zero. One thread per (position, tap, 4 channels). */
+__global__ __launch_bounds__(256) void vae_downsample_gather_kernel(bf16 *__restrict__ out, const float *__restrict__ x, int hp, int wp, int C) {
+    const int quads = C >> 2;
+    const int H2 = (hp - 2) >> 1, W2 = (wp - 2) >> 1, hp2 = H2 + 2, wp2 = W2 + 2;
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)hp2 * wp2 * 9 * quads) return;
+    const int q = (int)(idx % quads);
+    const size_t pt = idx / quads;
+    const int tap = (int)(pt % 9), p = (int)(pt / 9);
+    const int y = p / wp2, xx = p - y * wp2;
+    bf16x4 o = {(bf16)0.0f, (bf16)0.0f, (bf16)0.0f, (bf16)0.0f};
+    if (y >= 1 && y <= H2 && xx >= 1 && xx <= W2) {
+        const int ky = tap / 3, kx = tap - ky * 3;
+        const int sy = 2 * (y - 1) + ky + 1, sx = 2 * (xx - 1) + kx + 1; /* bordered input coordinates, at most hp-1 / wp-1 */
+        const f32x4 v = *(const f32x4 *)(x + ((size_t)sy * wp + sx) * C + q * 4);
+#pragma unroll
+        for (int e = 0; e < 4; e++) o[e] = (bf16)v[e];
+    }
+    *(bf16x4 *)(out + ((size_t)p * 9 + tap) * C + q * 4) = o;
+}
+
+/* Output of the quant convolution, fp32 [(2h+2)*(2w+2), ldx] (channels 0..31 = the posterior's
+ * mean, flux_vae.c:411-424) -> 2x2 patchify to 128 channels (flux_kernels.c:1038-1065) ->
+ * (v - running_mean) / sqrt(running_var + eps) (flux_kernels.c:555-575) -> latent [128, h, w]. */
+__global__ __launch_bounds__(256) void vae_latent_out_kernel(float *__restrict__ latent, const float *__restrict__ x, int ldx,
+                                                             const float *__restrict__ bn_mean, const float *__restrict__ bn_var, int h, int w,
+                                                             float eps) {
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= 128 * h * w) return;
+    const int lc = idx / (h * w), r = idx - lc * (h * w), ph = r / w, pw = r - ph * w;
+    const int c = lc >> 2, pi = (lc >> 1) & 1, pj = lc & 1, wp = 2 * w + 2;
+    const float v = x[((size_t)(2 * ph + pi + 1) * wp + (2 * pw + pj + 1)) * ldx + c];
+    latent[idx] = (v - bn_mean[lc]) / sqrtf(bn_var[lc] + eps);
+}
+
 /* ---- attention over all positions with one head (attnblock_forward, flux_vae.c:223-313).
  * Scores are materialised, as in the reference: S = q k^T (GEMM), P = softmax(S * scale + bias)
  * (below), O = P v (GEMM against v^T). Keys run over the bordered grid plus padding up to a
@@ -382,6 +443,31 @@ extern "C" int flux_hip_upsample2x(void *out_bf16, const float *x, int hp, int w
     hipLaunchKernelGGL(vae_upsample_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, flux_hip_stream_handle(), (bf16 *)out_bf16, x, hp,
                        wp, C);
     LAUNCH_OK("vae_upsample_kernel");
+    return 1;
+}
+
+extern "C" int flux_hip_vae_image_in(void *out_bf16, const float *img, int H, int W) {
+    if (H <= 0 || W <= 0) return flux_hip_fail("flux_hip_vae_image_in: bad shape");
+    const int rows = (H + 2) * (W + 2);
+    hipLaunchKernelGGL(vae_image_in_kernel, dim3((rows + 3) / 4), dim3(256), 0, flux_hip_stream_handle(), (bf16 *)out_bf16, img, H, W);
+    LAUNCH_OK("vae_image_in_kernel");
+    return 1;
+}
+
+extern "C" int flux_hip_downsample_gather(void *out_bf16, const float *x, int hp, int wp, int C) {
+    if (C <= 0 || (C & 3) || hp < 4 || wp < 4 || ((hp | wp) & 1)) return flux_hip_fail("flux_hip_downsample_gather: bad shape (the image must have even sides)");
+    const size_t total = (size_t)((hp - 2) / 2 + 2) * ((wp - 2) / 2 + 2) * 9 * (C / 4);
+    hipLaunchKernelGGL(vae_downsample_gather_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, flux_hip_stream_handle(), (bf16 *)out_bf16,
+                       x, hp, wp, C);
+    LAUNCH_OK("vae_downsample_gather_kernel");
+    return 1;
+}
+
+extern "C" int flux_hip_vae_latent_out(float *latent, const float *x, int ldx, const float *bn_mean, const float *bn_var, int h, int w, float eps) {
+    if (h <= 0 || w <= 0 || ldx < 32) return flux_hip_fail("flux_hip_vae_latent_out: bad shape");
+    hipLaunchKernelGGL(vae_latent_out_kernel, dim3((128 * h * w + 255) / 256), dim3(256), 0, flux_hip_stream_handle(), latent, x, ldx, bn_mean,
+                       bn_var, h, w, eps);
+    LAUNCH_OK("vae_latent_out_kernel");
     return 1;
 }
 

@@ -147,6 +147,10 @@ def lib():
     L.flux_hip_vae_free.argtypes = [vp]
     L.flux_hip_vae_decode.argtypes = [vp, vp, c_i, c_i, vp, vp]
     L.flux_hip_vae_set_attention_chunk.argtypes = [c_i]
+    L.flux_hip_vae_encode.argtypes = [vp, vp, c_i, c_i, vp]
+    L.flux_hip_vae_image_in.argtypes = [vp, vp, c_i, c_i]
+    L.flux_hip_downsample_gather.argtypes = [vp, vp, c_i, c_i, c_i]
+    L.flux_hip_vae_latent_out.argtypes = [vp, vp, c_i, vp, vp, c_i, c_i, c_f]
     L.flux_hip_rms_norm.argtypes = [vp, vp, vp, c_i, c_i, c_f]
     L.flux_hip_causal_attention.argtypes = [vp, vp, vp, c_i, vp, c_i, c_i, c_i]
     L.flux_hip_qwen3_new.restype = vp
@@ -432,7 +436,7 @@ def randn(n, seed=None):
 
 
 class Vae:
-    """The VAE decoder on the GPU, built from named tensors (uint16 = bf16, float32) or a safetensors file."""
+    """The VAE (decoder and encoder) on the GPU, built from named tensors (uint16 = bf16, float32) or a safetensors file."""
 
     def __init__(self, weights=None, path=None):
         init()
@@ -469,6 +473,15 @@ class Vae:
         u = np.empty((16 * h, 16 * w, 3), np.uint8)
         check(lib().flux_hip_vae_decode(self.h, latent.ctypes.data, h, w, u.ctypes.data, f.ctypes.data), "flux_hip_vae_decode")
         return f, u
+
+    def encode(self, img):
+        """img [3, H, W] in [-1, 1], H and W multiples of 16 -> normalised latent [128, H/16, W/16]."""
+        img = _f32(img)
+        assert img.ndim == 3 and img.shape[0] == 3
+        H, W = img.shape[1], img.shape[2]
+        lat = np.empty((128, max(H // 16, 1), max(W // 16, 1)), np.float32)
+        check(lib().flux_hip_vae_encode(self.h, img.ctypes.data, H, W, lat.ctypes.data), "flux_hip_vae_encode")
+        return lat
 
 
 class Qwen3:

@@ -334,9 +334,10 @@ int flux_hip_softmax_rows(void *p_bf16, const float *s, const float *key_bias, i
 int flux_hip_transpose_bf16(void *vt, int ld, const void *v, int ldv, int rows, int cols);
 
 typedef struct flux_hip_vae flux_hip_vae;
-/* Decoder weights from a VAE .safetensors file (tensor names as flux_vae_load_safetensors reads
- * them, flux_vae.c:1232-1330; encoder tensors are skipped), or from the reference's parsed-file
- * handle (safetensors_file_t *). NULL on failure. */
+/* VAE weights from a .safetensors file (tensor names as flux_vae_load_safetensors reads them,
+ * flux_vae.c:1232-1330), or from the reference's parsed-file handle (safetensors_file_t *). The
+ * decoder's tensors must all be there; a file without the encoder's loads, and encoding with it
+ * fails. NULL on failure. */
 flux_hip_vae *flux_hip_vae_load_file(const char *path);
 flux_hip_vae *flux_hip_vae_load_safetensors(void *safetensors_file);
 /* Piecewise construction: new, then one set_tensor per tensor (dtype 0 = f32, 1 = f16, 2 = bf16). */
@@ -346,17 +347,32 @@ void flux_hip_vae_free(flux_hip_vae *v);
 /* latent f32 [128, h, w] (host) -> rgb u8 [16h, 16w, 3] and/or rgb_f32 [3, 16h, 16w] (decoder output
  * before the conversion to 8 bits); either may be NULL. h, w <= 112. 1 = ok, 0 = failed. */
 int flux_hip_vae_decode(flux_hip_vae *v, const float *latent, int h, int w, uint8_t *rgb, float *rgb_f32);
+/* image f32 [3, H, W] in [-1, 1] (host; H, W multiples of 16, at most 1792) -> normalised latent f32
+ * [128, H/16, W/16] (host): flux_vae_encode, flux_vae.c:320-443, for one image. A residual block
+ * that widens computes skip + conv2(...) as written; the reference's plain-C build overwrites part
+ * of that convolution's input while it runs (flux_vae.c:203 with flux_kernels.c:441-470), its
+ * BLAS path in one tile does not. 1 = ok, 0 = failed. */
+int flux_hip_vae_encode(flux_hip_vae *v, const float *img, int H, int W, float *latent);
+/* Encoder pieces: img f32 [3, H, W] (device) -> bf16 [(H+2)*(W+2), 64], the 27 values under every
+ * 3x3 window first (conv_in as a GEMM with K = 64, flux_vae.c:336); x f32 [hp*wp, C] -> bf16
+ * [(H/2+2)*(W/2+2), 9*C], the nine taps of the stride-2 convolution side by side
+ * (flux_vae.c:363-377); quant-convolution output f32 [(2h+2)*(2w+2), ldx] -> latent f32 [128, h, w]
+ * (mean channels, patchify, latent normalisation, flux_vae.c:411-437). */
+int flux_hip_vae_image_in(void *out_bf16, const float *img, int H, int W);
+int flux_hip_downsample_gather(void *out_bf16, const float *x, int hp, int wp, int C);
+int flux_hip_vae_latent_out(float *latent, const float *x, int ldx, const float *bn_mean, const float *bn_var, int h, int w, float eps);
 /* Test hook: at most `rows` query rows per attention chunk (0 = default: 1 GB of fp32 scores per chunk). */
 void flux_hip_vae_set_attention_chunk(int rows);
-/* When set, called after each of the decoder's 15 blocks has been queued (role of
+/* When set, called after each of the decoder's 15 / the encoder's 11 blocks has been queued (role of
  * flux_vae_progress_callback, flux_kernels.h:292-293). */
 extern void (*flux_hip_vae_progress)(int block, int total);
 
-/* The reference's own VAE entry points (flux.c:36-43) over the device decoder; see
- * flux_vae_dropin.c for how an application keeps its CPU encoder beside them. The handles are
- * flux_vae_t * / flux_image * / safetensors_file_t * in the reference's headers. */
+/* The reference's own VAE entry points (flux.c:36-43) over the device VAE; see flux_vae_dropin.c
+ * for how an application links them (and how it keeps its CPU encoder if it wants to). The
+ * handles are flux_vae_t * / flux_image * / safetensors_file_t * in the reference's headers. */
 void *flux_vae_load_safetensors(void *safetensors_file);
 void *flux_vae_decode(void *vae, const float *latent, int batch, int latent_h, int latent_w);
+float *flux_vae_encode(void *vae, const float *img, int batch, int H, int W, int *out_h, int *out_w);
 void flux_vae_free(void *vae);
 
 /* ---------------------------------------------------------------- Qwen3 text encoder

@@ -1,13 +1,15 @@
-"""GPU parity tests of the VAE decoder: its operators through the C ABI against the CPU oracle
-(oracle/vae_oracle.c), and the whole decoder against the oracle and against the images the
-reference's own flux_vae_decode produced (tests/golden/vae.npz).
+"""GPU parity tests of the VAE: its operators through the C ABI against the CPU oracle
+(oracle/vae_oracle.c), the whole decoder against the oracle and against the images the
+reference's own flux_vae_decode produced (tests/golden/vae.npz), and the whole encoder against the
+oracle.
 
 Tolerances. Operators take bf16 inputs (the same rounded values go to the oracle) and accumulate in
 fp32: 2e-6 relative for fp32 outputs, 4e-3 for bf16 outputs (one rounding, 2^-9 per element).
 The decoder keeps its residual stream in fp32 and rounds what feeds each convolution to bf16
 (about 30 layers): the unquantised image must agree with the fp32 oracle to 2e-2 relative L2,
 the 8-bit image to a mean absolute difference of 1.5 levels (the reference's own end-to-end threshold
-is 20, run_test.py:96-104).
+is 20, run_test.py:96-104). The encoder is built the same way (about 25 layers): its latent, a
+quantity of unit scale, must agree with the fp32 oracle to 2e-2 relative L2.
 """
 import os
 
@@ -15,7 +17,7 @@ import numpy as np
 import pytest
 
 from metrics import rel_l2
-from model_spec import normal_f32, f32_to_bf16, bf16_to_f32, make_vae_weights
+from model_spec import normal_f32, f32_to_bf16, bf16_to_f32, make_vae_weights, vae_test_image
 
 pytestmark = pytest.mark.gpu
 
@@ -323,6 +325,118 @@ def test_vae_decode_large(vae_pair, side):
     diff = np.abs(u.astype(np.int32) - uo.astype(np.int32))
     print(f"vae decode {16 * side}^2: rel_l2={r:.3e} mean|d|={diff.mean():.3f} max|d|={diff.max()}", flush=True)
     assert r <= 2e-2 and diff.mean() <= 1.5
+
+
+# ---- encoder ----
+
+def test_encoder_input_rows(hip):
+    """Every position's 3x3 window over the three colour planes, tap-major, in one row of 64."""
+    H, W = 6, 9
+    img = normal_f32((3, H, W), 61, 1)
+    rows = (H + 2) * (W + 2)
+    out = hip.DevBuf.from_array(np.full((rows, 64), 0x4040, np.uint16))
+    dimg = hip.DevBuf.from_array(img)
+    hip.check(hip.lib().flux_hip_vae_image_in(out.ptr, dimg.ptr, H, W))
+    got = bf16_to_f32(out.to_array(np.uint16, (rows, 64))).reshape(H + 2, W + 2, 64)
+    pad = np.zeros((3, H + 4, W + 4), np.float32)
+    pad[:, 2:-2, 2:-2] = img
+    want = np.zeros((H + 2, W + 2, 64), np.float32)
+    for ky in range(3):
+        for kx in range(3):
+            for c in range(3):
+                want[:, :, (ky * 3 + kx) * 3 + c] = pad[c, ky:ky + H + 2, kx:kx + W + 2]
+    np.testing.assert_array_equal(got, q(want))
+
+
+@pytest.mark.parametrize("shape", [(128, 8, 6), (256, 4, 10)])
+def test_downsample_step(hip, oracle_mod, shape):
+    """Gather of the nine stride-2 taps + one GEMM over K = 9 C against the oracle's downsampling convolution."""
+    C, H, W = shape
+    cout = 128
+    x = q(normal_f32((C, H, W), 62, 1))
+    w = q(normal_f32((cout, C, 3, 3), 62, 2, 0.0, 0.05))
+    b = normal_f32((cout,), 62, 3)
+    L = hip.lib()
+    H2, W2 = H // 2, W // 2
+    rows2 = (H2 + 2) * (W2 + 2)
+    a = hip.DevBuf.from_array(np.full((rows2, 9 * C), 0x4040, np.uint16))
+    dx = hip.DevBuf.from_array(to_padded(x))
+    hip.check(L.flux_hip_downsample_gather(a.ptr, dx.ptr, H + 2, W + 2, C))
+    ga = bf16_to_f32(a.to_array(np.uint16, (rows2, 9 * C))).reshape(H2 + 2, W2 + 2, 9, C)
+    assert not (ga[0].any() or ga[-1].any() or ga[:, 0].any() or ga[:, -1].any())
+    xp = np.zeros((C, H + 1, W + 1), np.float32)
+    xp[:, :H, :W] = x
+    for ky in range(3):
+        for kx in range(3):
+            np.testing.assert_array_equal(ga[1:-1, 1:-1, ky * 3 + kx].transpose(2, 0, 1), xp[:, ky:ky + H:2, kx:kx + W:2][:, :H2, :W2])
+    out = hip.DevBuf.from_array(np.full((rows2, cout), 3.0, np.float32))
+    dw, db = hip.DevBuf.from_array(conv_weight(w)), hip.DevBuf.from_array(b)
+    hip.check(L.flux_hip_conv(hip.EPI_CONV_F32, a.ptr, dw.ptr, db.ptr, None, out.ptr, rows2, W2 + 2, 9 * C, cout, 1))
+    got = out.to_array(np.float32, (rows2, cout))
+    assert border_is_zero(got, H2, W2)
+    assert rel_l2(from_padded(got, H2, W2), oracle_mod.conv2d_down(x, w, b)) <= 2e-6
+
+
+def test_encoder_latent_out(hip, oracle_mod):
+    """Mean channels -> 2x2 patchify -> latent normalisation."""
+    h, w, ldx = 3, 5, 64
+    x = normal_f32((ldx, 2 * h, 2 * w), 63, 1)
+    mean, var = normal_f32((128,), 63, 2), 1.0 + np.abs(normal_f32((128,), 63, 3))
+    lat = hip.DevBuf.from_array(np.zeros((128, h, w), np.float32))
+    dx, dm, dv = hip.DevBuf.from_array(to_padded(x)), hip.DevBuf.from_array(mean), hip.DevBuf.from_array(var)
+    hip.check(hip.lib().flux_hip_vae_latent_out(lat.ptr, dx.ptr, ldx, dm.ptr, dv.ptr, h, w, 1e-4))
+    want = (oracle_mod.patchify(x[:32]) - mean[:, None, None]) / np.sqrt(var + np.float32(1e-4))[:, None, None]
+    np.testing.assert_allclose(lat.to_array(np.float32, (128, h, w)), want, rtol=2e-6, atol=2e-6)
+
+
+@pytest.mark.parametrize("case", [(32, 32, 311), (48, 32, 312), (64, 112, 313), (256, 256, 314)])
+def test_vae_encode(vae_pair, case):
+    dev, cpu = vae_pair
+    H, W, seed = case
+    img = vae_test_image(H, W, seed)
+    got, want = dev.encode(img), cpu.encode(img)
+    r = rel_l2(got, want)
+    print(f"vae encode {H}x{W}: rel_l2={r:.3e} max|d|={np.abs(got - want).max():.3e} std={want.std():.3f}", flush=True)
+    assert got.shape == (128, H // 16, W // 16) and want.std() > 0.2
+    assert r <= 2e-2
+
+
+def test_vae_encode_after_decode(vae_pair):
+    """Encoder and decoder share their work buffers; neither depends on what ran before."""
+    dev, cpu = vae_pair
+    img = vae_test_image(64, 48, 315)
+    a = dev.encode(img)
+    dev.decode(normal_f32((128, 5, 4), 305, 1), 5, 4)
+    dev.encode(vae_test_image(96, 96, 316))
+    np.testing.assert_array_equal(dev.encode(img), a)
+
+
+@pytest.mark.parametrize("side", [512, 1024])
+def test_vae_encode_large(vae_pair, side):
+    """Full-size encodes against the oracle (chunked attention at 1024; about half a minute of CPU work on 16 cores)."""
+    dev, cpu = vae_pair
+    img = vae_test_image(side, side, 317)
+    got, want = dev.encode(img), cpu.encode(img)
+    r = rel_l2(got, want)
+    print(f"vae encode {side}^2: rel_l2={r:.3e} max|d|={np.abs(got - want).max():.3e}", flush=True)
+    assert r <= 2e-2
+
+
+def test_vae_encode_errors(hip, vae_pair):
+    dev, _ = vae_pair
+    L = hip.lib()
+    lat = np.zeros((128, 4, 4), np.float32)
+    img = np.zeros((3, 40, 32), np.float32)
+    assert L.flux_hip_vae_encode(dev.h, img.ctypes.data, 40, 32, lat.ctypes.data) == 0      # 40 is not a multiple of 16
+    assert b"multiples of 16" in L.flux_hip_last_error()
+    assert L.flux_hip_vae_encode(dev.h, None, 32, 32, lat.ctypes.data) == 0
+    W = {k: v for k, v in make_vae_weights().items() if not (k.startswith("encoder.") or k.startswith("quant_conv"))}
+    v = hip.Vae(W)                                                                          # a decoder-only file
+    f, u = v.decode(normal_f32((128, 2, 2), 301, 1), 2, 2)
+    assert np.isfinite(f).all()
+    assert L.flux_hip_vae_encode(v.h, np.zeros((3, 32, 32), np.float32).ctypes.data, 32, 32, lat.ctypes.data) == 0
+    assert b"encoder." in L.flux_hip_last_error()
+    v.close()
 
 
 def test_vae_missing_tensor_fails(hip):
