@@ -129,11 +129,11 @@ def test_reference_cli_links_against_the_library():
         assert re.search(rf"\bU {name}\b", syms), name
     for name in ("flux_vae_decode_cpu", "flux_vae_encode", "flux_generate_with_embeddings"):
         assert re.search(rf"\bT {name}\b", syms), name
-    # all three stages from the backend: flux_qwen3.c is left out, the tokenizer stays
+    # all stages from the backend: the VAE encoder is an import too, flux_qwen3.c is left out, the tokenizer stays
     r = subprocess.run(["make", "-C", os.path.join(ROOT, "oracle"), "pipeline_gpuall"], capture_output=True, text=True)
     assert r.returncode == 0 and "linked _ref/libfluxpipe_gpuall.so" in r.stdout, r.stdout + r.stderr
     syms = subprocess.run(["nm", "-D", os.path.join(ROOT, "oracle", "_ref", "libfluxpipe_gpuall.so")], capture_output=True, text=True).stdout
-    for name in ("qwen3_encoder_load", "qwen3_encode_text", "qwen3_encoder_free", "flux_vae_decode", "flux_sample_euler"):
+    for name in ("qwen3_encoder_load", "qwen3_encode_text", "qwen3_encoder_free", "flux_vae_decode", "flux_vae_encode", "flux_sample_euler"):
         assert re.search(rf"\bU {name}\b", syms), name
-    for name in ("qwen3_tokenizer_load", "qwen3_tokenize_chat", "flux_generate"):
+    for name in ("qwen3_tokenizer_load", "qwen3_tokenize_chat", "flux_generate", "flux_img2img", "flux_image_to_tensor"):
         assert re.search(rf"\bT {name}\b", syms), name

@@ -231,7 +231,18 @@ ctypes.c_void_p.in_dll(P, "flux_text_progress_callback").value = ctypes.cast(cb,
 ctx = P.flux_load_dir(model_dir.encode())
 assert ctx, P.flux_get_error()
 prm = FluxParams(width, height, steps, seed, 0.0, 0, 0, 2.0)
-img_p = P.flux_generate(ctx, prompt.encode(), ctypes.byref(prm))
+if len(sys.argv) > 9:                                  # image-to-image: the input picture as uint8 [H, W, 3]
+    src = np.ascontiguousarray(np.load(sys.argv[9]))
+    P.flux_img2img.restype = vp
+    P.flux_img2img.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(FluxImage), ctypes.POINTER(FluxParams)]
+    blocks = []
+    vcb = CB(lambda b, t: blocks.append((b, t)))
+    ctypes.c_void_p.in_dll(P, "flux_vae_progress_callback").value = ctypes.cast(vcb, vp).value
+    inp = FluxImage(src.shape[1], src.shape[0], 3, src.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)))
+    img_p = P.flux_img2img(ctx, prompt.encode(), ctypes.byref(inp), ctypes.byref(prm))
+    assert (0, 11) in blocks and (10, 11) in blocks and (14, 15) in blocks, blocks[:4]   # encoder's 11 blocks, then the decoder's 15
+else:
+    img_p = P.flux_generate(ctx, prompt.encode(), ctypes.byref(prm))
 assert img_p, P.flux_get_error()
 im = ctypes.cast(img_p, ctypes.POINTER(FluxImage)).contents
 np.save(out, np.ctypeslib.as_array(im.data, shape=(im.height, im.width, im.channels)).copy())
@@ -259,15 +270,18 @@ def _byte_level_tokenizer_json():
 
 
 @pytest.mark.skipif(not (os.path.exists(PIPE_GPUALL) and os.path.exists(REF)), reason="reference-built libraries not present")
-@pytest.mark.parametrize("distilled", [True, False])
-def test_prompt_to_image_with_all_stages_on_the_device(oracle_mod, tmp_path, distilled):
-    """flux_generate(ctx, prompt) through the reference's flux.c: its tokenizer on the CPU, then text encoder,
-    denoising loop (Euler, or CFG with the empty prompt for a non-distilled model) and VAE decoder on the
-    device. Expected image: the reference's tokenizer, then the CPU oracles of the three stages."""
+@pytest.mark.parametrize("mode", ["distilled", "cfg", "img2img", "img2img_cfg"])
+def test_prompt_to_image_with_all_stages_on_the_device(oracle_mod, tmp_path, mode):
+    """flux_generate(ctx, prompt) / flux_img2img(ctx, prompt, picture) through the reference's flux.c: its
+    tokenizer on the CPU, then text encoder, (VAE encoder of the input picture,) denoising loop (Euler, or
+    CFG with the empty prompt for a non-distilled model; the picture's latent as reference tokens) and VAE
+    decoder on the device. Expected image: the reference's tokenizer, then the CPU oracles of the stages."""
     import subprocess
     import sys
     from dataclasses import replace
-    from model_spec import QwenConfig, make_qwen3_weights
+    from model_spec import QwenConfig, make_qwen3_weights, vae_test_image
+    distilled = mode in ("distilled", "img2img")
+    img2img = mode.startswith("img2img")
     cfg = SMALL
     qcfg = QwenConfig(hidden=cfg.text_dim // 3, intermediate=384, heads=4, kv_heads=2, layers=27, vocab=151936)
     W, VW, QW = make_weights(cfg, 42, 0.05, "sharp"), make_vae_weights(), make_qwen3_weights(qcfg)
@@ -283,8 +297,13 @@ def test_prompt_to_image_with_all_stages_on_the_device(oracle_mod, tmp_path, dis
     (tmp_path / "model_index.json").write_text('{"is_distilled": true}' if distilled else '{"_class_name": "Flux2Pipeline"}')
     width, height, steps, seed, prompt = 64, 64, 3, 21, "a small red fox"
     out = str(tmp_path / "img.npy")
+    extra = []
+    if img2img:                                      # the input picture, 8 bits per channel, at the output size
+        picture = np.clip((vae_test_image(height, width, 41).transpose(1, 2, 0) + 1.0) * 127.5, 0, 255).astype(np.uint8)
+        np.save(str(tmp_path / "input.npy"), picture)
+        extra = [str(tmp_path / "input.npy")]
     r = subprocess.run([sys.executable, "-c", _CHILD_PROMPT, PIPE_GPUALL, str(tmp_path), out,
-                        str(width), str(height), str(steps), str(seed), prompt], capture_output=True, text=True, timeout=900)
+                        str(width), str(height), str(steps), str(seed), prompt] + extra, capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, r.stdout + r.stderr
     got = np.load(out)
 
@@ -315,20 +334,34 @@ def test_prompt_to_image_with_all_stages_on_the_device(oracle_mod, tmp_path, dis
     q.close()
     R.qwen3_tokenizer_free(tok)
     lh, lw = height // 16, width // 16
+    vo = oracle_mod.VaeOracle(VW)
+    refs = None
+    if img2img:
+        # flux_image_to_tensor (flux_vae.c:1110-1135), the encoder, and the latent as reference tokens at time offset 10 (flux.c:806)
+        tensor = (picture.astype(np.float32) / np.float32(255.0) * np.float32(2.0) - np.float32(1.0)).transpose(2, 0, 1)
+        refs = [(vo.encode(tensor), lh, lw, 10)]
     o = oracle_mod.Oracle(cfg, W)
     z0 = oracle_mod.init_noise(cfg.channels, lh, lw, seed)
     sched = oracle_mod.official_schedule(steps, lh * lw)
     if distilled:
-        latent = o.sample_euler(z0, lh, lw, emb, sched)
+        latent = o.sample_euler(z0, lh, lw, emb, sched, refs=refs)
     else:
-        latent = o.sample_euler_cfg(z0, lh, lw, emb, emb_u, 4.0, sched)    # default guidance of a base model, flux.c:222
+        latent = o.sample_euler_cfg(z0, lh, lw, emb, emb_u, 4.0, sched, refs=refs)    # default guidance of a base model, flux.c:222
+    if img2img:                                      # the picture matters: without it the expected image is another one
+        plain = o.sample_euler(z0, lh, lw, emb, sched) if distilled else o.sample_euler_cfg(z0, lh, lw, emb, emb_u, 4.0, sched)
+        _, other = vo.decode(plain, lh, lw)
     o.close()
-    vo = oracle_mod.VaeOracle(VW)
     _, want = vo.decode(latent, lh, lw)
     vo.close()
+    if img2img:
+        effect = np.abs(want.astype(np.int32) - other.astype(np.int32)).mean()
+        print(f"effect of the input picture on the expected image: mean abs diff {effect:.2f}", flush=True)
+        assert effect > 1.5
     diff = np.abs(got.astype(np.int32) - want.astype(np.int32))
-    print(f"prompt -> image, all stages on the device (distilled={distilled}): mean abs diff {diff.mean():.3f}, max {diff.max()}, "
+    print(f"prompt -> image, all stages on the device ({mode}): mean abs diff {diff.mean():.3f}, max {diff.max()}, "
           f"image std {want.std():.1f}", flush=True)
     assert got.shape == (height, width, 3) and want.std() > 5.0
     assert diff.mean() <= 20.0                   # the reference's own acceptance threshold
     assert diff.mean() <= 2.0
+    if img2img:
+        assert diff.mean() <= 0.5 * effect       # well inside what the picture itself changes
