@@ -16,8 +16,9 @@ Also measured in the same run:
                 extrapolated to the 5 + 20 blocks of a step
 
 --workload vae_c2 | vae_c3 | vae_c4 measures the step after the sampling loop instead: one "step" is
-one VAE decode of a 16/32/64-wide latent to a 256/512/1024-pixel image. --workload qwen3 measures the
-step before it: one forward of the text encoder over 512 tokens.
+one VAE decode of a 16/32/64-wide latent to a 256/512/1024-pixel image; vae_enc_c2 | vae_enc_c3 |
+vae_enc_c4 the VAE encoder on a picture of those sizes (the input of image-to-image generation).
+--workload qwen3 measures the step before the loop: one forward of the text encoder over 512 tokens.
 """
 import argparse
 import json
@@ -114,57 +115,76 @@ def cpu_baseline(cfg, n_img, n_txt):
     }
 
 
-VAE_WORKLOADS = {"vae_c2": 16, "vae_c3": 32, "vae_c4": 64}   # latent side: 256^2, 512^2, 1024^2 images
+VAE_WORKLOADS = {"vae_c2": 16, "vae_c3": 32, "vae_c4": 64,   # latent side: 256^2, 512^2, 1024^2 images
+                 "vae_enc_c2": 16, "vae_enc_c3": 32, "vae_enc_c4": 64}   # the same sizes through the encoder
 
 
-def vae_cpu_baseline(flops_decode):
-    """The CPU oracle's decoder (OpenMP loops) on a 128x128 image; its FLOP rate carried to the
-    benchmarked size."""
+def vae_cpu_baseline(flops_step, encode=False):
+    """The CPU oracle's decoder / encoder (OpenMP loops) on a 128x128 (256x256) image; its FLOP rate
+    carried to the benchmarked size."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import oracle as O
-    from model_spec import make_vae_weights, vae_decode_flops
+    from model_spec import make_vae_weights, vae_decode_flops, vae_encode_flops, vae_test_image
     o = O.VaeOracle(make_vae_weights())
-    lat = normal_f32((128, 8, 8), 9, 1)
-    o.decode(normal_f32((128, 2, 2), 9, 2), 2, 2)
-    t0 = time.perf_counter()
-    o.decode(lat, 8, 8)
-    dt = time.perf_counter() - t0
+    if encode:
+        o.encode(vae_test_image(32, 32, 9))
+        img = vae_test_image(256, 256, 9)
+        t0 = time.perf_counter()
+        o.encode(img)
+        dt = time.perf_counter() - t0
+        rate, what, unit = vae_encode_flops(256, 256) / dt, "256x256 encode", "encodes/s"
+    else:
+        lat = normal_f32((128, 8, 8), 9, 1)
+        o.decode(normal_f32((128, 2, 2), 9, 2), 2, 2)
+        t0 = time.perf_counter()
+        o.decode(lat, 8, 8)
+        dt = time.perf_counter() - t0
+        rate, what, unit = vae_decode_flops(8, 8) / dt, "128x128 decode", "decodes/s"
     o.close()
-    rate = vae_decode_flops(8, 8) / dt
-    return {"value": rate / flops_decode, "unit": "decodes/s", "cores": O.lib().fo_num_threads(), "kind": "port",
-            "sample": f"one 128x128 decode ({dt:.1f} s, {rate / 1e9:.1f} GFLOP/s, OpenMP loops of the CPU oracle), "
+    return {"value": rate / flops_step, "unit": unit, "cores": O.lib().fo_num_threads(), "kind": "port",
+            "sample": f"one {what} ({dt:.1f} s, {rate / 1e9:.1f} GFLOP/s, OpenMP loops of the CPU oracle), "
                       f"carried to this size by FLOP count"}
 
 
 def bench_vae(args):
     """One step = one decode of a latent to an 8-bit image through flux_hip_vae_decode (host latent in,
-    host image out: 0.5 + 3 MB over PCIe at 1024^2, inside the timed region)."""
+    host image out: 0.5 + 3 MB over PCIe at 1024^2, inside the timed region), or (vae_enc_*) one encode
+    of an fp32 image to a latent through flux_hip_vae_encode (12.6 + 0.5 MB over PCIe at 1024^2)."""
     import ctypes
-    from model_spec import make_vae_weights, vae_decode_convs, vae_decode_flops
+    from model_spec import make_vae_weights, vae_decode_convs, vae_decode_flops, vae_encode_convs, vae_encode_flops, vae_test_image
     side = VAE_WORKLOADS[args.workload]
+    enc = args.workload.startswith("vae_enc")
     K, Wm = args.steps, args.warmup
     fluxhip.init()
     if args.tile_mask:
         fluxhip.lib().flux_hip_linear_tile_mask(args.tile_mask)
     v = fluxhip.Vae(make_vae_weights())
-    lat = normal_f32((128, side, side), 321, 1)
-    for _ in range(max(Wm, 1)):
-        f, u = v.decode(lat, side, side)
-    assert np.isfinite(f).all() and u.std() > 5.0
+    if enc:
+        img = vae_test_image(16 * side, 16 * side, 322)
+        step = lambda: v.encode(img)
+        for _ in range(max(Wm, 1)):
+            z = step()
+        assert np.isfinite(z).all() and z.std() > 0.2
+    else:
+        lat = normal_f32((128, side, side), 321, 1)
+        step = lambda: v.decode(lat, side, side)
+        for _ in range(max(Wm, 1)):
+            f, u = step()
+        assert np.isfinite(f).all() and u.std() > 5.0
     L = fluxhip.lib()
     if not args.no_kernel_timing:
         L.flux_hip_linear_probe(-2)          # events around every convolution launch
     t0 = time.perf_counter()
     for _ in range(K):
-        v.decode(lat, side, side)
+        step()
     wall = time.perf_counter() - t0
-    flops = vae_decode_flops(side, side)
+    flops = vae_encode_flops(16 * side, 16 * side) if enc else vae_decode_flops(side, side)
     roof = None
     if not args.no_kernel_timing:
         # launch i of a decode is convolution i of vae_decode_convs (after the post-quant one, which the
         # input kernel does); a kernel (= tile shape) runs layers of several shapes, so its figure is
         # (sum of its launches' algorithmic FLOPs) / (sum of their durations). Dominant = most time.
-        convs = vae_decode_convs(side, side)[1:]
+        convs = vae_encode_convs(16 * side, 16 * side) if enc else vae_decode_convs(side, side)[1:]
         cap = K * len(convs)
         tiles = np.zeros(cap, np.int32)
         ms = np.zeros(cap, np.float32)
@@ -182,17 +202,20 @@ def bench_vae(args):
                     "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": None,
                     "kernel": names.get(dom, f"tile {dom}") + ": 3x3 / 1x1 convolutions as GEMMs with bias, residual and border epilogue",
                     "launches_timed": t_n, "ms_per_launch": round(t_ms / t_n, 4), "flops_per_launch": t_fl / t_n,
-                    "launches_per_decode": t_n // K,
-                    "all_conv_kernels": {names.get(t, str(t)): {"launches_per_decode": c // K, "ms_per_decode": round(m / K, 3),
+                    "launches_per_step": t_n // K,
+                    "all_conv_kernels": {names.get(t, str(t)): {"launches_per_step": c // K, "ms_per_step": round(m / K, 3),
                                                                 "tflops": round(f / (m * 1e-3) / 1e12, 1)} for t, (m, f, c) in per_tile.items()}}
     v.close()
-    cpu = None if args.no_cpu_baseline else vae_cpu_baseline(flops)
+    cpu = None if args.no_cpu_baseline else vae_cpu_baseline(flops, enc)
+    what = "encodes" if enc else "decodes"
     print(json.dumps({
-        "metric": f"VAE decodes/s ({16 * side}x{16 * side} image, 1 GPU)", "value": round(K / wall, 3), "unit": "decodes/s",
+        "metric": f"VAE {what}/s ({16 * side}x{16 * side} image, 1 GPU)", "value": round(K / wall, 3), "unit": f"{what}/s",
         "n_gpus": 1, "steps": K, "warmup": Wm, "ms_per_step": round(wall * 1000.0 / K, 3), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: FLUX.2 VAE decoder (84 M parameters, random-init bf16), latent "
-                               f"[128,{side},{side}] -> {16 * side}x{16 * side} RGB, batch 1, host buffers in and out"},
+        "config": {"workload": (f"{args.workload}: FLUX.2 VAE encoder (random-init bf16), {16 * side}x{16 * side} RGB fp32 -> latent "
+                                f"[128,{side},{side}], batch 1, host buffers in and out") if enc else
+                               (f"{args.workload}: FLUX.2 VAE decoder (84 M parameters, random-init bf16), latent "
+                                f"[128,{side},{side}] -> {16 * side}x{16 * side} RGB, batch 1, host buffers in and out")},
         "tflops": round(flops * K / wall / 1e12, 1), "flops_per_step": flops, "roofline": roof, "cpu_baseline": cpu}))
 
 

@@ -242,19 +242,25 @@ __global__ __launch_bounds__(256) void vae_upsample_kernel(bf16 *__restrict__ ou
 /* image [3, H, W] fp32 -> the 3x3 neighbourhood of every position as one row of 64 bf16:
  * element (ky*3 + kx)*3 + c = img[c, y-1+ky, x-1+kx] (zero outside the image), elements 27..63
  * zero. The first convolution (3 -> 128 channels, flux_vae.c:336-338) is then a GEMM with K = 64
- * over these rows. Four positions per workgroup of 256 threads. */
+ * over these rows. 32 positions per workgroup of 256 threads. */
 __global__ __launch_bounds__(256) void vae_image_in_kernel(bf16 *__restrict__ out, const float *__restrict__ img, int H, int W) {
     const int wp = W + 2, rows = (H + 2) * wp;
-    const int p = blockIdx.x * 4 + (threadIdx.x >> 6), k = threadIdx.x & 63;
+    const int p = blockIdx.x * 32 + (threadIdx.x >> 3), k0 = (threadIdx.x & 7) * 8; /* eight elements (16 bytes) per thread */
     if (p >= rows) return;
-    float v = 0.0f;
-    if (k < 27) {
-        const int tap = k / 3, c = k - tap * 3, ky = tap / 3, kx = tap - ky * 3;
-        const int py = p / wp, px = p - py * wp;
-        const int y = py - 2 + ky, x = px - 2 + kx; /* image coordinates: bordered position minus 1, tap offset minus 1 */
-        if (y >= 0 && y < H && x >= 0 && x < W) v = img[((size_t)c * H + y) * W + x];
+    const int py = p / wp, px = p - py * wp;
+    bf16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const int k = k0 + e;
+        float v = 0.0f;
+        if (k < 27) {
+            const int tap = k / 3, c = k - tap * 3, ky = tap / 3, kx = tap - ky * 3;
+            const int y = py - 2 + ky, x = px - 2 + kx; /* image coordinates: bordered position minus 1, tap offset minus 1 */
+            if (y >= 0 && y < H && x >= 0 && x < W) v = img[((size_t)c * H + y) * W + x];
+        }
+        o[e] = (bf16)v;
     }
-    out[(size_t)p * 64 + k] = (bf16)v;
+    *(bf16x8 *)(out + (size_t)p * 64 + k0) = o;
 }
 
 /* The downsampling step (flux_vae.c:363-377: one row of zeros below and one column on the right,
@@ -449,7 +455,7 @@ extern "C" int flux_hip_upsample2x(void *out_bf16, const float *x, int hp, int w
 extern "C" int flux_hip_vae_image_in(void *out_bf16, const float *img, int H, int W) {
     if (H <= 0 || W <= 0) return flux_hip_fail("flux_hip_vae_image_in: bad shape");
     const int rows = (H + 2) * (W + 2);
-    hipLaunchKernelGGL(vae_image_in_kernel, dim3((rows + 3) / 4), dim3(256), 0, flux_hip_stream_handle(), (bf16 *)out_bf16, img, H, W);
+    hipLaunchKernelGGL(vae_image_in_kernel, dim3((rows + 31) / 32), dim3(256), 0, flux_hip_stream_handle(), (bf16 *)out_bf16, img, H, W);
     LAUNCH_OK("vae_image_in_kernel");
     return 1;
 }

@@ -286,6 +286,45 @@ def vae_decode_flops(h, w):
     return conv + 4.0 * n * n * 512
 
 
+def vae_encode_convs(H, W):
+    """The encoder's convolutions for an H x W image, in execution order (flux_vae_encode,
+    flux_vae.c:320-443): (name, output H, output W, cin, cout, taps); one flux_hip_conv launch each,
+    in this order."""
+    mult = [1, 2, 4, 4]
+    out = [("conv_in", H, W, 3, 128, 9)]
+
+    def res(name, i, o):
+        out.append((name + ".conv1", H, W, i, o, 9))
+        if i != o:
+            out.append((name + ".conv_shortcut", H, W, i, o, 1))
+        out.append((name + ".conv2", H, W, o, o, 9))
+
+    prev = 128
+    for lvl in range(4):
+        ch = 128 * mult[lvl]
+        for r in range(2):
+            res(f"down.{lvl}.{r}", prev if r == 0 else ch, ch)
+        if lvl < 3:
+            H, W = H // 2, W // 2
+            out.append((f"down.{lvl}.downsample", H, W, ch, ch, 9))
+        prev = ch
+    res("mid.0", 512, 512)
+    out.append(("mid.attn.to_qkv", H, W, 512, 1536, 1))
+    out.append(("mid.attn.to_out", H, W, 512, 512, 1))
+    res("mid.1", 512, 512)
+    out.append(("conv_out", H, W, 512, 64, 9))
+    out.append(("quant_conv", H, W, 64, 64, 1))
+    return out
+
+
+def vae_encode_flops(H, W):
+    """Algorithmic FLOPs of one encode: convolutions over the real image and channel counts, plus the
+    mid-block attention's two products over (H/8 * W/8) positions at width 512."""
+    conv = sum(2.0 * h * w * ci * co * t for _, h, w, ci, co, t in vae_encode_convs(H, W))
+    n = (H // 8) * (W // 8)
+    return conv + 4.0 * n * n * 512
+
+
 @dataclass(frozen=True)
 class QwenConfig:
     """Qwen3 text encoder (flux_qwen3.h:22-39): the hidden states after three layers, side by side,
