@@ -231,16 +231,22 @@ ctypes.c_void_p.in_dll(P, "flux_text_progress_callback").value = ctypes.cast(cb,
 ctx = P.flux_load_dir(model_dir.encode())
 assert ctx, P.flux_get_error()
 prm = FluxParams(width, height, steps, seed, 0.0, 0, 0, 2.0)
-if len(sys.argv) > 9:                                  # image-to-image: the input picture as uint8 [H, W, 3]
-    src = np.ascontiguousarray(np.load(sys.argv[9]))
-    P.flux_img2img.restype = vp
-    P.flux_img2img.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(FluxImage), ctypes.POINTER(FluxParams)]
+if len(sys.argv) > 9:                                  # image-to-image: the input pictures as uint8 [H, W, 3]
+    srcs = [np.ascontiguousarray(np.load(a)) for a in sys.argv[9:]]
     blocks = []
     vcb = CB(lambda b, t: blocks.append((b, t)))
     ctypes.c_void_p.in_dll(P, "flux_vae_progress_callback").value = ctypes.cast(vcb, vp).value
-    inp = FluxImage(src.shape[1], src.shape[0], 3, src.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)))
-    img_p = P.flux_img2img(ctx, prompt.encode(), ctypes.byref(inp), ctypes.byref(prm))
-    assert (0, 11) in blocks and (10, 11) in blocks and (14, 15) in blocks, blocks[:4]   # encoder's 11 blocks, then the decoder's 15
+    inps = [FluxImage(a.shape[1], a.shape[0], 3, a.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8))) for a in srcs]
+    if len(inps) == 1:
+        P.flux_img2img.restype = vp
+        P.flux_img2img.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(FluxImage), ctypes.POINTER(FluxParams)]
+        img_p = P.flux_img2img(ctx, prompt.encode(), ctypes.byref(inps[0]), ctypes.byref(prm))
+    else:
+        P.flux_multiref.restype = vp
+        P.flux_multiref.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(ctypes.POINTER(FluxImage)), c_i, ctypes.POINTER(FluxParams)]
+        arr = (ctypes.POINTER(FluxImage) * len(inps))(*[ctypes.pointer(i) for i in inps])
+        img_p = P.flux_multiref(ctx, prompt.encode(), arr, len(inps), ctypes.byref(prm))
+    assert blocks.count((0, 11)) == len(inps) and (10, 11) in blocks and (14, 15) in blocks, blocks[:4]   # encoder's 11 blocks per picture, then the decoder's 15
 else:
     img_p = P.flux_generate(ctx, prompt.encode(), ctypes.byref(prm))
 assert img_p, P.flux_get_error()
@@ -270,9 +276,10 @@ def _byte_level_tokenizer_json():
 
 
 @pytest.mark.skipif(not (os.path.exists(PIPE_GPUALL) and os.path.exists(REF)), reason="reference-built libraries not present")
-@pytest.mark.parametrize("mode", ["distilled", "cfg", "img2img", "img2img_cfg"])
+@pytest.mark.parametrize("mode", ["distilled", "cfg", "img2img", "img2img_cfg", "multiref"])
 def test_prompt_to_image_with_all_stages_on_the_device(oracle_mod, tmp_path, mode):
-    """flux_generate(ctx, prompt) / flux_img2img(ctx, prompt, picture) through the reference's flux.c: its
+    """flux_generate(ctx, prompt) / flux_img2img(ctx, prompt, picture) / flux_multiref(ctx, prompt, two pictures
+    of different sizes) through the reference's flux.c: its
     tokenizer on the CPU, then text encoder, (VAE encoder of the input picture,) denoising loop (Euler, or
     CFG with the empty prompt for a non-distilled model; the picture's latent as reference tokens) and VAE
     decoder on the device. Expected image: the reference's tokenizer, then the CPU oracles of the stages."""
@@ -280,8 +287,8 @@ def test_prompt_to_image_with_all_stages_on_the_device(oracle_mod, tmp_path, mod
     import sys
     from dataclasses import replace
     from model_spec import QwenConfig, make_qwen3_weights, vae_test_image
-    distilled = mode in ("distilled", "img2img")
-    img2img = mode.startswith("img2img")
+    distilled = mode in ("distilled", "img2img", "multiref")
+    img2img = mode.startswith("img2img") or mode == "multiref"
     cfg = SMALL
     qcfg = QwenConfig(hidden=cfg.text_dim // 3, intermediate=384, heads=4, kv_heads=2, layers=27, vocab=151936)
     W, VW, QW = make_weights(cfg, 42, 0.05, "sharp"), make_vae_weights(), make_qwen3_weights(qcfg)
@@ -298,10 +305,12 @@ def test_prompt_to_image_with_all_stages_on_the_device(oracle_mod, tmp_path, mod
     width, height, steps, seed, prompt = 64, 64, 3, 21, "a small red fox"
     out = str(tmp_path / "img.npy")
     extra = []
-    if img2img:                                      # the input picture, 8 bits per channel, at the output size
-        picture = np.clip((vae_test_image(height, width, 41).transpose(1, 2, 0) + 1.0) * 127.5, 0, 255).astype(np.uint8)
-        np.save(str(tmp_path / "input.npy"), picture)
-        extra = [str(tmp_path / "input.npy")]
+    pictures = []
+    if img2img:                                      # the input pictures, 8 bits per channel: one at the output size, or two of other sizes
+        for i, (ph, pw) in enumerate([(height, width)] if mode != "multiref" else [(48, 64), (32, 32)]):
+            pictures.append(np.clip((vae_test_image(ph, pw, 41 + i).transpose(1, 2, 0) + 1.0) * 127.5, 0, 255).astype(np.uint8))
+            np.save(str(tmp_path / f"input{i}.npy"), pictures[-1])
+            extra.append(str(tmp_path / f"input{i}.npy"))
     r = subprocess.run([sys.executable, "-c", _CHILD_PROMPT, PIPE_GPUALL, str(tmp_path), out,
                         str(width), str(height), str(steps), str(seed), prompt] + extra, capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, r.stdout + r.stderr
@@ -337,9 +346,11 @@ def test_prompt_to_image_with_all_stages_on_the_device(oracle_mod, tmp_path, mod
     vo = oracle_mod.VaeOracle(VW)
     refs = None
     if img2img:
-        # flux_image_to_tensor (flux_vae.c:1110-1135), the encoder, and the latent as reference tokens at time offset 10 (flux.c:806)
-        tensor = (picture.astype(np.float32) / np.float32(255.0) * np.float32(2.0) - np.float32(1.0)).transpose(2, 0, 1)
-        refs = [(vo.encode(tensor), lh, lw, 10)]
+        # flux_image_to_tensor (flux_vae.c:1110-1135), the encoder, and the latents as reference tokens at time offsets 10, 20 (flux.c:806, 987)
+        refs = []
+        for i, pic in enumerate(pictures):
+            tensor = (pic.astype(np.float32) / np.float32(255.0) * np.float32(2.0) - np.float32(1.0)).transpose(2, 0, 1)
+            refs.append((vo.encode(tensor), pic.shape[0] // 16, pic.shape[1] // 16, 10 * (i + 1)))
     o = oracle_mod.Oracle(cfg, W)
     z0 = oracle_mod.init_noise(cfg.channels, lh, lw, seed)
     sched = oracle_mod.official_schedule(steps, lh * lw)
