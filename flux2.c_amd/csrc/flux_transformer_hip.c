@@ -371,6 +371,10 @@ int fh_forward_device_n(flux_transformer_t *tf, int nb, const fh_rope *const *rp
     float *x = tf->x;
     const float *mt = mod_ptr(tf, 0, step), *mi = mod_ptr(tf, 1, step), *ms = mod_ptr(tf, 2, step), *mf = mod_ptr(tf, 3, step);
     flux_hip_linear_part p[4];
+    flux_hip_adaln_part an[4];
+    /* normed: xn already holds the AdaLN output that the next projection reads, written by the
+     * second pass of the residual projection before it (flux_hip_linear_resid_adaln) */
+    int normed = 0;
 
     if (ev) fh_event_record(ev, 0);
     /* inputs -> hidden (flux_transformer.c:3156-3196) */
@@ -383,7 +387,7 @@ int fh_forward_device_n(flux_transformer_t *tf, int nb, const fh_rope *const *rp
     /* double-stream blocks (flux_transformer.c:1774-1986); per sequence: text rows, then image rows */
     for (int i = 0; i < c->n_double; i++) {
         const fh_double *blk = &tf->dbl[i];
-        for (int b = 0; b < nb; b++)
+        for (int b = 0; b < nb && !normed; b++)
             if (!flux_hip_adaln_norm(xn + (size_t)R[b] * H * 2, H, x + (size_t)R[b] * H, N[b], H, Nt[b], mt, mt + H, mi, mi + H, eps)) return 0;
         for (int b = 0; b < nb; b++) {
             p[2 * b] = (flux_hip_linear_part){xn + (size_t)R[b] * H * 2, blk->qkv[0], qkv + (size_t)R[b] * 3 * H * 2, NULL, Nt[b]};
@@ -401,8 +405,12 @@ int fh_forward_device_n(flux_transformer_t *tf, int nb, const fh_rope *const *rp
             p[2 * b] = (flux_hip_linear_part){cat + (size_t)R[b] * ldcat * 2, blk->proj[0], x + (size_t)R[b] * H, mt + 2 * H, Nt[b]};
             p[2 * b + 1] = (flux_hip_linear_part){cat + (size_t)(R[b] + Nt[b]) * ldcat * 2, blk->proj[1], x + (size_t)(R[b] + Nt[b]) * H, mi + 2 * H, Ni};
         }
-        if (!flux_hip_linear(FLUX_HIP_EPI_RESID, 2 * nb, p, H, H, ldcat, H, H, 0, 0)) return 0;
-        for (int b = 0; b < nb; b++)
+        for (int b = 0; b < nb; b++) {
+            an[2 * b] = (flux_hip_adaln_part){xn + (size_t)R[b] * H * 2, mt + 3 * H, mt + 4 * H};
+            an[2 * b + 1] = (flux_hip_adaln_part){xn + (size_t)(R[b] + Nt[b]) * H * 2, mi + 3 * H, mi + 4 * H};
+        }
+        if (!flux_hip_linear_resid_adaln(2 * nb, p, H, H, ldcat, H, H, an, eps, &normed)) return 0;
+        for (int b = 0; b < nb && !normed; b++)
             if (!flux_hip_adaln_norm(xn + (size_t)R[b] * H * 2, H, x + (size_t)R[b] * H, N[b], H, Nt[b], mt + 3 * H, mt + 4 * H, mi + 3 * H, mi + 4 * H, eps)) return 0;
         /* linear_in rows are [gate ; up] (flux_transformer.c:4503-4523) */
         for (int b = 0; b < nb; b++) {
@@ -414,7 +422,13 @@ int fh_forward_device_n(flux_transformer_t *tf, int nb, const fh_rope *const *rp
             p[2 * b] = (flux_hip_linear_part){cat + ((size_t)R[b] * ldcat + H) * 2, blk->ff_out[0], x + (size_t)R[b] * H, mt + 5 * H, Nt[b]};
             p[2 * b + 1] = (flux_hip_linear_part){cat + ((size_t)(R[b] + Nt[b]) * ldcat + H) * 2, blk->ff_out[1], x + (size_t)(R[b] + Nt[b]) * H, mi + 5 * H, Ni};
         }
-        if (!flux_hip_linear(FLUX_HIP_EPI_RESID, 2 * nb, p, H, M, ldcat, M, H, 0, 0)) return 0;
+        /* what reads x next: the next double block's first AdaLN, or the first single block's */
+        const int more = i + 1 < c->n_double;
+        for (int b = 0; b < nb; b++) {
+            an[2 * b] = (flux_hip_adaln_part){xn + (size_t)R[b] * H * 2, more ? mt : ms, more ? mt + H : ms + H};
+            an[2 * b + 1] = (flux_hip_adaln_part){xn + (size_t)(R[b] + Nt[b]) * H * 2, more ? mi : ms, more ? mi + H : ms + H};
+        }
+        if (!flux_hip_linear_resid_adaln(2 * nb, p, H, M, ldcat, M, H, more || c->n_single > 0 ? an : NULL, eps, &normed)) return 0;
         if (flux_substep_callback) flux_substep_callback(FLUX_SUBSTEP_DOUBLE_BLOCK, i, c->n_double);
     }
     if (ev) fh_event_record(ev, 1);
@@ -422,7 +436,7 @@ int fh_forward_device_n(flux_transformer_t *tf, int nb, const fh_rope *const *rp
     /* single-stream blocks (flux_transformer.c:2992-3109): fused rows [Q | K | V | gate | up]; all rows of all sequences at once */
     for (int i = 0; i < c->n_single; i++) {
         const fh_single *blk = &tf->sgl[i];
-        if (!flux_hip_adaln_norm(xn, H, x, Ntot, H, Ntot, ms, ms + H, NULL, NULL, eps)) return 0;
+        if (!normed && !flux_hip_adaln_norm(xn, H, x, Ntot, H, Ntot, ms, ms + H, NULL, NULL, eps)) return 0;
         if (!linear1(FLUX_HIP_EPI_BF16, xn, blk->qkv_mlp, qkv, NULL, Ntot, 3 * H, H, H, H, 3 * H, 0, 0)) return 0;
         if (!linear1(FLUX_HIP_EPI_SWIGLU, xn, blk->qkv_mlp, cat + (size_t)H * 2, NULL, Ntot, 2 * M, H, H, H, ldcat, 3 * H, 3 * H + M)) return 0;
         for (int b = 0; b < nb; b++) {
@@ -432,7 +446,9 @@ int fh_forward_device_n(flux_transformer_t *tf, int nb, const fh_rope *const *rp
             if (!flux_hip_attention(cat + (size_t)R[b] * ldcat * 2, ldcat, q_b, 3 * H, kn + (size_t)R[b] * H * 2, vt + vt_off[b], ldvt[b], N[b], N[b],
                                     heads, N[b], blk->norm_q, NULL, rp[b]->cos, rp[b]->sin, eps)) return 0;
         }
-        if (!linear1(FLUX_HIP_EPI_RESID, cat, blk->out, x, ms + 2 * H, Ntot, H, H + M, ldcat, H + M, H, 0, 0)) return 0;
+        p[0] = (flux_hip_linear_part){cat, blk->out, x, ms + 2 * H, Ntot};
+        an[0] = (flux_hip_adaln_part){xn, ms, ms + H};
+        if (!flux_hip_linear_resid_adaln(1, p, H, H + M, ldcat, H + M, H, i + 1 < c->n_single ? an : NULL, eps, &normed)) return 0;
         if (flux_substep_callback) flux_substep_callback(FLUX_SUBSTEP_SINGLE_BLOCK, i, c->n_single);
     }
     if (ev) fh_event_record(ev, 2);

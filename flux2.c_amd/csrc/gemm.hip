@@ -580,12 +580,125 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(GemmArgs g) {
     }
 }
 
+/* What follows a residual projection in every block is the AdaLN of the updated rows
+ * (apply_adaln, flux_transformer.c:979-1048). When the projection ran as K slices, this kernel is
+ * its second pass and that normalisation in one: a workgroup owns one row, sums the slices in
+ * the fixed order, updates x (as splitk_finish_kernel<RESID> does), and while the row is still in
+ * registers computes mean and biased variance (two passes) and writes
+ * (1 + scale) * (x - mean) / sqrt(var + eps) + shift as bf16. One read of the partial sums, one
+ * read and write of x, one write of the normalised row. N <= 4096. */
+struct AdalnArgs {
+    bf16 *out[GEMM_MAX_PARTS];
+    const float *shift[GEMM_MAX_PARTS], *scale[GEMM_MAX_PARTS];
+    int ldo;
+    float eps;
+};
+
+__device__ __forceinline__ float block_sum_256(float v, float *red) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    __syncthreads(); /* red is free again */
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+__global__ __launch_bounds__(256) void splitk_finish_adaln_kernel(GemmArgs g, AdalnArgs a) {
+    __shared__ float red[4];
+    const int row = blockIdx.x;
+    const int prob = (row >= g.moff[1]) + (row >= g.moff[2]) + (row >= g.moff[3]);
+    const int m = row - g.moff[prob];
+    const int N = g.N;
+    f32x4 v[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) v[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    /* slices four at a time, so that a row with many short slices keeps enough loads in flight;
+     * the additions stay in slice order */
+    const size_t slice = (size_t)g.ws_rows * N;
+    const float *w0 = g.ws + (size_t)row * N;
+    int s = 0;
+    for (; s + 4 <= g.ksplit; s += 4) {
+        f32x4 t[4][4];
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int c = (i * 256 + threadIdx.x) * 4;
+                if (c < N) t[u][i] = *(const f32x4 *)(w0 + (size_t)(s + u) * slice + c);
+            }
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int c = (i * 256 + threadIdx.x) * 4;
+                if (c < N) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[i][e] += t[u][i][e];
+                }
+            }
+    }
+    for (; s < g.ksplit; s++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int c = (i * 256 + threadIdx.x) * 4;
+            if (c < N) {
+                const f32x4 t = *(const f32x4 *)(w0 + (size_t)s * slice + c);
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[i][e] += t[e];
+            }
+        }
+    }
+    float *xr = (float *)g.C[prob] + (size_t)m * g.ldc;
+    float s1 = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int c = (i * 256 + threadIdx.x) * 4;
+        if (c < N) {
+            f32x4 x = *(f32x4 *)(xr + c);
+            const f32x4 gt = *(const f32x4 *)(g.gate[prob] + c);
+#pragma unroll
+            for (int e = 0; e < 4; e++) x[e] += gt[e] * v[i][e];
+            *(f32x4 *)(xr + c) = x;
+            v[i] = x;
+            s1 += (x[0] + x[1]) + (x[2] + x[3]);
+        }
+    }
+    const float mean = block_sum_256(s1, red) / (float)N;
+    float q = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int c = (i * 256 + threadIdx.x) * 4;
+        if (c < N) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) { const float d = v[i][e] - mean; q += d * d; }
+        }
+    }
+    const float inv = 1.0f / sqrtf(block_sum_256(q, red) / (float)N + a.eps);
+    bf16 *o = a.out[prob] + (size_t)m * a.ldo;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int c = (i * 256 + threadIdx.x) * 4;
+        if (c < N) {
+            const f32x4 sh = *(const f32x4 *)(a.shift[prob] + c), sc = *(const f32x4 *)(a.scale[prob] + c);
+            bf16x4 r;
+#pragma unroll
+            for (int e = 0; e < 4; e++) r[e] = (bf16)((1.0f + sc[e]) * ((v[i][e] - mean) * inv) + sh[e]);
+            *(bf16x4 *)(o + c) = r;
+        }
+    }
+}
+
 template <int EPI>
 static int launch_split(GemmArgs &g, int tile) {
     if (!launch_epi<EPI_PARTIAL>(g, tile)) return 0;
     const size_t total = (size_t)g.ws_rows * ((EPI == FLUX_HIP_EPI_SWIGLU ? g.N >> 1 : g.N) >> 2);
     hipLaunchKernelGGL(splitk_finish_kernel<EPI>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, flux_hip_stream_handle(), g);
     return hipGetLastError() == hipSuccess ? 1 : flux_hip_fail("split-K reduction launch failed");
+}
+
+static int launch_split_adaln(GemmArgs &g, int tile, const AdalnArgs &a) {
+    if (!launch_epi<EPI_PARTIAL>(g, tile)) return 0;
+    hipLaunchKernelGGL(splitk_finish_adaln_kernel, dim3((unsigned)g.ws_rows), dim3(256), 0, flux_hip_stream_handle(), g, a);
+    return hipGetLastError() == hipSuccess ? 1 : flux_hip_fail("split-K reduction + AdaLN launch failed");
 }
 
 extern "C" void flux_hip_linear_release(void);
@@ -675,7 +788,8 @@ static int probe_slot(int epilogue) {
 }
 
 /* Tile and K-split choice, then the launch; `allowed` has bit t set for every tile id that may be used. */
-static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, int *tile_out = nullptr) {
+static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, int *tile_out = nullptr, const AdalnArgs *adaln = nullptr,
+                         int *adaln_done = nullptr) {
     /* Choose tile and K split with a small cost model: workgroups run in rounds over
      * 256 CUs x occupancy; a workgroup's time is its FLOPs at the tile's measured rate plus a
      * fixed prologue/epilogue cost; the launch cannot beat the time to stream its operands,
@@ -749,7 +863,14 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
         case FLUX_HIP_EPI_BF16: ok = split ? launch_split<FLUX_HIP_EPI_BF16>(g, tile) : launch_epi<FLUX_HIP_EPI_BF16>(g, tile); break;
         case FLUX_HIP_EPI_F32: ok = split ? launch_split<FLUX_HIP_EPI_F32>(g, tile) : launch_epi<FLUX_HIP_EPI_F32>(g, tile); break;
         case FLUX_HIP_EPI_F32_T: ok = launch_epi<FLUX_HIP_EPI_F32_T>(g, tile); break;
-        case FLUX_HIP_EPI_RESID: ok = split ? launch_split<FLUX_HIP_EPI_RESID>(g, tile) : launch_epi<FLUX_HIP_EPI_RESID>(g, tile); break;
+        case FLUX_HIP_EPI_RESID:
+            if (split && adaln) {
+                ok = launch_split_adaln(g, tile, *adaln);
+                if (adaln_done) *adaln_done = ok;
+            } else {
+                ok = split ? launch_split<FLUX_HIP_EPI_RESID>(g, tile) : launch_epi<FLUX_HIP_EPI_RESID>(g, tile);
+            }
+            break;
         case FLUX_HIP_EPI_SWIGLU: ok = split ? launch_split<FLUX_HIP_EPI_SWIGLU>(g, tile) : launch_epi<FLUX_HIP_EPI_SWIGLU>(g, tile); break;
         case FLUX_HIP_EPI_CONV_BF16: ok = launch_conv<FLUX_HIP_EPI_CONV_BF16>(g, tile); break;
         case FLUX_HIP_EPI_CONV_F32: ok = launch_conv<FLUX_HIP_EPI_CONV_F32>(g, tile); break;
@@ -759,8 +880,8 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
     return ok;
 }
 
-extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
-                               int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1) {
+static int linear_impl(int epilogue, int nparts, const flux_hip_linear_part *parts, int N, int K, int lda, int ldw, int ldc, int w_row0,
+                       int w_row1, const flux_hip_adaln_part *norm, float eps, int *fused) {
     if (epilogue < FLUX_HIP_EPI_BF16 || epilogue > FLUX_HIP_EPI_SWIGLU) return flux_hip_fail("flux_hip_linear: unknown epilogue %d", epilogue);
     if (nparts < 1 || nparts > GEMM_MAX_PARTS) return flux_hip_fail("flux_hip_linear: nparts=%d (1 to %d)", nparts, GEMM_MAX_PARTS);
     if (K <= 0 || (K & 63)) return flux_hip_fail("flux_hip_linear: K=%d must be a positive multiple of 64", K);
@@ -769,6 +890,7 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
         return flux_hip_fail("flux_hip_linear: lda=%d ldw=%d must be >= K and multiples of 8", lda, ldw);
     if (epilogue != FLUX_HIP_EPI_F32_T && (ldc & 3)) return flux_hip_fail("flux_hip_linear: ldc=%d must be a multiple of 4", ldc);
     GemmArgs g = {};
+    AdalnArgs a = {};
     int maxm = 0;
     for (int i = 0; i < nparts; i++) {
         if (parts[i].M < 0) return flux_hip_fail("flux_hip_linear: negative row count");
@@ -789,13 +911,43 @@ extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_p
         g.C[np] = parts[i].C;
         g.gate[np] = parts[i].gate;
         g.M[np] = parts[i].M;
+        if (norm) {
+            a.out[np] = (bf16 *)norm[i].out_bf16;
+            a.shift[np] = norm[i].shift;
+            a.scale[np] = norm[i].scale;
+        }
         if (parts[i].M > maxm) maxm = parts[i].M;
         np++;
     }
     if (np == 0) return 1;
     g.N = N; g.K = K; g.lda = lda; g.ldw = ldw; g.ldc = ldc; g.w_row0 = w_row0; g.w_row1 = w_row1;
-    return gemm_dispatch(g, np, epilogue, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0xFFu);
+    a.ldo = N;
+    a.eps = eps;
+    return gemm_dispatch(g, np, epilogue, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0xFFu, nullptr, norm ? &a : nullptr, fused);
 }
+
+extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
+                               int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1) {
+    return linear_impl(epilogue, nparts, parts, N, K, lda, ldw, ldc, w_row0, w_row1, nullptr, 0.0f, nullptr);
+}
+
+/* The residual projection, and - when it runs as K slices - the AdaLN of the updated rows in its
+ * second pass, see the header. */
+extern "C" int flux_hip_linear_resid_adaln(int nparts, const flux_hip_linear_part *parts, int N, int K, int lda, int ldw, int ldc,
+                                           const flux_hip_adaln_part *norm, float eps, int *fused) {
+    if (!fused) return flux_hip_fail("flux_hip_linear_resid_adaln: fused must not be NULL");
+    *fused = 0;
+    if (norm) {
+        if (N > 4096) return flux_hip_fail("flux_hip_linear_resid_adaln: N=%d (at most 4096 columns per row)", N);
+        for (int i = 0; i < nparts && i < GEMM_MAX_PARTS; i++)
+            if (parts[i].M > 0 && (!norm[i].out_bf16 || !norm[i].shift || !norm[i].scale ||
+                                   (((uintptr_t)norm[i].out_bf16 | (uintptr_t)norm[i].shift | (uintptr_t)norm[i].scale) & 15)))
+                return flux_hip_fail("flux_hip_linear_resid_adaln: NULL or unaligned AdaLN operand");
+    }
+    return linear_impl(FLUX_HIP_EPI_RESID, nparts, parts, N, K, lda, ldw, ldc, 0, 0, norm, eps, fused);
+}
+
+
 
 /* Convolution over a zero-bordered channels-last image as one GEMM, see the header. */
 extern "C" int flux_hip_conv_stats(int epilogue, const void *in, const void *w, const float *bias, const float *res, void *out, int rows,

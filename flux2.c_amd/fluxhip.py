@@ -131,6 +131,7 @@ def lib():
     L.flux_linear_schedule.argtypes = [c_i]
     L.flux_power_schedule.argtypes = [c_i, c_f]
     L.flux_official_schedule.argtypes = [c_i, c_i]
+    L.flux_hip_linear_resid_adaln.argtypes = [c_i, vp, c_i, c_i, c_i, c_i, c_i, vp, c_f, ctypes.POINTER(c_i)]
     L.flux_hip_conv.argtypes = [c_i, vp, vp, vp, vp, vp, c_i, c_i, c_i, c_i, c_i]
     L.flux_hip_group_norm.argtypes = [vp, vp, vp, c_i, vp, vp, vp, c_i, c_i, c_i, c_f, c_i]
     L.flux_hip_conv_stats.argtypes = [c_i, vp, vp, vp, vp, vp, c_i, c_i, c_i, c_i, c_i, vp, ctypes.POINTER(c_i)]
@@ -229,6 +230,26 @@ def linear(epilogue, parts, N, K, lda, ldw, ldc, w_row0=0, w_row1=0):
     for i, (A, W, C, g, M) in enumerate(parts):
         arr[i] = _Part(A, W, C, g, M)
     check(lib().flux_hip_linear(epilogue, len(parts), arr, N, K, lda, ldw, ldc, w_row0, w_row1), "flux_hip_linear")
+
+
+class _AdalnPart(ctypes.Structure):
+    _fields_ = [("out_bf16", vp), ("shift", vp), ("scale", vp)]
+
+
+def linear_resid_adaln(parts, N, K, lda, ldw, ldc, norms, eps=1e-6):
+    """parts as for linear() with the residual epilogue; norms: list of (out_bf16_ptr, shift_ptr, scale_ptr) per
+    part, or None. Returns True when the AdaLN outputs were written (the projection ran as K slices)."""
+    arr = (_Part * len(parts))()
+    for i, (A, W, C, g, M) in enumerate(parts):
+        arr[i] = _Part(A, W, C, g, M)
+    na = None
+    if norms is not None:
+        na = (_AdalnPart * len(parts))()
+        for i, (o, sh, sc) in enumerate(norms):
+            na[i] = _AdalnPart(o, sh, sc)
+    fused = c_i(0)
+    check(lib().flux_hip_linear_resid_adaln(len(parts), arr, N, K, lda, ldw, ldc, na, eps, ctypes.byref(fused)), "flux_hip_linear_resid_adaln")
+    return bool(fused.value)
 
 
 def _f32(a):

@@ -92,6 +92,22 @@ int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
                     int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1);
 
 /*
+ * flux_hip_linear with FLUX_HIP_EPI_RESID, with the AdaLN that follows every residual projection
+ * (apply_adaln, flux_transformer.c:979-1048, called at :1845, :1919, :3030) folded into it when the
+ * projection runs as K slices (few rows, long K): the pass that sums the slices and updates x then
+ * also writes (1 + scale) * LayerNorm(x) + shift as bf16 [M, N] (row stride N) per part, and
+ * *fused = 1. Otherwise (*fused = 0) only the projection has run and the caller normalises with
+ * flux_hip_adaln_norm. norm = NULL: plain projection. N <= 4096.
+ */
+typedef struct {
+    void *out_bf16;       /* bf16 [M, N] */
+    const float *shift;   /* f32 [N] */
+    const float *scale;   /* f32 [N] */
+} flux_hip_adaln_part;
+int flux_hip_linear_resid_adaln(int nparts, const flux_hip_linear_part *parts, int N, int K, int lda, int ldw, int ldc,
+                                const flux_hip_adaln_part *norm, float eps, int *fused);
+
+/*
  * 3x3 (taps = 9, padding 1, stride 1) or 1x1 (taps = 1) convolution with bias as one MFMA GEMM
  * over a channels-last image. Replaces flux_conv2d (flux_kernels.c:342-470; im2col + sgemm
  * there) for the VAE decoder's layers, with the residual add of resblock_forward /

@@ -184,6 +184,54 @@ def test_linear_split_k(hip, oracle_mod, tile):
     assert rel_l2(dres.to_array(np.float32, (40, 128)), r + g0[:128] * oracle_mod.linear(x, W)) < 2e-6
 
 
+@pytest.mark.parametrize("shape", [(64, 16, 768, 4096), (80, 0, 3072, 12288), (300, 212, 256, 256)])
+def test_linear_residual_then_adaln(hip, oracle_mod, shape):
+    """A residual projection that runs as K slices also writes the AdaLN of the rows it updated; x is then
+    bit for bit what the plain two-pass form gives, the normalised rows agree with the stand-alone kernel
+    and with the oracle. A projection that does not split reports that it left the normalisation to the caller."""
+    M0, M1, N, K = shape
+    a = q(normal_f32((M0 + M1, K), 24, 1))
+    W0, W1 = q(normal_f32((N, K), 24, 2, 0.0, 0.05)), q(normal_f32((N, K), 24, 3, 0.0, 0.05))
+    res = normal_f32((M0 + M1, N), 24, 4)
+    g0, g1 = normal_f32((N,), 24, 5), normal_f32((N,), 24, 6)
+    sh = [normal_f32((N,), 24, 7 + i, 0.0, 0.3) for i in range(2)]
+    sc = [normal_f32((N,), 24, 9 + i, 0.0, 0.3) for i in range(2)]
+    da, dW0, dW1 = dev_bf16(hip, a), dev_bf16(hip, W0), dev_bf16(hip, W1)
+    dg0, dg1 = hip.DevBuf.from_array(g0), hip.DevBuf.from_array(g1)
+    dsh, dsc = [hip.DevBuf.from_array(v) for v in sh], [hip.DevBuf.from_array(v) for v in sc]
+    parts = lambda dres: [(da.ptr, dW0.ptr, dres.ptr, dg0.ptr, M0), (da.at(M0 * K * 2), dW1.ptr, dres.at(M0 * N * 4), dg1.ptr, M1)]
+    # plain: projection, then the stand-alone AdaLN kernel
+    dres = hip.DevBuf.from_array(res)
+    hip.linear(hip.EPI_RESID, parts(dres), N, K, K, K, N)
+    x_plain = dres.to_array(np.float32, (M0 + M1, N))
+    dn = hip.DevBuf((M0 + M1) * N * 2)
+    hip.check(hip.lib().flux_hip_adaln_norm(dn.ptr, N, dres.ptr, M0 + M1, N, M0, dsh[0].ptr, dsc[0].ptr, dsh[1].ptr, dsc[1].ptr, 1e-6))
+    n_plain = bf16_to_f32(dn.to_array(np.uint16, (M0 + M1, N)))
+    # fused
+    dres2 = hip.DevBuf.from_array(res)
+    dn2 = hip.DevBuf.from_array(np.full((M0 + M1, N), 0x7fc0, np.uint16))
+    fused = hip.linear_resid_adaln(parts(dres2), N, K, K, K, N, [(dn2.ptr, dsh[0].ptr, dsc[0].ptr), (dn2.at(M0 * N * 2), dsh[1].ptr, dsc[1].ptr)])
+    x_fused = dres2.to_array(np.float32, (M0 + M1, N))
+    assert fused == (K > 256)                              # K = 256 is too short to slice
+    np.testing.assert_array_equal(x_fused, x_plain)
+    want_x = res.copy()
+    want_x[:M0] += g0 * oracle_mod.linear(a[:M0], W0)
+    if M1:
+        want_x[M0:] += g1 * oracle_mod.linear(a[M0:], W1)
+    assert rel_l2(x_fused, want_x) < 2e-6
+    if fused:
+        n_fused = bf16_to_f32(dn2.to_array(np.uint16, (M0 + M1, N)))
+        want_n = oracle_mod.adaln(want_x[:M0], sh[0], sc[0])
+        if M1:
+            want_n = np.concatenate([want_n, oracle_mod.adaln(want_x[M0:], sh[1], sc[1])])
+        assert rel_l2(n_fused, want_n) < 4e-3
+        assert rel_l2(n_fused, n_plain) < 2e-3 and (n_fused != n_plain).mean() < 0.02     # same values up to the order of the row sums
+    # no AdaLN asked for: the plain projection, never "fused"
+    dres3 = hip.DevBuf.from_array(res)
+    assert hip.linear_resid_adaln(parts(dres3), N, K, K, K, N, None) is False
+    np.testing.assert_array_equal(dres3.to_array(np.float32, (M0 + M1, N)), x_plain)
+
+
 def test_linear_rejects_bad_shapes(hip):
     d = hip.DevBuf(1024)
     with pytest.raises(hip.FluxHipError):
