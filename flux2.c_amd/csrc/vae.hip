@@ -349,6 +349,54 @@ __global__ __launch_bounds__(256) void vae_softmax_kernel(bf16 *__restrict__ P, 
     }
 }
 
+/* The same for rows of up to 1024 * SOFTMAX_REG_V4 * 4 columns (1024x1024 images have 17024), with
+ * the row held in registers between the three steps: S is read once. */
+#define SOFTMAX_REG_V4 20
+__global__ __launch_bounds__(256) void vae_softmax_reg_kernel(bf16 *__restrict__ P, const float *__restrict__ S, const float *__restrict__ key_bias,
+                                                              int ld, float scale) {
+    __shared__ float red[4];
+    const float *s = S + (size_t)blockIdx.x * ld;
+    bf16 *p = P + (size_t)blockIdx.x * ld;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    f32x4 v[SOFTMAX_REG_V4];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < SOFTMAX_REG_V4; i++) {
+        const int c = (i * 256 + threadIdx.x) * 4;
+        if (c < ld) {
+            const f32x4 t = *(const f32x4 *)(s + c), kb = *(const f32x4 *)(key_bias + c);
+#pragma unroll
+            for (int e = 0; e < 4; e++) { v[i][e] = t[e] * scale + kb[e]; mx = fmaxf(mx, v[i][e]); }
+        }
+    }
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    if (lane == 0) red[wave] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < SOFTMAX_REG_V4; i++)
+        if ((i * 256 + threadIdx.x) * 4 < ld) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) { v[i][e] = __expf(v[i][e] - mx); sum += v[i][e]; }
+        }
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+    if (lane == 0) red[wave] = sum;
+    __syncthreads();
+    const float inv = 1.0f / (red[0] + red[1] + red[2] + red[3]);
+#pragma unroll
+    for (int i = 0; i < SOFTMAX_REG_V4; i++) {
+        const int c = (i * 256 + threadIdx.x) * 4;
+        if (c < ld) {
+            bf16x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; e++) o[e] = (bf16)(v[i][e] * inv);
+            *(bf16x4 *)(p + c) = o;
+        }
+    }
+}
+
 /* vt[c][j] = v[j][c] for j < rows, 0 for rows <= j < ld: the value matrix as the "weight" operand
  * of the second attention GEMM. 64 x 64 tiles through LDS. */
 __global__ __launch_bounds__(256) void vae_transpose_kernel(bf16 *__restrict__ vt, int ld, const bf16 *__restrict__ v, int ldv, int rows) {
@@ -485,7 +533,10 @@ extern "C" int flux_hip_vae_key_bias(float *bias, int n, int hp, int wp) {
 
 extern "C" int flux_hip_softmax_rows(void *p_bf16, const float *s, const float *key_bias, int rows, int ld, float scale) {
     if (rows <= 0 || ld <= 0 || (ld & 3)) return flux_hip_fail("flux_hip_softmax_rows: bad shape %d x %d", rows, ld);
-    hipLaunchKernelGGL(vae_softmax_kernel, dim3(rows), dim3(256), 0, flux_hip_stream_handle(), (bf16 *)p_bf16, s, key_bias, ld, scale);
+    if (ld <= 1024 * SOFTMAX_REG_V4)
+        hipLaunchKernelGGL(vae_softmax_reg_kernel, dim3(rows), dim3(256), 0, flux_hip_stream_handle(), (bf16 *)p_bf16, s, key_bias, ld, scale);
+    else
+        hipLaunchKernelGGL(vae_softmax_kernel, dim3(rows), dim3(256), 0, flux_hip_stream_handle(), (bf16 *)p_bf16, s, key_bias, ld, scale);
     LAUNCH_OK("vae_softmax_kernel");
     return 1;
 }

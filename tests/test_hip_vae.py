@@ -228,8 +228,11 @@ def test_upsample(hip, oracle_mod):
     np.testing.assert_array_equal(from_padded(got, 2 * H, 2 * W), q(oracle_mod.upsample_nearest(x)))
 
 
-def test_softmax_rows_and_transpose(hip, oracle_mod):
-    rows, ld, valid = 37, 384, 300
+@pytest.mark.parametrize("shape", [(37, 384, 300), (3, 17024, 16900), (3, 20608, 20500)])
+def test_softmax_rows_and_transpose(hip, oracle_mod, shape):
+    """Rows of up to 20480 columns go through the kernel that keeps the row in registers, longer ones
+    (images beyond about 1100 pixels a side) through the three-pass kernel."""
+    rows, ld, valid = shape
     s = normal_f32((rows, ld), 56, 1, 0.0, 6.0)
     kb = np.zeros(ld, np.float32)
     kb[valid:] = -np.inf
