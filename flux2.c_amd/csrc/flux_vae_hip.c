@@ -266,7 +266,8 @@ int flux_hip_vae_set_tensor(flux_hip_vae *v, const char *name, int dtype, const 
         ok = flux_hip_upload(s->dst, tmp, sizeof(float) * (size_t)numel);
         free(tmp);
     } else {
-        /* [cout][cin][ky][kx] -> bf16 [cout][(ky*3+kx) * cin_pad + cin]: K runs tap-major */
+        /* [cout][cin][ky][kx] -> bf16 [cout][cin_pad / 64][ky*3+kx][64]: the nine taps of a 64-channel
+         * chunk side by side (flux_hip_conv's K order); for a 1x1 convolution that is [cout][cin_pad] */
         const int cout = s->rows, cin = s->cols, cp = s->cin_pad;
         uint16_t *tmp = (uint16_t *)calloc((size_t)cout * taps * cp, 2);
         if (!tmp) return flux_hip_fail("out of host memory");
@@ -275,7 +276,7 @@ int flux_hip_vae_set_tensor(flux_hip_vae *v, const char *name, int dtype, const 
         for (int o = 0; o < cout; o++)
             for (int c = 0; c < cin; c++)
                 for (int t = 0; t < taps; t++)
-                    tmp[packed ? (size_t)o * cp + t * cin + c : ((size_t)o * taps + t) * cp + c] =
+                    tmp[packed ? (size_t)o * cp + t * cin + c : (size_t)o * taps * cp + ((size_t)(c >> 6) * taps + t) * 64 + (c & 63)] =
                         to_bf16(fh_tensor_value(dtype, data, ((int64_t)o * cin + c) * taps + t));
         ok = flux_hip_upload(s->dst, tmp, packed ? (size_t)cout * cp * 2 : (size_t)cout * taps * cp * 2);
         free(tmp);
@@ -527,7 +528,7 @@ int flux_hip_vae_encode(flux_hip_vae *v, const float *img, int H, int W, float *
             if (!flux_hip_downsample_gather(s.A, s.x, s.hp, s.wp, c->cin)) return 0;
             s.hp = (s.hp - 2) / 2 + 2;
             s.wp = (s.wp - 2) / 2 + 2;
-            /* the nine taps sit side by side in every row of A: a 1x1 convolution over 9 * cin channels */
+            /* the nine taps sit side by side in every row of A, in the weights' K order: a 1x1 convolution over 9 * cin channels */
             if (!flux_hip_conv_stats(FLUX_HIP_EPI_CONV_F32, s.A, c->w, c->b, NULL, s.x, s.hp * s.wp, s.wp, 9 * c->cin_pad, c->cout_pad, 1, v->st_x,
                                      &s.x_rows))
                 return 0;

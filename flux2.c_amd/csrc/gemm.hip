@@ -54,10 +54,12 @@ struct GemmArgs {
     float *ws;
     int moff[GEMM_MAX_PARTS], ws_rows;
     /* convolution epilogues (see flux_hip_conv): rows are the positions of a zero-bordered
-     * conv_hp x conv_wp image with channels contiguous. With 9 taps K runs tap-major over
-     * 9 x cin and K step kt reads the activation rows shifted by its tap's (dy, dx);
-     * conv_kshift = log2(cin / 64) */
-    int conv_taps, conv_kshift, conv_wp, conv_hp;
+     * conv_hp x conv_wp image with channels contiguous. With 9 taps K runs over
+     * [cin / 64 channel chunks][9 taps][64 channels]: K step kt = 9 * chunk + tap reads the
+     * activation rows shifted by its tap's (dy, dx). The nine taps of a chunk follow each other so
+     * that what one tap fetched is still in L2 when the next asks for the neighbouring rows
+     * (tap-major order re-fetched wide images 3 to 10 times from HBM). */
+    int conv_taps, conv_wp, conv_hp;
     const float *bias, *res;
     /* optional: per (row-tile half, 4-channel group) sums and sums of squares of what a convolution
      * epilogue writes, [prow][N/4][2], for the group norm that follows */
@@ -67,14 +69,14 @@ struct GemmArgs {
 template <int EPI> struct IsConv { static constexpr bool value = EPI == FLUX_HIP_EPI_CONV_BF16 || EPI == FLUX_HIP_EPI_CONV_F32; };
 
 /* Element offset of K step kt within an activation row. Plain GEMM: kt * 64. 3x3 convolution:
- * tap = kt / (cin/64) selects a neighbour dy*Wp + dx rows away (uniform for the whole launch,
- * because border positions are rows of the matrix too), the remainder a 64-channel slice. */
+ * kt = 9 * chunk + tap; the tap selects a neighbour dy*Wp + dx rows away (uniform for the whole
+ * launch, because border positions are rows of the matrix too), the chunk a 64-channel slice. */
 template <int EPI>
 __device__ __forceinline__ int a_step_offset(const GemmArgs &g, int kt) {
     if (IsConv<EPI>::value && g.conv_taps == 9) {
-        const int tap = kt >> g.conv_kshift, kc = kt - (tap << g.conv_kshift);
-        const int dy = (tap * 11) >> 5, dx = tap - dy * 3; /* tap / 3, tap % 3 for tap < 9 */
-        return ((dy - 1) * g.conv_wp + (dx - 1)) * g.lda + kc * 64;
+        const int chunk = (kt * 7282) >> 16, tap = kt - 9 * chunk; /* kt / 9, kt % 9 for kt < 2048 */
+        const int dy = (tap * 11) >> 5, dx = tap - dy * 3;         /* tap / 3, tap % 3 for tap < 9 */
+        return ((dy - 1) * g.conv_wp + (dx - 1)) * g.lda + chunk * 64;
     }
     return kt * 64;
 }
@@ -966,10 +968,8 @@ extern "C" int flux_hip_conv_stats(int epilogue, const void *in, const void *w, 
     if (taps != 1 && taps != 9) return flux_hip_fail("flux_hip_conv: taps=%d (1 or 9)", taps);
     if (rows <= 0 || cin <= 0 || (cin & 63) || cout <= 0 || (cout & 63))
         return flux_hip_fail("flux_hip_conv: rows=%d cin=%d cout=%d (channels must be multiples of 64)", rows, cin, cout);
-    int kshift = 0;
-    while ((64 << kshift) < cin) kshift++;
-    if (taps == 9 && ((64 << kshift) != cin || wp < 3 || rows % wp || rows / wp < 3))
-        return flux_hip_fail("flux_hip_conv: a 3x3 convolution needs cin = 64 * 2^k and a bordered image (rows=%d wp=%d cin=%d)", rows, wp, cin);
+    if (taps == 9 && (wp < 3 || rows % wp || rows / wp < 3 || cin > 64 * 227))
+        return flux_hip_fail("flux_hip_conv: a 3x3 convolution needs a bordered image (rows=%d wp=%d cin=%d)", rows, wp, cin);
     if (wp > 0 && rows % wp) return flux_hip_fail("flux_hip_conv: rows=%d is not a multiple of the image width %d", rows, wp);
     if (!in || !w || !bias || !out) return flux_hip_fail("flux_hip_conv: NULL operand");
     if ((((uintptr_t)in | (uintptr_t)w | (uintptr_t)bias | (uintptr_t)res | (uintptr_t)out) & 15))
@@ -981,7 +981,7 @@ extern "C" int flux_hip_conv_stats(int epilogue, const void *in, const void *w, 
     g.C[0] = out;
     g.M[0] = rows;
     g.N = cout; g.K = taps * cin; g.lda = cin; g.ldw = taps * cin; g.ldc = cout;
-    g.conv_taps = taps; g.conv_kshift = kshift; g.conv_wp = wp; g.conv_hp = wp > 0 ? rows / wp : 0;
+    g.conv_taps = taps; g.conv_wp = wp; g.conv_hp = wp > 0 ? rows / wp : 0;
     g.bias = bias; g.res = res; g.stats = stats;
     if (stats && (!stats_rows || ((uintptr_t)stats & 7))) return flux_hip_fail("flux_hip_conv_stats: stats needs stats_rows and 8-byte alignment");
     const unsigned conv_tiles = 0x0F; /* 64x128, 128x128, 256x256 (4 waves), 64x64 */

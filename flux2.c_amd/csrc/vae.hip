@@ -265,8 +265,9 @@ __global__ __launch_bounds__(256) void vae_image_in_kernel(bf16 *__restrict__ ou
 
 /* The downsampling step (flux_vae.c:363-377: one row of zeros below and one column on the right,
  * then a 3x3 convolution with stride 2): fp32 [hp*wp, C] -> bf16 [hp2*wp2, 9*C] over the bordered
- * half-size grid, row (y', x') holding in[2(y'-1)+ky, 2(x'-1)+kx] for the nine taps, tap-major,
- * so that the convolution is a GEMM with K = 9*C over these rows. The input's own zero border
+ * half-size grid, row (y', x') holding in[2(y'-1)+ky, 2(x'-1)+kx] for the nine taps, in the K order
+ * of flux_hip_conv's weights ([C/64 chunks][9 taps][64 channels]), so that the convolution is a
+ * plain GEMM with K = 9*C over these rows. The input's own zero border
  * supplies the padding: the furthest row read is its bottom border. Border rows of the output
  * are zero. One thread per (position, tap, 4 channels). */
 __global__ __launch_bounds__(256) void vae_downsample_gather_kernel(bf16 *__restrict__ out, const float *__restrict__ x, int hp, int wp, int C) {
@@ -286,7 +287,8 @@ __global__ __launch_bounds__(256) void vae_downsample_gather_kernel(bf16 *__rest
 #pragma unroll
         for (int e = 0; e < 4; e++) o[e] = (bf16)v[e];
     }
-    *(bf16x4 *)(out + ((size_t)p * 9 + tap) * C + q * 4) = o;
+    const int c = q * 4;
+    *(bf16x4 *)(out + (size_t)p * 9 * C + ((c >> 6) * 9 + tap) * 64 + (c & 63)) = o;
 }
 
 /* Output of the quant convolution, fp32 [(2h+2)*(2w+2), ldx] (channels 0..31 = the posterior's

@@ -116,10 +116,12 @@ int flux_hip_linear_resid_adaln(int nparts, const flux_hip_linear_part *parts, i
  *        positions in row-major order, wp = W+2. With 9 taps the kernel reads up to wp+1 rows
  *        before `in` and after its end: the allocation must extend that far (contents there
  *        only reach border outputs, which are written as zeros).
- *   w    bf16 [cout, taps * cin], tap-major: w[o][(ky*3+kx) * cin + c]
+ *   w    bf16 [cout, taps * cin]; with 9 taps K runs over [cin/64 chunks][9 taps][64 channels]:
+ *        w[o][((c / 64) * 9 + ky*3+kx) * 64 + c % 64] (the nine taps of a channel chunk are
+ *        consecutive K steps, so that neighbouring rows are fetched while they are still cached)
  *   bias f32 [cout]; res f32 [rows, cout] or NULL (may be `out` itself); out [rows, cout]
  * Border positions of `out` are written as zeros, so it can feed the next convolution. wp = 0
- * (1x1 only) treats every row as interior. cin, cout: multiples of 64; 9 taps: cin = 64 * 2^k.
+ * (1x1 only) treats every row as interior. cin, cout: multiples of 64.
  */
 int flux_hip_conv(int epilogue, const void *in, const void *w, const float *bias, const float *res,
                   void *out, int rows, int wp, int cin, int cout, int taps);
@@ -371,8 +373,8 @@ int flux_hip_vae_decode(flux_hip_vae *v, const float *latent, int h, int w, uint
 int flux_hip_vae_encode(flux_hip_vae *v, const float *img, int H, int W, float *latent);
 /* Encoder pieces: img f32 [3, H, W] (device) -> bf16 [(H+2)*(W+2), 64], the 27 values under every
  * 3x3 window first (conv_in as a GEMM with K = 64, flux_vae.c:336); x f32 [hp*wp, C] -> bf16
- * [(H/2+2)*(W/2+2), 9*C], the nine taps of the stride-2 convolution side by side
- * (flux_vae.c:363-377); quant-convolution output f32 [(2h+2)*(2w+2), ldx] -> latent f32 [128, h, w]
+ * [(H/2+2)*(W/2+2), 9*C], the nine taps of the stride-2 convolution side by side in flux_hip_conv's
+ * K order (flux_vae.c:363-377); quant-convolution output f32 [(2h+2)*(2w+2), ldx] -> latent f32 [128, h, w]
  * (mean channels, patchify, latent normalisation, flux_vae.c:411-437). */
 int flux_hip_vae_image_in(void *out_bf16, const float *img, int H, int W);
 int flux_hip_downsample_gather(void *out_bf16, const float *x, int hp, int wp, int C);

@@ -65,13 +65,13 @@ class Guarded:
 
 
 def conv_weight(w):
-    """[cout, cin, k, k] -> bf16 [cout, k*k*cin], tap-major."""
+    """[cout, cin, k, k] -> bf16 [cout, cin/64, k*k, 64] flattened: the K order of flux_hip_conv."""
     co, ci, k, _ = w.shape
-    return f32_to_bf16(np.ascontiguousarray(w.transpose(0, 2, 3, 1)).reshape(co, k * k * ci))
+    return f32_to_bf16(np.ascontiguousarray(w.reshape(co, ci // 64, 64, k * k).transpose(0, 1, 3, 2)).reshape(co, k * k * ci))
 
 
 @pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3])
-@pytest.mark.parametrize("shape", [(9, 7, 64, 256), (5, 12, 128, 256), (20, 17, 256, 256)])
+@pytest.mark.parametrize("shape", [(9, 7, 64, 256), (5, 12, 128, 256), (20, 17, 256, 256), (6, 9, 192, 256)])
 def test_conv3x3(hip, oracle_mod, tile, shape):
     H, W, cin, cout = shape
     hip.lib().flux_hip_linear_force_tile(tile)
@@ -144,8 +144,9 @@ def test_conv1x1(hip, oracle_mod):
 def test_conv_rejects_bad_arguments(hip):
     L = hip.lib()
     d = hip.DevBuf(1 << 16)
-    assert L.flux_hip_conv(hip.EPI_CONV_F32, d.ptr, d.ptr, d.ptr, None, d.ptr, 30, 6, 96, 64, 9) == 0     # cin not 64 * 2^k
-    assert L.flux_hip_conv(hip.EPI_CONV_F32, d.ptr, d.ptr, d.ptr, None, d.ptr, 30, 6, 192, 64, 9) == 0
+    assert L.flux_hip_conv(hip.EPI_CONV_F32, d.ptr, d.ptr, d.ptr, None, d.ptr, 30, 6, 96, 64, 9) == 0     # cin not a multiple of 64
+    assert L.flux_hip_conv(hip.EPI_CONV_F32, d.ptr, d.ptr, d.ptr, None, d.ptr, 30, 6, 64, 96, 9) == 0     # nor cout
+    assert L.flux_hip_conv(hip.EPI_CONV_F32, d.ptr, d.ptr, d.ptr, None, d.ptr, 30, 2, 64, 64, 9) == 0     # no room for a border
     assert L.flux_hip_conv(hip.EPI_CONV_F32, d.ptr, d.ptr, d.ptr, None, d.ptr, 31, 6, 64, 64, 9) == 0     # rows not a multiple of wp
     assert L.flux_hip_conv(hip.EPI_BF16, d.ptr, d.ptr, d.ptr, None, d.ptr, 30, 6, 64, 64, 9) == 0         # not a conv epilogue
     assert L.flux_hip_conv(hip.EPI_CONV_F32, d.ptr, d.ptr, None, None, d.ptr, 30, 6, 64, 64, 9) == 0      # bias is required
@@ -365,7 +366,7 @@ def test_downsample_step(hip, oracle_mod, shape):
     a = hip.DevBuf.from_array(np.full((rows2, 9 * C), 0x4040, np.uint16))
     dx = hip.DevBuf.from_array(to_padded(x))
     hip.check(L.flux_hip_downsample_gather(a.ptr, dx.ptr, H + 2, W + 2, C))
-    ga = bf16_to_f32(a.to_array(np.uint16, (rows2, 9 * C))).reshape(H2 + 2, W2 + 2, 9, C)
+    ga = bf16_to_f32(a.to_array(np.uint16, (rows2, 9 * C))).reshape(H2 + 2, W2 + 2, C // 64, 9, 64).transpose(0, 1, 3, 2, 4).reshape(H2 + 2, W2 + 2, 9, C)
     assert not (ga[0].any() or ga[-1].any() or ga[:, 0].any() or ga[:, -1].any())
     xp = np.zeros((C, H + 1, W + 1), np.float32)
     xp[:, :H, :W] = x
