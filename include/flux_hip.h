@@ -14,8 +14,8 @@
  * (as the reference's GPU operators do, flux_metal.h:232-234); functions
  * returning pointers give NULL on failure. flux_hip_last_error() then holds a
  * message. Nothing here falls back to a CPU path: without a usable GPU every
- * call fails. Not thread-safe (neither is the reference, SURVEY of
- * flux_kernels.c:32-45 globals): one forward at a time per process.
+ * call fails. Not thread-safe (neither is the reference: see the globals at
+ * flux_kernels.c:32-45): one forward at a time per process.
  */
 #ifndef FLUX_HIP_H
 #define FLUX_HIP_H
