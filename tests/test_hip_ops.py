@@ -184,12 +184,14 @@ def test_linear_split_k(hip, oracle_mod, tile):
     assert rel_l2(dres.to_array(np.float32, (40, 128)), r + g0[:128] * oracle_mod.linear(x, W)) < 2e-6
 
 
+@pytest.mark.parametrize("tile", [-1, 1, 6])
 @pytest.mark.parametrize("shape", [(64, 16, 768, 4096), (80, 0, 3072, 12288), (300, 212, 256, 256)])
-def test_linear_residual_then_adaln(hip, oracle_mod, shape):
+def test_linear_residual_then_adaln(hip, oracle_mod, shape, tile):
     """A residual projection that runs as K slices also writes the AdaLN of the rows it updated; x is then
     bit for bit what the plain two-pass form gives, the normalised rows agree with the stand-alone kernel
     and with the oracle. A projection that does not split reports that it left the normalisation to the caller."""
     M0, M1, N, K = shape
+    hip.lib().flux_hip_linear_force_tile(tile)             # a forced tile that does not divide N is ignored
     a = q(normal_f32((M0 + M1, K), 24, 1))
     W0, W1 = q(normal_f32((N, K), 24, 2, 0.0, 0.05)), q(normal_f32((N, K), 24, 3, 0.0, 0.05))
     res = normal_f32((M0 + M1, N), 24, 4)
@@ -230,6 +232,7 @@ def test_linear_residual_then_adaln(hip, oracle_mod, shape):
     dres3 = hip.DevBuf.from_array(res)
     assert hip.linear_resid_adaln(parts(dres3), N, K, K, K, N, None) is False
     np.testing.assert_array_equal(dres3.to_array(np.float32, (M0 + M1, N)), x_plain)
+    hip.lib().flux_hip_linear_force_tile(-1)
 
 
 def test_linear_rejects_bad_shapes(hip):
