@@ -333,7 +333,27 @@ extern int *qwen3_pad_tokens(int *tokens, int num_tokens, int max_len, int *atte
 typedef void (*text_progress_fn)(int layer, int total);
 extern text_progress_fn flux_text_progress_callback __attribute__((weak)); /* flux_kernels.h */
 
-typedef struct { qwen3_tokenizer_t *tokenizer; flux_hip_qwen3 *model; } dropin_encoder; /* qwen3_encoder_t, flux_qwen3.h:117-120 */
+typedef struct { qwen3_tokenizer_t *tokenizer; flux_hip_qwen3 *model; char dir[600]; } dropin_encoder; /* qwen3_encoder_t, flux_qwen3.h:117-120 */
+
+/* The reference frees the text encoder after every prompt to make room for the transformer
+ * (flux_release_text_encoder, flux.c:285-295) and loads it again for the next one; its weights are
+ * a memory map, so that is cheap there. Here a load is a 6 GB upload, and 288 GB of HBM hold encoder
+ * and transformer side by side: the weights of the encoder freed last stay on the device and the
+ * next qwen3_encoder_load of the same directory takes them over. */
+static struct { char dir[600]; flux_hip_qwen3 *model; } g_kept;
+static int g_keep_resident = 1;
+int flux_hip_qwen3_resident_hits = 0;
+
+void flux_hip_qwen3_drop_resident(void) {
+    flux_hip_qwen3_free(g_kept.model);
+    g_kept.model = NULL;
+    g_kept.dir[0] = 0;
+}
+
+void flux_hip_qwen3_keep_resident(int on) {
+    g_keep_resident = on != 0;
+    if (!on) flux_hip_qwen3_drop_resident();
+}
 
 void *qwen3_model_load(const char *model_dir) { return flux_hip_qwen3_load_dir(model_dir); }
 /* weights live on the device either way */
@@ -356,8 +376,14 @@ void *qwen3_encoder_load(const char *model_dir, int use_mmap) {
     snprintf(path, sizeof path, "%s/tokenizer/tokenizer.json", model_dir);
     enc->tokenizer = qwen3_tokenizer_load(path);
     if (!enc->tokenizer) { flux_hip_fail("qwen3_encoder_load: failed to load %s", path); free(enc); return NULL; }
-    snprintf(path, sizeof path, "%s/text_encoder", model_dir);
-    enc->model = flux_hip_qwen3_load_dir(path);
+    snprintf(enc->dir, sizeof enc->dir, "%s/text_encoder", model_dir);
+    if (g_kept.model && !strcmp(g_kept.dir, enc->dir)) {
+        enc->model = g_kept.model;
+        g_kept.model = NULL;
+        flux_hip_qwen3_resident_hits++;
+    } else {
+        enc->model = flux_hip_qwen3_load_dir(enc->dir);
+    }
     if (!enc->model) { qwen3_tokenizer_free(enc->tokenizer); free(enc); return NULL; }
     return enc;
 }
@@ -366,7 +392,13 @@ void qwen3_encoder_free(void *p) {
     dropin_encoder *enc = (dropin_encoder *)p;
     if (!enc) return;
     if (qwen3_tokenizer_free) qwen3_tokenizer_free(enc->tokenizer);
-    flux_hip_qwen3_free(enc->model);
+    if (g_keep_resident && enc->model) {
+        flux_hip_qwen3_drop_resident();
+        g_kept.model = enc->model;
+        snprintf(g_kept.dir, sizeof g_kept.dir, "%s", enc->dir);
+    } else {
+        flux_hip_qwen3_free(enc->model);
+    }
     free(enc);
 }
 

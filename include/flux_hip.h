@@ -431,6 +431,15 @@ float *flux_hip_qwen3_forward(flux_hip_qwen3 *q, const int *input_ids, const int
 /* When set, called after each layer has been queued (role of flux_text_progress_callback). */
 extern void (*flux_hip_qwen3_progress)(int layer, int total);
 
+/* qwen3_encoder_free keeps the encoder's weights on the device and the next qwen3_encoder_load of the
+ * same directory takes them over instead of uploading 6 GB again (the reference frees its encoder
+ * after every prompt, flux.c:285-295; its weights are a memory map). keep_resident(0) switches that
+ * off and frees what is kept, drop_resident() frees it once; resident_hits counts the loads served
+ * from the kept weights. The files are not checked for changes in between. */
+void flux_hip_qwen3_keep_resident(int on);
+void flux_hip_qwen3_drop_resident(void);
+extern int flux_hip_qwen3_resident_hits;
+
 /* The reference's own entry points (flux_qwen3.h:93-141) over the device encoder: an application
  * keeps flux_qwen3_tokenizer.c and leaves flux_qwen3.c out of its link. Declared here only when the
  * reference's header has not been included (its declarations use its own opaque types). */

@@ -253,8 +253,20 @@ assert img_p, P.flux_get_error()
 im = ctypes.cast(img_p, ctypes.POINTER(FluxImage)).contents
 np.save(out, np.ctypeslib.as_array(im.data, shape=(im.height, im.width, im.channels)).copy())
 P.flux_image_free(img_p)
-P.flux_free(ctx)
 assert layers and layers[0] == (0, 27) and layers[-1] == (26, 27), layers[:3]
+if len(sys.argv) <= 9:
+    # a second prompt on the same context: flux.c has freed the text encoder and loads it again;
+    # the weights were kept on the device, and the same request gives the same image
+    hits = ctypes.c_int.in_dll(P, "flux_hip_qwen3_resident_hits")
+    before = hits.value
+    img2 = P.flux_generate(ctx, prompt.encode(), ctypes.byref(prm))
+    assert img2, P.flux_get_error()
+    im2 = ctypes.cast(img2, ctypes.POINTER(FluxImage)).contents
+    again = np.ctypeslib.as_array(im2.data, shape=(im2.height, im2.width, im2.channels)).copy()
+    P.flux_image_free(img2)
+    assert hits.value == before + 1, (before, hits.value)
+    assert np.array_equal(again, np.load(out))
+P.flux_free(ctx)
 print("child ok", len(layers))
 """
 
