@@ -426,6 +426,26 @@ def test_vae_encode_large(vae_pair, side):
     assert r <= 2e-2
 
 
+def test_vae_maximum_sizes(vae_pair):
+    """The largest images the reference accepts (1792 pixels a side, flux.h:52), where the oracle would take
+    many minutes: size-independent properties only. The row softmax takes its three-pass form here (51200
+    score columns), the attention runs in 12 chunks."""
+    dev, _ = vae_pair
+    lat = normal_f32((128, 112, 109), 320, 1)
+    f, u = dev.decode(lat, 112, 109)
+    f2, u2 = dev.decode(lat, 112, 109)
+    assert f.shape == (3, 1792, 1744) and np.isfinite(f).all() and u.std() > 20.0
+    np.testing.assert_array_equal(u, u2)
+    np.testing.assert_array_equal(f, f2)
+    img = vae_test_image(1792, 1776, 321)
+    z = dev.encode(img)
+    assert z.shape == (128, 112, 111) and np.isfinite(z).all() and 0.2 < z.std() < 2.0
+    np.testing.assert_array_equal(z, dev.encode(img))
+    # and a small one afterwards, on the same (now large) work buffers, still agrees with the oracle
+    small = normal_f32((128, 2, 3), 304, 1)
+    assert rel_l2(dev.decode(small, 2, 3)[0], vae_pair[1].decode(small, 2, 3)[0]) <= 2e-2
+
+
 def test_vae_encode_errors(hip, vae_pair):
     dev, _ = vae_pair
     L = hip.lib()
