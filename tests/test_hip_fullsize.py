@@ -82,3 +82,20 @@ def test_c5_cfg_with_reference_first_step(models):
     check(vg[0], vo[0], "c5 uncond")
     check(vg[1], vo[1], "c5 cond")
     assert psnr(zg, zo) >= 35.0
+
+
+def test_maximum_size_properties(models):
+    """1792 x 1792 (12544 image + 512 text tokens, the largest image the reference accepts, flux.h:52), alone
+    and with two reference images of other sizes (14244 tokens): the oracle would need half an hour per
+    forward, so only what does not depend on it - finite velocities of unit scale, the same bits on a second run."""
+    fluxhip, m, _ = models
+    for h, w, nt, refs in ((112, 112, 512, []), (112, 109, 300, [(40, 37, 10), (16, 16, 20)])):
+        z = normal_f32((128, h, w), 124, 1)
+        txt = normal_f32((nt, 7680), 124, 2)
+        rf = [(normal_f32((128, rh, rw), 124, 10 + i), rh, rw, t) for i, (rh, rw, t) in enumerate(refs)]
+        s = fluxhip.schedule("official", 4, h * w)[:2]
+        z1, v1 = m.sample(z, h, w, txt, s, refs=rf, trace=True)
+        z2, v2 = m.sample(z, h, w, txt, s, refs=rf, trace=True)
+        assert v1[0].shape == (128 * h * w,) and np.isfinite(v1[0]).all() and 0.3 < v1[0].std() < 3.0
+        np.testing.assert_array_equal(v1[0], v2[0])
+        np.testing.assert_array_equal(z1, z2)
