@@ -301,16 +301,23 @@ float *flux_hip_qwen3_forward(flux_hip_qwen3 *q, const int *input_ids, const int
     if (attention_mask && !flux_hip_upload(q->mask, attention_mask, (size_t)S * 4)) return NULL;
     const int *mask = attention_mask ? q->mask : NULL;
     if (!flux_hip_qwen3_embed(q->x, q->embed, q->ids, S, H, c->vocab)) return NULL;
+    /* normed: xn already holds the RMS norm that the next projection reads, written by the second pass
+     * of the residual projection before it (flux_hip_linear_resid_adaln in its RMS form) */
+    int normed = 0;
     for (int li = 0; li < q->n_run; li++) {
         const qlayer *l = &q->layer[li];
-        if (!flux_hip_rms_norm(q->xn, q->x, l->in_norm, S, H, c->eps)) return NULL;
+        if (!normed && !flux_hip_rms_norm(q->xn, q->x, l->in_norm, S, H, c->eps)) return NULL;
         if (!linear1(FLUX_HIP_EPI_BF16, q->xn, l->qkv, q->qkv, NULL, S, W, H, H, W, 0, 0)) return NULL;
         if (!flux_hip_qwen3_qk_rope(q->qkv, q->vt, QW_MAX_SEQ, l->q_norm, l->k_norm, q->rope_cos, q->rope_sin, S, c->heads, c->kv_heads, c->eps)) return NULL;
         if (!flux_hip_causal_attention(q->att, q->qkv, q->vt, QW_MAX_SEQ, mask, S, c->heads, c->kv_heads)) return NULL;
-        if (!linear1(FLUX_HIP_EPI_RESID, q->att, l->o, q->x, q->ones, S, H, QD, QD, H, 0, 0)) return NULL;
-        if (!flux_hip_rms_norm(q->xn, q->x, l->post_norm, S, H, c->eps)) return NULL;
+        flux_hip_linear_part po = {q->att, l->o, q->x, q->ones, S};
+        flux_hip_adaln_part no = {q->xn, NULL, l->post_norm};
+        if (!flux_hip_linear_resid_adaln(1, &po, H, QD, QD, QD, H, &no, c->eps, &normed)) return NULL;
+        if (!normed && !flux_hip_rms_norm(q->xn, q->x, l->post_norm, S, H, c->eps)) return NULL;
         if (!linear1(FLUX_HIP_EPI_SWIGLU, q->xn, l->gate_up, q->act, NULL, S, 2 * I, H, H, I, 0, I)) return NULL;
-        if (!linear1(FLUX_HIP_EPI_RESID, q->act, l->down, q->x, q->ones, S, H, I, I, H, 0, 0)) return NULL;
+        flux_hip_linear_part pd = {q->act, l->down, q->x, q->ones, S};
+        flux_hip_adaln_part nd = {q->xn, NULL, li + 1 < q->n_run ? q->layer[li + 1].in_norm : NULL};
+        if (!flux_hip_linear_resid_adaln(1, &pd, H, I, I, I, H, nd.scale ? &nd : NULL, c->eps, &normed)) return NULL;
         for (int j = 0; j < 3; j++)
             if (c->out_layer[j] == li && !flux_hip_qwen3_collect(q->out, 3 * H, j * H, q->x, S, H)) return NULL;
         if (flux_hip_qwen3_progress) flux_hip_qwen3_progress(li, q->n_run);

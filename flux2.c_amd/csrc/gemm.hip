@@ -591,7 +591,7 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(GemmArgs g) {
  * read and write of x, one write of the normalised row. N <= 4096. */
 struct AdalnArgs {
     bf16 *out[GEMM_MAX_PARTS];
-    const float *shift[GEMM_MAX_PARTS], *scale[GEMM_MAX_PARTS];
+    const float *shift[GEMM_MAX_PARTS], *scale[GEMM_MAX_PARTS]; /* RMS form: scale = the norm's weight, shift unused */
     int ldo;
     float eps;
 };
@@ -604,6 +604,9 @@ __device__ __forceinline__ float block_sum_256(float v, float *red) {
     return (red[0] + red[1]) + (red[2] + red[3]);
 }
 
+/* RMS = true: the norm that follows is x / sqrt(mean(x^2) + eps) * weight instead (qwen3_rms_norm,
+ * flux_qwen3.c:177-197) */
+template <bool RMS>
 __global__ __launch_bounds__(256) void splitk_finish_adaln_kernel(GemmArgs g, AdalnArgs a) {
     __shared__ float red[4];
     const int row = blockIdx.x;
@@ -664,7 +667,7 @@ __global__ __launch_bounds__(256) void splitk_finish_adaln_kernel(GemmArgs g, Ad
             s1 += (x[0] + x[1]) + (x[2] + x[3]);
         }
     }
-    const float mean = block_sum_256(s1, red) / (float)N;
+    const float mean = RMS ? 0.0f : block_sum_256(s1, red) / (float)N;
     float q = 0.0f;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -680,10 +683,16 @@ __global__ __launch_bounds__(256) void splitk_finish_adaln_kernel(GemmArgs g, Ad
     for (int i = 0; i < 4; i++) {
         const int c = (i * 256 + threadIdx.x) * 4;
         if (c < N) {
-            const f32x4 sh = *(const f32x4 *)(a.shift[prob] + c), sc = *(const f32x4 *)(a.scale[prob] + c);
+            const f32x4 sc = *(const f32x4 *)(a.scale[prob] + c);
             bf16x4 r;
+            if (RMS) {
 #pragma unroll
-            for (int e = 0; e < 4; e++) r[e] = (bf16)((1.0f + sc[e]) * ((v[i][e] - mean) * inv) + sh[e]);
+                for (int e = 0; e < 4; e++) r[e] = (bf16)(v[i][e] * inv * sc[e]);
+            } else {
+                const f32x4 sh = *(const f32x4 *)(a.shift[prob] + c);
+#pragma unroll
+                for (int e = 0; e < 4; e++) r[e] = (bf16)((1.0f + sc[e]) * ((v[i][e] - mean) * inv) + sh[e]);
+            }
             *(bf16x4 *)(o + c) = r;
         }
     }
@@ -699,7 +708,10 @@ static int launch_split(GemmArgs &g, int tile) {
 
 static int launch_split_adaln(GemmArgs &g, int tile, const AdalnArgs &a) {
     if (!launch_epi<EPI_PARTIAL>(g, tile)) return 0;
-    hipLaunchKernelGGL(splitk_finish_adaln_kernel, dim3((unsigned)g.ws_rows), dim3(256), 0, flux_hip_stream_handle(), g, a);
+    if (a.shift[0])
+        hipLaunchKernelGGL(splitk_finish_adaln_kernel<false>, dim3((unsigned)g.ws_rows), dim3(256), 0, flux_hip_stream_handle(), g, a);
+    else
+        hipLaunchKernelGGL(splitk_finish_adaln_kernel<true>, dim3((unsigned)g.ws_rows), dim3(256), 0, flux_hip_stream_handle(), g, a);
     return hipGetLastError() == hipSuccess ? 1 : flux_hip_fail("split-K reduction + AdaLN launch failed");
 }
 
@@ -942,9 +954,9 @@ extern "C" int flux_hip_linear_resid_adaln(int nparts, const flux_hip_linear_par
     if (norm) {
         if (N > 4096) return flux_hip_fail("flux_hip_linear_resid_adaln: N=%d (at most 4096 columns per row)", N);
         for (int i = 0; i < nparts && i < GEMM_MAX_PARTS; i++)
-            if (parts[i].M > 0 && (!norm[i].out_bf16 || !norm[i].shift || !norm[i].scale ||
+            if (parts[i].M > 0 && (!norm[i].out_bf16 || !norm[i].scale || (!norm[i].shift) != (!norm[0].shift) ||
                                    (((uintptr_t)norm[i].out_bf16 | (uintptr_t)norm[i].shift | (uintptr_t)norm[i].scale) & 15)))
-                return flux_hip_fail("flux_hip_linear_resid_adaln: NULL or unaligned AdaLN operand");
+                return flux_hip_fail("flux_hip_linear_resid_adaln: NULL or unaligned norm operand (shift must be given for all parts or for none)");
     }
     return linear_impl(FLUX_HIP_EPI_RESID, nparts, parts, N, K, lda, ldw, ldc, 0, 0, norm, eps, fused);
 }

@@ -98,10 +98,13 @@ int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
  * also writes (1 + scale) * LayerNorm(x) + shift as bf16 [M, N] (row stride N) per part, and
  * *fused = 1. Otherwise (*fused = 0) only the projection has run and the caller normalises with
  * flux_hip_adaln_norm. norm = NULL: plain projection. N <= 4096.
+ * With shift = NULL in every part the norm is the text encoder's RMS norm instead (qwen3_rms_norm,
+ * flux_qwen3.c:177-197, which follows both residual projections of a layer): x / sqrt(mean(x^2) +
+ * eps) * scale, scale being that norm's weight; *fused = 0 then leaves it to flux_hip_rms_norm.
  */
 typedef struct {
     void *out_bf16;       /* bf16 [M, N] */
-    const float *shift;   /* f32 [N] */
+    const float *shift;   /* f32 [N], or NULL for the RMS form */
     const float *scale;   /* f32 [N] */
 } flux_hip_adaln_part;
 int flux_hip_linear_resid_adaln(int nparts, const flux_hip_linear_part *parts, int N, int K, int lda, int ldw, int ldc,

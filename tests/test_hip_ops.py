@@ -235,6 +235,29 @@ def test_linear_residual_then_adaln(hip, oracle_mod, shape, tile):
     hip.lib().flux_hip_linear_force_tile(-1)
 
 
+def test_linear_residual_then_rms_norm(hip, oracle_mod):
+    """The same second pass with the text encoder's RMS norm (no shift, scale = the norm's weight)."""
+    M, N, K = 96, 2560, 4096
+    a = q(normal_f32((M, K), 25, 1))
+    W = q(normal_f32((N, K), 25, 2, 0.0, 0.05))
+    res = normal_f32((M, N), 25, 3)
+    g = np.ones(N, np.float32)
+    wn = normal_f32((N,), 25, 4, 1.0, 0.2)
+    da, dW, dg, dwn = dev_bf16(hip, a), dev_bf16(hip, W), hip.DevBuf.from_array(g), hip.DevBuf.from_array(wn)
+    dres = hip.DevBuf.from_array(res)
+    dn = hip.DevBuf.from_array(np.full((M, N), 0x7fc0, np.uint16))
+    fused = hip.linear_resid_adaln([(da.ptr, dW.ptr, dres.ptr, dg.ptr, M)], N, K, K, K, N, [(dn.ptr, None, dwn.ptr)])
+    assert fused
+    x = dres.to_array(np.float32, (M, N))
+    want_x = res + oracle_mod.linear(a, W)
+    assert rel_l2(x, want_x) < 2e-6
+    assert rel_l2(bf16_to_f32(dn.to_array(np.uint16, (M, N))), oracle_mod.qwen3_rms_norm(want_x, wn, 1e-6)) < 4e-3
+    # shift given for one part only: rejected before anything runs
+    with pytest.raises(hip.FluxHipError):
+        hip.linear_resid_adaln([(da.ptr, dW.ptr, dres.ptr, dg.ptr, 64), (da.ptr, dW.ptr, dres.ptr, dg.ptr, 32)], N, K, K, K, N,
+                               [(dn.ptr, None, dwn.ptr), (dn.ptr, dwn.ptr, dwn.ptr)])
+
+
 def test_linear_rejects_bad_shapes(hip):
     d = hip.DevBuf(1024)
     with pytest.raises(hip.FluxHipError):
