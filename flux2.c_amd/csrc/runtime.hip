@@ -7,11 +7,14 @@
 #include "../../include/flux_hip.h"
 #include <stdarg.h>
 #include <string.h>
+#include <stdlib.h>
 
 static char g_err[512] = "";
 static hipStream_t g_stream = nullptr;
 static int g_ready = 0;
 static hipEvent_t g_ev0 = nullptr, g_ev1 = nullptr;
+static void *g_stage = nullptr; /* pinned staging buffer of flux_hip_download */
+static size_t g_stage_bytes = 0;
 
 extern "C" int flux_hip_fail(const char *fmt, ...) {
     va_list ap;
@@ -51,6 +54,9 @@ extern "C" void flux_hip_cleanup(void) {
     if (!g_ready) return;
     (void)hipStreamSynchronize(g_stream);
     flux_hip_linear_release();
+    if (g_stage) (void)hipHostFree(g_stage);
+    g_stage = nullptr;
+    g_stage_bytes = 0;
     (void)hipEventDestroy(g_ev0);
     (void)hipEventDestroy(g_ev1);
     (void)hipStreamDestroy(g_stream);
@@ -87,9 +93,29 @@ extern "C" int flux_hip_upload(void *dst, const void *src, size_t bytes) {
     return 1;
 }
 
+/* Large results go through a pinned staging buffer (kept, grown on demand) and a host copy: a
+ * device-to-host copy into pageable memory runs at a fraction of the link's rate. */
+#define STAGE_MIN ((size_t)1 << 20)
+#define STAGE_MAX ((size_t)256 << 20)
+
 extern "C" int flux_hip_download(void *dst, const void *src, size_t bytes) {
     if (!flux_hip_available()) return 0;
     if (!bytes) return 1;
+    if (bytes >= STAGE_MIN && bytes <= STAGE_MAX) {
+        if (bytes > g_stage_bytes) {
+            if (g_stage) (void)hipHostFree(g_stage);
+            g_stage = nullptr;
+            g_stage_bytes = 0;
+            if (hipHostMalloc(&g_stage, bytes, hipHostMallocDefault) == hipSuccess) g_stage_bytes = bytes;
+            else { g_stage = nullptr; (void)hipGetLastError(); }
+        }
+        if (g_stage) {
+            HIP_OK(hipMemcpyAsync(g_stage, src, bytes, hipMemcpyDeviceToHost, g_stream));
+            HIP_OK(hipStreamSynchronize(g_stream));
+            memcpy(dst, g_stage, bytes);
+            return 1;
+        }
+    }
     HIP_OK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
     HIP_OK(hipStreamSynchronize(g_stream));
     return 1;
