@@ -287,20 +287,10 @@ def _byte_level_tokenizer_json():
     return json.dumps({"model": {"vocab": vocab, "merges": []}, "added_tokens": []}, ensure_ascii=False)
 
 
-@pytest.mark.skipif(not (os.path.exists(PIPE_GPUALL) and os.path.exists(REF)), reason="reference-built libraries not present")
-@pytest.mark.parametrize("mode", ["distilled", "cfg", "img2img", "img2img_cfg", "multiref"])
-def test_prompt_to_image_with_all_stages_on_the_device(oracle_mod, tmp_path, mode):
-    """flux_generate(ctx, prompt) / flux_img2img(ctx, prompt, picture) / flux_multiref(ctx, prompt, two pictures
-    of different sizes) through the reference's flux.c: its
-    tokenizer on the CPU, then text encoder, (VAE encoder of the input picture,) denoising loop (Euler, or
-    CFG with the empty prompt for a non-distilled model; the picture's latent as reference tokens) and VAE
-    decoder on the device. Expected image: the reference's tokenizer, then the CPU oracles of the stages."""
-    import subprocess
-    import sys
-    from dataclasses import replace
-    from model_spec import QwenConfig, make_qwen3_weights, vae_test_image
-    distilled = mode in ("distilled", "img2img", "multiref")
-    img2img = mode.startswith("img2img") or mode == "multiref"
+def _write_model_dir(tmp_path, distilled):
+    """A model directory as flux_load_dir reads it (flux.c:142-250): transformer, VAE, text encoder in two
+    shards, tokenizer, model_index.json. Small transformer and text encoder, full-size VAE, random weights."""
+    from model_spec import QwenConfig, make_qwen3_weights
     cfg = SMALL
     qcfg = QwenConfig(hidden=cfg.text_dim // 3, intermediate=384, heads=4, kv_heads=2, layers=27, vocab=151936)
     W, VW, QW = make_weights(cfg, 42, 0.05, "sharp"), make_vae_weights(), make_qwen3_weights(qcfg)
@@ -314,6 +304,23 @@ def test_prompt_to_image_with_all_stages_on_the_device(oracle_mod, tmp_path, mod
     write_safetensors(str(tmp_path / "text_encoder" / "model-00002-of-00002.safetensors"), {n: QW[n] for n in names[half:]})
     (tmp_path / "tokenizer" / "tokenizer.json").write_text(_byte_level_tokenizer_json(), encoding="utf-8")
     (tmp_path / "model_index.json").write_text('{"is_distilled": true}' if distilled else '{"_class_name": "Flux2Pipeline"}')
+    return cfg, qcfg, W, VW, QW
+
+
+@pytest.mark.skipif(not (os.path.exists(PIPE_GPUALL) and os.path.exists(REF)), reason="reference-built libraries not present")
+@pytest.mark.parametrize("mode", ["distilled", "cfg", "img2img", "img2img_cfg", "multiref"])
+def test_prompt_to_image_with_all_stages_on_the_device(oracle_mod, tmp_path, mode):
+    """flux_generate(ctx, prompt) / flux_img2img(ctx, prompt, picture) / flux_multiref(ctx, prompt, two pictures
+    of different sizes) through the reference's flux.c: its
+    tokenizer on the CPU, then text encoder, (VAE encoder of the input picture,) denoising loop (Euler, or
+    CFG with the empty prompt for a non-distilled model; the picture's latent as reference tokens) and VAE
+    decoder on the device. Expected image: the reference's tokenizer, then the CPU oracles of the stages."""
+    import subprocess
+    import sys
+    from model_spec import vae_test_image
+    distilled = mode in ("distilled", "img2img", "multiref")
+    img2img = mode.startswith("img2img") or mode == "multiref"
+    cfg, qcfg, W, VW, QW = _write_model_dir(tmp_path, distilled)
     width, height, steps, seed, prompt = 64, 64, 3, 21, "a small red fox"
     out = str(tmp_path / "img.npy")
     extra = []
@@ -388,3 +395,46 @@ def test_prompt_to_image_with_all_stages_on_the_device(oracle_mod, tmp_path, mod
     assert diff.mean() <= 2.0
     if img2img:
         assert diff.mean() <= 0.5 * effect       # well inside what the picture itself changes
+
+
+CLI = os.path.join(ROOT, "oracle", "_ref", "flux")
+
+
+@pytest.mark.skipif(not (os.path.exists(CLI) and os.path.exists(PIPE_GPUALL)), reason="reference-built programs not present")
+@pytest.mark.parametrize("mode", ["text", "picture", "two_pictures"])
+def test_reference_command_line_program(tmp_path, mode):
+    """The reference's own command-line program (main.c: options, seed, PNG in and out), linked against the
+    device library (make -C oracle cli), as a user runs it and as the reference's run_test.py:57-77 starts
+    it: -d DIR -p PROMPT --seed N --steps N -W N -H N -o OUT.png [-i IN.png ...]. The PNG it writes must
+    hold the image that the library level gives for the same request; that image is held against the CPU
+    oracles in test_prompt_to_image_with_all_stages_on_the_device."""
+    import subprocess
+    import sys
+    from PIL import Image
+    from model_spec import vae_test_image
+    _write_model_dir(tmp_path, True)
+    width, height, steps, seed, prompt = 64, 64, 3, 21, "a small red fox"
+    sizes = {"text": [], "picture": [(height, width)], "two_pictures": [(48, 64), (32, 32)]}[mode]
+    cli_in, lib_in = [], []
+    for i, (ph, pw) in enumerate(sizes):
+        pic = np.clip((vae_test_image(ph, pw, 41 + i).transpose(1, 2, 0) + 1.0) * 127.5, 0, 255).astype(np.uint8)
+        Image.fromarray(pic).save(str(tmp_path / f"input{i}.png"))
+        np.save(str(tmp_path / f"input{i}.npy"), pic)
+        cli_in += ["-i", str(tmp_path / f"input{i}.png")]
+        lib_in.append(str(tmp_path / f"input{i}.npy"))
+    out_png, out_npy = str(tmp_path / "out.png"), str(tmp_path / "img.npy")
+    cmd = [CLI, "-d", str(tmp_path), "-p", prompt, "--seed", str(seed), "--steps", str(steps),
+           "-W", str(width), "-H", str(height), "-o", out_png] + cli_in
+    print("running", " ".join(cmd[:1] + cmd[3:]), flush=True)
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    got = np.array(Image.open(out_png))
+    assert got.shape == (height, width, 3) and got.std() > 5.0
+    r = subprocess.run([sys.executable, "-c", _CHILD_PROMPT, PIPE_GPUALL, str(tmp_path), out_npy,
+                        str(width), str(height), str(steps), str(seed), prompt] + lib_in, capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0, r.stdout + r.stderr
+    want = np.load(out_npy)
+    diff = np.abs(got.astype(np.int32) - want.astype(np.int32))
+    print(f"command-line program vs library level ({mode}): mean abs diff {diff.mean():.3f}, max {diff.max()}", flush=True)
+    assert diff.mean() <= 20.0                   # run_test.py:96-104
+    assert np.array_equal(got, want)             # the same calls underneath: the same bits
