@@ -287,16 +287,29 @@ def _byte_level_tokenizer_json():
     return json.dumps({"model": {"vocab": vocab, "merges": []}, "added_tokens": []}, ensure_ascii=False)
 
 
-def _write_model_dir(tmp_path, distilled):
+def _write_model_dir(tmp_path, distilled, full_size=False):
     """A model directory as flux_load_dir reads it (flux.c:142-250): transformer, VAE, text encoder in two
-    shards, tokenizer, model_index.json. Small transformer and text encoder, full-size VAE, random weights."""
-    from model_spec import QwenConfig, make_qwen3_weights
-    cfg = SMALL
-    qcfg = QwenConfig(hidden=cfg.text_dim // 3, intermediate=384, heads=4, kv_heads=2, layers=27, vocab=151936)
-    W, VW, QW = make_weights(cfg, 42, 0.05, "sharp"), make_vae_weights(), make_qwen3_weights(qcfg)
+    shards, tokenizer, model_index.json. Random weights: a full-size VAE with a small transformer and text
+    encoder, or (full_size) the 4B transformer and layers 0-26 of the 4B text encoder, 14 GB on disk."""
+    from dataclasses import replace
+    from model_spec import KLEIN_4B, QWEN3_4B, QwenConfig, make_qwen3_weights
+    if full_size:
+        cfg, qcfg = KLEIN_4B, replace(QWEN3_4B, layers=27)
+        W = make_weights(cfg, 42, 0.02, "sharp")
+    else:
+        cfg = SMALL
+        qcfg = QwenConfig(hidden=cfg.text_dim // 3, intermediate=384, heads=4, kv_heads=2, layers=27, vocab=151936)
+        W = make_weights(cfg, 42, 0.05, "sharp")
+    if full_size:
+        print("transformer weights made", flush=True)
+    VW, QW = make_vae_weights(), make_qwen3_weights(qcfg)
+    if full_size:
+        print("text encoder weights made", flush=True)
     for d in ("transformer", "vae", "text_encoder", "tokenizer"):
         os.makedirs(tmp_path / d)
     write_safetensors(str(tmp_path / "transformer" / "diffusion_pytorch_model.safetensors"), W)
+    if full_size:
+        print("transformer file written", flush=True)
     write_safetensors(str(tmp_path / "vae" / "diffusion_pytorch_model.safetensors"), VW)
     names = list(QW)
     half = len(names) // 2
@@ -305,6 +318,59 @@ def _write_model_dir(tmp_path, distilled):
     (tmp_path / "tokenizer" / "tokenizer.json").write_text(_byte_level_tokenizer_json(), encoding="utf-8")
     (tmp_path / "model_index.json").write_text('{"is_distilled": true}' if distilled else '{"_class_name": "Flux2Pipeline"}')
     return cfg, qcfg, W, VW, QW
+
+
+def _expected_images(oracle_mod, tmp_path, cfg, qcfg, W, VW, QW, prompt, width, height, steps, seed, distilled, pictures):
+    """The image the pipeline should give, on the CPU: the reference's tokenizer, then the oracles of text
+    encoder, (VAE encoder,) sampling loop and VAE decoder. Returns (image, image without the input pictures or None)."""
+    R = ctypes.CDLL(REF)
+    R.qwen3_tokenizer_load.restype = vp
+    R.qwen3_tokenizer_load.argtypes = [ctypes.c_char_p]
+    R.qwen3_tokenize_chat.restype = ctypes.POINTER(c_i)
+    R.qwen3_tokenize_chat.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(c_i), c_i]
+    R.qwen3_tokenizer_free.argtypes = [vp]
+    tok = R.qwen3_tokenizer_load(str(tmp_path / "tokenizer" / "tokenizer.json").encode())
+    assert tok
+
+    def encode(text, q):
+        n = c_i(0)
+        p = R.qwen3_tokenize_chat(tok, text.encode(), ctypes.byref(n), 512)
+        ids = np.full(512, 151643, np.int32)                 # padded with <|endoftext|> (flux_qwen3_tokenizer.c:1059-1075)
+        ids[:n.value] = np.ctypeslib.as_array(p, shape=(n.value,))
+        mask = np.zeros(512, np.int32)
+        mask[:n.value] = 1
+        assert 10 < n.value < 64
+        return q.forward(ids, mask)
+
+    # ... then the three oracles
+    q = oracle_mod.Qwen3Oracle(qcfg, QW)
+    emb = encode(prompt, q)
+    emb_u = None if distilled else encode("", q)
+    q.close()
+    R.qwen3_tokenizer_free(tok)
+    lh, lw = height // 16, width // 16
+    vo = oracle_mod.VaeOracle(VW)
+    refs = None
+    if pictures:
+        # flux_image_to_tensor (flux_vae.c:1110-1135), the encoder, and the latents as reference tokens at time offsets 10, 20 (flux.c:806, 987)
+        refs = []
+        for i, pic in enumerate(pictures):
+            tensor = (pic.astype(np.float32) / np.float32(255.0) * np.float32(2.0) - np.float32(1.0)).transpose(2, 0, 1)
+            refs.append((vo.encode(tensor), pic.shape[0] // 16, pic.shape[1] // 16, 10 * (i + 1)))
+    o = oracle_mod.Oracle(cfg, W)
+    z0 = oracle_mod.init_noise(cfg.channels, lh, lw, seed)
+    sched = oracle_mod.official_schedule(steps, lh * lw)
+    if distilled:
+        latent = o.sample_euler(z0, lh, lw, emb, sched, refs=refs)
+    else:
+        latent = o.sample_euler_cfg(z0, lh, lw, emb, emb_u, 4.0, sched, refs=refs)    # default guidance of a base model, flux.c:222
+    if pictures:                                      # the picture matters: without it the expected image is another one
+        plain = o.sample_euler(z0, lh, lw, emb, sched) if distilled else o.sample_euler_cfg(z0, lh, lw, emb, emb_u, 4.0, sched)
+        _, other = vo.decode(plain, lh, lw)
+    o.close()
+    _, want = vo.decode(latent, lh, lw)
+    vo.close()
+    return want, (other if pictures else None)
 
 
 @pytest.mark.skipif(not (os.path.exists(PIPE_GPUALL) and os.path.exists(REF)), reason="reference-built libraries not present")
@@ -335,54 +401,7 @@ def test_prompt_to_image_with_all_stages_on_the_device(oracle_mod, tmp_path, mod
     assert r.returncode == 0, r.stdout + r.stderr
     got = np.load(out)
 
-    # expected, on the CPU: the reference's tokenizer ...
-    R = ctypes.CDLL(REF)
-    R.qwen3_tokenizer_load.restype = vp
-    R.qwen3_tokenizer_load.argtypes = [ctypes.c_char_p]
-    R.qwen3_tokenize_chat.restype = ctypes.POINTER(c_i)
-    R.qwen3_tokenize_chat.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(c_i), c_i]
-    R.qwen3_tokenizer_free.argtypes = [vp]
-    tok = R.qwen3_tokenizer_load(str(tmp_path / "tokenizer" / "tokenizer.json").encode())
-    assert tok
-
-    def encode(text, q):
-        n = c_i(0)
-        p = R.qwen3_tokenize_chat(tok, text.encode(), ctypes.byref(n), 512)
-        ids = np.full(512, 151643, np.int32)                 # padded with <|endoftext|> (flux_qwen3_tokenizer.c:1059-1075)
-        ids[:n.value] = np.ctypeslib.as_array(p, shape=(n.value,))
-        mask = np.zeros(512, np.int32)
-        mask[:n.value] = 1
-        assert 10 < n.value < 64
-        return q.forward(ids, mask)
-
-    # ... then the three oracles
-    q = oracle_mod.Qwen3Oracle(qcfg, QW)
-    emb = encode(prompt, q)
-    emb_u = None if distilled else encode("", q)
-    q.close()
-    R.qwen3_tokenizer_free(tok)
-    lh, lw = height // 16, width // 16
-    vo = oracle_mod.VaeOracle(VW)
-    refs = None
-    if img2img:
-        # flux_image_to_tensor (flux_vae.c:1110-1135), the encoder, and the latents as reference tokens at time offsets 10, 20 (flux.c:806, 987)
-        refs = []
-        for i, pic in enumerate(pictures):
-            tensor = (pic.astype(np.float32) / np.float32(255.0) * np.float32(2.0) - np.float32(1.0)).transpose(2, 0, 1)
-            refs.append((vo.encode(tensor), pic.shape[0] // 16, pic.shape[1] // 16, 10 * (i + 1)))
-    o = oracle_mod.Oracle(cfg, W)
-    z0 = oracle_mod.init_noise(cfg.channels, lh, lw, seed)
-    sched = oracle_mod.official_schedule(steps, lh * lw)
-    if distilled:
-        latent = o.sample_euler(z0, lh, lw, emb, sched, refs=refs)
-    else:
-        latent = o.sample_euler_cfg(z0, lh, lw, emb, emb_u, 4.0, sched, refs=refs)    # default guidance of a base model, flux.c:222
-    if img2img:                                      # the picture matters: without it the expected image is another one
-        plain = o.sample_euler(z0, lh, lw, emb, sched) if distilled else o.sample_euler_cfg(z0, lh, lw, emb, emb_u, 4.0, sched)
-        _, other = vo.decode(plain, lh, lw)
-    o.close()
-    _, want = vo.decode(latent, lh, lw)
-    vo.close()
+    want, other = _expected_images(oracle_mod, tmp_path, cfg, qcfg, W, VW, QW, prompt, width, height, steps, seed, distilled, pictures)
     if img2img:
         effect = np.abs(want.astype(np.int32) - other.astype(np.int32)).mean()
         print(f"effect of the input picture on the expected image: mean abs diff {effect:.2f}", flush=True)
@@ -438,3 +457,63 @@ def test_reference_command_line_program(tmp_path, mode):
     print(f"command-line program vs library level ({mode}): mean abs diff {diff.mean():.3f}, max {diff.max()}", flush=True)
     assert diff.mean() <= 20.0                   # run_test.py:96-104
     assert np.array_equal(got, want)             # the same calls underneath: the same bits
+
+
+def _room_for_full_size(path):
+    """The full-size run writes a 14 GB model directory and holds about 45 GB of host memory."""
+    import shutil
+    try:
+        avail = int(next(l for l in open("/proc/meminfo") if l.startswith("MemAvailable")).split()[1]) >> 20
+    except (OSError, StopIteration, ValueError):
+        avail = 0
+    return shutil.disk_usage(path).free >> 30 >= 24 and avail >= 80
+
+
+@pytest.mark.skipif(os.environ.get("FLUX_SKIP_FULLSIZE_E2E") == "1", reason="switched off by FLUX_SKIP_FULLSIZE_E2E=1")
+@pytest.mark.skipif(not (os.path.exists(CLI) and os.path.exists(REF)), reason="reference-built programs not present")
+def test_full_size_model_through_the_command_line_program(oracle_mod, tmp_path):
+    """The model at its real sizes (4B transformer, layers 0-26 of the 4B text encoder, the VAE; random
+    weights in bf16 safetensors files laid out like the published model directory) through the reference's
+    command-line program with all stages on the device. At 64x64 the PNG is held against the CPU oracles of
+    all stages; at 1024x1024 (the headline size) the run is timed, repeated, and must give the same PNG."""
+    import subprocess
+    import time
+    from PIL import Image
+    if not _room_for_full_size(str(tmp_path)):
+        pytest.skip("needs 24 GB of disk under the temporary directory and 80 GB of free host memory")
+    t0 = time.time()
+    cfg, qcfg, W, VW, QW = _write_model_dir(tmp_path, True, full_size=True)
+    print(f"model directory written in {time.time() - t0:.0f} s", flush=True)
+    prompt, seed, steps = "a lighthouse on a cliff at dawn", 7, 4
+
+    def run(width, height, out):
+        cmd = [CLI, "-d", str(tmp_path), "-p", prompt, "--seed", str(seed), "--steps", str(steps),
+               "-W", str(width), "-H", str(height), "-o", out, "-v"]
+        t = time.time()
+        r = subprocess.run(cmd, capture_output=True, text=True, timeout=900)
+        dt = time.time() - t
+        assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
+        return np.array(Image.open(out)), dt, r.stdout + r.stderr
+
+    got, dt, log = run(64, 64, str(tmp_path / "small.png"))
+    print(f"64x64, {steps} steps: {dt:.1f} s wall for the process", flush=True)
+    want, _ = _expected_images(oracle_mod, tmp_path, cfg, qcfg, W, VW, QW, prompt, 64, 64, steps, seed, True, [])
+    diff = np.abs(got.astype(np.int32) - want.astype(np.int32))
+    print(f"full-size model, prompt -> 64x64 PNG vs CPU oracles: mean abs diff {diff.mean():.3f}, max {diff.max()}, image std {want.std():.1f}", flush=True)
+    assert got.shape == (64, 64, 3) and want.std() > 5.0
+    assert diff.mean() <= 20.0                   # run_test.py:96-104
+    assert diff.mean() <= 2.0
+    del W, QW
+    big = []
+    for rep in range(2):
+        img, dt, log = run(1024, 1024, str(tmp_path / f"big{rep}.png"))
+        print(f"1024x1024, {steps} steps, run {rep}: {dt:.1f} s wall for the process (load, encode, denoise, decode, PNG)", flush=True)
+        for line in log.splitlines():
+            if any(k in line.lower() for k in ("load", "encod", "denois", "step", "decod", "total", "sav")) and len(line) < 160:
+                print("    | " + line.strip(), flush=True)
+        assert img.shape == (1024, 1024, 3) and img.std() > 5.0
+        big.append(img)
+    import shutil
+    for d in ("transformer", "text_encoder", "vae"):      # 14 GB that no later test needs
+        shutil.rmtree(str(tmp_path / d), ignore_errors=True)
+    assert np.array_equal(big[0], big[1])
