@@ -304,6 +304,8 @@ float *flux_hip_qwen3_forward(flux_hip_qwen3 *q, const int *input_ids, const int
     /* normed: xn already holds the RMS norm that the next projection reads, written by the second pass
      * of the residual projection before it (flux_hip_linear_resid_adaln in its RMS form) */
     int normed = 0;
+    int parts = 1;   /* 1: parts travel as they are produced; 0: no staging buffer, one download at the end */
+    const size_t part_bytes = (size_t)S * H * 4;
     for (int li = 0; li < q->n_run; li++) {
         const qlayer *l = &q->layer[li];
         if (!normed && !flux_hip_rms_norm(q->xn, q->x, l->in_norm, S, H, c->eps)) return NULL;
@@ -318,13 +320,34 @@ float *flux_hip_qwen3_forward(flux_hip_qwen3 *q, const int *input_ids, const int
         flux_hip_linear_part pd = {q->act, l->down, q->x, q->ones, S};
         flux_hip_adaln_part nd = {q->xn, NULL, li + 1 < q->n_run ? q->layer[li + 1].in_norm : NULL};
         if (!flux_hip_linear_resid_adaln(1, &pd, H, I, I, I, H, nd.scale ? &nd : NULL, c->eps, &normed)) return NULL;
-        for (int j = 0; j < 3; j++)
-            if (c->out_layer[j] == li && !flux_hip_qwen3_collect(q->out, 3 * H, j * H, q->x, S, H)) return NULL;
+        /* a captured layer goes to its third of q->out ([3][S][H], layer-major) and from there to the
+         * host at once, on the copy stream, while the layers after it run */
+        for (int j = 0; j < 3; j++) {
+            if (c->out_layer[j] != li) continue;
+            if (!flux_hip_qwen3_collect(q->out + (size_t)j * S * H, H, 0, q->x, S, H)) return NULL;
+            if (parts > 0) parts = flux_hip_download_part_begin(j, j * part_bytes, 3 * part_bytes, q->out + (size_t)j * S * H, part_bytes);
+            if (parts < 0) return NULL;
+        }
         if (flux_hip_qwen3_progress) flux_hip_qwen3_progress(li, q->n_run);
     }
     float *out = (float *)malloc((size_t)S * 3 * H * sizeof(float));
     if (!out) { flux_hip_fail("out of host memory"); return NULL; }
-    if (!flux_hip_download(out, q->out, (size_t)S * 3 * H * 4)) { free(out); return NULL; }
+    float *whole = NULL;    /* without a staging buffer (results under 1 MB): one download at the end */
+    if (!parts) {
+        whole = (float *)malloc(3 * part_bytes);
+        if (!whole || !flux_hip_download(whole, q->out, 3 * part_bytes)) {
+            if (!whole) flux_hip_fail("out of host memory");
+            free(whole); free(out);
+            return NULL;
+        }
+    }
+    /* [3][S][H] -> [S][3H]: the first two parts are interleaved while the device still computes */
+    for (int j = 0; j < 3; j++) {
+        const float *part = whole ? whole + (size_t)j * S * H : (const float *)flux_hip_download_part_wait(j);
+        if (!part) { free(out); return NULL; }
+        for (int r = 0; r < S; r++) memcpy(out + ((size_t)r * 3 + j) * H, part + (size_t)r * H, (size_t)H * 4);
+    }
+    free(whole);
     return out;
 }
 

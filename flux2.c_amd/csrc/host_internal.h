@@ -81,4 +81,8 @@ float fh_tensor_value(int dtype, const void *data, int64_t i);
 #ifdef __cplusplus
 }
 #endif
+/* runtime.hip: a result copied to the host part by part while later work runs (see there) */
+int flux_hip_download_part_begin(int part, size_t stage_offset, size_t stage_total, const void *src, size_t bytes);
+const void *flux_hip_download_part_wait(int part);
+
 #endif

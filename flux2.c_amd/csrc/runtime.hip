@@ -15,6 +15,10 @@ static int g_ready = 0;
 static hipEvent_t g_ev0 = nullptr, g_ev1 = nullptr;
 static void *g_stage = nullptr; /* pinned staging buffer of flux_hip_download */
 static size_t g_stage_bytes = 0;
+#define DOWNLOAD_PARTS 4
+static hipStream_t g_copy_stream = nullptr; /* carries flux_hip_download_part_begin's copies beside the main stream */
+static hipEvent_t g_part_ready[DOWNLOAD_PARTS], g_part_done[DOWNLOAD_PARTS];
+static const void *g_part_at[DOWNLOAD_PARTS];
 
 extern "C" int flux_hip_fail(const char *fmt, ...) {
     va_list ap;
@@ -42,6 +46,11 @@ extern "C" int flux_hip_init(void) {
     HIP_OK(hipStreamCreate(&g_stream));
     HIP_OK(hipEventCreate(&g_ev0));
     HIP_OK(hipEventCreate(&g_ev1));
+    HIP_OK(hipStreamCreateWithFlags(&g_copy_stream, hipStreamNonBlocking));
+    for (int i = 0; i < DOWNLOAD_PARTS; i++) {
+        HIP_OK(hipEventCreateWithFlags(&g_part_ready[i], hipEventDisableTiming));
+        HIP_OK(hipEventCreateWithFlags(&g_part_done[i], hipEventDisableTiming));
+    }
     g_ready = 1;
     return 1;
 }
@@ -59,6 +68,13 @@ extern "C" void flux_hip_cleanup(void) {
     g_stage_bytes = 0;
     (void)hipEventDestroy(g_ev0);
     (void)hipEventDestroy(g_ev1);
+    (void)hipStreamSynchronize(g_copy_stream);
+    for (int i = 0; i < DOWNLOAD_PARTS; i++) {
+        (void)hipEventDestroy(g_part_ready[i]);
+        (void)hipEventDestroy(g_part_done[i]);
+    }
+    (void)hipStreamDestroy(g_copy_stream);
+    g_copy_stream = nullptr;
     (void)hipStreamDestroy(g_stream);
     g_stream = nullptr;
     g_ready = 0;
@@ -118,6 +134,45 @@ extern "C" int flux_hip_download(void *dst, const void *src, size_t bytes) {
     HIP_OK(hipStreamSynchronize(g_stream));
     if (stage) memcpy(dst, stage, bytes);
     return 1;
+}
+
+/* A result whose parts become final one after the other (the captured layers of the text encoder):
+ * part_begin queues, on a second stream, the copy of one part into the pinned staging buffer at
+ * stage_offset, to start when the work queued so far on the main stream has run; the main stream goes
+ * on meanwhile. part_wait returns the part's host address once it has arrived. All parts of one
+ * result name the same stage_total. part_begin returns 1, 0 when there is no staging buffer of that
+ * size (the caller then downloads the whole result at the end), -1 on an error. */
+extern "C" int flux_hip_download_part_begin(int part, size_t stage_offset, size_t stage_total, const void *src, size_t bytes) {
+    if (!flux_hip_available()) return -1;
+    if (part < 0 || part >= DOWNLOAD_PARTS || stage_offset + bytes > stage_total) {
+        flux_hip_fail("flux_hip_download_part_begin: bad part");
+        return -1;
+    }
+    char *stage = (char *)stage_buffer(stage_total);
+    if (!stage) return 0;
+    if (hipEventRecord(g_part_ready[part], g_stream) != hipSuccess ||
+        hipStreamWaitEvent(g_copy_stream, g_part_ready[part], 0) != hipSuccess ||
+        hipMemcpyAsync(stage + stage_offset, src, bytes, hipMemcpyDeviceToHost, g_copy_stream) != hipSuccess ||
+        hipEventRecord(g_part_done[part], g_copy_stream) != hipSuccess) {
+        flux_hip_fail("flux_hip_download_part_begin: %s", hipGetErrorString(hipGetLastError()));
+        return -1;
+    }
+    g_part_at[part] = stage + stage_offset;
+    return 1;
+}
+
+extern "C" const void *flux_hip_download_part_wait(int part) {
+    if (!g_ready || part < 0 || part >= DOWNLOAD_PARTS || !g_part_at[part]) {
+        flux_hip_fail("flux_hip_download_part_wait: no such part");
+        return nullptr;
+    }
+    if (hipEventSynchronize(g_part_done[part]) != hipSuccess) {
+        flux_hip_fail("flux_hip_download_part_wait: %s", hipGetErrorString(hipGetLastError()));
+        return nullptr;
+    }
+    const void *at = g_part_at[part];
+    g_part_at[part] = nullptr;
+    return at;
 }
 
 extern "C" int flux_hip_memset(void *dst, int value, size_t bytes) {
