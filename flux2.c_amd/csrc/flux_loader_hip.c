@@ -159,8 +159,16 @@ int fh_safetensors_walk(const char *path, fh_tensor_cb cb, void *ctx) {
                             unsigned long long v = strtoull(p, &end, 10);
                             if (end == p) { flux_hip_fail("%s: malformed entry %s", path, name); goto fail; }
                             p = end;
-                            if (is_shape) numel *= (int64_t)v;
-                            else { if (idx == 0) off0 = v; else off1 = v; have_off = 1; }
+                            if (is_shape) {
+                                /* no product of sizes in a file that fits an address space comes near 2^62 */
+                                if (v > ((uint64_t)1 << 40) || (v && numel > (((int64_t)1 << 62) / (int64_t)v))) {
+                                    flux_hip_fail("%s: tensor %s has an impossible shape", path, name);
+                                    goto fail;
+                                }
+                                numel *= (int64_t)v;
+                            } else if (idx == 0) { off0 = v; have_off = 1; }
+                            else if (idx == 1) off1 = v;
+                            else { flux_hip_fail("%s: tensor %s has more than two data offsets", path, name); goto fail; }
                             idx++;
                             p = skip_ws(p, e);
                             if (p < e && *p == ',') p++;
@@ -174,6 +182,11 @@ int fh_safetensors_walk(const char *path, fh_tensor_cb cb, void *ctx) {
                 }
                 int dt = !strcmp(dtype, "BF16") ? DT_BF16 : !strcmp(dtype, "F32") ? DT_F32 : !strcmp(dtype, "F16") ? DT_F16 : -1;
                 size_t esz = dt == DT_F32 ? 4 : 2;
+                if (dt < 0) {   /* a type this library has no use for (integers, fp64, fp8): not handed on */
+                    p = skip_ws(p, e);
+                    if (p < e && *p == ',') p++;
+                    continue;
+                }
                 if (!have_off || off1 < off0 || off1 > dsize || (off1 - off0) != (uint64_t)numel * esz) {
                     flux_hip_fail("%s: tensor %s has inconsistent offsets", path, name);
                     goto fail;
@@ -192,7 +205,9 @@ fail:
 }
 
 static int transformer_tensor_cb(void *ctx, const char *name, int dtype, const void *data, int64_t numel) {
-    return set_from((flux_transformer_t *)ctx, name, dtype, data, numel);
+    if (set_from((flux_transformer_t *)ctx, name, dtype, data, numel)) return 1;
+    /* files may carry tensors this path does not use; only real failures abort */
+    return strstr(flux_hip_last_error(), "is not part of the transformer") != NULL;
 }
 
 flux_transformer_t *flux_hip_transformer_load_file(const char *path, const flux_hip_config *cfg) {
@@ -237,15 +252,34 @@ void fh_safetensors_close_compat(void *p) {
     free(sf);
 }
 
+/* Entry i of a parsed handle: where its data lies and how many elements it has. The handle comes
+ * from the reference's parser; what is checked here is that reading the entry stays inside the
+ * mapping it describes. */
+static int handle_entry(const ref_safetensors_file *sf, int i, const char **data, int64_t *numel) {
+    const ref_safetensor *t = &sf->tensors[i];
+    if (t->ndim < 0 || t->ndim > 8) return flux_hip_fail("safetensors handle: tensor %d has %d dimensions", i, t->ndim);
+    int64_t n = 1;
+    for (int d = 0; d < t->ndim; d++) {
+        if (t->shape[d] < 0 || (t->shape[d] && n > (((int64_t)1 << 62) / t->shape[d]))) return flux_hip_fail("safetensors handle: tensor %.200s has an impossible shape", t->name);
+        n *= t->shape[d];
+    }
+    const size_t esz = t->dtype == DT_F32 ? 4 : 2, head = 8 + sf->header_size;
+    if (head > sf->file_size || t->data_offset > sf->file_size - head || (uint64_t)n * esz > sf->file_size - head - t->data_offset)
+        return flux_hip_fail("safetensors handle: tensor %.200s lies outside its file", t->name);
+    *data = (const char *)sf->data + head + t->data_offset;
+    *numel = n;
+    return 1;
+}
+
 int fh_safetensors_walk_handle(void *p, fh_tensor_cb cb, void *ctx) {
     ref_safetensors_file *sf = (ref_safetensors_file *)p;
     if (!sf || !sf->data) return flux_hip_fail("safetensors handle is NULL");
     if (sf->num_tensors < 0 || sf->num_tensors > 512) return flux_hip_fail("safetensors handle: bad tensor count");
     for (int i = 0; i < sf->num_tensors; i++) {
-        const ref_safetensor *t = &sf->tensors[i];
-        int64_t numel = 1;
-        for (int d = 0; d < t->ndim; d++) numel *= t->shape[d];
-        if (!cb(ctx, t->name, t->dtype, (const char *)sf->data + 8 + sf->header_size + t->data_offset, numel)) return 0;
+        const char *data;
+        int64_t numel;
+        if (!handle_entry(sf, i, &data, &numel)) return 0;
+        if (!cb(ctx, sf->tensors[i].name, sf->tensors[i].dtype, data, numel)) return 0;
     }
     return 1;
 }
@@ -296,9 +330,9 @@ static flux_transformer_t *load_from_handle(void *p) {
     if (!tf) return NULL;
     for (int i = 0; i < sf->num_tensors; i++) {
         const ref_safetensor *t = &sf->tensors[i];
-        int64_t numel = 1;
-        for (int d = 0; d < t->ndim; d++) numel *= t->shape[d];
-        const char *data = (const char *)sf->data + 8 + sf->header_size + t->data_offset;
+        const char *data;
+        int64_t numel;
+        if (!handle_entry(sf, i, &data, &numel)) { flux_transformer_free(tf); return NULL; }
         if (!set_from(tf, t->name, t->dtype, data, numel)) {
             /* files may carry tensors this path does not use; only real failures abort */
             if (strstr(flux_hip_last_error(), "is not part of the transformer")) continue;

@@ -174,6 +174,63 @@ def test_safetensors_file_loader(hip, oracle_mod, tmp_path):
         hip.Transformer(cfg, path=str(p))
 
 
+def test_malformed_weight_files_are_refused(hip, tmp_path):
+    """Every way a .safetensors file can lie about itself ends in an error with a reason, never in a read
+    outside the mapping; tensors of other types or names are passed over."""
+    import json
+    import struct
+    cfg = TINY
+    W = make_weights(cfg, 42, 0.02, "sharp")
+    good = tmp_path / "good.safetensors"
+    write_safetensors(str(good), W)
+    raw = good.read_bytes()
+    hlen = struct.unpack("<Q", raw[:8])[0]
+    header, data = json.loads(raw[8:8 + hlen]), raw[8 + hlen:]
+
+    def write(name, hdr, payload=data, hlen_override=None):
+        hj = json.dumps(hdr, separators=(",", ":")).encode() if isinstance(hdr, dict) else hdr
+        q = tmp_path / name
+        q.write_bytes(struct.pack("<Q", len(hj) if hlen_override is None else hlen_override) + hj + payload)
+        return str(q)
+
+    def altered(fn):
+        h = json.loads(json.dumps(header))
+        fn(h)
+        return h
+
+    first = next(iter(header))
+    bad = {
+        "truncated data": write("a.safetensors", header, data[:len(data) // 2]),
+        "header length beyond the file": write("b.safetensors", header, hlen_override=1 << 40),
+        "header length zero": write("c.safetensors", header, hlen_override=0),
+        "not JSON": write("d.safetensors", b"[1, 2, 3]" + b" " * 7),
+        "cut-off JSON": write("e.safetensors", json.dumps(header).encode()[:hlen // 2]),
+        "shape larger than the byte range": write("f.safetensors", altered(lambda h: h[first].update(shape=[h[first]["shape"][0] * 2] + h[first]["shape"][1:]))),
+        "shape that overflows": write("g.safetensors", altered(lambda h: h[first].update(shape=[1 << 39, 1 << 39]))),
+        "offsets reversed": write("h.safetensors", altered(lambda h: h[first].update(data_offsets=h[first]["data_offsets"][::-1]))),
+        "offsets beyond the data": write("i.safetensors", altered(lambda h: h[first].update(data_offsets=[len(data), len(data) + h[first]["data_offsets"][1]]))),
+        "no offsets": write("j.safetensors", altered(lambda h: h[first].pop("data_offsets"))),
+    }
+    (tmp_path / "k.safetensors").write_bytes(b"abc")
+    bad["shorter than its length field"] = str(tmp_path / "k.safetensors")
+    bad["missing file"] = str(tmp_path / "nothing.safetensors")
+    for what, path in bad.items():
+        with pytest.raises(hip.FluxHipError) as err:
+            hip.Transformer(cfg, path=path)
+        print(f"{what}: {err.value}", flush=True)
+        assert len(str(err.value)) > 20
+    # passed over: a tensor of a type the library has no use for, and one under a name it does not know
+    extra = altered(lambda h: (h.update({"step_count": {"dtype": "I64", "shape": [1], "data_offsets": [len(data), len(data) + 8]}}),
+                               h.update({"ema.decay": {"dtype": "BF16", "shape": [4], "data_offsets": [len(data) + 8, len(data) + 16]}}),
+                               h.update({"__metadata__": {"format": "pt"}})))
+    a = hip.Transformer(cfg, path=write("l.safetensors", extra, data + bytes(16)))
+    b = hip.Transformer(cfg, path=str(good))
+    lat = normal_f32((cfg.channels, 4, 4), 14, 1)
+    txt = normal_f32((16, cfg.text_dim), 14, 2)
+    assert np.array_equal(a.forward(lat, 4, 4, txt, 0.5), b.forward(lat, 4, 4, txt, 0.5))
+    a.close(); b.close()
+
+
 def test_error_paths(hip):
     cfg = TINY
     m = hip.Transformer(cfg)          # no weights yet
