@@ -29,6 +29,12 @@
  * so the loop is software-pipelined by hand: fragments are double-buffered in registers, every
  * fourth MFMA is followed by one LDS read for the next half-step and (in the second half) one
  * global->LDS load for the stage after next, and there is one barrier per 64-wide K step.
+ * A lone wave cannot keep its SIMD's matrix pipe busy: back-to-back independent 16x16x32 MFMAs
+ * from one wave fill 64 % of the issue slots, from two waves 97 % (measured with operands in
+ * registers; counters put this kernel at 71 %). The same loop therefore also exists over a
+ * WGM x WGN grid of waves; with 8 waves (2 x 4, 128 x 64 each, two per SIMD) on the 256 x 256
+ * tile it runs at the speed of the 4-wave form, its extra issue slots spent waiting at the
+ * barrier, and is kept for comparison runs (tile id 4).
  *
  * LDS rows are 128 bytes (64 bf16); the 16-byte chunk index is XOR-swizzled with a function of
  * the row so that the 16 rows a fragment read touches spread over all banks. A direct-to-LDS
@@ -350,10 +356,13 @@ __device__ __forceinline__ void acc_fence(f32x4 (&acc)[TN][TM]) {
 
 template <bool V> struct BoolC { static constexpr bool value = V; };
 
-template <int TM, int TN, int EPI>
-__global__ __launch_bounds__(256) void gemm4w_kernel(GemmArgs g) {
-    constexpr int BM = 32 * TM, BN = 32 * TN, WGN = 2, WM = 16 * TM, WN = 16 * TN;
-    constexpr int NL = TM + TN;     /* global->LDS loads per wave and stage: 8 tile rows each */
+template <int TM, int TN, int EPI, int WGM = 2, int WGN = 2>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm4w_kernel(GemmArgs g) {
+    constexpr int WM = 16 * TM, WN = 16 * TN, BM = WGM * WM, BN = WGN * WN;
+    constexpr int RPP = 8 * WGM * WGN; /* tile rows one pass of the workgroup's loads covers: 8 per wave instruction */
+    static_assert(BM % RPP == 0 && BN % RPP == 0, "tile rows must divide evenly over the waves' loads");
+    constexpr int LA = BM / RPP, LB = BN / RPP;
+    constexpr int NL = LA + LB;     /* global->LDS loads per wave and stage: 8 tile rows each */
     constexpr int NF = TM + TN;     /* fragments per K half-step: TN weight side, TM activation side */
     constexpr int NM = TM * TN;     /* MFMAs per K half-step */
     constexpr int RD = NM / NF;     /* one LDS read (and one load) every RD MFMAs */
@@ -375,21 +384,21 @@ __global__ __launch_bounds__(256) void gemm4w_kernel(GemmArgs g) {
     const int wm = wave / WGN, wn = wave % WGN;
     const int lrow = tid >> 3, lchunk = tid & 7;
 
-    /* Load i of a stage by this wave covers tile rows lrow + 32 i (8 rows of 128 bytes per wave
-     * instruction): activation rows for i < TM, weight rows after. Rows 32 apart share a swizzle.
+    /* Load i of a stage by this wave covers tile rows lrow + RPP i (8 rows of 128 bytes per wave
+     * instruction): activation rows for i < LA, weight rows after. Rows RPP apart share a swizzle.
      * The K offset of this workgroup's slice is folded into the per-lane sources. */
     const int kt_begin = t.ks * g.kt_per;
     const int KT = min(g.K >> 6, kt_begin + g.kt_per) - kt_begin;
     const int chunk = ((lchunk ^ lds_swz(lrow)) << 3) + kt_begin * 64;
     const bf16 *src[NL];
 #pragma unroll
-    for (int i = 0; i < TM; i++) src[i] = A + (size_t)min(m0 + lrow + i * 32, M - 1) * g.lda + chunk;
+    for (int i = 0; i < LA; i++) src[i] = A + (size_t)min(m0 + lrow + i * RPP, M - 1) * g.lda + chunk;
 #pragma unroll
-    for (int i = 0; i < TN; i++) src[TM + i] = W + (size_t)weight_row<BN, WN, EPI>(g, tn, lrow + i * 32) * g.ldw + chunk;
+    for (int i = 0; i < LB; i++) src[LA + i] = W + (size_t)weight_row<BN, WN, EPI>(g, tn, lrow + i * RPP) * g.ldw + chunk;
     /* (convolutions never split K, so for them kt below is the absolute K step) */
     auto issue1 = [&](int kt, int stage, int i) {
-        const int off = i < TM ? a_step_offset<EPI>(g, kt) : kt * 64;
-        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src[i] + off), LDS_PTR(smem + stage * STAGE + (lrow - (lane >> 3) + i * 32) * 128), 16, 0, 0);
+        const int off = i < LA ? a_step_offset<EPI>(g, kt) : kt * 64;
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src[i] + off), LDS_PTR(smem + stage * STAGE + (lrow - (lane >> 3) + i * RPP) * 128), 16, 0, 0);
     };
 #pragma unroll
     for (int i = 0; i < NL; i++) issue1(0, 0, i);
@@ -461,7 +470,7 @@ __global__ __launch_bounds__(256) void gemm4w_kernel(GemmArgs g) {
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); /* the last MFMA results retire before they are read */
     acc_fence<TM, TN>(acc);
 
-    store_tile<BN, WM, WN, EPI>(g, t, acc, m0, M, wm, wn, l15, lq, t.tm * 2 + wm);
+    store_tile<BN, WM, WN, EPI>(g, t, acc, m0, M, wm, wn, l15, lq, t.tm * WGM + wm);
 }
 
 /* ------------------------------------------------------------------ host side */
@@ -494,11 +503,11 @@ static int launch_cfg(GemmArgs &g) {
     return 1;
 }
 
-template <int TM, int TN, int EPI>
+template <int TM, int TN, int EPI, int WGM = 2, int WGN = 2>
 static int launch_4w(GemmArgs &g) {
-    constexpr int BM = 32 * TM, BN = 32 * TN, LDS = 2 * (BM + BN) * 128;
+    constexpr int BM = 16 * TM * WGM, BN = 16 * TN * WGN, LDS = 2 * (BM + BN) * 128;
     static bool attr_done = false;
-    auto kern = gemm4w_kernel<TM, TN, EPI>;
+    auto kern = gemm4w_kernel<TM, TN, EPI, WGM, WGN>;
     if (!attr_done) {
         HIP_OK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
         attr_done = true;
@@ -507,7 +516,7 @@ static int launch_4w(GemmArgs &g) {
     g.ntiles = g.N / BN;
     g.total_tiles = g.mtiles * g.ntiles;
     int grid = (g.total_tiles * g.ksplit + 7) & ~7;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), LDS, flux_hip_stream_handle(), g);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WGM * WGN), LDS, flux_hip_stream_handle(), g);
     HIP_OK(hipGetLastError());
     return 1;
 }
@@ -519,7 +528,7 @@ static int launch_epi(GemmArgs &g, int tile) {
         case 5: return launch_4w<9, 6, EPI>(g);
         case 6: return launch_4w<6, 6, EPI>(g);
         case 7: return launch_4w<8, 6, EPI>(g);
-        case 4: return launch_cfg<256, 256, 2, 4, EPI>(g); /* 8-wave form of the same tile, for comparison runs */
+        case 4: return launch_4w<8, 4, EPI, 2, 4>(g); /* 8 waves, two per SIMD, on the 256x256 tile */
         case 1: return launch_cfg<128, 128, 2, 2, EPI>(g);
         case 3: return launch_cfg<64, 64, 2, 2, EPI>(g);
         default: return launch_cfg<64, 128, 2, 2, EPI>(g);
@@ -736,7 +745,7 @@ extern "C" void flux_hip_linear_release(void) {
 }
 
 static int g_force_tile = -1;
-static unsigned g_tile_mask = 0xEF; /* tiles the automatic choice may use: all but the 8-wave comparison form */
+static unsigned g_tile_mask = 0xEF; /* tiles the automatic choice may use: all but the 8-wave form of 256 x 256 */
 static int g_splitk_enabled = 1;
 extern "C" void flux_hip_linear_force_tile(int tile) { g_force_tile = tile; }
 extern "C" void flux_hip_linear_tile_mask(unsigned mask) { g_tile_mask = mask ? mask : 0xEF; }
