@@ -398,7 +398,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm4w_kernel(GemmArgs g) {
     /* (convolutions never split K, so for them kt below is the absolute K step) */
     auto issue1 = [&](int kt, int stage, int i) {
         const int off = i < LA ? a_step_offset<EPI>(g, kt) : kt * 64;
-        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src[i] + off), LDS_PTR(smem + stage * STAGE + (lrow - (lane >> 3) + i * RPP) * 128), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src[i] + off), LDS_PTR(smem + stage * STAGE + (wave * 8 + i * RPP) * 128), 16, 0, 0);
     };
 #pragma unroll
     for (int i = 0; i < NL; i++) issue1(0, 0, i);
