@@ -27,14 +27,28 @@
  * limit is what buys throughput (1020 -> 1145 TFLOP/s sustained back to back on the
  * 4608 x 18432 x 3072 projection). With a single wave per SIMD nothing hides latency for free,
  * so the loop is software-pipelined by hand: fragments are double-buffered in registers, every
- * fourth MFMA is followed by one LDS read for the next half-step and (in the second half) one
- * global->LDS load for the stage after next, and there is one barrier per 64-wide K step.
- * A lone wave cannot keep its SIMD's matrix pipe busy: back-to-back independent 16x16x32 MFMAs
- * from one wave fill 64 % of the issue slots, from two waves 97 % (measured with operands in
- * registers; counters put this kernel at 71 %). The same loop therefore also exists over a
- * WGM x WGN grid of waves; with 8 waves (2 x 4, 128 x 64 each, two per SIMD) on the 256 x 256
- * tile it runs at the speed of the 4-wave form, its extra issue slots spent waiting at the
- * barrier, and is kept for comparison runs (tile id 4).
+ * third or fourth MFMA is followed by one LDS read for the next half-step and (in the second half) one
+ * global->LDS load for the stage after next, and there is one barrier per 64-wide K step. The
+ * reads come after their MFMA, not before it, so that the half-step opens with an MFMA whose
+ * operands arrived long ago: the compiler puts an lgkmcnt(0) wait in front of the first MFMA after
+ * the loop's back edge, and with a read issued just before it that wait exposed a full LDS latency
+ * per K step. Global sources are a scalar base plus a 32-bit offset per lane, so stepping along K
+ * is scalar work. Blocks are walked in serpentine order (one MFMA operand changes at a time).
+ * A workgroup goes on to further tiles (one workgroup per compute unit is launched) and requests the
+ * next tile's first stage before it stores the finished one.
+ * One wave per SIMD does keep the matrix pipe full when its MFMAs are written by hand: a register-
+ * resident loop of independent v_mfma_f32_16x16x32_bf16 reaches 2.4 PFLOP/s on zero operands and
+ * 1.86 on random bits with 256 threads per compute unit, accumulators in VGPRs or AGPRs alike (the
+ * same loop left to the compiler's builtin gets 1.46: it shuffles accumulators between the two
+ * register files). Cycle stamps in this kernel on zero operands (4608 x 18432 x 3072, clocks near
+ * their maximum) put 91 % of a wave's life in the K loop, 7 % in the epilogue and next-tile
+ * set-up, 4 % in the mid-step wait and barrier; the K loop ran at 75 % of the MFMA issue rate
+ * before the reads moved behind their MFMAs. On real operands the chip is at its power limit, in a
+ * denoising step as well as back to back: removing those stalls made the kernel 5 % faster back to
+ * back and the step 1 % faster.
+ * The same loop also exists over a WGM x WGN grid of waves; with 8 waves (2 x 4, 128 x 64 each, two
+ * per SIMD) on the 256 x 256 tile it runs at the speed of the 4-wave form and is kept for comparison
+ * runs (tile id 4).
  *
  * LDS rows are 128 bytes (64 bf16); the 16-byte chunk index is XOR-swizzled with a function of
  * the row so that the 16 rows a fragment read touches spread over all banks. A direct-to-LDS
@@ -53,6 +67,7 @@ struct GemmArgs {
     int M[GEMM_MAX_PARTS];
     int mt_end[GEMM_MAX_PARTS]; /* row tiles of parts 0..i together; unused parts repeat the total */
     int mtiles, ntiles, total_tiles;
+    int vgrid; /* workgroups' worth of tiles (a multiple of 8); a launch with fewer workgroups walks them in strides of its size */
     int N, K, lda, ldw, ldc, w_row0, w_row1;
     /* split-K: workgroup (tile, s) multiplies K-steps [s*kt_per, (s+1)*kt_per) and stores its
      * fp32 partial tile into ws[s][moff[part] + m][n]; a second kernel sums the slices */
@@ -104,10 +119,9 @@ __device__ __forceinline__ int lds_swz(int r) { return ((r >> 1) & 7) ^ ((r & 1)
 struct TileId {
     int ks, tm, tn, prob, tml;
 };
-__device__ __forceinline__ bool decode_tile(const GemmArgs &g, TileId &t) {
-    int nb = gridDim.x;
-    int per_xcd = nb >> 3;
-    int logical = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+__device__ __forceinline__ bool decode_tile(const GemmArgs &g, int vb, TileId &t) {
+    int per_xcd = g.vgrid >> 3;
+    int logical = (vb & 7) * per_xcd + (vb >> 3);
     if (logical >= g.total_tiles * g.ksplit) return false;
     t.ks = logical / g.total_tiles;
     logical -= t.ks * g.total_tiles;
@@ -242,7 +256,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     TileId t;
-    if (!decode_tile(g, t)) return;
+    if (!decode_tile(g, blockIdx.x, t)) return;
     const int ks = t.ks, tn = t.tn, prob = t.prob;
     const bf16 *__restrict__ A = g.A[prob];
     const bf16 *__restrict__ W = g.W[prob];
@@ -355,6 +369,9 @@ __device__ __forceinline__ void acc_fence(f32x4 (&acc)[TN][TM]) {
 }
 
 template <bool V> struct BoolC { static constexpr bool value = V; };
+/* whether a workgroup of gemm4w_kernel goes on to further tiles (the 4-wave form of the transformer's epilogues;
+ * with the convolution epilogues the values kept across tiles would spill) */
+template <int EPI, int WAVES> struct Walks4w { static constexpr bool value = !IsConv<EPI>::value && WAVES == 4; };
 
 template <int TM, int TN, int EPI, int WGM = 2, int WGN = 2>
 __global__ __launch_bounds__(64 * WGM * WGN) void gemm4w_kernel(GemmArgs g) {
@@ -371,48 +388,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm4w_kernel(GemmArgs g) {
     static_assert(RD >= 2 && RD * (NF - 1) + 1 < NM, "reads and loads must fit between the MFMAs");
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
-    TileId t;
-    if (!decode_tile(g, t)) return;
-    const int tn = t.tn, prob = t.prob;
-    const bf16 *__restrict__ A = g.A[prob];
-    const bf16 *__restrict__ W = g.W[prob];
-    const int M = g.M[prob];
-    const int m0 = t.tml * BM;
-
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WGN, wn = wave % WGN;
     const int lrow = tid >> 3, lchunk = tid & 7;
-
-    /* Load i of a stage by this wave covers tile rows lrow + RPP i (8 rows of 128 bytes per wave
-     * instruction): activation rows for i < LA, weight rows after. Rows RPP apart share a swizzle.
-     * The K offset of this workgroup's slice is folded into the per-lane sources. */
-    const int kt_begin = t.ks * g.kt_per;
-    const int KT = min(g.K >> 6, kt_begin + g.kt_per) - kt_begin;
-    const int chunk = ((lchunk ^ lds_swz(lrow)) << 3) + kt_begin * 64;
-    const bf16 *src[NL];
-#pragma unroll
-    for (int i = 0; i < LA; i++) src[i] = A + (size_t)min(m0 + lrow + i * RPP, M - 1) * g.lda + chunk;
-#pragma unroll
-    for (int i = 0; i < LB; i++) src[LA + i] = W + (size_t)weight_row<BN, WN, EPI>(g, tn, lrow + i * RPP) * g.ldw + chunk;
-    /* (convolutions never split K, so for them kt below is the absolute K step) */
-    auto issue1 = [&](int kt, int stage, int i) {
-        const int off = i < LA ? a_step_offset<EPI>(g, kt) : kt * 64;
-        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(src[i] + off), LDS_PTR(smem + stage * STAGE + (wave * 8 + i * RPP) * 128), 16, 0, 0);
-    };
-#pragma unroll
-    for (int i = 0; i < NL; i++) issue1(0, 0, i);
-
-    f32x4 acc[TN][TM];
-#pragma unroll
-    for (int i = 0; i < TN; i++)
-#pragma unroll
-        for (int j = 0; j < TM; j++)
-#pragma unroll
-            for (int e = 0; e < 4; e++) acc[i][j][e] = 0.0f;
-    acc_fence<TM, TN>(acc); /* the zeroes are written, and a few cycles pass, before the first MFMA reads them */
-    asm volatile("s_nop 7" ::: "memory");
-
     const int l15 = lane & 15, lq = lane >> 4;
     const int swzl = lds_swz(l15);
     const int a_frag = (wm * WM + l15) * 128;
@@ -422,58 +401,136 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm4w_kernel(GemmArgs g) {
     auto frag = [&](const char *st, int coff, int q) -> bf16x8 {
         return q < TN ? *(const bf16x8 *)(st + b_frag + q * 2048 + coff) : *(const bf16x8 *)(st + a_frag + (q - TN) * 2048 + coff);
     };
-    bf16x8 f0[NF], f1[NF];
 
-    WAIT_VMCNT0();
-    __syncthreads();
-    if (KT > 1) {
-#pragma unroll
-        for (int i = 0; i < NL; i++) issue1(1, 1, i);
-    }
-#pragma unroll
-    for (int q = 0; q < NF; q++) f0[q] = frag(smem, coff0, q);
+    /* A launch has at most one workgroup per compute unit; each walks the tiles vb, vb + gridDim.x, ...
+     * of the virtual grid, so that a tile's stores drain, and the next tile's first stage arrives,
+     * while the matrix pipes already work again (with one workgroup per tile, the end of one and the
+     * start of the next on a compute unit cost 5-14 us of a 60 us tile). */
+    int vb = blockIdx.x;
+    TileId t;
+    if (!decode_tile(g, vb, t)) return;
 
-    auto step = [&](int kt, auto more_c, auto more2_c) {
-        constexpr bool more = decltype(more_c)::value, more2 = decltype(more2_c)::value;
-        auto &accr = acc;
-        const int cur = kt & 1;
-        const char *st = smem + cur * STAGE;
-        const char *nx = smem + (cur ^ 1) * STAGE;
-        /* first K half of the stage from f0, while the second half's fragments arrive in f1 */
+    /* Load i of a stage by this wave covers tile rows lrow + RPP i (8 rows of 128 bytes per wave
+     * instruction): activation rows for i < LA, weight rows after. Rows RPP apart share a swizzle.
+     * The K offset of this workgroup's slice is folded into the per-lane sources. */
+    /* Sources are a uniform base per operand (tile's matrix + this workgroup's K slice + the K step, all scalar
+     * arithmetic) plus a 32-bit byte offset per lane and load, so that stepping along K costs no vector work. */
+    unsigned voff[NL];
+    const char *baseA, *baseW;
+    auto set_sources = [&](const TileId &tt) {
+        const int M = g.M[tt.prob], m0 = tt.tml * BM;
+        const int chunk = (lchunk ^ lds_swz(lrow)) << 3;
+        baseA = (const char *)(g.A[tt.prob] + tt.ks * g.kt_per * 64);
+        baseW = (const char *)(g.W[tt.prob] + tt.ks * g.kt_per * 64);
 #pragma unroll
-        for (int b = 0; b < NM; b++) {
-            if (b % RD == 0 && b / RD < NF) f1[b / RD] = frag(st, coff1, b / RD);
-            MFMA_AGPR(accr[b % TN][b / TN], f0[b % TN], f0[TN + b / TN]);
-        }
-        if (more) {
-            /* the next stage has landed for this wave; past the barrier it has for all, and
-             * everyone has finished reading this stage, which is refilled below */
-            WAIT_VMCNT0();
-            __syncthreads();
-        }
-        /* second half from f1, while the next stage's first fragments arrive in f0 and the stage
-         * after next is requested; at most one other instruction between two MFMAs */
+        for (int i = 0; i < LA; i++) voff[i] = ((unsigned)min(m0 + lrow + i * RPP, M - 1) * (unsigned)g.lda + chunk) * 2u;
 #pragma unroll
-        for (int b = 0; b < NM; b++) {
-            if (more && b % RD == 0 && b / RD < NF) f0[b / RD] = frag(nx, coff0, b / RD);
-            if (more2 && b % RD == 1 && b / RD < NL) issue1(kt + 2, cur, b / RD);
-            MFMA_AGPR(accr[b % TN][b / TN], f1[b % TN], f1[TN + b / TN]);
-        }
+        for (int i = 0; i < LB; i++) voff[LA + i] = ((unsigned)weight_row<BN, WN, EPI>(g, tt.tn, lrow + i * RPP) * (unsigned)g.ldw + chunk) * 2u;
     };
-    int kt = 0;
-    for (; kt < KT - 2; kt++) step(kt, BoolC<true>{}, BoolC<true>{});
-    if (kt < KT - 1) {
-        step(kt, BoolC<true>{}, BoolC<false>{});
-        kt++;
-    }
-    step(kt, BoolC<false>{}, BoolC<false>{});
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); /* the last MFMA results retire before they are read */
-    acc_fence<TM, TN>(acc);
+    /* (convolutions never split K, so for them kt below is the absolute K step) */
+    auto issue1 = [&](int kt, int stage, int i) {
+        const char *base = i < LA ? baseA + (ptrdiff_t)a_step_offset<EPI>(g, kt) * 2 : baseW + kt * 128;
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(base + voff[i]), LDS_PTR(smem + stage * STAGE + (wave * 8 + i * RPP) * 128), 16, 0, 0);
+    };
+    set_sources(t);
+#pragma unroll
+    for (int i = 0; i < NL; i++) issue1(0, 0, i);
 
-    store_tile<BN, WM, WN, EPI>(g, t, acc, m0, M, wm, wn, l15, lq, t.tm * WGM + wm);
+    for (;;) {
+        const int kt_begin = t.ks * g.kt_per;
+        const int KT = min(g.K >> 6, kt_begin + g.kt_per) - kt_begin;
+
+        f32x4 acc[TN][TM];
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+#pragma unroll
+            for (int j = 0; j < TM; j++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[i][j][e] = 0.0f;
+        acc_fence<TM, TN>(acc); /* the zeroes are written, and a few cycles pass, before the first MFMA reads them */
+        asm volatile("s_nop 7" ::: "memory");
+
+        bf16x8 f0[NF], f1[NF];
+
+        WAIT_VMCNT0();
+        __syncthreads();
+        if (KT > 1) {
+#pragma unroll
+            for (int i = 0; i < NL; i++) issue1(1, 1, i);
+        }
+#pragma unroll
+        for (int q = 0; q < NF; q++) f0[q] = frag(smem, coff0, q);
+
+        /* The blocks of a half-step are walked in serpentine order: exactly one MFMA operand changes from one
+         * instruction to the next (the matrix pipes draw less power that way than when the weight fragment
+         * wraps around together with a new activation fragment). */
+        auto serp = [](int b) { return ((b / TN) & 1) ? TN - 1 - b % TN : b % TN; };
+        auto step = [&](int kt, auto more_c, auto more2_c) {
+            constexpr bool more = decltype(more_c)::value, more2 = decltype(more2_c)::value;
+            auto &accr = acc;
+            const int cur = kt & 1;
+            const char *st = smem + cur * STAGE;
+            const char *nx = smem + (cur ^ 1) * STAGE;
+            /* first K half of the stage from f0, while the second half's fragments arrive in f1 */
+#pragma unroll
+            for (int b = 0; b < NM; b++) {
+                MFMA_AGPR(accr[serp(b)][b / TN], f0[serp(b)], f0[TN + b / TN]);
+                if (b % RD == 0 && b / RD < NF) f1[b / RD] = frag(st, coff1, b / RD);
+            }
+            if (more) {
+                /* the next stage has landed for this wave; past the barrier it has for all, and
+                 * everyone has finished reading this stage, which is refilled below */
+                WAIT_VMCNT0();
+                __syncthreads();
+            }
+            /* second half from f1, while the next stage's first fragments arrive in f0 and the stage
+             * after next is requested; at most one other instruction between two MFMAs */
+#pragma unroll
+            for (int b = 0; b < NM; b++) {
+                MFMA_AGPR(accr[serp(b)][b / TN], f1[serp(b)], f1[TN + b / TN]);
+                if (more && b % RD == 0 && b / RD < NF) f0[b / RD] = frag(nx, coff0, b / RD);
+                if (more2 && b % RD == 1 && b / RD < NL) issue1(kt + 2, cur, b / RD);
+            }
+        };
+        int kt = 0;
+        for (; kt < KT - 2; kt++) step(kt, BoolC<true>{}, BoolC<true>{});
+        if (kt < KT - 1) {
+            step(kt, BoolC<true>{}, BoolC<false>{});
+            kt++;
+        }
+        step(kt, BoolC<false>{}, BoolC<false>{});
+
+        /* The next tile's first stage is requested before this tile is stored: every wave has taken
+         * its last fragments out of LDS once it is past this barrier. */
+        const TileId done = t;
+        vb += gridDim.x;
+        const bool again = Walks4w<EPI, WGM * WGN>::value && vb < g.vgrid && decode_tile(g, vb, t);
+        if (again) {
+            __syncthreads();
+            set_sources(t);
+#pragma unroll
+            for (int i = 0; i < NL; i++) issue1(0, 0, i);
+        }
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); /* the last MFMA results retire before they are read */
+        acc_fence<TM, TN>(acc);
+
+        store_tile<BN, WM, WN, EPI>(g, done, acc, done.tml * BM, g.M[done.prob], wm, wn, l15, lq, done.tm * WGM + wm);
+        if (!again) break;
+    }
 }
 
 /* ------------------------------------------------------------------ host side */
+
+static int g_persistent = 1;
+extern "C" void flux_hip_linear_persistent(int on) { g_persistent = on; }
+static int compute_units() {
+    static int n = 0;
+    if (!n) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 8) n = 256;
+    }
+    return n;
+}
 
 static void set_row_tiles(GemmArgs &g, int BM) {
     int end = 0;
@@ -498,6 +555,7 @@ static int launch_cfg(GemmArgs &g) {
     g.ntiles = g.N / BN;
     g.total_tiles = g.mtiles * g.ntiles;
     int grid = (g.total_tiles * g.ksplit + 7) & ~7;
+    g.vgrid = grid;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(T), LDS, flux_hip_stream_handle(), g);
     HIP_OK(hipGetLastError());
     return 1;
@@ -515,7 +573,13 @@ static int launch_4w(GemmArgs &g) {
     set_row_tiles(g, BM);
     g.ntiles = g.N / BN;
     g.total_tiles = g.mtiles * g.ntiles;
-    int grid = (g.total_tiles * g.ksplit + 7) & ~7;
+    /* the kernel addresses operand rows with 32-bit byte offsets from the matrix base */
+    size_t span = ((size_t)max(g.w_row0, g.w_row1) + g.N) * g.ldw * 2;
+    for (int i = 0; i < GEMM_MAX_PARTS; i++) span = max(span, (size_t)g.M[i] * g.lda * 2);
+    if (span >= ((size_t)1 << 32)) return g.N % 128 == 0 ? launch_cfg<128, 128, 2, 2, EPI>(g) : launch_cfg<64, 64, 2, 2, EPI>(g);
+    /* one workgroup fits on a compute unit (registers, LDS): launch at most that many, each walks its share of the tiles */
+    g.vgrid = (g.total_tiles * g.ksplit + 7) & ~7;
+    const int grid = g_persistent && Walks4w<EPI, WGM * WGN>::value ? min(g.vgrid, compute_units() & ~7) : g.vgrid;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WGM * WGN), LDS, flux_hip_stream_handle(), g);
     HIP_OK(hipGetLastError());
     return 1;

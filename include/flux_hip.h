@@ -144,6 +144,8 @@ void flux_hip_linear_force_tile(int tile);
 /* bit t set = the automatic choice may use tile t (default 0xEF: all but tile 4; 0 restores it) */
 void flux_hip_linear_tile_mask(unsigned mask);
 void flux_hip_linear_enable_splitk(int on);
+/* 1 (default): the 4-wave GEMM launches at most one workgroup per compute unit and each walks several tiles; 0: one workgroup per tile */
+void flux_hip_linear_persistent(int on);
 /* 0 = 128-query workgroups, 1 = 256-query workgroups, -1 = automatic */
 void flux_hip_attention_force_variant(int v);
 int flux_hip_linear_probe(int epilogue);
