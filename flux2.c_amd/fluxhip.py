@@ -70,6 +70,7 @@ def lib():
     L.flux_hip_linear_force_tile.argtypes = [c_i]
     L.flux_hip_set_batched_cfg.argtypes = [c_i]
     L.flux_hip_linear_enable_splitk.argtypes = [c_i]
+    L.flux_hip_linear_persistent.argtypes = [c_i]
     L.flux_hip_attention_force_variant.argtypes = [c_i]
     L.flux_hip_linear_probe.argtypes = [c_i]
     L.flux_hip_linear_probe_read.argtypes = [ctypes.POINTER(c_i), ctypes.POINTER(c_f)]

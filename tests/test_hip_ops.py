@@ -112,6 +112,46 @@ def test_linear_large_tile_k_steps(hip, oracle_mod, K, tile):
     hip.lib().flux_hip_linear_force_tile(-1)
 
 
+@pytest.mark.parametrize("tile", [2, 5, 6, 7])
+def test_linear_workgroups_walk_several_tiles(hip, oracle_mod, tile):
+    """More tiles than compute units: a workgroup of the 4-wave kernel goes on to further tiles (and requests the
+    next tile's first stage before it stores the finished one). Ragged row counts, two row ranges, every epilogue
+    of the transformer; the result must also be bit for bit what one workgroup per tile gives."""
+    L = hip.lib()
+    L.flux_hip_linear_force_tile(tile)
+    K, N = 192, 6144
+    Ms = (1500, 1200)
+    xs = [q(normal_f32((M, K), 41, 1 + i)) for i, M in enumerate(Ms)]
+    W = q(normal_f32((N, K), 41, 5, 0.0, 0.1))
+    gate = normal_f32((N,), 41, 6)
+    res0 = [normal_f32((M, N), 41, 7 + i) for i, M in enumerate(Ms)]
+    dxs, dW, dg = [dev_bf16(hip, x) for x in xs], dev_bf16(hip, W), hip.DevBuf.from_array(gate)
+    outs = {}
+    for persistent in (1, 0):
+        L.flux_hip_linear_persistent(persistent)
+        # bf16 store
+        ob = [hip.DevBuf(M * N * 2) for M in Ms]
+        hip.linear(hip.EPI_BF16, [(dx.ptr, dW.ptr, o.ptr, None, M) for dx, o, M in zip(dxs, ob, Ms)], N, K, K, K, N, 0, 0)
+        # gated residual
+        orr = [hip.DevBuf.from_array(r) for r in res0]
+        hip.linear(hip.EPI_RESID, [(dx.ptr, dW.ptr, o.ptr, dg.ptr, M) for dx, o, M in zip(dxs, orr, Ms)], N, K, K, K, N, 0, 0)
+        # silu(gate) * up with the gate rows in the first half of W and the up rows in the second
+        osw = [hip.DevBuf(M * (N // 2) * 2) for M in Ms]
+        hip.linear(hip.EPI_SWIGLU, [(dx.ptr, dW.ptr, o.ptr, None, M) for dx, o, M in zip(dxs, osw, Ms)], N, K, K, K, N // 2, 0, N // 2)
+        outs[persistent] = ([o.to_array(np.uint16, (M, N)) for o, M in zip(ob, Ms)],
+                            [o.to_array(np.float32, (M, N)) for o, M in zip(orr, Ms)],
+                            [o.to_array(np.uint16, (M, N // 2)) for o, M in zip(osw, Ms)])
+    L.flux_hip_linear_persistent(1)
+    L.flux_hip_linear_force_tile(-1)
+    for i, (x, M) in enumerate(zip(xs, Ms)):
+        want = oracle_mod.linear(x, W)
+        assert rel_l2(bf16_to_f32(outs[1][0][i]), want) < 4e-3
+        assert rel_l2(outs[1][1][i], res0[i] + gate[None, :] * want) < 2e-6
+        assert rel_l2(bf16_to_f32(outs[1][2][i]), oracle_mod.silu(want[:, :N // 2]) * want[:, N // 2:]) < 4e-3
+        for k in range(3):
+            assert np.array_equal(outs[1][k][i], outs[0][k][i])
+
+
 @pytest.mark.parametrize("tile", [-1, 0, 1, 6])
 def test_linear_split_k_other_epilogues(hip, oracle_mod, tile):
     """Few rows, long K: the bf16, fp32 and SwiGLU epilogues also run as K slices plus a finishing pass
