@@ -18,6 +18,7 @@
  */
 #include "common.h"
 #include "../../include/flux_hip.h"
+#include "../../include/flux_hip_debug.h"
 
 #define HD 128
 
@@ -347,8 +348,11 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
         if (__any(grow)) {
 #pragma unroll
             for (int u = 0; u < 2; u++) {
-                const float d = (EDGE && t == 0) ? m_new[u] : fmaxf(m_new[u], 0.0f);
-                const float alpha = fast_exp2(-d);
+                /* on the first tile the accumulators are still zero and stay so: the tile's maximum may lie
+                 * far below zero, and 2^-d would then be infinite (0 * inf) */
+                const bool first = EDGE && t == 0;
+                const float d = first ? m_new[u] : fmaxf(m_new[u], 0.0f);
+                const float alpha = first ? 1.0f : fast_exp2(-d);
                 m_run[u] += d;
 #pragma unroll
                 for (int e = 0; e < 4; e++) l_acc[u][e] *= alpha;

@@ -252,6 +252,11 @@ void fh_safetensors_close_compat(void *p) {
     free(sf);
 }
 
+/* Tensors of other types (integers, fp64, fp8, booleans: the reference's numbering goes on past 2,
+ * flux_safetensors.h:20-28) are passed over, as the file walker above does; their element size is
+ * not known here, so they are not sized either. */
+static int usable_dtype(int dtype) { return dtype == DT_F32 || dtype == DT_F16 || dtype == DT_BF16; }
+
 /* Entry i of a parsed handle: where its data lies and how many elements it has. The handle comes
  * from the reference's parser; what is checked here is that reading the entry stays inside the
  * mapping it describes. */
@@ -278,6 +283,7 @@ int fh_safetensors_walk_handle(void *p, fh_tensor_cb cb, void *ctx) {
     for (int i = 0; i < sf->num_tensors; i++) {
         const char *data;
         int64_t numel;
+        if (!usable_dtype(sf->tensors[i].dtype)) continue;
         if (!handle_entry(sf, i, &data, &numel)) return 0;
         if (!cb(ctx, sf->tensors[i].name, sf->tensors[i].dtype, data, numel)) return 0;
     }
@@ -332,6 +338,7 @@ static flux_transformer_t *load_from_handle(void *p) {
         const ref_safetensor *t = &sf->tensors[i];
         const char *data;
         int64_t numel;
+        if (!usable_dtype(t->dtype)) continue;
         if (!handle_entry(sf, i, &data, &numel)) { flux_transformer_free(tf); return NULL; }
         if (!set_from(tf, t->name, t->dtype, data, numel)) {
             /* files may carry tensors this path does not use; only real failures abort */

@@ -10,6 +10,7 @@
  * The host thread only queues work; step callbacks therefore fire at queue time.
  */
 #include "../../include/flux_hip.h"
+#include "../../include/flux_hip_debug.h"
 #include "host_internal.h"
 #include <hip/hip_runtime_api.h>
 #include <math.h>
@@ -235,11 +236,11 @@ void flux_hip_session_free(flux_hip_session *s) {
     free(s);
 }
 
-flux_hip_session *flux_hip_session_begin(void *transformer, const float *z, int channels, int h, int w,
-                                         const flux_ref_t *refs, int num_refs,
-                                         const float *text_emb_cond, int text_seq_cond,
-                                         const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
-                                         const float *schedule, int num_steps) {
+static flux_hip_session *session_begin_impl(void *transformer, const float *z, int channels, int h, int w,
+                                            const flux_ref_t *refs, int num_refs,
+                                            const float *text_emb_cond, int text_seq_cond,
+                                            const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
+                                            const float *schedule, int num_steps, int reset_timing) {
     flux_transformer_t *tf = (flux_transformer_t *)transformer;
     if (!tf || !z || !text_emb_cond || !schedule) { flux_hip_fail("sampler: NULL argument"); return NULL; }
     if (!fh_model_complete(tf)) return NULL;
@@ -284,11 +285,20 @@ flux_hip_session *flux_hip_session_begin(void *transformer, const float *z, int 
     if (!flux_hip_upload(s->z_dev, z, s->n_lat * 4)) goto fail;
     if (!upload_ref_tokens(tf, s->n_target, refs, num_refs)) goto fail;
     s->ev = events_begin(num_steps * (cfg ? 2 : 1));
-    flux_reset_timing();
+    if (reset_timing) flux_reset_timing();
     return s;
 fail:
     flux_hip_session_free(s);
     return NULL;
+}
+
+flux_hip_session *flux_hip_session_begin(void *transformer, const float *z, int channels, int h, int w,
+                                         const flux_ref_t *refs, int num_refs,
+                                         const float *text_emb_cond, int text_seq_cond,
+                                         const float *text_emb_uncond, int text_seq_uncond, float guidance_scale,
+                                         const float *schedule, int num_steps) {
+    return session_begin_impl(transformer, z, channels, h, w, refs, num_refs, text_emb_cond, text_seq_cond, text_emb_uncond,
+                              text_seq_uncond, guidance_scale, schedule, num_steps, 1);
 }
 
 int flux_hip_session_step(flux_hip_session *s, int step, float *v_trace) {
@@ -592,22 +602,34 @@ float *flux_generate_latent(void *ctx_ptr, const float *text_emb, int text_seq, 
 void (*flux_progress_callback)(int, int) = NULL;
 void flux_set_progress_callback(void (*callback)(int, int)) { flux_progress_callback = callback; }
 
-/* One forward = a one-step schedule whose velocity is returned instead of applied
- * (flux_transformer.c:3115, 3605, 3815; used by flux_denoise_step, flux.c:1109). */
+/* One forward (flux_transformer.c:3115, 3605, 3815; used by flux_denoise_step, flux.c:1109): the
+ * device state of a one-step run is set up, the forward is queued and its velocity read back. As in
+ * the reference, a forward fires no step callback, moves no latent and adds its stage times to the
+ * flux_timing_transformer_* counters instead of starting them afresh (flux_transformer.c:3561-3564);
+ * the block-level flux_substep_callback fires as it does there. */
 float *flux_transformer_forward_with_multi_refs(flux_transformer_t *tf, const float *img_latent, int img_h, int img_w,
                                                 const flux_ref_t *refs, int num_refs,
                                                 const float *txt_emb, int txt_seq, float timestep) {
     if (!tf || !img_latent || !txt_emb) { flux_hip_fail("forward: NULL argument"); return NULL; }
     if (img_h <= 0 || img_w <= 0 || txt_seq <= 0) { flux_hip_fail("forward: bad sizes"); return NULL; }
     const size_t n = (size_t)tf->c.channels * img_h * img_w;
-    float sched[2] = {timestep, timestep};
+    const float sched[2] = {timestep, timestep};
+    flux_hip_session *s = session_begin_impl(tf, img_latent, tf->c.channels, img_h, img_w, refs, refs ? num_refs : 0, txt_emb,
+                                             txt_seq, NULL, 0, 0.0f, sched, 1, 0);
+    if (!s) return NULL;
     float *v = (float *)malloc(n * 4);
-    if (!v) { flux_hip_fail("out of host memory"); return NULL; }
-    float *z = flux_hip_sample_traced(tf, img_latent, tf->c.channels, img_h, img_w, refs, refs ? num_refs : 0,
-                                      txt_emb, txt_seq, NULL, 0, 0.0f, sched, 1, v);
-    if (!z) { free(v); return NULL; }
-    free(z);
-    return v;
+    if (!v) flux_hip_fail("out of host memory");
+    if (v && fh_forward_device(tf, s->rp_c, s->z_dev, s->n_target, s->txt_c, 0, s->v_c, s->ev)) {
+        if (s->ev) s->ev->used++;
+        if (flux_hip_download(v, s->v_c, n * 4)) {
+            events_collect(s->ev);
+            flux_hip_session_free(s);
+            return v;
+        }
+    }
+    free(v);
+    flux_hip_session_free(s);
+    return NULL;
 }
 
 float *flux_transformer_forward(flux_transformer_t *tf, const float *img_latent, int img_h, int img_w,

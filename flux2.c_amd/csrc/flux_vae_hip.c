@@ -20,6 +20,7 @@
  * attention as two GEMMs around a row softmax; everything else is in vae.hip.
  */
 #include "../../include/flux_hip.h"
+#include "../../include/flux_hip_debug.h"
 #include "host_internal.h"
 #include <hip/hip_runtime_api.h>
 #include <math.h>

@@ -57,6 +57,7 @@
  */
 #include "common.h"
 #include "../../include/flux_hip.h"
+#include "../../include/flux_hip_debug.h"
 
 #define GEMM_MAX_PARTS 4
 struct GemmArgs {

@@ -16,6 +16,10 @@
  * message. Nothing here falls back to a CPU path: without a usable GPU every
  * call fails. Not thread-safe (neither is the reference: see the globals at
  * flux_kernels.c:32-45): one forward at a time per process.
+ *
+ * Switches that pin a tile, a kernel variant or a code path for tests and measurements, and the
+ * launch probe the benchmark reads, are process-wide state and no part of this interface: they are
+ * declared in flux_hip_debug.h.
  */
 #ifndef FLUX_HIP_H
 #define FLUX_HIP_H
@@ -134,27 +138,6 @@ int flux_hip_conv(int epilogue, const void *in, const void *w, const float *bias
  * the image (flux_hip_group_norm_stats). */
 int flux_hip_conv_stats(int epilogue, const void *in, const void *w, const float *bias, const float *res, void *out, int rows,
                         int wp, int cin, int cout, int taps, float *stats, int *stats_rows);
-
-/* Measurement hooks. force_tile: 0/1/2/3/5/6/7 pins the GEMM tile (64x128, 128x128, 256x256, 64x64,
- * 288x192, 192x192, 256x192; 4 = 256x256 in its 8-wave form, never chosen automatically), -1 restores the automatic
- * choice (a tile whose width does not divide N is skipped; if none is left the 128x128 tile runs); enable_splitk(0) turns the split-K path off. probe(epilogue) records HIP events around every later
- * flux_hip_linear launch with that epilogue (-1 stops); probe_read waits for them and returns
- * their count and summed duration. */
-void flux_hip_linear_force_tile(int tile);
-/* bit t set = the automatic choice may use tile t (default 0xEF: all but tile 4; 0 restores it) */
-void flux_hip_linear_tile_mask(unsigned mask);
-void flux_hip_linear_enable_splitk(int on);
-/* 1 (default): the 4-wave GEMM launches at most one workgroup per compute unit and each walks several tiles; 0: one workgroup per tile */
-void flux_hip_linear_persistent(int on);
-/* 0 = 128-query workgroups, 1 = 256-query workgroups, -1 = automatic */
-void flux_hip_attention_force_variant(int v);
-int flux_hip_linear_probe(int epilogue);
-int flux_hip_linear_probe_read(int *launches, float *total_ms);
-/* the same for the recorded launches that used one tile id (see force_tile) */
-int flux_hip_linear_probe_read_tile(int tile, int *launches, float *total_ms);
-/* probe(-2) records every flux_hip_conv launch. read_launches copies out, in launch order, the
- * tile id and duration (ms) of up to `max` recorded launches and returns their number (-1 on error). */
-int flux_hip_linear_probe_read_launches(int max, int *tiles, float *ms);
 
 /*
  * out = (1 + scale) * LayerNorm(x) + shift per row, x f32 [rows, hidden], out bf16.
@@ -384,8 +367,6 @@ int flux_hip_vae_encode(flux_hip_vae *v, const float *img, int H, int W, float *
 int flux_hip_vae_image_in(void *out_bf16, const float *img, int H, int W);
 int flux_hip_downsample_gather(void *out_bf16, const float *x, int hp, int wp, int C);
 int flux_hip_vae_latent_out(float *latent, const float *x, int ldx, const float *bn_mean, const float *bn_var, int h, int w, float eps);
-/* Test hook: at most `rows` query rows per attention chunk (0 = default: 1 GB of fp32 scores per chunk). */
-void flux_hip_vae_set_attention_chunk(int rows);
 /* When set, called after each of the decoder's 15 / the encoder's 11 blocks has been queued (role of
  * flux_vae_progress_callback, flux_kernels.h:292-293). */
 extern void (*flux_hip_vae_progress)(int block, int total);
@@ -466,10 +447,8 @@ float *qwen3_encode_text(void *enc, const char *prompt);
  * waits and copies the current latent out. The samplers above are built from these.
  */
 /* A CFG step's unconditional and conditional forwards run as one batch of two sequences (each weight
- * matrix streamed once, twice the rows per GEMM); 0 switches back to two separate forwards, the
- * reference's order (flux_sample.c:485-493). Takes effect at the next session_begin. */
-void flux_hip_set_batched_cfg(int on);
-
+ * matrix streamed once, twice the rows per GEMM); flux_hip_set_batched_cfg(0) in flux_hip_debug.h
+ * switches back to two separate forwards, the reference's order (flux_sample.c:485-493). */
 typedef struct flux_hip_session flux_hip_session;
 flux_hip_session *flux_hip_session_begin(void *transformer, const float *z, int channels, int h, int w,
                                          const flux_ref_t *refs, int num_refs,

@@ -1,0 +1,51 @@
+/*
+ * flux_hip_debug.h - test and measurement switches of libflux_hip.so.
+ *
+ * None of these has a counterpart in the reference and none is needed to use the library; an
+ * application includes flux_hip.h only. They are process-wide mutable state (like the reference's
+ * own globals, flux_kernels.c:32-45): set one, run, and restore the default. tests/conftest.py
+ * restores all of them before every test module.
+ */
+#ifndef FLUX_HIP_DEBUG_H
+#define FLUX_HIP_DEBUG_H
+
+#include "flux_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* force_tile: 0/1/2/3/5/6/7 pins the GEMM tile of flux_hip_linear (64x128, 128x128, 256x256, 64x64,
+ * 288x192, 192x192, 256x192; 4 = 256x256 in its 8-wave form, never chosen automatically), -1 restores
+ * the automatic choice (a tile whose width does not divide N is skipped; if none is left the 128x128
+ * tile runs). */
+void flux_hip_linear_force_tile(int tile);
+/* bit t set = the automatic choice may use tile t (default 0xEF: all but tile 4; 0 restores it) */
+void flux_hip_linear_tile_mask(unsigned mask);
+/* 0 turns the split-K path off (default 1) */
+void flux_hip_linear_enable_splitk(int on);
+/* 1 (default): the 4-wave GEMM launches at most one workgroup per compute unit and each walks several
+ * tiles; 0: one workgroup per tile */
+void flux_hip_linear_persistent(int on);
+/* 0 = 128-query workgroups, 1 = 256-query workgroups, -1 = automatic (default) */
+void flux_hip_attention_force_variant(int v);
+/* 1 (default): a CFG step runs its two forwards as one batch of two sequences; 0: one after the other.
+ * Takes effect at the next flux_hip_session_begin. */
+void flux_hip_set_batched_cfg(int on);
+/* VAE attention: at most `rows` query rows per chunk (0 = default: 1 GB of fp32 scores per chunk). */
+void flux_hip_vae_set_attention_chunk(int rows);
+
+/* Launch probe: probe(epilogue) records HIP events around every later flux_hip_linear launch with
+ * that epilogue (-2: every flux_hip_conv launch; -1 stops); probe_read waits for them and returns
+ * their count and summed duration, probe_read_tile the same for the launches that used one tile id,
+ * probe_read_launches copies out, in launch order, the tile id and duration (ms) of up to `max`
+ * recorded launches and returns their number (-1 on error). */
+int flux_hip_linear_probe(int epilogue);
+int flux_hip_linear_probe_read(int *launches, float *total_ms);
+int flux_hip_linear_probe_read_tile(int tile, int *launches, float *total_ms);
+int flux_hip_linear_probe_read_launches(int max, int *tiles, float *ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLUX_HIP_DEBUG_H */

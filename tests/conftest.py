@@ -24,3 +24,29 @@ def oracle_mod():
 @pytest.fixture(scope="session")
 def golden_dir():
     return os.path.join(ROOT, "tests", "golden")
+
+
+@pytest.fixture(autouse=True, scope="module")
+def _default_switches(request):
+    """The switches of include/flux_hip_debug.h are process-wide: every GPU test module starts from the
+    defaults, whatever an earlier module (or a failed assertion in it) left behind."""
+    mark = getattr(request.module, "pytestmark", None)
+    marks = list(mark) if isinstance(mark, (list, tuple)) else [mark] if mark is not None else []
+    if not any(getattr(m, "name", "") == "gpu" for m in marks):
+        yield
+        return
+    import fluxhip
+    L = fluxhip.lib()
+
+    def restore():
+        L.flux_hip_linear_force_tile(-1)
+        L.flux_hip_linear_tile_mask(0)
+        L.flux_hip_linear_enable_splitk(1)
+        L.flux_hip_linear_persistent(1)
+        L.flux_hip_attention_force_variant(-1)
+        L.flux_hip_set_batched_cfg(1)
+        L.flux_hip_vae_set_attention_chunk(0)
+        L.flux_hip_linear_probe(-1)
+    restore()
+    yield
+    restore()

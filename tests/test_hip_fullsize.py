@@ -3,17 +3,22 @@ N(0, 0.02) seed 42, against the fp32 CPU oracle on the same inputs.
 
 c2: 256 image + 512 text tokens, full 4-step distilled schedule (velocities + final latent)
 c3: 1024 + 512 tokens, first step of the 4-step schedule
-c4: 4096 + 512 tokens (headline shape), first step
+c4: 4096 + 512 tokens (headline shape), full 4-step schedule
 c5: CFG + one reference image, (1024 + 1024) + 512 tokens, first step = two forwards
-The oracle needs seconds to a minute per forward at these sizes, so c3-c5 check one step; the
-remaining steps run the same kernels at the same shapes with other modulation vectors.
 Gates: velocity rel-L2 <= 2e-2, cosine >= 0.999, latent PSNR >= 35 dB.
+
+Two weight sets. "literal": every tensor N(0, 0.02), the QK-norm weights included; attention logits
+are then of order 1e-4, the softmax is uniform and an error in RoPE, QK-norm or softmax cannot move
+the velocity beyond the gate. "sharp": the same tensors with the QK-norm weights at 1.0 (logits of
+order one); c3, c4 and c5 run their first step with it as well, and a control shows that an oracle
+whose image RoPE axes are swapped fails the gate there (flux_transformer.c:719-741, 1052-1106,
+1335-1460 are what these cases can see and the literal ones cannot).
 """
 import numpy as np
 import pytest
 
 from metrics import rel_l2, cosine, psnr
-from model_spec import KLEIN_4B, tensor_shapes, make_weights, normal_f32
+from model_spec import KLEIN_4B, tensor_shapes, make_weights, normal_f32, is_qk_norm
 
 pytestmark = pytest.mark.gpu
 
@@ -34,6 +39,23 @@ def models(oracle_mod):
     yield fluxhip, hip_m, ora
     hip_m.close()
     ora.close()
+
+
+def set_qk_norm(models, oracle_mod, mode):
+    """Replaces the QK-norm weights of both models: "literal" = N(0, 0.02), "sharp" = 1.0."""
+    _, hip_m, ora = models
+    for name in tensor_shapes(KLEIN_4B):
+        if is_qk_norm(name):
+            a = make_weights(KLEIN_4B, 42, 0.02, mode, only=[name])[name]
+            hip_m.set_tensor(name, a)
+            assert oracle_mod.lib().fo_model_set_bf16(ora.h, name.encode(), a.ctypes.data, a.size) == 0
+
+
+@pytest.fixture
+def sharp(models, oracle_mod):
+    set_qk_norm(models, oracle_mod, "sharp")
+    yield
+    set_qk_norm(models, oracle_mod, "literal")
 
 
 def check(vg, vo, what):
@@ -57,8 +79,7 @@ def test_c2_full_schedule(models):
     assert p >= 35.0
 
 
-@pytest.mark.parametrize("name,h,w", [("c3", 32, 32), ("c4", 64, 64)])
-def test_first_step(models, name, h, w):
+def first_step(models, name, h, w):
     fluxhip, m, o = models
     z = normal_f32((128, h, w), 123, 1)
     txt = normal_f32((512, 7680), 123, 2)
@@ -67,9 +88,50 @@ def test_first_step(models, name, h, w):
     zg, vg = m.sample(z, h, w, txt, s, trace=True)
     check(vg[0], vo[0], f"{name} step 0")
     assert psnr(zg, zo) >= 35.0
+    return z, txt, s, vg[0], vo[0]
 
 
-def test_c5_cfg_with_reference_first_step(models):
+def test_c3_first_step(models):
+    first_step(models, "c3", 32, 32)
+
+
+def test_c4_full_schedule(models):
+    """The headline shape through all four steps of its schedule: every step's velocity and the final latent."""
+    fluxhip, m, o = models
+    h = w = 64
+    z = normal_f32((128, h, w), 123, 1)
+    txt = normal_f32((512, 7680), 123, 2)
+    s = fluxhip.schedule("official", 4, h * w)
+    zo, vo = o.sample_euler(z, h, w, txt, s, trace=True)
+    zg, vg = m.sample(z, h, w, txt, s, trace=True)
+    for i in range(4):
+        check(vg[i], vo[i], f"c4 step {i}")
+    p = psnr(zg, zo)
+    print(f"c4 final latent PSNR {p:.1f} dB", flush=True)
+    assert p >= 35.0
+
+
+def test_c3_sharp_first_step_and_rope_control(models, sharp):
+    """QK-norm weights of 1.0: RoPE, QK-norm and softmax decide the output (24 heads x 1536 tokens). Against an oracle
+    whose image rows and columns are swapped the same velocity must FAIL the gate; if it passed, this fixture
+    would say nothing about the attention side either."""
+    fluxhip, m, o = models
+    z, txt, s, vg, vo = first_step(models, "c3 sharp", 32, 32)
+    h = w = 32
+    zt = z.reshape(128, h, w).transpose(0, 2, 1).copy()
+    _, vw = o.sample_euler(zt, h, w, txt, s, trace=True)
+    wrong = vw[0].reshape(128, h, w).transpose(0, 2, 1).ravel()
+    r = rel_l2(vg, wrong)
+    print(f"c3 sharp against the mirrored oracle: rel_l2={r:.3e}", flush=True)
+    assert r > 3 * 2e-2, r
+
+
+def test_c4_sharp_first_step(models, sharp):
+    """24 heads x 4608 tokens with logits of order one: the 256-query workgroups and the head order over the XCDs."""
+    first_step(models, "c4 sharp", 64, 64)
+
+
+def c5_first_step(models, what):
     fluxhip, m, o = models
     h = w = 32
     z = normal_f32((128, h, w), 123, 1)
@@ -79,9 +141,18 @@ def test_c5_cfg_with_reference_first_step(models):
     s = fluxhip.schedule("official", 50, h * w)[:2]
     zo, vo = o.sample_euler_cfg(z, h, w, txt, txt_u, 4.0, s, refs=[ref], trace=True)
     zg, vg = m.sample(z, h, w, txt, s, refs=[ref], txt_uncond=txt_u, guidance=4.0, trace=True)
-    check(vg[0], vo[0], "c5 uncond")
-    check(vg[1], vo[1], "c5 cond")
+    check(vg[0], vo[0], f"{what} uncond")
+    check(vg[1], vo[1], f"{what} cond")
     assert psnr(zg, zo) >= 35.0
+
+
+def test_c5_cfg_with_reference_first_step(models):
+    c5_first_step(models, "c5")
+
+
+def test_c5_sharp_cfg_with_reference_first_step(models, sharp):
+    """Batched CFG (two sequences, per-sequence K / V^T offsets) and the reference image's T offset with sharp logits."""
+    c5_first_step(models, "c5 sharp")
 
 
 def test_maximum_size_properties(models):

@@ -223,12 +223,35 @@ def test_malformed_weight_files_are_refused(hip, tmp_path):
     extra = altered(lambda h: (h.update({"step_count": {"dtype": "I64", "shape": [1], "data_offsets": [len(data), len(data) + 8]}}),
                                h.update({"ema.decay": {"dtype": "BF16", "shape": [4], "data_offsets": [len(data) + 8, len(data) + 16]}}),
                                h.update({"__metadata__": {"format": "pt"}})))
-    a = hip.Transformer(cfg, path=write("l.safetensors", extra, data + bytes(16)))
+    extra_path = write("l.safetensors", extra, data + bytes(16))
+    a = hip.Transformer(cfg, path=extra_path)
     b = hip.Transformer(cfg, path=str(good))
     lat = normal_f32((cfg.channels, 4, 4), 14, 1)
     txt = normal_f32((16, cfg.text_dim), 14, 2)
-    assert np.array_equal(a.forward(lat, 4, 4, txt, 0.5), b.forward(lat, 4, 4, txt, 0.5))
+    want = b.forward(lat, 4, 4, txt, 0.5)
+    assert np.array_equal(a.forward(lat, 4, 4, txt, 0.5), want)
     a.close(); b.close()
+    # the same file through the handle the reference's own parser makes of it (its dtype numbering goes on past
+    # BF16: I32 = 3, I64 = 4, BOOL = 5, flux_safetensors.h:20-28): the I64 entry is passed over there too
+    import ctypes
+    ref_so = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "oracle", "_ref", "libfluxref.so")
+    if os.path.exists(ref_so):
+        R = ctypes.CDLL(os.path.realpath(ref_so))
+        R.safetensors_open.restype = ctypes.c_void_p
+        R.safetensors_open.argtypes = [ctypes.c_char_p]
+        sf = R.safetensors_open(extra_path.encode())
+        assert sf
+        L = hip.lib()
+        L.flux_transformer_load_safetensors_mmap.restype = ctypes.c_void_p
+        L.flux_transformer_load_safetensors_mmap.argtypes = [ctypes.c_void_p]
+        tf = L.flux_transformer_load_safetensors_mmap(sf)
+        assert tf, L.flux_hip_last_error()
+        p = L.flux_transformer_forward(tf, lat.ctypes.data, 4, 4, txt.ctypes.data, 16, ctypes.c_float(0.5))
+        assert p, L.flux_hip_last_error()
+        got = np.ctypeslib.as_array(ctypes.cast(p, ctypes.POINTER(ctypes.c_float)), shape=(cfg.channels * 16,)).copy()
+        hip.libc_free(p)
+        L.flux_transformer_free(tf)            # closes the handle it took over
+        assert np.array_equal(got.reshape(want.shape), want)
 
 
 def test_error_paths(hip):
@@ -363,6 +386,15 @@ def test_callbacks_fire_in_order(hip):
                                 sched.ctypes.data, 2, prog_cb)
         assert p
         hip.libc_free(p)
+        # a single forward (flux_transformer.c:3115) fires the block callbacks only and ADDS to the stage timers
+        sampler_log, log[:] = list(log), []
+        total = ctypes.c_double.in_dll(L, "flux_timing_transformer_total")
+        t0 = total.value
+        m.forward(z, 2, 2, txt, 0.5)
+        t1 = total.value
+        m.forward(z, 2, 2, txt, 0.5)
+        assert t0 > 0 and t1 > t0 and total.value > t1
+        forward_log, log[:] = list(log), sampler_log
     finally:
         ctypes.c_void_p.in_dll(L, "flux_step_callback").value = None
         ctypes.c_void_p.in_dll(L, "flux_substep_callback").value = None
@@ -372,4 +404,5 @@ def test_callbacks_fire_in_order(hip):
     for s in (1, 2):
         want += [("step", s, 2)] + per_step + [("progress", s, 2)]
     assert log == want
+    assert forward_log == per_step + per_step
     m.close()
