@@ -789,6 +789,36 @@ static int launch_split_adaln(GemmArgs &g, int tile, const AdalnArgs &a) {
     return hipGetLastError() == hipSuccess ? 1 : flux_hip_fail("split-K reduction + AdaLN launch failed");
 }
 
+/* Workspace of flux_hip_linear_static: the K slices' partial sums live in this array instead of in
+ * memory from hipMalloc. Each GPU that loads the library holds its own copy until the process ends.
+ * In host code the array's name is only a handle for hipGetSymbolAddress; the address a kernel can
+ * use is asked for once per device (static_ws_for_current_device) and kept. */
+#define STATIC_WS_BYTES ((size_t)FLUX_HIP_LINEAR_STATIC_BYTES)
+static __device__ __align__(256) float g_static_ws[STATIC_WS_BYTES / sizeof(float)];
+#define STATIC_WS_MAX_DEVICES 64
+static float *g_static_ws_ptr[STATIC_WS_MAX_DEVICES];
+
+static float *static_ws_for_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= STATIC_WS_MAX_DEVICES) {
+        flux_hip_fail("flux_hip_linear_static: no current device (or a device number beyond %d)", STATIC_WS_MAX_DEVICES - 1);
+        return nullptr;
+    }
+    if (!g_static_ws_ptr[dev]) {
+        float *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(g_static_ws));
+        if (e != hipSuccess || !p) {
+            flux_hip_fail("flux_hip_linear_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+            return nullptr;
+        }
+        g_static_ws_ptr[dev] = p;
+    }
+    return g_static_ws_ptr[dev];
+}
+
+/* called by flux_hip_init with its device current */
+extern "C" int flux_hip_linear_static_init(void) { return static_ws_for_current_device() != nullptr; }
+
 extern "C" void flux_hip_linear_release(void);
 static float *g_ws = nullptr;
 static size_t g_ws_bytes = 0;
@@ -877,7 +907,7 @@ static int probe_slot(int epilogue) {
 
 /* Tile and K-split choice, then the launch; `allowed` has bit t set for every tile id that may be used. */
 static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, int *tile_out = nullptr, const AdalnArgs *adaln = nullptr,
-                         int *adaln_done = nullptr) {
+                         int *adaln_done = nullptr, float *fixed_ws = nullptr, size_t fixed_ws_bytes = 0) {
     /* Choose tile and K split with a small cost model: workgroups run in rounds over
      * 256 CUs x occupancy; a workgroup's time is its FLOPs at the tile's measured rate plus a
      * fixed prologue/epilogue cost; the launch cannot beat the time to stream its operands,
@@ -909,6 +939,7 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
             for (int si = 0; si < 10; si++) {
                 const int sp = splits[si];
                 if (sp > 1 && (!can_split || kt_total / sp < 4)) break;
+                if (sp > 1 && fixed_ws && (double)sp * rows * N * sizeof(float) > (double)fixed_ws_bytes) break; /* the slices must fit the given workspace */
                 const int per = (kt_total + sp - 1) / sp;
                 const long blocks = tiles * ((kt_total + per - 1) / per);
                 const long slots = 256L * occ[t];
@@ -937,8 +968,12 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
             g.moff[i] = g.ws_rows;
             g.ws_rows += g.M[i];
         }
-        if (!ensure_ws((size_t)g.ksplit * g.ws_rows * g.N * sizeof(float))) return 0;
-        g.ws = g_ws;
+        if (fixed_ws) {
+            g.ws = fixed_ws;
+        } else {
+            if (!ensure_ws((size_t)g.ksplit * g.ws_rows * g.N * sizeof(float))) return 0;
+            g.ws = g_ws;
+        }
     }
 
     if (tile_out) *tile_out = tile;
@@ -969,7 +1004,7 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
 }
 
 static int linear_impl(int epilogue, int nparts, const flux_hip_linear_part *parts, int N, int K, int lda, int ldw, int ldc, int w_row0,
-                       int w_row1, const flux_hip_adaln_part *norm, float eps, int *fused) {
+                       int w_row1, const flux_hip_adaln_part *norm, float eps, int *fused, float *fixed_ws = nullptr, size_t fixed_ws_bytes = 0) {
     if (epilogue < FLUX_HIP_EPI_BF16 || epilogue > FLUX_HIP_EPI_SWIGLU) return flux_hip_fail("flux_hip_linear: unknown epilogue %d", epilogue);
     if (nparts < 1 || nparts > GEMM_MAX_PARTS) return flux_hip_fail("flux_hip_linear: nparts=%d (1 to %d)", nparts, GEMM_MAX_PARTS);
     if (K <= 0 || (K & 63)) return flux_hip_fail("flux_hip_linear: K=%d must be a positive multiple of 64", K);
@@ -1011,12 +1046,32 @@ static int linear_impl(int epilogue, int nparts, const flux_hip_linear_part *par
     g.N = N; g.K = K; g.lda = lda; g.ldw = ldw; g.ldc = ldc; g.w_row0 = w_row0; g.w_row1 = w_row1;
     a.ldo = N;
     a.eps = eps;
-    return gemm_dispatch(g, np, epilogue, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0xFFu, nullptr, norm ? &a : nullptr, fused);
+    return gemm_dispatch(g, np, epilogue, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0xFFu, nullptr, norm ? &a : nullptr, fused,
+                         fixed_ws, fixed_ws_bytes);
 }
 
 extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
                                int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1) {
     return linear_impl(epilogue, nparts, parts, N, K, lda, ldw, ldc, w_row0, w_row1, nullptr, 0.0f, nullptr);
+}
+
+/* flux_hip_linear for callers that must not allocate: the partial sums of the K slices go to the
+ * static device array above. Nothing here or below it calls hipMalloc, hipFree or an allocating
+ * library routine. Every partial sum the second pass reads has been written by the first pass of the
+ * same call, so the array needs no clearing between calls; calls that overlap on one GPU (two
+ * streams, two host threads) would share it and race. */
+extern "C" int flux_hip_linear_static(int epilogue, int nparts, const flux_hip_linear_part *parts,
+                                      int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1) {
+    if (nparts < 1 || nparts > GEMM_MAX_PARTS) return flux_hip_fail("flux_hip_linear_static: nparts=%d (1 to %d)", nparts, GEMM_MAX_PARTS);
+    long long rows = 0;
+    for (int i = 0; i < nparts; i++) rows += parts[i].M > 0 ? parts[i].M : 0;
+    if (N > 0 && rows * (long long)N > (long long)FLUX_HIP_LINEAR_STATIC_MAX_OUTPUTS)
+        return flux_hip_fail("flux_hip_linear_static: %lld rows x %d columns = %lld outputs, beyond the maximum of %lld "
+                             "(two K slices of fp32 partial sums must fit the %zu MiB static workspace)",
+                             rows, N, rows * (long long)N, (long long)FLUX_HIP_LINEAR_STATIC_MAX_OUTPUTS, STATIC_WS_BYTES >> 20);
+    float *ws = static_ws_for_current_device();
+    if (!ws) return 0;
+    return linear_impl(epilogue, nparts, parts, N, K, lda, ldw, ldc, w_row0, w_row1, nullptr, 0.0f, nullptr, ws, STATIC_WS_BYTES);
 }
 
 /* The residual projection, and - when it runs as K slices - the AdaLN of the updated rows in its

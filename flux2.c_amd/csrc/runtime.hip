@@ -34,6 +34,8 @@ extern "C" const char *flux_hip_last_error(void) { return g_err; }
 extern "C" hipStream_t flux_hip_stream_handle(void) { return g_stream; }
 extern "C" void *flux_hip_stream(void) { return (void *)g_stream; }
 
+extern "C" int flux_hip_linear_static_init(void);
+
 extern "C" int flux_hip_init(void) {
     if (g_ready) return 1;
     int n = 0;
@@ -51,6 +53,7 @@ extern "C" int flux_hip_init(void) {
         HIP_OK(hipEventCreateWithFlags(&g_part_ready[i], hipEventDisableTiming));
         HIP_OK(hipEventCreateWithFlags(&g_part_done[i], hipEventDisableTiming));
     }
+    if (!flux_hip_linear_static_init()) return 0; /* device address of the static workspace, with device 0 current */
     g_ready = 1;
     return 1;
 }

@@ -96,6 +96,24 @@ int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
                     int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1);
 
 /*
+ * flux_hip_linear that allocates nothing. No counterpart in the reference: it is for callers that
+ * cannot call hipMalloc - code under HIP graph capture, tight serving loops, harnesses that forbid
+ * allocation. flux_hip_linear takes a workspace from hipMalloc (kept and grown on demand) when it
+ * runs a projection with few rows and a long K as K slices; this entry point keeps the slices'
+ * fp32 partial sums in a static device array of FLUX_HIP_LINEAR_STATIC_BYTES instead, which every GPU
+ * the library runs on holds until the process ends, and considers only as many slices as fit there.
+ * Same arguments, epilogues and results (to fp32 summation order when the number of slices differs)
+ * as flux_hip_linear. Fails, before anything is launched, when the row counts of all parts together
+ * times N exceed FLUX_HIP_LINEAR_STATIC_MAX_OUTPUTS (two slices must fit). All calls on one GPU share
+ * the array: calls that overlap there (two streams, two host threads) race. The array's contents need
+ * no clearing between calls.
+ */
+#define FLUX_HIP_LINEAR_STATIC_BYTES (64u << 20)
+#define FLUX_HIP_LINEAR_STATIC_MAX_OUTPUTS (FLUX_HIP_LINEAR_STATIC_BYTES / 8u) /* rows * N */
+int flux_hip_linear_static(int epilogue, int nparts, const flux_hip_linear_part *parts,
+                           int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1);
+
+/*
  * flux_hip_linear with FLUX_HIP_EPI_RESID, with the AdaLN that follows every residual projection
  * (apply_adaln, flux_transformer.c:979-1048, called at :1845, :1919, :3030) folded into it when the
  * projection runs as K slices (few rows, long K): the pass that sums the slices and updates x then
