@@ -12,13 +12,14 @@ Also measured in the same run:
   roofline      the dominant kernel (gate/up projection GEMM with the SiLU*up epilogue) launched
                 alone at the workload's shape and timed with HIP events on the backend's stream
   cpu_baseline  the CPU oracle (fp32, BLAS when available) on a bounded sample of the same
-                workload: one double-stream and two single-stream blocks at full shape,
-                extrapolated to the 5 + 20 blocks of a step
+                workload: one whole forward at full shape after a small warm-up forward
 
 --workload vae_c2 | vae_c3 | vae_c4 measures the step after the sampling loop instead: one "step" is
 one VAE decode of a 16/32/64-wide latent to a 256/512/1024-pixel image; vae_enc_c2 | vae_enc_c3 |
 vae_enc_c4 the VAE encoder on a picture of those sizes (the input of image-to-image generation).
 --workload qwen3 measures the step before the loop: one forward of the text encoder over 512 tokens.
+--workload mfma_peak measures no part of the model: what the matrix pipes sustain on their own (the measured
+peak beside the datasheet's 2.5 PFLOP/s).
 """
 import argparse
 import json
@@ -79,39 +80,38 @@ def time_dominant_kernel(cfg, tokens, launches=20):
     return ms, flops
 
 
-def cpu_baseline(cfg, n_img, n_txt):
-    """Oracle timing on this host: 1 double + 2 single blocks at full shape -> steps/s."""
+def cpu_baseline(cfg, wl, forwards):
+    """The CPU oracle on this host: ONE whole forward of the workload (input projections, timestep MLP and
+    modulation, all double- and single-stream blocks, final layer) at full shape, timed after a small warm-up
+    forward that touches every weight -> steps/s (a CFG step is two such forwards)."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import oracle as O
     blas = O.enable_blas()
-    sub = FluxConfig(**{**cfg.as_dict(), "n_double": 1, "n_single": 1})
-    names = [n for n in tensor_shapes(sub) if n.startswith(("transformer_blocks.0.", "single_transformer_blocks.0."))]
-    W = make_weights(sub, 42, 0.02, "literal", only=names)
-    o = O.Oracle(sub, W)
-    del W
-    H = cfg.hidden
-    n = n_img + n_txt
-    ic, isn = O.rope_image(1, n_img)
-    tc, ts = O.rope_text(n_txt)
-    ih, th = normal_f32((n_img, H), 9, 1), normal_f32((n_txt, H), 9, 2)
-    im, tm = normal_f32((6 * H,), 9, 3, 0.0, 0.1), normal_f32((6 * H,), 9, 4, 0.0, 0.1)
-    O.linear(normal_f32((256, 256), 9, 5), normal_f32((256, 256), 9, 6))   # wake the BLAS threads
+    o = O.Oracle(cfg, {})
+    for name in tensor_shapes(cfg):                      # one tensor at a time on the host (15.5 GB as fp32 in the oracle)
+        a = make_weights(cfg, 42, 0.02, "literal", only=[name])[name]
+        assert O.lib().fo_model_set_bf16(o.h, name.encode(), a.ctypes.data, a.size) == 0, name
+    h, w, nt = wl["h"], wl["w"], wl["txt"]
+    refs = [(normal_f32((cfg.channels, rh, rw), 123, 10 + i), rh, rw, t) for i, (rh, rw, t) in enumerate(wl["refs"])]
+    o.forward(normal_f32((cfg.channels, 2, 2), 9, 1), 2, 2, normal_f32((8, cfg.text_dim), 9, 2), 1.0)   # warm-up: 12 tokens
+    z = normal_f32((cfg.channels, h, w), 123, 1)
+    txt = normal_f32((nt, cfg.text_dim), 123, 2)
     t0 = time.time()
-    o.double_block(0, ih, th, im, tm, ic, isn, tc, ts)
-    t_d = time.time() - t0
-    x = normal_f32((n, H), 9, 7)
-    t_s = []
-    for _ in range(2):
-        t0 = time.time()
-        o.single_block(0, x, im[:3 * H], ic, isn, tc, ts, n_txt)
-        t_s.append(time.time() - t0)
+    v = o.forward(z, h, w, txt, 1.0, refs=refs)
+    t_fwd = time.time() - t0
+    assert np.isfinite(v).all()
     o.close()
-    t_step = cfg.n_double * t_d + cfg.n_single * min(t_s)
+    n = h * w + sum(rh * rw for rh, rw, _ in wl["refs"]) + nt
+    threads = int(O.lib().fo_num_threads())
     return {
-        "value": 1.0 / t_step, "unit": "steps/s", "cores": int(O.lib().fo_num_threads()), "kind": "port",
-        "sample": f"1 double-stream block ({t_d:.2f} s) + 2 single-stream blocks ({min(t_s):.2f} s each) at full shape "
-                  f"({n} tokens), extrapolated to {cfg.n_double}+{cfg.n_single} blocks; "
-                  f"{'OpenBLAS sgemm ' + os.path.basename(blas) if blas else 'built-in OpenMP loops'}",
+        "value": 1.0 / (forwards * t_fwd), "unit": "steps/s", "cores": threads, "kind": "port",
+        "sample": f"1 full forward of the CPU oracle ({t_fwd:.2f} s: embedders, {cfg.n_double} double- and {cfg.n_single} single-stream "
+                  f"blocks, final layer; {n} tokens) after a 12-token warm-up forward"
+                  + (f", times {forwards} forwards per step" if forwards > 1 else "") + "; "
+                  + (f"GEMMs: OpenBLAS sgemm ({os.path.basename(blas)}) on {threads} threads" if blas else f"GEMMs: built-in OpenMP loops on {threads} threads")
+                  + f", os.cpu_count() = {os.cpu_count()}; the oracle's other loops (AdaLN, QK-norm, RoPE, softmax, SiLU) are OpenMP-parallel "
+                    "on the same threads, where the reference runs them on one thread (flux_transformer.c:1021-1046), so this "
+                    "baseline is at least as fast as the reference's BLAS build would be on this host",
     }
 
 
@@ -294,18 +294,54 @@ def bench_qwen3(args):
         "tflops": round(flops * K / wall / 1e12, 1), "flops_per_step": flops, "roofline": roof, "cpu_baseline": cpu}))
 
 
+def bench_mfma_peak(args):
+    """The matrix pipes on their own (flux_hip_mfma_peak: register-resident loops of independent bf16 MFMAs on every
+    compute unit, no memory traffic), for both instruction shapes, one and two waves per SIMD, and operand data of
+    three kinds. One "step" is one launch of about 5 ms; the figure is the best of --steps launches after --warmup."""
+    import ctypes
+    fluxhip.init()
+    L = fluxhip.lib()
+    L.flux_hip_mfma_peak.argtypes = [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_float)]
+    shapes = {0: "v_mfma_f32_16x16x32_bf16", 1: "v_mfma_f32_32x32x16_bf16"}
+    patterns = {0: "all zeros", 1: "1.0 <= x < 2.0, random low byte", 2: "random bit patterns"}
+    iters = 12000                       # x 16 MFMAs per wave: about 5 ms per launch at two waves per SIMD
+    table = []
+    for waves in (2, 1):
+        for pat in patterns:
+            row = {"operands": patterns[pat], "waves_per_simd": waves}
+            for sh in shapes:
+                t = ctypes.c_float(0.0)
+                for _ in range(max(args.warmup, 0)):
+                    fluxhip.check(L.flux_hip_mfma_peak(sh, pat, waves, iters, 1, ctypes.byref(t)), "flux_hip_mfma_peak")
+                fluxhip.check(L.flux_hip_mfma_peak(sh, pat, waves, iters, max(args.steps, 1), ctypes.byref(t)), "flux_hip_mfma_peak")
+                row[shapes[sh]] = round(t.value, 1)
+            table.append(row)
+    best = max(r[shapes[0]] for r in table if r["operands"] == "random bit patterns")
+    zeros = max(max(r[shapes[0]], r[shapes[1]]) for r in table if r["operands"] == "all zeros")
+    print(json.dumps({
+        "metric": "MFMA-only bf16 throughput, operands in registers (TFLOP/s, 1 GPU)", "value": best, "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "mfma_peak: one workgroup per compute unit, 16 independent accumulator blocks (64 registers) per wave, "
+                               f"{iters} x 16 MFMAs per wave and launch; value = v_mfma_f32_16x16x32_bf16 on random bit patterns"},
+        "datasheet_peak": PEAK_BF16_TFLOPS, "best_on_zero_operands": zeros, "frac_of_datasheet_on_random_bits": round(best / PEAK_BF16_TFLOPS, 4),
+        "table": table, "roofline": None, "cpu_baseline": None}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=8)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + sorted(VAE_WORKLOADS) + ["qwen3"])
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + sorted(VAE_WORKLOADS) + ["qwen3", "mfma_peak"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     ap.add_argument("--tile-mask", type=lambda v: int(v, 0), default=0,
                     help="restrict the GEMM tiles the backend may choose (bit t = tile id t), for A/B runs")
     ap.add_argument("--sequential-cfg", action="store_true",
                     help="run the two forwards of a CFG step one after the other instead of as one batch (A/B runs)")
+    ap.add_argument("--fused-qkv-mlp", type=int, default=1, choices=[0, 1],
+                    help="single-stream blocks: 1 = QKV and gate/up projections as one launch (default), 0 = as two (A/B runs)")
     ap.add_argument("--calibrate", action="store_true",
                     help="launch only a streaming kernel of known size (f32->bf16 over 64 Mi elements: reads 256 MiB, "
                          "writes 128 MiB) and the dominant GEMM, for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
@@ -319,6 +355,8 @@ def main():
         return bench_vae(args)
     if args.workload == "qwen3":
         return bench_qwen3(args)
+    if args.workload == "mfma_peak":
+        return bench_mfma_peak(args)
     cfg = KLEIN_4B
     wl = WORKLOADS[args.workload]
     if args.calibrate:
@@ -346,6 +384,7 @@ def main():
         fluxhip.lib().flux_hip_linear_tile_mask(args.tile_mask)
     if args.sequential_cfg:
         fluxhip.lib().flux_hip_set_batched_cfg(0)
+    fluxhip.lib().flux_hip_set_fused_qkv_mlp(args.fused_qkv_mlp)
     model = load_model(cfg)
     z = normal_f32((cfg.channels, h, w), 123, 1)
     txt = normal_f32((nt, cfg.text_dim), 123, 2)
@@ -415,7 +454,7 @@ def main():
 
     cpu = None
     if not args.no_cpu_baseline:
-        cpu = cpu_baseline(cfg, n_img, nt)
+        cpu = cpu_baseline(cfg, wl, forwards)
 
     out = {
         "metric": "transformer denoise steps/s at 1024^2 (1 GPU); achieved TFLOP/s vs bf16 peak"

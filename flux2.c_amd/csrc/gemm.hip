@@ -70,6 +70,11 @@ struct GemmArgs {
     int mtiles, ntiles, total_tiles;
     int vgrid; /* workgroups' worth of tiles (a multiple of 8); a launch with fewer workgroups walks them in strides of its size */
     int N, K, lda, ldw, ldc, w_row0, w_row1;
+    /* fused [Q | K | V | gate | up] projection (EPI_QKV_SWIGLU): the first nq_cols columns (weight rows from w_row0)
+     * are stored as bf16 to C, the other N - nq_cols are gate / up pairs (gate rows from w_row1, up rows from
+     * w_row2) whose silu(gate) * up goes to C2; nq_tiles = nq_cols / tile width */
+    int w_row2, nq_cols, nq_tiles, ldc2;
+    void *C2;
     /* split-K: workgroup (tile, s) multiplies K-steps [s*kt_per, (s+1)*kt_per) and stores its
      * fp32 partial tile into ws[s][moff[part] + m][n]; a second kernel sums the slices */
     int ksplit, kt_per;
@@ -105,6 +110,8 @@ __device__ __forceinline__ int a_step_offset(const GemmArgs &g, int kt) {
 
 /* internal epilogue: fp32 partial sums of one K slice (see split-K above) */
 #define EPI_PARTIAL 5
+/* internal epilogue of flux_hip_linear_qkv_swiglu: bf16 store for the leading column tiles, SiLU(gate) * up beyond */
+#define EPI_QKV_SWIGLU 8
 
 __device__ __forceinline__ int lds_swz(int r) { return ((r >> 1) & 7) ^ ((r & 1) << 2); }
 
@@ -142,9 +149,10 @@ __device__ __forceinline__ bool decode_tile(const GemmArgs &g, int vb, TileId &t
  * gate, up so that a lane ends up holding matching pairs. */
 template <int BN, int WN, int EPI>
 __device__ __forceinline__ int weight_row(const GemmArgs &g, int tn, int v) {
-    if (EPI == FLUX_HIP_EPI_SWIGLU) {
+    if (EPI == FLUX_HIP_EPI_SWIGLU || (EPI == EPI_QKV_SWIGLU && tn >= g.nq_tiles)) {
         int wv = v / WN, blk = (v % WN) >> 4;
         int idx = wv * (WN / 2) + (blk >> 1) * 16 + (v & 15);
+        if (EPI == EPI_QKV_SWIGLU) return ((blk & 1) ? g.w_row2 : g.w_row1) + (tn - g.nq_tiles) * (BN / 2) + idx;
         return ((blk & 1) ? g.w_row1 : g.w_row0) + tn * (BN / 2) + idx;
     }
     return g.w_row0 + tn * BN + v;
@@ -153,10 +161,10 @@ __device__ __forceinline__ int weight_row(const GemmArgs &g, int tn, int v) {
 /* Accumulator element e of block (i, j): feature n = 4*(lane/16) + e of the 16-column block,
  * token m = lane%16 of the 16-row block. */
 template <int BN, int WM, int WN, int EPI>
-__device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f32x4 (&acc)[WN / 16][WM / 16], int m0, int M,
-                                           int wm, int wn, int l15, int lq, int prow) {
+__device__ __forceinline__ void store_tile_to(const GemmArgs &g, const TileId &t, f32x4 (&acc)[WN / 16][WM / 16], int m0, int M,
+                                              int wm, int wn, int l15, int lq, int prow, void *Cp, const int ldc, const int tn) {
     constexpr int TM = WM / 16, TN = WN / 16;
-    const int ldc = g.ldc, prob = t.prob, tn = t.tn, n0 = tn * BN, ks = t.ks;
+    const int prob = t.prob, n0 = tn * BN, ks = t.ks;
     float st_s[TN], st_q[TN]; /* convolutions with statistics: this lane's sums per 16-column block */
 #pragma unroll
     for (int i = 0; i < TN; i++) st_s[i] = st_q[i] = 0.0f;
@@ -170,7 +178,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f
             inside = y >= 1 && y < g.conv_hp - 1 && x >= 1 && x < g.conv_wp - 1;
         }
         if (EPI == FLUX_HIP_EPI_SWIGLU) {
-            bf16 *C = (bf16 *)g.C[prob] + (size_t)m * ldc + tn * (BN / 2) + wn * (WN / 2) + lq * 4;
+            bf16 *C = (bf16 *)Cp + (size_t)m * ldc + tn * (BN / 2) + wn * (WN / 2) + lq * 4;
 #pragma unroll
             for (int i = 0; i < TN; i += 2) {
                 bf16x4 o;
@@ -186,16 +194,16 @@ __device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f
                     bf16x4 o;
 #pragma unroll
                     for (int e = 0; e < 4; e++) o[e] = (bf16)acc[i][j][e];
-                    *(bf16x4 *)((bf16 *)g.C[prob] + (size_t)m * ldc + n) = o;
+                    *(bf16x4 *)((bf16 *)Cp + (size_t)m * ldc + n) = o;
                 } else if (EPI == EPI_PARTIAL) {
                     *(f32x4 *)(g.ws + ((size_t)ks * g.ws_rows + g.moff[prob] + m) * g.N + n) = acc[i][j];
                 } else if (EPI == FLUX_HIP_EPI_F32) {
-                    *(f32x4 *)((float *)g.C[prob] + (size_t)m * ldc + n) = acc[i][j];
+                    *(f32x4 *)((float *)Cp + (size_t)m * ldc + n) = acc[i][j];
                 } else if (EPI == FLUX_HIP_EPI_F32_T) {
 #pragma unroll
-                    for (int e = 0; e < 4; e++) ((float *)g.C[prob])[(size_t)(n + e) * ldc + m] = acc[i][j][e];
+                    for (int e = 0; e < 4; e++) ((float *)Cp)[(size_t)(n + e) * ldc + m] = acc[i][j][e];
                 } else if (EPI == FLUX_HIP_EPI_RESID) {
-                    float *p = (float *)g.C[prob] + (size_t)m * ldc + n;
+                    float *p = (float *)Cp + (size_t)m * ldc + n;
                     f32x4 x = *(f32x4 *)p;
                     f32x4 gt = *(const f32x4 *)(g.gate[prob] + n);
 #pragma unroll
@@ -211,7 +219,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f
                         st_s[i] += v;
                         st_q[i] += v * v;
                     }
-                    *(bf16x4 *)((bf16 *)g.C[prob] + (size_t)m * ldc + n) = o;
+                    *(bf16x4 *)((bf16 *)Cp + (size_t)m * ldc + n) = o;
                 } else if (EPI == FLUX_HIP_EPI_CONV_F32) {
                     const f32x4 bv = *(const f32x4 *)(g.bias + n);
                     f32x4 r = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -222,7 +230,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f
                         st_s[i] += r[e];
                         st_q[i] += r[e] * r[e];
                     }
-                    *(f32x4 *)((float *)g.C[prob] + (size_t)m * ldc + n) = r;
+                    *(f32x4 *)((float *)Cp + (size_t)m * ldc + n) = r;
                 }
             }
         }
@@ -245,6 +253,19 @@ __device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f
     }
 }
 
+/* Cp, ldc, tn: where the tile goes - the part's output, or for the fused [Q|K|V|gate|up] projection the output of the
+ * side of the boundary the tile lies on (the tile width divides nq_cols, so a tile is wholly on one side) */
+template <int BN, int WM, int WN, int EPI>
+__device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f32x4 (&acc)[WN / 16][WM / 16], int m0, int M,
+                                           int wm, int wn, int l15, int lq, int prow) {
+    if constexpr (EPI == EPI_QKV_SWIGLU) {
+        if (t.tn < g.nq_tiles) store_tile_to<BN, WM, WN, FLUX_HIP_EPI_BF16>(g, t, acc, m0, M, wm, wn, l15, lq, prow, g.C[0], g.ldc, t.tn);
+        else store_tile_to<BN, WM, WN, FLUX_HIP_EPI_SWIGLU>(g, t, acc, m0, M, wm, wn, l15, lq, prow, g.C2, g.ldc2, t.tn - g.nq_tiles);
+    } else {
+        store_tile_to<BN, WM, WN, EPI>(g, t, acc, m0, M, wm, wn, l15, lq, prow, g.C[t.prob], g.ldc, t.tn);
+    }
+}
+
 template <int BM, int BN, int WGM, int WGN, int EPI>
 __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
     constexpr int T = WGM * WGN * 64;
@@ -253,7 +274,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
     constexpr int PA = BM / RPP, PB = BN / RPP;
     constexpr int STAGE = (BM + BN) * 128;
     static_assert(BM % RPP == 0 && BN % RPP == 0, "tile rows must divide evenly over threads");
-    static_assert(EPI != FLUX_HIP_EPI_SWIGLU || (TN % 2 == 0), "swiglu pairs 16-column blocks");
+    static_assert((EPI != FLUX_HIP_EPI_SWIGLU && EPI != EPI_QKV_SWIGLU) || (TN % 2 == 0), "swiglu pairs 16-column blocks");
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     TileId t;
@@ -385,7 +406,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm4w_kernel(GemmArgs g) {
     constexpr int NM = TM * TN;     /* MFMAs per K half-step */
     constexpr int RD = NM / NF;     /* one LDS read (and one load) every RD MFMAs */
     constexpr int STAGE = (BM + BN) * 128;
-    static_assert(EPI != FLUX_HIP_EPI_SWIGLU || (TN % 2 == 0), "swiglu pairs 16-column blocks");
+    static_assert((EPI != FLUX_HIP_EPI_SWIGLU && EPI != EPI_QKV_SWIGLU) || (TN % 2 == 0), "swiglu pairs 16-column blocks");
     static_assert(RD >= 2 && RD * (NF - 1) + 1 < NM, "reads and loads must fit between the MFMAs");
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -554,6 +575,7 @@ static int launch_cfg(GemmArgs &g) {
     }
     set_row_tiles(g, BM);
     g.ntiles = g.N / BN;
+    g.nq_tiles = g.nq_cols / BN;
     g.total_tiles = g.mtiles * g.ntiles;
     int grid = (g.total_tiles * g.ksplit + 7) & ~7;
     g.vgrid = grid;
@@ -573,9 +595,10 @@ static int launch_4w(GemmArgs &g) {
     }
     set_row_tiles(g, BM);
     g.ntiles = g.N / BN;
+    g.nq_tiles = g.nq_cols / BN;
     g.total_tiles = g.mtiles * g.ntiles;
     /* the kernel addresses operand rows with 32-bit byte offsets from the matrix base */
-    size_t span = ((size_t)max(g.w_row0, g.w_row1) + g.N) * g.ldw * 2;
+    size_t span = ((size_t)max(max(g.w_row0, g.w_row1), g.w_row2) + g.N) * g.ldw * 2;
     for (int i = 0; i < GEMM_MAX_PARTS; i++) span = max(span, (size_t)g.M[i] * g.lda * 2);
     if (span >= ((size_t)1 << 32)) return g.N % 128 == 0 ? launch_cfg<128, 128, 2, 2, EPI>(g) : launch_cfg<64, 64, 2, 2, EPI>(g);
     /* one workgroup fits on a compute unit (registers, LDS): launch at most that many, each walks its share of the tiles */
@@ -931,7 +954,7 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
         double rows = 0.0;
         for (int i = 0; i < np; i++) rows += g.M[i];
         for (int t = 0; t < NT; t++) {
-            if (N % bn[t]) continue;
+            if (N % bn[t] || g.nq_cols % bn[t]) continue;
             if (!((allowed >> t) & 1)) continue;
             long tiles = 0;
             for (int i = 0; i < np; i++) tiles += (g.M[i] + bm[t] - 1) / bm[t];
@@ -995,6 +1018,7 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
             }
             break;
         case FLUX_HIP_EPI_SWIGLU: ok = split ? launch_split<FLUX_HIP_EPI_SWIGLU>(g, tile) : launch_epi<FLUX_HIP_EPI_SWIGLU>(g, tile); break;
+        case EPI_QKV_SWIGLU: ok = launch_epi<EPI_QKV_SWIGLU>(g, tile); break;
         case FLUX_HIP_EPI_CONV_BF16: ok = launch_conv<FLUX_HIP_EPI_CONV_BF16>(g, tile); break;
         case FLUX_HIP_EPI_CONV_F32: ok = launch_conv<FLUX_HIP_EPI_CONV_F32>(g, tile); break;
         default: return flux_hip_fail("flux_hip_linear: unknown epilogue %d", epilogue);
@@ -1053,6 +1077,30 @@ static int linear_impl(int epilogue, int nparts, const flux_hip_linear_part *par
 extern "C" int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
                                int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1) {
     return linear_impl(epilogue, nparts, parts, N, K, lda, ldw, ldc, w_row0, w_row1, nullptr, 0.0f, nullptr);
+}
+
+/* One launch for the fused projection of a single-stream block, see the header. Never split along K. */
+extern "C" int flux_hip_linear_qkv_swiglu(const void *A, const void *W, void *qkv_out, void *mlp_out, int M, int qkv_cols, int mlp, int K,
+                                          int lda, int ldw, int ld_qkv, int ld_mlp) {
+    if (M <= 0) return 1;
+    if (K <= 0 || (K & 63)) return flux_hip_fail("flux_hip_linear_qkv_swiglu: K=%d must be a positive multiple of 64", K);
+    if (qkv_cols <= 0 || (qkv_cols & 127) || mlp <= 0 || (mlp & 63))
+        return flux_hip_fail("flux_hip_linear_qkv_swiglu: qkv_cols=%d must be a multiple of 128, mlp=%d of 64", qkv_cols, mlp);
+    if (lda < K || ldw < K || (lda & 7) || (ldw & 7) || (ld_qkv & 3) || (ld_mlp & 3))
+        return flux_hip_fail("flux_hip_linear_qkv_swiglu: bad leading dimensions");
+    if (!A || !W || !qkv_out || !mlp_out) return flux_hip_fail("flux_hip_linear_qkv_swiglu: NULL operand");
+    if ((((uintptr_t)A | (uintptr_t)W) & 15) || (((uintptr_t)qkv_out | (uintptr_t)mlp_out) & 7))
+        return flux_hip_fail("flux_hip_linear_qkv_swiglu: operands must be 16-byte aligned (outputs 8-byte)");
+    GemmArgs g = {};
+    g.A[0] = (const bf16 *)A; g.W[0] = (const bf16 *)W; g.C[0] = qkv_out; g.C2 = mlp_out; g.M[0] = M;
+    g.N = qkv_cols + 2 * mlp; g.K = K; g.lda = lda; g.ldw = ldw; g.ldc = ld_qkv; g.ldc2 = ld_mlp;
+    g.w_row0 = 0; g.w_row1 = qkv_cols; g.w_row2 = qkv_cols + mlp; g.nq_cols = qkv_cols;
+    int tile = -1;
+    const int saved = g_splitk_enabled;
+    g_splitk_enabled = 0;
+    const int ok = gemm_dispatch(g, 1, EPI_QKV_SWIGLU, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0xFFu, &tile);
+    g_splitk_enabled = saved;
+    return ok;
 }
 
 /* flux_hip_linear for callers that must not allocate: the partial sums of the K slices go to the

@@ -96,6 +96,19 @@ int flux_hip_linear(int epilogue, int nparts, const flux_hip_linear_part *parts,
                     int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1);
 
 /*
+ * The fused projection of a single-stream block in one launch: the reference runs one linear
+ * hidden -> 3*hidden + 2*mlp whose output rows are [Q, K, V, gate, up] (flux_transformer.c:3034-3058).
+ * Here A bf16 [M, lda] is multiplied by W bf16 [qkv_cols + 2*mlp, ldw] once; output columns
+ * [0, qkv_cols) are stored as bf16 to qkv_out [M, ld_qkv], and for the rest silu(gate) * up
+ * (weight rows qkv_cols.. are the gate, qkv_cols + mlp.. the up features) goes as bf16 to
+ * mlp_out [M, ld_mlp] (mlp columns). Bit for bit what flux_hip_linear gives in two launches with
+ * FLUX_HIP_EPI_BF16 and FLUX_HIP_EPI_SWIGLU on the same tile; the activations are read once and
+ * one launch has all the column tiles. qkv_cols % 128 == 0, mlp % 64 == 0, K % 64 == 0.
+ */
+int flux_hip_linear_qkv_swiglu(const void *A, const void *W, void *qkv_out, void *mlp_out, int M, int qkv_cols, int mlp, int K,
+                               int lda, int ldw, int ld_qkv, int ld_mlp);
+
+/*
  * flux_hip_linear that allocates nothing. No counterpart in the reference: it is for callers that
  * cannot call hipMalloc - code under HIP graph capture, tight serving loops, harnesses that forbid
  * allocation. flux_hip_linear takes a workspace from hipMalloc (kept and grown on demand) when it

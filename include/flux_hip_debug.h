@@ -32,6 +32,9 @@ void flux_hip_attention_force_variant(int v);
 /* 1 (default): a CFG step runs its two forwards as one batch of two sequences; 0: one after the other.
  * Takes effect at the next flux_hip_session_begin. */
 void flux_hip_set_batched_cfg(int on);
+/* The fused projection of a single-stream block: 1 (default) = one launch (flux_hip_linear_qkv_swiglu), 0 = two
+ * (QKV, then gate/up). */
+void flux_hip_set_fused_qkv_mlp(int on);
 /* VAE attention: at most `rows` query rows per chunk (0 = default: 1 GB of fp32 scores per chunk). */
 void flux_hip_vae_set_attention_chunk(int rows);
 
@@ -44,6 +47,13 @@ int flux_hip_linear_probe(int epilogue);
 int flux_hip_linear_probe_read(int *launches, float *total_ms);
 int flux_hip_linear_probe_read_tile(int tile, int *launches, float *total_ms);
 int flux_hip_linear_probe_read_launches(int max, int *tiles, float *ms);
+
+/* What the matrix pipes sustain on their own: a register-resident loop of independent bf16 MFMAs on every
+ * compute unit (one workgroup each, waves_per_simd = 1 or 2 waves per SIMD; `iters` x 16 MFMAs per wave),
+ * run launches + 1 times; the best launch's rate in TFLOP/s goes to *tflops. shape 0 =
+ * v_mfma_f32_16x16x32_bf16, 1 = v_mfma_f32_32x32x16_bf16; pattern 0 = all-zero operands, 1 = values in
+ * [1, 2) with a random low byte, 2 = random bit patterns. `bench.py --workload mfma_peak` prints the table. */
+int flux_hip_mfma_peak(int shape, int pattern, int waves_per_simd, int iters, int launches, float *tflops);
 
 #ifdef __cplusplus
 }

@@ -45,6 +45,7 @@ def _default_switches(request):
         L.flux_hip_linear_persistent(1)
         L.flux_hip_attention_force_variant(-1)
         L.flux_hip_set_batched_cfg(1)
+        L.flux_hip_set_fused_qkv_mlp(1)
         L.flux_hip_vae_set_attention_chunk(0)
         L.flux_hip_linear_probe(-1)
     restore()

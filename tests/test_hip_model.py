@@ -131,6 +131,31 @@ def test_batched_cfg_equals_two_forwards(hip, oracle_mod):
     m.close(); o.close()
 
 
+def test_single_stream_projection_as_one_or_two_launches(hip, oracle_mod):
+    """A single-stream block's [Q | K | V | gate | up] projection runs as one launch (the default) or as two: both
+    within the gate of the oracle, and equal up to the tile choice's summation order. 30 tokens (where the two
+    launches run as K slices) and 300."""
+    cfg = SMALL
+    W = make_weights(cfg, 42, 0.05, "sharp")
+    o = oracle_mod.Oracle(cfg, W)
+    m = hip.Transformer(cfg, W)
+    L = hip.lib()
+    try:
+        for h, w, nt in ((4, 5, 10), (16, 17, 28)):
+            lat = normal_f32((cfg.channels, h, w), 19, 1)
+            txt = normal_f32((nt, cfg.text_dim), 19, 2)
+            want = o.forward(lat, h, w, txt, 0.6)
+            got = {}
+            for mode in (0, 1):
+                L.flux_hip_set_fused_qkv_mlp(mode)
+                got[mode] = m.forward(lat, h, w, txt, 0.6)
+                gate(got[mode], want, f"{h}x{w}+{nt} tokens, fused projection mode {mode}")
+            assert rel_l2(got[1], got[0]) < 5e-3      # bf16 intermediates round differently when the K slices of the two-launch form sum in another order
+    finally:
+        L.flux_hip_set_fused_qkv_mlp(1)
+    m.close(); o.close()
+
+
 def test_broken_rope_would_be_caught(hip, oracle_mod):
     """Sensitivity check: against an oracle whose image RoPE is mirrored the gate must fail,
     otherwise the sharp fixture would say nothing about RoPE in the HIP kernels."""

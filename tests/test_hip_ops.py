@@ -298,6 +298,42 @@ def test_linear_residual_then_rms_norm(hip, oracle_mod):
                                [(dn.ptr, None, dwn.ptr), (dn.ptr, dwn.ptr, dwn.ptr)])
 
 
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6, 7])
+@pytest.mark.parametrize("M", [45, 700])
+def test_linear_qkv_swiglu_one_launch(hip, oracle_mod, tile, M):
+    """The fused projection of a single-stream block (rows [Q, K, V, gate, up], flux_transformer.c:3034-3058) as ONE
+    launch: bit for bit what the two launches (bf16 store, SiLU(gate) * up) give on the same tile, and right
+    against the oracle. Strided outputs; nothing written outside them."""
+    import ctypes
+    L = hip.lib()
+    L.flux_hip_linear_qkv_swiglu.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 8
+    L.flux_hip_linear_force_tile(tile)
+    K, qc, mlp = 192, 768, 1536                         # both widths are multiples of every tile width (64 ... 256)
+    ldq, ldm = qc + 64, mlp + 128
+    x = q(normal_f32((M, K), 61, 1))
+    W = q(normal_f32((qc + 2 * mlp, K), 61, 2, 0.0, 0.1))
+    dx, dW = dev_bf16(hip, x), dev_bf16(hip, W)
+    fq = hip.DevBuf.from_array(np.zeros((M, ldq), np.uint16))
+    fm = hip.DevBuf.from_array(np.zeros((M, ldm), np.uint16))
+    hip.check(L.flux_hip_linear_qkv_swiglu(dx.ptr, dW.ptr, fq.ptr, fm.at(64 * 2), M, qc, mlp, K, K, K, ldq, ldm), "flux_hip_linear_qkv_swiglu")
+    tq = hip.DevBuf.from_array(np.zeros((M, ldq), np.uint16))
+    tm = hip.DevBuf.from_array(np.zeros((M, ldm), np.uint16))
+    L.flux_hip_linear_enable_splitk(0)
+    try:
+        hip.linear(hip.EPI_BF16, [(dx.ptr, dW.ptr, tq.ptr, None, M)], qc, K, K, K, ldq, 0, 0)
+        hip.linear(hip.EPI_SWIGLU, [(dx.ptr, dW.ptr, tm.at(64 * 2), None, M)], 2 * mlp, K, K, K, ldm, qc, qc + mlp)
+    finally:
+        L.flux_hip_linear_enable_splitk(1)
+        L.flux_hip_linear_force_tile(-1)
+    got_q, got_m = fq.to_array(np.uint16, (M, ldq)), fm.to_array(np.uint16, (M, ldm))
+    np.testing.assert_array_equal(got_q, tq.to_array(np.uint16, (M, ldq)))
+    np.testing.assert_array_equal(got_m, tm.to_array(np.uint16, (M, ldm)))
+    lin = oracle_mod.linear(x, W)
+    assert rel_l2(bf16_to_f32(got_q[:, :qc]), lin[:, :qc]) < 4e-3
+    assert rel_l2(bf16_to_f32(got_m[:, 64:64 + mlp]), oracle_mod.silu(lin[:, qc:qc + mlp]) * lin[:, qc + mlp:]) < 4e-3
+    assert not got_q[:, qc:].any() and not got_m[:, :64].any() and not got_m[:, 64 + mlp:].any()
+
+
 def test_linear_rejects_bad_shapes(hip):
     d = hip.DevBuf(1024)
     with pytest.raises(hip.FluxHipError):
