@@ -423,6 +423,328 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
     }
 }
 
+
+/* ---------------------------------------------------------------------------------------
+ * The same attention with 16 NQ queries per wave (NQ = 1 .. 4) and four waves, one per SIMD, per
+ * workgroup: 64 NQ queries per workgroup. A K or V^T fragment read from LDS now feeds NQ MFMAs instead
+ * of two, so a 64-query wave needs half the LDS bytes and fragment reads per FLOP of the 32-query
+ * waves above. The price is registers - 32 NQ for the output accumulators, 16 NQ each for the scores
+ * and the Q fragments - which is why there is one wave per SIMD and why the MFMAs are written as inline
+ * assembly: the output accumulators and the Q fragments are pinned to AGPRs, the scores to VGPRs, and
+ * nothing migrates between the register files (left to the register allocator, a kernel of this
+ * shape moves some two hundred registers per key tile between them).
+ * Hazards the compiler cannot see in inline assembly are kept apart by construction: the same
+ * accumulator is written again only after at least four other MFMAs, and vector code reads MFMA
+ * results only behind an explicit run of idle cycles (mfma_results_fence).
+ * --------------------------------------------------------------------------------------- */
+#define MFMA_ACC_A(acc, a, b) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b))
+#define MFMA_ACC_V(acc, a, b) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b))
+#define MFMA_ACC_VQ(acc, a, q) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(q))
+#define MFMA_NEW_VQ(acc, a, q, c) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %3" : "=&v"(acc) : "v"(a), "a"(q), "v"(c))
+/* Guarded forms, for MFMAs whose operands a vector instruction may have written just before (the bf16
+ * probabilities, a start value the compiler re-creates, a register copy it slips in): two idle issue slots travel
+ * inside the statement, so nothing can come between them and the MFMA. */
+#define MFMA_NEW_VQ_GUARDED(acc, a, q, c) \
+    asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %3" : "=&v"(acc) : "v"(a), "a"(q), "v"(c))
+#define MFMA_ACC_V_ONES_GUARDED(acc, ones, b) asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc) : "a"(ones), "v"(b))
+
+/* Idle cycles until the last MFMAs have written their results, then every listed accumulator passes
+ * through an empty asm statement ordered with the MFMAs, so that reads of them stay behind it. */
+template <int N>
+__device__ __forceinline__ void mfma_results_fence_v(f32x4 (&acc)[4][N]) {
+    asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < N; j++) asm volatile("" : "+v"(acc[i][j]));
+}
+template <int N>
+__device__ __forceinline__ void mfma_results_fence_a(f32x4 (&acc)[8][N]) {
+    asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < N; j++) asm volatile("" : "+a"(acc[i][j]));
+}
+
+template <int NQ>
+__global__ __launch_bounds__(256, 1) void attention_wide_kernel(bf16 *__restrict__ out, int ldo, const bf16 *__restrict__ q, int ldq,
+                                                                const bf16 *__restrict__ k, const bf16 *__restrict__ vt, int ld_vt,
+                                                                int seq_q, int seq_k, int heads, int split,
+                                                                const float *__restrict__ q_w0, const float *__restrict__ q_w1,
+                                                                const float *__restrict__ rope_cos, const float *__restrict__ rope_sin,
+                                                                float eps) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    constexpr int NW = 4, WQ = 16 * NQ, BQ = NW * WQ, LP = 16 / NW;
+    /* every XCD gets a contiguous run of (head, query block) pairs, as above */
+    const int nqb = (seq_q + BQ - 1) / BQ;
+    const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    if (logical >= nqb * heads) return;
+    const int h = logical / nqb, qb = logical - h * nqb;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l15 = lane & 15, lq = lane >> 4;
+    const int H = heads * HD;
+
+    /* ---- tile loader: as in attention_kernel<4> ---- */
+    const int ntiles = (seq_k + 63) >> 6;
+    const bf16 *k_src[LP];
+    const bf16 *v_src[LP];
+    int k_dst[LP], v_dst[LP], k_row[LP];
+#pragma unroll
+    for (int i = 0; i < LP; i++) {
+        int r = wave * 4 + i * (NW * 4) + (lane >> 4);
+        {
+            int ib = r >> 4, jj = (r >> 2) & 3, ee = r & 3;
+            k_row[i] = 32 * (ib >> 1) + 8 * jj + 4 * (ib & 1) + ee;
+        }
+        k_src[i] = k + h * HD + (((lane & 15) ^ (r & 15)) << 3);
+        k_dst[i] = (wave * 4 + i * (NW * 4)) * 256;
+        int d = wave * 8 + i * (NW * 8) + (lane >> 3);
+        v_src[i] = vt + (size_t)(h * HD + d) * ld_vt + (((lane & 7) ^ vt_swz(d)) << 3);
+        v_dst[i] = (wave * 8 + i * (NW * 8)) * 128;
+    }
+    auto issue_k = [&](int t) {
+        char *base = smem + (t & 1) * (64 * 256);
+        const int key0 = t * 64;
+#pragma unroll
+        for (int i = 0; i < LP; i++) {
+            int r = min(key0 + k_row[i], seq_k - 1);
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(k_src[i] + (size_t)r * H), LDS_PTR(base + k_dst[i]), 16, 0, 0);
+        }
+    };
+    auto issue_v = [&](int t) {
+        char *base = smem + 2 * (64 * 256) + (t & 1) * (128 * 128);
+        const int key0 = t * 64;
+#pragma unroll
+        for (int i = 0; i < LP; i++)
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(v_src[i] + key0), LDS_PTR(base + v_dst[i]), 16, 0, 0);
+    };
+    issue_k(0);
+    issue_v(0);
+
+    /* ---- Q fragments (B operand) with RMSNorm * weight, RoPE and the softmax scale; they live in AGPRs ---- */
+    bf16x8 qf[NQ][4];
+    int qrow[NQ];
+#pragma unroll
+    for (int t = 0; t < NQ; t++) {
+        qrow[t] = qb * BQ + wave * WQ + t * 16 + l15;
+        const int qrc = min(qrow[t], seq_q - 1);
+        const bf16 *qp = q + (size_t)qrc * ldq + h * HD + lq * 8;
+        float x[4][8];
+        float ss = 0.0f;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            bf16x8 v = *(const bf16x8 *)(qp + kk * 32);
+#pragma unroll
+            for (int e = 0; e < 8; e++) { x[kk][e] = (float)v[e]; ss += x[kk][e] * x[kk][e]; }
+        }
+        ss += __shfl_xor(ss, 16, 64);
+        ss += __shfl_xor(ss, 32, 64);
+        const float inv = 1.0f / sqrtf(ss * (1.0f / HD) + eps);
+        const float fold = 0.08838834764831845f * 1.44269504088896341f; /* 1/sqrt(128) and log2(e): scores are base-2 logits */
+        const float *w = (qrc < split ? q_w0 : q_w1) + lq * 8;
+        const float *cs = rope_cos + (size_t)qrc * HD + lq * 8;
+        const float *sn = rope_sin + (size_t)qrc * HD + lq * 8;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            f32x4 w0 = *(const f32x4 *)(w + kk * 32), w1 = *(const f32x4 *)(w + kk * 32 + 4);
+            f32x4 c0 = *(const f32x4 *)(cs + kk * 32), c1 = *(const f32x4 *)(cs + kk * 32 + 4);
+            f32x4 s0 = *(const f32x4 *)(sn + kk * 32), s1 = *(const f32x4 *)(sn + kk * 32 + 4);
+            float wv[8] = {w0[0], w0[1], w0[2], w0[3], w1[0], w1[1], w1[2], w1[3]};
+            float cv[8] = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
+            float sv[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
+#pragma unroll
+            for (int e = 0; e < 8; e += 2) {
+                float a = x[kk][e] * inv * wv[e], b = x[kk][e + 1] * inv * wv[e + 1];
+                qf[t][kk][e] = (bf16)((a * cv[e] - b * sv[e]) * fold);
+                qf[t][kk][e + 1] = (bf16)((b * cv[e] + a * sv[e]) * fold);
+            }
+            asm volatile("" : "+a"(qf[t][kk])); /* one aligned AGPR quad per fragment from here on */
+        }
+    }
+
+    f32x4 o_acc[8][NQ]; /* AGPRs */
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < NQ; j++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) o_acc[i][j][e] = 0.0f;
+    /* neg_m: minus the reference maximum of the online softmax, four copies per query block: the start value
+     * of the score accumulators (see attention_kernel) */
+    f32x4 neg_m[NQ];
+    f32x4 l_acc[NQ];
+#pragma unroll
+    for (int j = 0; j < NQ; j++) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) { neg_m[j][e] = 0.0f; l_acc[j][e] = 0.0f; }
+    }
+    bf16x8 ones;
+#pragma unroll
+    for (int e = 0; e < 8; e++) ones[e] = (bf16)1.0f;
+    /* from here on a value the compiler cannot re-create: it stays in four AGPRs instead of being written anew
+     * right in front of the MFMA that reads it (the compiler does not know that its inline assembly is an MFMA,
+     * which must not read a register in the two issue slots after a vector instruction wrote it) */
+    asm volatile("" : "+a"(ones));
+    f32x4 s_acc[4][NQ];
+
+    /* One key tile, as in attention_kernel: S^T = K Q^T - m_run (16 NQ MFMAs), online softmax with the lazily
+     * moved maximum, O^T += V^T P^T (16 NQ MFMAs) and the row sums (2 NQ). */
+    auto step = [&](int t, auto edge_c) {
+        constexpr bool EDGE = decltype(edge_c)::value;
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        if (t + 1 < ntiles) {
+            issue_k(t + 1);
+            issue_v(t + 1);
+        }
+        const char *kt = smem + (t & 1) * (64 * 256);
+        const char *vtile = smem + 2 * (64 * 256) + (t & 1) * (128 * 128);
+        auto kread = [&](int kk, bf16x8 (&dst)[4]) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) dst[i] = *(const bf16x8 *)(kt + (i * 16 + l15) * 256 + (((kk * 4 + lq) ^ l15) << 4));
+        };
+        auto vread = [&](int b, bf16x8 (&dst)[4]) {
+#pragma unroll
+            for (int f = 0; f < 4; f++) {
+                const int d = ((b & 1) * 4 + f) * 16 + l15;
+                dst[f] = *(const bf16x8 *)(vtile + d * 128 + (((4 * (b >> 1) + lq) ^ vt_swz(d)) << 4));
+            }
+        };
+        bf16x8 fa[4], fb[4];
+        {
+            kread(0, fa);
+            kread(1, fb);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                bf16x8 (&cur)[4] = (kk & 1) ? fb : fa;
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int j = 0; j < NQ; j++) {
+                        if (kk == 0 && i == 0) MFMA_NEW_VQ_GUARDED(s_acc[i][j], cur[i], qf[j][0], neg_m[j]); /* first reader of neg_m[j] */
+                        else if (kk == 0) MFMA_NEW_VQ(s_acc[i][j], cur[i], qf[j][0], neg_m[j]);
+                        else MFMA_ACC_VQ(s_acc[i][j], cur[i], qf[j][kk]);
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+                if (kk + 2 < 4) kread(kk + 2, cur);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        vread(0, fa); /* in flight during the softmax */
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_results_fence_v<NQ>(s_acc);
+
+        if (EDGE && t == ntiles - 1 && (seq_k & 63)) {
+            const int key0 = t * 64;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    if (key0 + 32 * (i >> 1) + 8 * lq + 4 * (i & 1) + e >= seq_k) {
+#pragma unroll
+                        for (int j = 0; j < NQ; j++) s_acc[i][j][e] = -1e30f;
+                    }
+        }
+        bool grow = EDGE && t == 0;
+        float m_new[NQ];
+#pragma unroll
+        for (int j = 0; j < NQ; j++) {
+            float mx = fmaxf(fmaxf(s_acc[0][j][0], s_acc[0][j][1]), fmaxf(s_acc[0][j][2], s_acc[0][j][3]));
+#pragma unroll
+            for (int i = 1; i < 4; i++) mx = fmaxf(fmaxf(mx, fmaxf(s_acc[i][j][0], s_acc[i][j][1])), fmaxf(s_acc[i][j][2], s_acc[i][j][3]));
+            m_new[j] = mx; /* this lane's keys only; relative to m_run */
+            grow = grow || (mx > 8.0f);
+        }
+        if (__any(grow)) {
+            /* rare: some score lies more than 2^8 above the reference (or this is the first tile). The exact row
+             * maxima (a query's scores sit in lanes l, l^16, l^32, l^48) move the references; see attention_kernel. */
+            if (t > 0) mfma_results_fence_a<NQ>(o_acc);
+#pragma unroll
+            for (int j = 0; j < NQ; j++) {
+                float mx = m_new[j];
+                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                const bool first = EDGE && t == 0;
+                const float d = first ? mx : fmaxf(mx, 0.0f);
+                const float alpha = first ? 1.0f : fast_exp2(-d);
+#pragma unroll
+                for (int e = 0; e < 4; e++) { neg_m[j][e] -= d; l_acc[j][e] *= alpha; }
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) s_acc[i][j][e] -= d;
+#pragma unroll
+                for (int i = 0; i < 8; i++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) o_acc[i][j][e] *= alpha;
+            }
+        }
+        bf16x8 pf[2][NQ];
+#pragma unroll
+        for (int j = 0; j < NQ; j++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) s_acc[i][j][e] = fast_exp2(s_acc[i][j][e]);
+#pragma unroll
+            for (int c = 0; c < 2; c++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    pf[c][j][e] = (bf16)s_acc[2 * c][j][e];
+                    pf[c][j][4 + e] = (bf16)s_acc[2 * c + 1][j][e];
+                }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        /* the row sums are the first readers of each probability fragment */
+#pragma unroll
+        for (int j = 0; j < NQ; j++) MFMA_ACC_V_ONES_GUARDED(l_acc[j], ones, pf[0][j]);
+        __builtin_amdgcn_sched_barrier(0);
+        vread(1, fb);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            bf16x8 (&cur)[4] = (b & 1) ? fb : fa;
+            if (b == 2) {
+#pragma unroll
+                for (int j = 0; j < NQ; j++) MFMA_ACC_V_ONES_GUARDED(l_acc[j], ones, pf[1][j]);
+            }
+#pragma unroll
+            for (int f = 0; f < 4; f++)
+#pragma unroll
+                for (int j = 0; j < NQ; j++) MFMA_ACC_A(o_acc[(b & 1) * 4 + f][j], cur[f], pf[b >> 1][j]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (b + 2 < 4) vread(b + 2, cur);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    step(0, AttFlag<true>{});
+    for (int t = 1; t < ntiles - 1; t++) step(t, AttFlag<false>{});
+    if (ntiles > 1) step(ntiles - 1, AttFlag<true>{});
+
+    mfma_results_fence_a<NQ>(o_acc);
+    asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
+#pragma unroll
+    for (int j = 0; j < NQ; j++) asm volatile("" : "+v"(l_acc[j]));
+#pragma unroll
+    for (int j = 0; j < NQ; j++) {
+        const float inv_l = 1.0f / l_acc[j][0];
+        if (qrow[j] < seq_q) {
+            bf16 *op = out + (size_t)qrow[j] * ldo + h * HD + lq * 4;
+#pragma unroll
+            for (int dt = 0; dt < 8; dt++) {
+                bf16x4 r;
+#pragma unroll
+                for (int e = 0; e < 4; e++) r[e] = (bf16)(o_acc[dt][j][e] * inv_l);
+                *(bf16x4 *)(op + dt * 16) = r;
+            }
+        }
+    }
+}
+
 static int g_att_force = -1;
 extern "C" void flux_hip_attention_force_variant(int v) { g_att_force = v; }
 
@@ -443,11 +765,23 @@ extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ld
     const int big = g_att_force >= 0 ? g_att_force : (((seq_q + 255) / 256) * heads >= 256);
     static bool attr_done = false;
     if (!attr_done) {
+        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
+        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
+        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<3>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
+        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
         HIP_OK(hipFuncSetAttribute((const void *)attention_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
         HIP_OK(hipFuncSetAttribute((const void *)attention_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
         attr_done = true;
     }
-    if (big) {
+    if (big >= 11 && big <= 14) {
+        /* 16 NQ queries per wave, four waves per workgroup (variants 11 .. 14 = NQ 1 .. 4) */
+        const int nq = big - 10, bq = 64 * nq;
+        const int blocks = ((seq_q + bq - 1) / bq) * heads;
+        auto kern = nq == 1 ? attention_wide_kernel<1> : nq == 2 ? attention_wide_kernel<2> : nq == 3 ? attention_wide_kernel<3> : attention_wide_kernel<4>;
+        hipLaunchKernelGGL(kern, dim3((blocks + 7) & ~7), dim3(256), 2 * ATT_STAGE, flux_hip_stream_handle(),
+                           (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,
+                           heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps);
+    } else if (big) {
         const int blocks = ((seq_q + 255) / 256) * heads;
         hipLaunchKernelGGL(attention_kernel<8>, dim3((blocks + 7) & ~7), dim3(512), 2 * ATT_STAGE, flux_hip_stream_handle(),
                            (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,

@@ -1,0 +1,140 @@
+"""Register hazards around hand-written MFMAs, checked on the compiler's assembly output (CPU test, no GPU).
+
+The GEMM and attention kernels issue their MFMAs through inline assembly so that accumulators stay in the register
+file they were put in. The compiler does not know that those statements are matrix instructions, so it neither inserts
+the idle cycles the hardware wants around them nor keeps its own register copies away from them:
+  * a vector instruction that writes a register an MFMA reads needs two issue slots in between;
+  * a vector, LDS or memory instruction that touches an MFMA's result register needs the MFMA to have finished
+    (passes + 4 issue slots for this 4-pass instruction; the kernels place sixteen idle cycles, and this test asks for 8).
+The kernels keep these apart by construction; this test compiles the files the way the Makefile does and checks every
+MFMA in the inline-assembly kernels, so that a register copy the allocator slips in front of an MFMA fails here
+instead of giving wrong numbers on the GPU. Instructions are taken in layout order (branches are not followed), which
+is how the straight-line loops of these kernels run.
+"""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "flux2.c_amd", "csrc")
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "--cuda-device-only", "-S"]
+
+VALU_TO_MFMA_SLOTS = 2
+MFMA_RESULT_SLOTS = 8
+
+
+def regs(tok):
+    """'v[4:7]' -> {('v',4..7)}, 'a12' -> {('a',12)}; anything else -> empty."""
+    m = re.fullmatch(r"([va])\[(\d+):(\d+)\]", tok)
+    if m:
+        return {(m.group(1), i) for i in range(int(m.group(2)), int(m.group(3)) + 1)}
+    m = re.fullmatch(r"([va])(\d+)", tok)
+    if m:
+        return {(m.group(1), int(m.group(2)))}
+    return set()
+
+
+def parse(line):
+    line = line.split(";")[0].strip()
+    if not line or line.endswith(":") or line.startswith("."):
+        return None
+    parts = line.split(None, 1)
+    op = parts[0]
+    ops = [t.strip() for t in re.split(r",\s*", parts[1])] if len(parts) > 1 else []
+    ops = [t.split()[0] if t else t for t in ops]          # drop modifiers such as 'offset:16'
+    return op, ops
+
+
+def kernel_bodies(asm):
+    out, name, body = {}, None, []
+    for line in asm.splitlines():
+        m = re.match(r"^(_Z\w+):", line)
+        if m:
+            name, body = m.group(1), []
+            continue
+        if name:
+            body.append(line)
+            if "s_endpgm" in line:
+                out[name] = body
+                name = None
+    return out
+
+
+def lint(body):
+    """Returns a list of (line number in the kernel, message)."""
+    problems = []
+    recent_valu = []      # (slots ago, registers written, text)
+    recent_mfma = []      # (slots ago, result registers, text)
+    for ln, line in enumerate(body):
+        p = parse(line)
+        if not p:
+            continue
+        op, ops = p
+        slots = 1
+        if op == "s_nop":
+            slots = int(ops[0]) + 1
+        is_mfma = op.startswith("v_mfma")
+        written, read = set(), set()
+        if is_mfma:
+            written = regs(ops[0])
+            for t in ops[1:4]:
+                read |= regs(t)
+        elif op.startswith("v_") and not op.startswith("v_cmp"):
+            written = regs(ops[0]) if ops else set()
+            for t in ops[1:]:
+                read |= regs(t)
+        elif op.startswith(("ds_read", "global_load", "buffer_load", "scratch_load")):
+            written = regs(ops[0]) if ops and not op.startswith("global_load_lds") else set()
+            for t in ops[1:] if written else ops:
+                read |= regs(t)
+        else:
+            for t in ops:
+                read |= regs(t)
+        if is_mfma:
+            for ago, w, text in recent_valu:
+                if ago < VALU_TO_MFMA_SLOTS and w & read:
+                    problems.append((ln, f"MFMA reads a register {ago} slot(s) after '{text}' wrote it: {line.strip()}"))
+        else:
+            for ago, w, text in recent_mfma:
+                if ago < MFMA_RESULT_SLOTS and w & (read | written):
+                    problems.append((ln, f"'{line.strip()}' touches the result of '{text}' {ago} slot(s) after it was issued"))
+        recent_valu = [(a + slots, w, t) for a, w, t in recent_valu if a + slots < 4]
+        recent_mfma = [(a + slots, w, t) for a, w, t in recent_mfma if a + slots < MFMA_RESULT_SLOTS + 2]
+        if is_mfma:
+            recent_mfma.append((0, written, line.strip()))
+        elif op.startswith("v_") and written:
+            recent_valu.append((0, written, line.strip()))
+    return problems
+
+
+@pytest.mark.parametrize("src,extra,pattern", [("attention.hip", ["-fno-honor-nans"], "attention_wide_kernel"),
+                                               ("gemm.hip", [], "gemm4w_kernel")])
+def test_inline_asm_mfma_hazards(src, extra, pattern, tmp_path):
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc is not installed")
+    out = tmp_path / (src + ".s")
+    r = subprocess.run([hipcc] + FLAGS + extra + [os.path.join(CSRC, src), "-o", str(out)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    kernels = {k: v for k, v in kernel_bodies(out.read_text()).items() if pattern in k}
+    assert kernels, f"no kernel named *{pattern}* in {src}"
+    report = []
+    for name, body in sorted(kernels.items()):
+        assert any("v_mfma" in l for l in body), name
+        for ln, msg in lint(body):
+            report.append(f"{name} +{ln}: {msg}")
+    assert not report, "\n".join(report[:40]) + f"\n({len(report)} in all)"
+
+
+def test_the_lint_sees_a_planted_hazard():
+    body = ["\tv_mov_b32_e32 v5, v9", "\tv_mfma_f32_16x16x32_bf16 v[0:3], v[4:7], v[8:11], v[0:3]", "\tv_add_f32_e32 v20, v1, v1",
+            "\ts_nop 7", "\tv_add_f32_e32 v21, v2, v2", "\ts_endpgm"]
+    found = lint(body)
+    assert len(found) == 2 and "MFMA reads" in found[0][1] and "touches the result" in found[1][1]
+    clean = ["\tv_mov_b32_e32 v5, v9", "\ts_nop 1", "\tv_mfma_f32_16x16x32_bf16 v[0:3], v[4:7], v[8:11], v[0:3]", "\ts_nop 7",
+             "\tv_add_f32_e32 v20, v1, v1", "\ts_endpgm"]
+    assert not lint(clean)
