@@ -130,11 +130,13 @@ extern "C" int flux_hip_kv_prepare(void *k_out, void *vt_out, int ld_vt, const v
  *                consecutive keys per lane, and A = V^T fragment is one 16-byte LDS read.
  * --------------------------------------------------------------------------------------- */
 #define ATT_STAGE (64 * 256 + 128 * 128)
+#define ATT_WIDE_LDS (6 * 16384) /* attention_wide_kernel: three K and three V^T slots */
 __device__ __forceinline__ int vt_swz(int d) { return ((d >> 1) & 7) ^ ((d & 1) << 2); }
 #define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
 
 template <bool V> struct AttFlag { static constexpr bool value = V; };
+template <int V> struct AttInt { static constexpr int value = V; };
 
 template <int NW>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf16 *__restrict__ out, int ldo,
@@ -143,7 +145,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
                                                            int seq_q, int seq_k, int heads, int split,
                                                            const float *__restrict__ q_w0, const float *__restrict__ q_w1,
                                                            const float *__restrict__ rope_cos,
-                                                           const float *__restrict__ rope_sin, float eps) {
+                                                           const float *__restrict__ rope_sin, float eps, int *redo) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     /* Workgroups are dealt round-robin to the 8 XCDs, each with its own L2. Give every XCD a
      * contiguous run of (head, query block) pairs, so that all query blocks of a head run on one
@@ -156,6 +158,13 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
     if (logical >= nqb * heads) return;
     const int h = logical / nqb, qb = logical - h * nqb;
     const int tid = threadIdx.x, lane = tid & 63;
+    if (redo) {
+        /* second pass behind attention_wide_kernel: only the query blocks it has marked are computed (again) here */
+        const int marked = redo[h * nqb + qb];
+        __syncthreads();
+        if (!marked) return;
+        if (tid == 0) redo[h * nqb + qb] = 0;
+    }
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l15 = lane & 15, lq = lane >> 4;
     const int H = heads * HD;
@@ -446,7 +455,9 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
  * inside the statement, so nothing can come between them and the MFMA. */
 #define MFMA_NEW_VQ_GUARDED(acc, a, q, c) \
     asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %3" : "=&v"(acc) : "v"(a), "a"(q), "v"(c))
-#define MFMA_ACC_V_ONES_GUARDED(acc, ones, b) asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc) : "a"(ones), "v"(b))
+#define MFMA_ACC_VQ_GUARDED(acc, a, q) asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "a"(q))
+#define MFMA_ACC_A_GUARDED(acc, a, b) asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b))
+#define MFMA_ACC_A_ONES_GUARDED(acc, ones, b) asm volatile("s_nop 1\n\tv_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "a"(ones), "v"(b))
 
 /* Idle cycles until the last MFMAs have written their results, then every listed accumulator passes
  * through an empty asm statement ordered with the MFMAs, so that reads of them stay behind it. */
@@ -467,13 +478,14 @@ __device__ __forceinline__ void mfma_results_fence_a(f32x4 (&acc)[8][N]) {
         for (int j = 0; j < N; j++) asm volatile("" : "+a"(acc[i][j]));
 }
 
+#define WIDE_BIAS 32.0f
 template <int NQ>
 __global__ __launch_bounds__(256, 1) void attention_wide_kernel(bf16 *__restrict__ out, int ldo, const bf16 *__restrict__ q, int ldq,
                                                                 const bf16 *__restrict__ k, const bf16 *__restrict__ vt, int ld_vt,
                                                                 int seq_q, int seq_k, int heads, int split,
                                                                 const float *__restrict__ q_w0, const float *__restrict__ q_w1,
                                                                 const float *__restrict__ rope_cos, const float *__restrict__ rope_sin,
-                                                                float eps) {
+                                                                float eps, int *redo) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     constexpr int NW = 4, WQ = 16 * NQ, BQ = NW * WQ, LP = 16 / NW;
     /* every XCD gets a contiguous run of (head, query block) pairs, as above */
@@ -486,50 +498,50 @@ __global__ __launch_bounds__(256, 1) void attention_wide_kernel(bf16 *__restrict
     const int l15 = lane & 15, lq = lane >> 4;
     const int H = heads * HD;
 
-    /* ---- tile loader: as in attention_kernel<4> ---- */
+    /* ---- tile loader: LDS layout and key permutation as in attention_kernel<4>; the global sources are a
+     * uniform base (scalar arithmetic per tile) plus one 32-bit byte offset per lane and load ---- */
     const int ntiles = (seq_k + 63) >> 6;
-    const bf16 *k_src[LP];
-    const bf16 *v_src[LP];
-    int k_dst[LP], v_dst[LP], k_row[LP];
+    const char *k_base = (const char *)(k + h * HD);
+    const char *v_base = (const char *)(vt + (size_t)h * HD * ld_vt);
+    int k_row[LP];       /* key of the tile that this lane fetches with load i */
+    unsigned v_off[LP];  /* byte offset of this lane's V^T chunk for load i */
+    const unsigned k_chunk = (unsigned)(((lane & 15) ^ ((wave * 4 + (lane >> 4)) & 15)) << 4);
 #pragma unroll
     for (int i = 0; i < LP; i++) {
-        int r = wave * 4 + i * (NW * 4) + (lane >> 4);
-        {
-            int ib = r >> 4, jj = (r >> 2) & 3, ee = r & 3;
-            k_row[i] = 32 * (ib >> 1) + 8 * jj + 4 * (ib & 1) + ee;
-        }
-        k_src[i] = k + h * HD + (((lane & 15) ^ (r & 15)) << 3);
-        k_dst[i] = (wave * 4 + i * (NW * 4)) * 256;
-        int d = wave * 8 + i * (NW * 8) + (lane >> 3);
-        v_src[i] = vt + (size_t)(h * HD + d) * ld_vt + (((lane & 7) ^ vt_swz(d)) << 3);
-        v_dst[i] = (wave * 8 + i * (NW * 8)) * 128;
+        const int r = wave * 4 + i * (NW * 4) + (lane >> 4); /* LDS row; (r & 15) is the same for every i */
+        const int ib = r >> 4, jj = (r >> 2) & 3, ee = r & 3;
+        k_row[i] = 32 * (ib >> 1) + 8 * jj + 4 * (ib & 1) + ee;
+        const int d = wave * 8 + i * (NW * 8) + (lane >> 3);
+        v_off[i] = ((unsigned)d * (unsigned)ld_vt + (unsigned)(((lane & 7) ^ vt_swz(d)) << 3)) * 2u;
     }
-    auto issue_k = [&](int t) {
-        char *base = smem + (t & 1) * (64 * 256);
-        const int key0 = t * 64;
+    /* LDS: three K slots of 16 KB, then three V^T slots of 16 KB; tile x lives in slot x % 3 of its ring.
+     * load i of tile `src` goes into slot `slot` (src is the tile the slot is for, except beyond the last tile,
+     * where the last one is fetched again into a slot nobody reads any more: no branches in the loop) */
+    auto issue_k1 = [&](int slot, int src, int i) {
+        const unsigned off = (unsigned)min(src * 64 + k_row[i], seq_k - 1) * (unsigned)(H * 2) + k_chunk;
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(k_base + off), LDS_PTR(smem + slot * 16384 + (wave * 4 + i * (NW * 4)) * 256), 16, 0, 0);
+    };
+    auto issue_v1 = [&](int slot, int src, int i) {
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(v_base + src * 128 + v_off[i]),
+                                         LDS_PTR(smem + 3 * 16384 + slot * 16384 + (wave * 8 + i * (NW * 8)) * 128), 16, 0, 0);
+    };
+    /* before the loop: K(0), V(0), K(1), V(1), K(2) */
 #pragma unroll
-        for (int i = 0; i < LP; i++) {
-            int r = min(key0 + k_row[i], seq_k - 1);
-            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(k_src[i] + (size_t)r * H), LDS_PTR(base + k_dst[i]), 16, 0, 0);
+    for (int x = 0; x < 3; x++) {
+        const int src = min(x, ntiles - 1);
+#pragma unroll
+        for (int i = 0; i < LP; i++) issue_k1(x, src, i);
+        if (x < 2) {
+#pragma unroll
+            for (int i = 0; i < LP; i++) issue_v1(x, src, i);
         }
-    };
-    auto issue_v = [&](int t) {
-        char *base = smem + 2 * (64 * 256) + (t & 1) * (128 * 128);
-        const int key0 = t * 64;
-#pragma unroll
-        for (int i = 0; i < LP; i++)
-            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(v_src[i] + key0), LDS_PTR(base + v_dst[i]), 16, 0, 0);
-    };
-    issue_k(0);
-    issue_v(0);
+    }
 
     /* ---- Q fragments (B operand) with RMSNorm * weight, RoPE and the softmax scale; they live in AGPRs ---- */
     bf16x8 qf[NQ][4];
-    int qrow[NQ];
 #pragma unroll
     for (int t = 0; t < NQ; t++) {
-        qrow[t] = qb * BQ + wave * WQ + t * 16 + l15;
-        const int qrc = min(qrow[t], seq_q - 1);
+        const int qrc = min(qb * BQ + wave * WQ + t * 16 + l15, seq_q - 1);
         const bf16 *qp = q + (size_t)qrc * ldq + h * HD + lq * 8;
         float x[4][8];
         float ss = 0.0f;
@@ -587,153 +599,246 @@ __global__ __launch_bounds__(256, 1) void attention_wide_kernel(bf16 *__restrict
      * right in front of the MFMA that reads it (the compiler does not know that its inline assembly is an MFMA,
      * which must not read a register in the two issue slots after a vector instruction wrote it) */
     asm volatile("" : "+a"(ones));
-    f32x4 s_acc[4][NQ];
 
-    /* One key tile, as in attention_kernel: S^T = K Q^T - m_run (16 NQ MFMAs), online softmax with the lazily
-     * moved maximum, O^T += V^T P^T (16 NQ MFMAs) and the row sums (2 NQ). */
-    auto step = [&](int t, auto edge_c) {
-        constexpr bool EDGE = decltype(edge_c)::value;
-        __builtin_amdgcn_s_waitcnt(0x0F70);
-        __syncthreads();
-        if (t + 1 < ntiles) {
-            issue_k(t + 1);
-            issue_v(t + 1);
-        }
-        const char *kt = smem + (t & 1) * (64 * 256);
-        const char *vtile = smem + 2 * (64 * 256) + (t & 1) * (128 * 128);
-        auto kread = [&](int kk, bf16x8 (&dst)[4]) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) dst[i] = *(const bf16x8 *)(kt + (i * 16 + l15) * 256 + (((kk * 4 + lq) ^ l15) << 4));
-        };
-        auto vread = [&](int b, bf16x8 (&dst)[4]) {
-#pragma unroll
-            for (int f = 0; f < 4; f++) {
-                const int d = ((b & 1) * 4 + f) * 16 + l15;
-                dst[f] = *(const bf16x8 *)(vtile + d * 128 + (((4 * (b >> 1) + lq) ^ vt_swz(d)) << 4));
-            }
-        };
-        bf16x8 fa[4], fb[4];
-        {
-            kread(0, fa);
-            kread(1, fb);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int kk = 0; kk < 4; kk++) {
-                bf16x8 (&cur)[4] = (kk & 1) ? fb : fa;
-#pragma unroll
-                for (int i = 0; i < 4; i++)
-#pragma unroll
-                    for (int j = 0; j < NQ; j++) {
-                        if (kk == 0 && i == 0) MFMA_NEW_VQ_GUARDED(s_acc[i][j], cur[i], qf[j][0], neg_m[j]); /* first reader of neg_m[j] */
-                        else if (kk == 0) MFMA_NEW_VQ(s_acc[i][j], cur[i], qf[j][0], neg_m[j]);
-                        else MFMA_ACC_VQ(s_acc[i][j], cur[i], qf[j][kk]);
-                    }
-                __builtin_amdgcn_sched_barrier(0);
-                if (kk + 2 < 4) kread(kk + 2, cur);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        vread(0, fa); /* in flight during the softmax */
-        __builtin_amdgcn_sched_barrier(0);
-        mfma_results_fence_v<NQ>(s_acc);
+    /* The loop is software-pipelined inside each wave, because with one wave per SIMD nothing else overlaps the
+     * softmax with the matrix pipe. The unit is a chunk of 32 keys (half a tile): while chunk u is exponentiated
+     * and multiplied into O, the scores of chunk u + 1 are already being computed:
+     *   phase 1: S(u+1) = K Q^T - m   (8 NQ MFMAs)  with  P(u) = 2^S(u) -> bf16 (12 NQ vector instructions)
+     *   phase 2: row sums and O += V^T P(u)^T (9 NQ MFMAs), the requests for the next fragments and loads
+     * Vector instructions sit one or two behind each MFMA; sched_barrier keeps them there. Two score buffers
+     * alternate, so one trip of the loop is one tile: an "even" step (second chunk's scores, first chunk's
+     * product) and an "odd" step (next tile's first chunk's scores, second chunk's product). One barrier per
+     * tile, at the start of the odd step: behind it K(t)'s and V(t-1)'s slots are free and take K(t+3) and
+     * V(t+2); everything read before the next barrier landed before this one (three slots per ring), so
+     * fragments are requested from LDS a phase ahead of their MFMAs, across the barrier too.
+     * The reference maxima are fixed on the first chunk, see first_reference. */
+    f32x4 s_a[2][NQ], s_b[2][NQ];
+    bf16x8 kf[4][2];  /* K fragments of a chunk: [32-dim step of the head dim][key block of the chunk] */
+    bf16x8 vf[2][4];  /* V^T fragments: [half of the head dim][16-row block] */
+    u32x4 pf[NQ];     /* P^T of the chunk as MFMA B fragments (8 bf16), per query block */
 
-        if (EDGE && t == ntiles - 1 && (seq_k & 63)) {
-            const int key0 = t * 64;
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    if (key0 + 32 * (i >> 1) + 8 * lq + 4 * (i & 1) + e >= seq_k) {
-#pragma unroll
-                        for (int j = 0; j < NQ; j++) s_acc[i][j][e] = -1e30f;
-                    }
+    /* Fragments are requested from LDS a whole phase before the MFMAs that read them (the chunk's eight K
+     * fragments during the product phase before, its eight V^T fragments during the score phase before), one
+     * read behind each of the phase's first eight MFMAs: no MFMA waits for LDS. */
+    auto kfrag1 = [&](int slot, int cp, int x) { /* x = 0..7: key block 2cp + x%2 of the tile, head dims 32 (x/2) .. +31 */
+        const int kk = x >> 1, i = x & 1;
+        kf[kk][i] = *(const bf16x8 *)(smem + slot * 16384 + ((2 * cp + i) * 16 + l15) * 256 + (((kk * 4 + lq) ^ l15) << 4));
+    };
+    auto vfrag1 = [&](int slot, int cp, int x) { /* x = 0..7: head-dim block x, keys of 32-key chunk cp */
+        const int d = x * 16 + l15;
+        vf[x >> 2][x & 3] = *(const bf16x8 *)(smem + 3 * 16384 + slot * 16384 + d * 128 + (((4 * cp + lq) ^ vt_swz(d)) << 4));
+    };
+    /* The vector instructions of the loop are inline assembly as well: an ordinary expression the compiler may
+     * sink to its use in the next phase, and then nothing overlaps.
+     * One instruction of the exponentiation of a chunk: k = 0 .. 12 NQ - 1, per query block eight exponentials and
+     * then four conversions of pairs (a conversion reads exponentials issued at least four instructions earlier). */
+    auto exp_op = [&](f32x4 (&sc)[2][NQ], int k) {
+        const int j = k / 12, r = k % 12;
+        if (r < 8) {
+            float x = sc[r >> 2][j][r & 3];
+            asm volatile("v_exp_f32_e32 %0, %0" : "+v"(x));
+            sc[r >> 2][j][r & 3] = x;
+        } else {
+            const int hh = r - 8, i = hh >> 1, e = 2 * (hh & 1);
+            unsigned w;
+            asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(w) : "v"(sc[i][j][e]), "v"(sc[i][j][e + 1]));
+            pf[j][hh] = w;
         }
-        bool grow = EDGE && t == 0;
-        float m_new[NQ];
+    };
+    /* lane-wise maximum of a chunk's scores, one instruction at a time: 4 per query block (three-operand maxima
+     * over the block's 8 values), the query blocks taking turns so that dependent instructions lie NQ apart */
+    float lmax[NQ];
+    auto max_op = [&](f32x4 (&sc)[2][NQ], int k) {
+        const int q4 = k / NQ, j = k % NQ;
+        auto v = [&](int idx) { return sc[idx >> 2][j][idx & 3]; };
+        if (q4 == 0) asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(lmax[j]) : "v"(v(0)), "v"(v(1)), "v"(v(2)));
+        else if (q4 < 3) asm volatile("v_max3_f32 %0, %0, %1, %2" : "+v"(lmax[j]) : "v"(v(2 * q4 + 1)), "v"(v(2 * q4 + 2)));
+        else asm volatile("v_max_f32_e32 %0, %0, %1" : "+v"(lmax[j]) : "v"(v(7)));
+    };
+    /* S = K Q^T - m for one chunk; kf must already hold (or be receiving) the chunk's fragments.
+     * between(m) runs behind MFMA m (m = 0 .. 8 NQ - 1). */
+    /* guard_c: outside the loop, where the register allocator may reconcile its assignments with copies right in
+     * front of an MFMA, every MFMA carries its two idle slots with it */
+    auto s_phase = [&](f32x4 (&sc)[2][NQ], auto &&between, auto guard_c) {
+        constexpr bool GUARD = decltype(guard_c)::value;
 #pragma unroll
-        for (int j = 0; j < NQ; j++) {
-            float mx = fmaxf(fmaxf(s_acc[0][j][0], s_acc[0][j][1]), fmaxf(s_acc[0][j][2], s_acc[0][j][3]));
+        for (int kk = 0; kk < 4; kk++) {
 #pragma unroll
-            for (int i = 1; i < 4; i++) mx = fmaxf(fmaxf(mx, fmaxf(s_acc[i][j][0], s_acc[i][j][1])), fmaxf(s_acc[i][j][2], s_acc[i][j][3]));
-            m_new[j] = mx; /* this lane's keys only; relative to m_run */
-            grow = grow || (mx > 8.0f);
-        }
-        if (__any(grow)) {
-            /* rare: some score lies more than 2^8 above the reference (or this is the first tile). The exact row
-             * maxima (a query's scores sit in lanes l, l^16, l^32, l^48) move the references; see attention_kernel. */
-            if (t > 0) mfma_results_fence_a<NQ>(o_acc);
+            for (int i = 0; i < 2; i++)
 #pragma unroll
-            for (int j = 0; j < NQ; j++) {
-                float mx = m_new[j];
-                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                const bool first = EDGE && t == 0;
-                const float d = first ? mx : fmaxf(mx, 0.0f);
-                const float alpha = first ? 1.0f : fast_exp2(-d);
-#pragma unroll
-                for (int e = 0; e < 4; e++) { neg_m[j][e] -= d; l_acc[j][e] *= alpha; }
-#pragma unroll
-                for (int i = 0; i < 4; i++)
-#pragma unroll
-                    for (int e = 0; e < 4; e++) s_acc[i][j][e] -= d;
-#pragma unroll
-                for (int i = 0; i < 8; i++)
-#pragma unroll
-                    for (int e = 0; e < 4; e++) o_acc[i][j][e] *= alpha;
-            }
-        }
-        bf16x8 pf[2][NQ];
-#pragma unroll
-        for (int j = 0; j < NQ; j++) {
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) s_acc[i][j][e] = fast_exp2(s_acc[i][j][e]);
-#pragma unroll
-            for (int c = 0; c < 2; c++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    pf[c][j][e] = (bf16)s_acc[2 * c][j][e];
-                    pf[c][j][4 + e] = (bf16)s_acc[2 * c + 1][j][e];
+                for (int j = 0; j < NQ; j++) {
+                    if (kk == 0 && (i == 0 || GUARD)) MFMA_NEW_VQ_GUARDED(sc[i][j], kf[0][i], qf[j][0], neg_m[j]); /* first reader of neg_m[j] */
+                    else if (kk == 0) MFMA_NEW_VQ(sc[i][j], kf[0][i], qf[j][0], neg_m[j]);
+                    else if (GUARD) MFMA_ACC_VQ_GUARDED(sc[i][j], kf[kk][i], qf[j][kk]);
+                    else MFMA_ACC_VQ(sc[i][j], kf[kk][i], qf[j][kk]);
+                    between((kk * 2 + i) * NQ + j);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
         }
-        __builtin_amdgcn_sched_barrier(0);
+    };
+    /* row sums and O^T += V^T P^T for one chunk; vf[0] and vf[1] must already hold (or be receiving) the chunk's
+     * fragments. between(m) runs behind PV MFMA m (m = 0 .. 8 NQ - 1). */
+    auto pv_phase = [&](auto &&between, auto guard_c) {
+        constexpr bool GUARD = decltype(guard_c)::value;
         /* the row sums are the first readers of each probability fragment */
 #pragma unroll
-        for (int j = 0; j < NQ; j++) MFMA_ACC_V_ONES_GUARDED(l_acc[j], ones, pf[0][j]);
-        __builtin_amdgcn_sched_barrier(0);
-        vread(1, fb);
+        for (int j = 0; j < NQ; j++) MFMA_ACC_A_ONES_GUARDED(l_acc[j], ones, pf[j]);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
-            bf16x8 (&cur)[4] = (b & 1) ? fb : fa;
-            if (b == 2) {
-#pragma unroll
-                for (int j = 0; j < NQ; j++) MFMA_ACC_V_ONES_GUARDED(l_acc[j], ones, pf[1][j]);
-            }
+        for (int g = 0; g < 2; g++)
 #pragma unroll
             for (int f = 0; f < 4; f++)
 #pragma unroll
-                for (int j = 0; j < NQ; j++) MFMA_ACC_A(o_acc[(b & 1) * 4 + f][j], cur[f], pf[b >> 1][j]);
-            __builtin_amdgcn_sched_barrier(0);
-            if (b + 2 < 4) vread(b + 2, cur);
-            __builtin_amdgcn_sched_barrier(0);
+                for (int j = 0; j < NQ; j++) {
+                    if (GUARD) MFMA_ACC_A_GUARDED(o_acc[g * 4 + f][j], vf[g][f], pf[j]);
+                    else MFMA_ACC_A(o_acc[g * 4 + f][j], vf[g][f], pf[j]);
+                    between((g * 4 + f) * NQ + j);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+    };
+    auto fence_scores = [&](f32x4 (&sc)[2][NQ]) {
+        asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < NQ; j++) asm volatile("" : "+v"(sc[i][j]));
+    };
+    auto mask_chunk = [&](f32x4 (&sc)[2][NQ], int u) { /* keys of chunk u beyond seq_k (chunks of the last tile only) */
+        if ((u + 1) * 32 <= seq_k) return;
+        fence_scores(sc);
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (u * 32 + 8 * lq + 4 * i + e >= seq_k) {
+#pragma unroll
+                    for (int j = 0; j < NQ; j++) sc[i][j][e] = -1e30f;
+                }
+    };
+    /* The references of the online softmax are set once, from the first chunk: its exact row maxima (a query's
+     * scores sit in lanes l, l^16, l^32, l^48) plus WIDE_BIAS. Probabilities then start near 2^-WIDE_BIAS, and a
+     * later score may exceed the first chunk's maximum by more than 100 base-2 logits (a factor of 2^100 between
+     * probabilities of one row) before anything leaves the range of fp32. The loop never looks at the scores'
+     * size again and never moves the references: maxima cost a vector instruction per two scores, and rescaling
+     * O with vector instructions inside the loop makes the register allocator carry O through VGPRs on every
+     * trip. Should a row overflow all the same, its sums show it at the end: the wave then marks its query blocks
+     * in `redo` instead of writing output, and attention_kernel<4>, launched behind this kernel, computes the
+     * marked blocks with its moving references. */
+    auto first_reference = [&](f32x4 (&sc)[2][NQ]) {
+#pragma unroll
+        for (int j = 0; j < NQ; j++) {
+            float mx = lmax[j];
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float d = mx + WIDE_BIAS;
+#pragma unroll
+            for (int e = 0; e < 4; e++) neg_m[j][e] = -d;
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) sc[i][j][e] -= d;
         }
     };
+    auto nothing = [](int) {};
+    /* ---- first chunk, not pipelined: S(0) and its exact maxima ---- */
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads(); /* K(0), V(0), K(1), V(1), K(2) are in LDS */
+#pragma unroll
+    for (int x = 0; x < 8; x++) kfrag1(0, 0, x);
+    s_phase(s_a, nothing, AttFlag<true>{});
+    fence_scores(s_a);
+    mask_chunk(s_a, 0);
+#pragma unroll
+    for (int k = 0; k < 4 * NQ; k++) max_op(s_a, k);
+    first_reference(s_a);
+#pragma unroll
+    for (int x = 0; x < 8; x++) kfrag1(0, 1, x);
 
-    step(0, AttFlag<true>{});
-    for (int t = 1; t < ntiles - 1; t++) step(t, AttFlag<false>{});
-    if (ntiles > 1) step(ntiles - 1, AttFlag<true>{});
+    /* Even step of tile t (slot sl = t % 3): scores of its second chunk into s_b, product of its first chunk.
+     * The first K fragments of the odd step's chunk (first chunk of tile t + 1, slot sn) are requested meanwhile. */
+    auto even_step = [&](int t, int sl, int sn, auto guard_c) {
+        s_phase(s_b, [&](int m) {
+            if (m < 8) vfrag1(sl, 0, m);
+#pragma unroll
+            for (int k = (m * 3) / 2; k < ((m + 1) * 3) / 2; k++) exp_op(s_a, k);
+        }, guard_c);
+        mask_chunk(s_b, 2 * t + 1);
+        pv_phase([&](int m) {
+            if (m < 8 && t + 1 < ntiles) kfrag1(sn, 0, m);
+        }, guard_c);
+    };
+    /* Odd step of tile t: the barrier, the loads of K(t+3) and V(t+2), scores of tile t+1's first chunk into s_a,
+     * product of tile t's second chunk. sp = (t + 2) % 3 is the slot V(t+2) goes to. */
+    auto odd_step = [&](int t, int sl, int sn, int sp) {
+        __builtin_amdgcn_s_waitcnt(0x0F70); /* this wave's parts of K(t+2) and V(t+1) are in LDS */
+        __syncthreads();
+        s_phase(s_a, [&](int m) {
+            if (m < 8) vfrag1(sl, 1, m);
+#pragma unroll
+            for (int k = (m * 3) / 2; k < ((m + 1) * 3) / 2; k++) exp_op(s_b, k);
+        }, AttFlag<false>{});
+        mask_chunk(s_a, 2 * t + 2);
+        pv_phase([&](int m) {
+            if (m < 8) kfrag1(sn, 1, m);
+            if (m >= 8 * NQ - 2 * LP) { /* the tile's eight loads behind the last eight MFMAs */
+                const int i = m - (8 * NQ - 2 * LP);
+                if (i & 1) issue_v1(sp, min(t + 2, ntiles - 1), i >> 1);
+                else issue_k1(sl, min(t + 3, ntiles - 1), i >> 1);
+            }
+        }, AttFlag<false>{});
+    };
+    /* the last chunk: nothing left to overlap */
+    auto last_step = [&](int sl) {
+#pragma unroll
+        for (int x = 0; x < 8; x++) vfrag1(sl, 1, x);
+#pragma unroll
+        for (int k = 0; k < 12 * NQ; k++) exp_op(s_b, k);
+        __builtin_amdgcn_sched_barrier(0);
+        pv_phase(nothing, AttFlag<true>{});
+    };
+    {
+        int sl = 0, sn = 1, sp = 2; /* slots of tiles t, t + 1, t + 2 */
+        for (int t = 0; t < ntiles - 1; t++) {
+            even_step(t, sl, sn, AttFlag<false>{});
+            odd_step(t, sl, sn, sp);
+            const int r = sl; sl = sn; sn = sp; sp = r;
+        }
+        even_step(ntiles - 1, sl, sn, AttFlag<true>{});
+        last_step(sl);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70); /* no load into LDS is left in flight */
 
     mfma_results_fence_a<NQ>(o_acc);
     asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
 #pragma unroll
-    for (int j = 0; j < NQ; j++) asm volatile("" : "+v"(l_acc[j]));
+    for (int j = 0; j < NQ; j++) asm volatile("" : "+a"(l_acc[j]));
+    /* Did a score come within reach of fp32 overflow (see first_reference)? Then a row sum or an accumulator is
+     * infinite, not a number, or beyond 2^100: tested on the exponent bits (this file is compiled to assume that
+     * there are no NaNs, so a floating-point comparison would not do). */
+    unsigned worst = 0;
+#pragma unroll
+    for (int j = 0; j < NQ; j++) {
+        worst = max(worst, __float_as_uint(l_acc[j][0]) & 0x7fffffffu);
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) worst = max(worst, __float_as_uint(o_acc[i][j][e]) & 0x7fffffffu);
+    }
+    if (__any(worst >= 0x71800000u)) {
+        /* attention_kernel<4> works on blocks of 128 queries: mark those this wave's queries lie in */
+        const int q0 = qb * BQ + wave * WQ, q1 = min(q0 + WQ, seq_q) - 1;
+        if (lane == 0 && q0 < seq_q) {
+            const int nqb128 = (seq_q + 127) >> 7;
+            for (int b128 = q0 >> 7; b128 <= q1 >> 7; b128++) redo[h * nqb128 + b128] = 1;
+        }
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < NQ; j++) {
         const float inv_l = 1.0f / l_acc[j][0];
-        if (qrow[j] < seq_q) {
-            bf16 *op = out + (size_t)qrow[j] * ldo + h * HD + lq * 4;
+        const int qr = qb * BQ + wave * WQ + j * 16 + l15;
+        if (qr < seq_q) {
+            bf16 *op = out + (size_t)qr * ldo + h * HD + lq * 4;
 #pragma unroll
             for (int dt = 0; dt < 8; dt++) {
                 bf16x4 r;
@@ -743,6 +848,22 @@ __global__ __launch_bounds__(256, 1) void attention_wide_kernel(bf16 *__restrict
             }
         }
     }
+}
+
+/* Marks of attention_wide_kernel for the second pass, one per (head, block of 128 queries); all zero between
+ * calls (the second pass clears what it finds). A static device array: attention allocates nothing. */
+#define ATT_REDO_MAX (1 << 16)
+static __device__ int g_att_redo[ATT_REDO_MAX];
+static int *g_att_redo_ptr[64];
+static int *att_redo_for_current_device() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    if (!g_att_redo_ptr[dev]) {
+        int *p = nullptr;
+        if (hipGetSymbolAddress((void **)&p, HIP_SYMBOL(g_att_redo)) != hipSuccess) return nullptr;
+        g_att_redo_ptr[dev] = p;
+    }
+    return g_att_redo_ptr[dev];
 }
 
 static int g_att_force = -1;
@@ -760,15 +881,22 @@ extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ld
         return flux_hip_fail("flux_hip_attention: operands must be 16-byte aligned (output 8-byte)");
     if ((ldo & 3) || (ldq & 7) || (ld_vt & 7) || ld_vt < (seq_k + 63) / 64 * 64)
         return flux_hip_fail("flux_hip_attention: bad leading dimensions (ldo=%d ldq=%d ld_vt=%d)", ldo, ldq, ld_vt);
-    /* 256-query workgroups (8 waves) share each K / V^T tile among twice as many queries;
-     * 128-query workgroups (two per CU) balance better when there are few of them. */
-    const int big = g_att_force >= 0 ? g_att_force : (((seq_q + 255) / 256) * heads >= 256);
+    /* Variants: 0 / 1 = attention_kernel with 128 / 256 queries per workgroup, 11 .. 14 = attention_wide_kernel with
+     * 16 NQ queries per wave (NQ = 1 .. 4; 64 NQ queries per workgroup, one workgroup per compute unit). Default: the
+     * widest wave that still gives about 0.7 workgroups per compute unit (measured at 24 heads: 4608 and 2560
+     * tokens NQ = 4, 1536 tokens NQ = 3, 768 and fewer NQ = 1). */
+    int big = g_att_force;
+    if (big < 0) {
+        int nq = 4;
+        while (nq > 1 && ((seq_q + 64 * nq - 1) / (64 * nq)) * heads < 180) nq--;
+        big = 10 + nq;
+    }
     static bool attr_done = false;
     if (!attr_done) {
-        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
-        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
-        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<3>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
-        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
+        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, ATT_WIDE_LDS));
+        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, ATT_WIDE_LDS));
+        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<3>, hipFuncAttributeMaxDynamicSharedMemorySize, ATT_WIDE_LDS));
+        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, ATT_WIDE_LDS));
         HIP_OK(hipFuncSetAttribute((const void *)attention_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
         HIP_OK(hipFuncSetAttribute((const void *)attention_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
         attr_done = true;
@@ -776,21 +904,27 @@ extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ld
     if (big >= 11 && big <= 14) {
         /* 16 NQ queries per wave, four waves per workgroup (variants 11 .. 14 = NQ 1 .. 4) */
         const int nq = big - 10, bq = 64 * nq;
-        const int blocks = ((seq_q + bq - 1) / bq) * heads;
+        const int blocks = ((seq_q + bq - 1) / bq) * heads, blocks128 = ((seq_q + 127) / 128) * heads;
+        int *redo = att_redo_for_current_device();
+        if (!redo || blocks128 > ATT_REDO_MAX) return flux_hip_fail("flux_hip_attention: no room for the second-pass marks");
         auto kern = nq == 1 ? attention_wide_kernel<1> : nq == 2 ? attention_wide_kernel<2> : nq == 3 ? attention_wide_kernel<3> : attention_wide_kernel<4>;
-        hipLaunchKernelGGL(kern, dim3((blocks + 7) & ~7), dim3(256), 2 * ATT_STAGE, flux_hip_stream_handle(),
+        hipLaunchKernelGGL(kern, dim3((blocks + 7) & ~7), dim3(256), ATT_WIDE_LDS, flux_hip_stream_handle(),
                            (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,
-                           heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps);
+                           heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps, redo);
+        /* second pass: the blocks of 128 queries the first one marked (normally none: every workgroup leaves at once) */
+        hipLaunchKernelGGL(attention_kernel<4>, dim3((blocks128 + 7) & ~7), dim3(256), 2 * ATT_STAGE, flux_hip_stream_handle(),
+                           (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,
+                           heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps, redo);
     } else if (big) {
         const int blocks = ((seq_q + 255) / 256) * heads;
         hipLaunchKernelGGL(attention_kernel<8>, dim3((blocks + 7) & ~7), dim3(512), 2 * ATT_STAGE, flux_hip_stream_handle(),
                            (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,
-                           heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps);
+                           heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps, (int *)nullptr);
     } else {
         const int blocks = ((seq_q + 127) / 128) * heads;
         hipLaunchKernelGGL(attention_kernel<4>, dim3((blocks + 7) & ~7), dim3(256), 2 * ATT_STAGE, flux_hip_stream_handle(),
                            (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,
-                           heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps);
+                           heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps, (int *)nullptr);
     }
     HIP_OK(hipGetLastError());
     return 1;

@@ -5,7 +5,9 @@ file they were put in. The compiler does not know that those statements are matr
 the idle cycles the hardware wants around them nor keeps its own register copies away from them:
   * a vector instruction that writes a register an MFMA reads needs two issue slots in between;
   * a vector, LDS or memory instruction that touches an MFMA's result register needs the MFMA to have finished
-    (passes + 4 issue slots for this 4-pass instruction; the kernels place sixteen idle cycles, and this test asks for 8).
+    (passes + 4 issue slots for this 4-pass instruction; the kernels place sixteen idle cycles, and this test asks for 8);
+  * the attention kernel also writes its exponentials as inline assembly: a transcendental's result must not be read
+    by the very next instruction.
 The kernels keep these apart by construction; this test compiles the files the way the Makefile does and checks every
 MFMA in the inline-assembly kernels, so that a register copy the allocator slips in front of an MFMA fails here
 instead of giving wrong numbers on the GPU. Instructions are taken in layout order (branches are not followed), which
@@ -24,6 +26,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-featu
          "--cuda-device-only", "-S"]
 
 VALU_TO_MFMA_SLOTS = 2
+TRANS = ("v_exp_", "v_log_", "v_rcp_", "v_rsq_", "v_sqrt_", "v_sin_", "v_cos_")
 MFMA_RESULT_SLOTS = 8
 
 
@@ -94,6 +97,9 @@ def lint(body):
         else:
             for t in ops:
                 read |= regs(t)
+        for ago, w, text in recent_valu:
+            if ago == 0 and text.startswith(TRANS) and w & read:
+                problems.append((ln, f"'{line.strip()}' reads the result of '{text}' in the next slot"))
         if is_mfma:
             for ago, w, text in recent_valu:
                 if ago < VALU_TO_MFMA_SLOTS and w & read:
@@ -135,6 +141,8 @@ def test_the_lint_sees_a_planted_hazard():
             "\ts_nop 7", "\tv_add_f32_e32 v21, v2, v2", "\ts_endpgm"]
     found = lint(body)
     assert len(found) == 2 and "MFMA reads" in found[0][1] and "touches the result" in found[1][1]
+    assert len(lint(["\tv_exp_f32_e32 v1, v1", "\tv_cvt_pk_bf16_f32 v2, v1, v3", "\ts_endpgm"])) == 1
+    assert not lint(["\tv_exp_f32_e32 v1, v1", "\tv_exp_f32_e32 v3, v3", "\tv_cvt_pk_bf16_f32 v2, v1, v4", "\ts_endpgm"])
     clean = ["\tv_mov_b32_e32 v5, v9", "\ts_nop 1", "\tv_mfma_f32_16x16x32_bf16 v[0:3], v[4:7], v[8:11], v[0:3]", "\ts_nop 7",
              "\tv_add_f32_e32 v20, v1, v1", "\ts_endpgm"]
     assert not lint(clean)
