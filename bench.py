@@ -18,6 +18,8 @@ Also measured in the same run:
 one VAE decode of a 16/32/64-wide latent to a 256/512/1024-pixel image; vae_enc_c2 | vae_enc_c3 |
 vae_enc_c4 the VAE encoder on a picture of those sizes (the input of image-to-image generation).
 --workload qwen3 measures the step before the loop: one forward of the text encoder over 512 tokens.
+--workload att_c2 | att_c3 | att_c4 | att_c5 measures the attention operator alone (K/V preparation + attention) at
+that workload's sequence length.
 --workload mfma_peak measures no part of the model: what the matrix pipes sustain on their own (the measured
 peak beside the datasheet's 2.5 PFLOP/s).
 """
@@ -294,6 +296,74 @@ def bench_qwen3(args):
         "tflops": round(flops * K / wall / 1e12, 1), "flops_per_step": flops, "roofline": roof, "cpu_baseline": cpu}))
 
 
+ATT_WORKLOADS = {"att_c2": 768, "att_c3": 1536, "att_c4": 4608, "att_c5": 2560}
+
+
+def bench_attention(args):
+    """The attention operator alone at a workload's sequence length (24 heads of 128, text split at 512): one "step"
+    is one flux_hip_kv_prepare + flux_hip_attention pair, back to back on resident buffers, as a single-stream
+    block runs them. The roofline object is the attention kernel by itself (HIP events around runs of it)."""
+    n, heads = ATT_WORKLOADS[args.workload], KLEIN_4B.heads
+    H = heads * 128
+    fluxhip.init()
+    L = fluxhip.lib()
+    L.flux_hip_attention_force_variant(args.attention_variant)
+    qkv = fluxhip.DevBuf.from_array(normal_bf16((n, 3 * H), 5, 1))
+    w = fluxhip.DevBuf.from_array(np.ones(128, np.float32))
+    ang = normal_f32((n, 128), 5, 2)
+    cos, sin = fluxhip.DevBuf.from_array(np.cos(ang)), fluxhip.DevBuf.from_array(np.sin(ang))
+    ldvt = (n + 63) // 64 * 64
+    kn, vt, out = fluxhip.DevBuf(n * H * 2), fluxhip.DevBuf(H * ldvt * 2), fluxhip.DevBuf(n * H * 2)
+
+    def prep():
+        fluxhip.check(L.flux_hip_kv_prepare(kn.ptr, vt.ptr, ldvt, qkv.ptr, 3 * H, H, 2 * H, n, heads, 512, w.ptr, w.ptr, cos.ptr, sin.ptr, 1e-6))
+
+    def att():
+        fluxhip.check(L.flux_hip_attention(out.ptr, H, qkv.ptr, 3 * H, kn.ptr, vt.ptr, ldvt, n, n, heads, 512, w.ptr, w.ptr, cos.ptr, sin.ptr, 1e-6))
+
+    for _ in range(max(args.warmup, 1)):
+        prep(); att()
+    fluxhip.sync()
+    t0 = time.perf_counter()
+    L.flux_hip_timer_start()
+    for _ in range(args.steps):
+        prep(); att()
+    ev_ms = L.flux_hip_timer_stop()
+    wall = time.perf_counter() - t0
+    L.flux_hip_timer_start()
+    for _ in range(args.steps):
+        att()
+    att_ms = L.flux_hip_timer_stop() / args.steps
+    L.flux_hip_timer_start()
+    for _ in range(args.steps):
+        prep()
+    prep_ms = L.flux_hip_timer_stop() / args.steps
+    res = bf16_to_f32_host(out.to_array(np.uint16, (n, H)))
+    assert np.isfinite(res).all()
+    flops = 4.0 * n * n * H
+    ach = flops / (att_ms * 1e-3) / 1e12
+    prep_bytes = 4.0 * n * H * 2
+    L.flux_hip_attention_force_variant(-1)
+    print(json.dumps({
+        "metric": f"attention calls/s ({n} tokens, {heads} heads, 1 GPU)", "value": round(args.steps / wall, 2), "unit": "calls/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1000.0 / args.steps, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: K/V preparation + joint attention over {n} tokens (512 text), {heads} heads x 128, N(0,1) bf16 "
+                               f"q/k/v, unit QK-norm weights, random RoPE angles; variant {args.attention_variant}"},
+        "device_ms_per_step_events": round(ev_ms / args.steps, 4),
+        "roofline": {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4),
+                     "traffic": None, "kernel": "attention_wide_kernel (+ its empty second pass): softmax(q k^T / sqrt(128)) v, 4 n^2 H FLOP",
+                     "ms_per_launch": round(att_ms, 4), "flops_per_launch": flops},
+        "kv_prepare": {"bound": "hbm", "ms_per_launch": round(prep_ms, 4), "bytes_per_launch": prep_bytes,
+                       "achieved_GBps": round(prep_bytes / (prep_ms * 1e-3) / 1e9, 1), "peak_GBps": 8000.0,
+                       "frac": round(prep_bytes / (prep_ms * 1e-3) / 8e12, 4)},
+        "cpu_baseline": None}))
+
+
+def bf16_to_f32_host(a):
+    return (a.astype(np.uint32) << 16).view(np.float32)
+
+
 def bench_mfma_peak(args):
     """The matrix pipes on their own (flux_hip_mfma_peak: register-resident loops of independent bf16 MFMAs on every
     compute unit, no memory traffic), for both instruction shapes, one and two waves per SIMD, and operand data of
@@ -333,7 +403,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=8)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + sorted(VAE_WORKLOADS) + ["qwen3", "mfma_peak"])
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + sorted(VAE_WORKLOADS) + sorted(ATT_WORKLOADS) + ["qwen3", "mfma_peak"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     ap.add_argument("--tile-mask", type=lambda v: int(v, 0), default=0,
@@ -342,6 +412,8 @@ def main():
                     help="run the two forwards of a CFG step one after the other instead of as one batch (A/B runs)")
     ap.add_argument("--fused-qkv-mlp", type=int, default=1, choices=[0, 1],
                     help="single-stream blocks: 1 = QKV and gate/up projections as one launch (default), 0 = as two (A/B runs)")
+    ap.add_argument("--attention-variant", type=int, default=-1,
+                    help="attention kernel variant (flux_hip_attention_force_variant; -1 = the backend's choice), for A/B runs")
     ap.add_argument("--calibrate", action="store_true",
                     help="launch only a streaming kernel of known size (f32->bf16 over 64 Mi elements: reads 256 MiB, "
                          "writes 128 MiB) and the dominant GEMM, for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs")
@@ -357,6 +429,8 @@ def main():
         return bench_qwen3(args)
     if args.workload == "mfma_peak":
         return bench_mfma_peak(args)
+    if args.workload in ATT_WORKLOADS:
+        return bench_attention(args)
     cfg = KLEIN_4B
     wl = WORKLOADS[args.workload]
     if args.calibrate:
@@ -385,6 +459,7 @@ def main():
     if args.sequential_cfg:
         fluxhip.lib().flux_hip_set_batched_cfg(0)
     fluxhip.lib().flux_hip_set_fused_qkv_mlp(args.fused_qkv_mlp)
+    fluxhip.lib().flux_hip_attention_force_variant(args.attention_variant)
     model = load_model(cfg)
     z = normal_f32((cfg.channels, h, w), 123, 1)
     txt = normal_f32((nt, cfg.text_dim), 123, 2)

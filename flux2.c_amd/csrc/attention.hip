@@ -479,20 +479,15 @@ __device__ __forceinline__ void mfma_results_fence_a(f32x4 (&acc)[8][N]) {
 }
 
 #define WIDE_BIAS 32.0f
+/* One workgroup's work: the 64 NQ queries from q0 on of head h. */
 template <int NQ>
-__global__ __launch_bounds__(256, 1) void attention_wide_kernel(bf16 *__restrict__ out, int ldo, const bf16 *__restrict__ q, int ldq,
-                                                                const bf16 *__restrict__ k, const bf16 *__restrict__ vt, int ld_vt,
-                                                                int seq_q, int seq_k, int heads, int split,
-                                                                const float *__restrict__ q_w0, const float *__restrict__ q_w1,
-                                                                const float *__restrict__ rope_cos, const float *__restrict__ rope_sin,
-                                                                float eps, int *redo) {
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-    constexpr int NW = 4, WQ = 16 * NQ, BQ = NW * WQ, LP = 16 / NW;
-    /* every XCD gets a contiguous run of (head, query block) pairs, as above */
-    const int nqb = (seq_q + BQ - 1) / BQ;
-    const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-    if (logical >= nqb * heads) return;
-    const int h = logical / nqb, qb = logical - h * nqb;
+__device__ __forceinline__ void attention_wide_body(char *smem, const int h, const int q0, bf16 *__restrict__ out, int ldo,
+                                                    const bf16 *__restrict__ q, int ldq, const bf16 *__restrict__ k,
+                                                    const bf16 *__restrict__ vt, int ld_vt, int seq_q, int seq_k, int heads, int split,
+                                                    const float *__restrict__ q_w0, const float *__restrict__ q_w1,
+                                                    const float *__restrict__ rope_cos, const float *__restrict__ rope_sin, float eps,
+                                                    int *redo) {
+    constexpr int NW = 4, WQ = 16 * NQ, LP = 16 / NW;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l15 = lane & 15, lq = lane >> 4;
@@ -541,7 +536,7 @@ __global__ __launch_bounds__(256, 1) void attention_wide_kernel(bf16 *__restrict
     bf16x8 qf[NQ][4];
 #pragma unroll
     for (int t = 0; t < NQ; t++) {
-        const int qrc = min(qb * BQ + wave * WQ + t * 16 + l15, seq_q - 1);
+        const int qrc = min(q0 + wave * WQ + t * 16 + l15, seq_q - 1);
         const bf16 *qp = q + (size_t)qrc * ldq + h * HD + lq * 8;
         float x[4][8];
         float ss = 0.0f;
@@ -826,17 +821,17 @@ __global__ __launch_bounds__(256, 1) void attention_wide_kernel(bf16 *__restrict
     }
     if (__any(worst >= 0x71800000u)) {
         /* attention_kernel<4> works on blocks of 128 queries: mark those this wave's queries lie in */
-        const int q0 = qb * BQ + wave * WQ, q1 = min(q0 + WQ, seq_q) - 1;
-        if (lane == 0 && q0 < seq_q) {
+        const int qw0 = q0 + wave * WQ, qw1 = min(qw0 + WQ, seq_q) - 1;
+        if (lane == 0 && qw0 < seq_q) {
             const int nqb128 = (seq_q + 127) >> 7;
-            for (int b128 = q0 >> 7; b128 <= q1 >> 7; b128++) redo[h * nqb128 + b128] = 1;
+            for (int b128 = qw0 >> 7; b128 <= qw1 >> 7; b128++) redo[h * nqb128 + b128] = 1;
         }
         return;
     }
 #pragma unroll
     for (int j = 0; j < NQ; j++) {
         const float inv_l = 1.0f / l_acc[j][0];
-        const int qr = qb * BQ + wave * WQ + j * 16 + l15;
+        const int qr = q0 + wave * WQ + j * 16 + l15;
         if (qr < seq_q) {
             bf16 *op = out + (size_t)qr * ldo + h * HD + lq * 4;
 #pragma unroll
@@ -847,6 +842,33 @@ __global__ __launch_bounds__(256, 1) void attention_wide_kernel(bf16 *__restrict
                 *(bf16x4 *)(op + dt * 16) = r;
             }
         }
+    }
+}
+
+/* The launch: every head's queries are cut into na blocks of 64 NQA queries followed by nb blocks of 64 NQB
+ * (NQB = NQA - 1): a launch whose workgroups are all alike leaves compute units idle in its last round (18 blocks
+ * of 256 queries per head, 24 heads: 432 workgroups, 1.69 rounds over 256 units, paid as 2), and with shorter
+ * blocks at the end the last round is a short one. Each XCD takes a contiguous run of heads, so that a head's K and
+ * V^T are fetched into one L2 only, and within its run the long blocks of all its heads come first (workgroups are
+ * dealt to the XCDs round-robin and started in order). */
+template <int NQA, int NQB>
+__global__ __launch_bounds__(256, 1) void attention_wide_kernel(bf16 *__restrict__ out, int ldo, const bf16 *__restrict__ q, int ldq,
+                                                                const bf16 *__restrict__ k, const bf16 *__restrict__ vt, int ld_vt,
+                                                                int seq_q, int seq_k, int heads, int split,
+                                                                const float *__restrict__ q_w0, const float *__restrict__ q_w1,
+                                                                const float *__restrict__ rope_cos, const float *__restrict__ rope_sin,
+                                                                float eps, int *redo, int na, int nb) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int xcd = blockIdx.x & 7, hx0 = xcd * heads / 8, nh = (xcd + 1) * heads / 8 - hx0;
+    int item = blockIdx.x >> 3;
+    if (item >= nh * (na + nb)) return;
+    if (item < nh * na) {
+        attention_wide_body<NQA>(smem, hx0 + item / na, (item % na) * 64 * NQA, out, ldo, q, ldq, k, vt, ld_vt, seq_q, seq_k, heads, split,
+                                 q_w0, q_w1, rope_cos, rope_sin, eps, redo);
+    } else {
+        item -= nh * na;
+        attention_wide_body<NQB>(smem, hx0 + item / nb, na * 64 * NQA + (item % nb) * 64 * NQB, out, ldo, q, ldq, k, vt, ld_vt, seq_q,
+                                 seq_k, heads, split, q_w0, q_w1, rope_cos, rope_sin, eps, redo);
     }
 }
 
@@ -866,6 +888,46 @@ static int *att_redo_for_current_device() {
     return g_att_redo_ptr[dev];
 }
 
+/* How a head's queries are cut into blocks: na blocks of 64 nqa queries, then nb blocks of 64 (nqa - 1). The choice
+ * minimises the time of the slowest XCD under a simple model: an XCD's compute units (one workgroup each at a
+ * time) take its blocks in order, and a block of 64 NQ queries costs cost[NQ] (relative times of one workgroup
+ * measured at 4608 keys: the per-tile work that does not depend on NQ - loads, barrier, fragment reads - makes short
+ * blocks dearer per query). */
+struct WidePlan { int nqa, na, nb; };
+static WidePlan wide_plan(int seq_q, int heads) {
+    static int c_seq = -1, c_heads = -1;
+    static WidePlan c_plan;
+    if (seq_q == c_seq && heads == c_heads) return c_plan;
+    static const double cost[5] = {0.0, 0.43, 0.54, 0.70, 1.0};
+    int cus = 256, dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 8) cus = 256;
+    const int per_xcd = cus / 8, nh = (heads + 7) / 8;
+    WidePlan best = {2, 0, (seq_q + 63) / 64};
+    double best_t = 1e30;
+    for (int nqa = 4; nqa >= 2; nqa--) {
+        const int la = 64 * nqa, lb = 64 * (nqa - 1);
+        for (int na = (seq_q + la - 1) / la; na >= 0; na--) {
+            const int rest = seq_q - na * la, nb = rest > 0 ? (rest + lb - 1) / lb : 0;
+            /* list scheduling of nh * na long blocks, then nh * nb short ones, on per_xcd units */
+            double busy[64];
+            const int units = per_xcd < 64 ? per_xcd : 64;
+            for (int u = 0; u < units; u++) busy[u] = 0.0;
+            for (int i = 0; i < nh * (na + nb); i++) {
+                int u0 = 0;
+                for (int u = 1; u < units; u++)
+                    if (busy[u] < busy[u0]) u0 = u;
+                busy[u0] += i < nh * na ? cost[nqa] : cost[nqa - 1];
+            }
+            double t = 0.0;
+            for (int u = 0; u < units; u++) t = busy[u] > t ? busy[u] : t;
+            t += 1e-4 * nh * (na + nb); /* ties: fewer workgroups */
+            if (t < best_t) { best_t = t; best = {nqa, na, nb}; }
+        }
+    }
+    c_seq = seq_q; c_heads = heads; c_plan = best;
+    return best;
+}
+
 static int g_att_force = -1;
 extern "C" void flux_hip_attention_force_variant(int v) { g_att_force = v; }
 
@@ -881,51 +943,49 @@ extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ld
         return flux_hip_fail("flux_hip_attention: operands must be 16-byte aligned (output 8-byte)");
     if ((ldo & 3) || (ldq & 7) || (ld_vt & 7) || ld_vt < (seq_k + 63) / 64 * 64)
         return flux_hip_fail("flux_hip_attention: bad leading dimensions (ldo=%d ldq=%d ld_vt=%d)", ldo, ldq, ld_vt);
-    /* Variants: 0 / 1 = attention_kernel with 128 / 256 queries per workgroup, 11 .. 14 = attention_wide_kernel with
-     * 16 NQ queries per wave (NQ = 1 .. 4; 64 NQ queries per workgroup, one workgroup per compute unit). Default: the
-     * widest wave that still gives about 0.7 workgroups per compute unit (measured at 24 heads: 4608 and 2560
-     * tokens NQ = 4, 1536 tokens NQ = 3, 768 and fewer NQ = 1). */
-    int big = g_att_force;
-    if (big < 0) {
-        int nq = 4;
-        while (nq > 1 && ((seq_q + 64 * nq - 1) / (64 * nq)) * heads < 180) nq--;
-        big = 10 + nq;
-    }
+    /* Variants: 0 / 1 = attention_kernel with 128 / 256 queries per workgroup; 11 .. 14 = attention_wide_kernel with
+     * 16 NQ queries per wave throughout (NQ = 1 .. 4); -1 (default) and 15 = attention_wide_kernel with the mix of
+     * block lengths that wide_plan() finds. */
     static bool attr_done = false;
     if (!attr_done) {
-        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, ATT_WIDE_LDS));
-        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, ATT_WIDE_LDS));
-        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<3>, hipFuncAttributeMaxDynamicSharedMemorySize, ATT_WIDE_LDS));
-        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, ATT_WIDE_LDS));
         HIP_OK(hipFuncSetAttribute((const void *)attention_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
         HIP_OK(hipFuncSetAttribute((const void *)attention_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * ATT_STAGE));
+        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<4, 3>, hipFuncAttributeMaxDynamicSharedMemorySize, ATT_WIDE_LDS));
+        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<3, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, ATT_WIDE_LDS));
+        HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<2, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, ATT_WIDE_LDS));
         attr_done = true;
     }
-    if (big >= 11 && big <= 14) {
-        /* 16 NQ queries per wave, four waves per workgroup (variants 11 .. 14 = NQ 1 .. 4) */
-        const int nq = big - 10, bq = 64 * nq;
-        const int blocks = ((seq_q + bq - 1) / bq) * heads, blocks128 = ((seq_q + 127) / 128) * heads;
-        int *redo = att_redo_for_current_device();
-        if (!redo || blocks128 > ATT_REDO_MAX) return flux_hip_fail("flux_hip_attention: no room for the second-pass marks");
-        auto kern = nq == 1 ? attention_wide_kernel<1> : nq == 2 ? attention_wide_kernel<2> : nq == 3 ? attention_wide_kernel<3> : attention_wide_kernel<4>;
-        hipLaunchKernelGGL(kern, dim3((blocks + 7) & ~7), dim3(256), ATT_WIDE_LDS, flux_hip_stream_handle(),
-                           (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,
-                           heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps, redo);
-        /* second pass: the blocks of 128 queries the first one marked (normally none: every workgroup leaves at once) */
-        hipLaunchKernelGGL(attention_kernel<4>, dim3((blocks128 + 7) & ~7), dim3(256), 2 * ATT_STAGE, flux_hip_stream_handle(),
-                           (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,
-                           heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps, redo);
-    } else if (big) {
-        const int blocks = ((seq_q + 255) / 256) * heads;
-        hipLaunchKernelGGL(attention_kernel<8>, dim3((blocks + 7) & ~7), dim3(512), 2 * ATT_STAGE, flux_hip_stream_handle(),
-                           (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,
-                           heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps, (int *)nullptr);
-    } else {
-        const int blocks = ((seq_q + 127) / 128) * heads;
-        hipLaunchKernelGGL(attention_kernel<4>, dim3((blocks + 7) & ~7), dim3(256), 2 * ATT_STAGE, flux_hip_stream_handle(),
-                           (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,
-                           heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps, (int *)nullptr);
+    const int variant = g_att_force;
+    if (variant == 0 || variant == 1) {
+        const int bq = variant ? 256 : 128, blocks = ((seq_q + bq - 1) / bq) * heads;
+        hipLaunchKernelGGL(variant ? attention_kernel<8> : attention_kernel<4>, dim3((blocks + 7) & ~7), dim3(variant ? 512 : 256), 2 * ATT_STAGE,
+                           flux_hip_stream_handle(), (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt,
+                           seq_q, seq_k, heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps, (int *)nullptr);
+        HIP_OK(hipGetLastError());
+        return 1;
     }
+    WidePlan plan;
+    if (variant >= 11 && variant <= 14) {
+        const int nq = variant - 10;
+        plan.nqa = nq > 1 ? nq : 2;
+        plan.na = nq > 1 ? (seq_q + 64 * nq - 1) / (64 * nq) : 0;
+        plan.nb = nq > 1 ? 0 : (seq_q + 63) / 64;
+    } else {
+        plan = wide_plan(seq_q, heads);
+    }
+    const int blocks128 = ((seq_q + 127) / 128) * heads;
+    int *redo = att_redo_for_current_device();
+    if (!redo || blocks128 > ATT_REDO_MAX) return flux_hip_fail("flux_hip_attention: no room for the second-pass marks");
+    const int max_nh = (heads + 7) / 8; /* the most heads one XCD takes */
+    const dim3 grid(8 * max_nh * (plan.na + plan.nb));
+    auto kern = plan.nqa == 4 ? attention_wide_kernel<4, 3> : plan.nqa == 3 ? attention_wide_kernel<3, 2> : attention_wide_kernel<2, 1>;
+    hipLaunchKernelGGL(kern, grid, dim3(256), ATT_WIDE_LDS, flux_hip_stream_handle(), (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq,
+                       (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k, heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps,
+                       redo, plan.na, plan.nb);
+    /* second pass: the blocks of 128 queries the first one marked (normally none: every workgroup leaves at once) */
+    hipLaunchKernelGGL(attention_kernel<4>, dim3((blocks128 + 7) & ~7), dim3(256), 2 * ATT_STAGE, flux_hip_stream_handle(),
+                       (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,
+                       heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps, redo);
     HIP_OK(hipGetLastError());
     return 1;
 }
