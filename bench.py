@@ -38,10 +38,11 @@ import fluxhip  # noqa: E402
 from model_spec import KLEIN_4B, FluxConfig, tensor_shapes, make_weights, normal_f32, normal_bf16, flops_per_forward  # noqa: E402
 
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA peak (datasheet)
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# `bench.py --calibrate` (profiles/gemm_swiglu_c4_traffic.txt), scaled by the same counters on a
-# streaming kernel of known size.
-TRAFFIC_BYTES = {"c4": 878_000_000}
+# Bytes per launch that the dominant kernel moves beyond its L2s, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# `bench.py --calibrate` (profiles/gemm_qkv_swiglu_c4_traffic.txt, profiles/gemm_swiglu_c4_traffic.txt), scaled by
+# the same counters on a streaming kernel of known size.
+PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E peak (datasheet)
+TRAFFIC_BYTES = {("c4", True): 1_551_000_000, ("c4", False): 878_000_000}   # keyed by (workload, fused [Q|K|V|gate|up] launch)
 
 # (latent h, w, text tokens, reference-image latents [(h, w, t_offset)], cfg, schedule steps)
 WORKLOADS = {
@@ -61,25 +62,48 @@ def load_model(cfg, seed=42, qk="literal"):
     return m
 
 
-def time_dominant_kernel(cfg, tokens, launches=20):
-    """Gate/up projection with SwiGLU epilogue at [tokens, hidden] x [2*mlp, hidden]^T, alone."""
+EPI_QKV_SWIGLU = 8          # flux_hip_linear_probe's number for the launches of flux_hip_linear_qkv_swiglu
+
+
+def dominant_kernel_cost(cfg, tokens, fused):
+    """Algorithmic FLOPs and bytes of one launch of the step's dominant kernel: the [Q|K|V|gate|up] projection of a
+    single-stream block (fused) or the gate/up projection with SwiGLU epilogue (not fused), each operand read once
+    and each output written once, bf16."""
     H, M = cfg.hidden, cfg.mlp
+    if fused:
+        return 2.0 * tokens * H * (3 * H + 2 * M), 2.0 * ((3 * H + 2 * M) * H + tokens * H + tokens * (3 * H + M))
+    return 2.0 * tokens * H * 2 * M, 2.0 * (2 * M * H + tokens * H + tokens * M)
+
+
+def time_dominant_kernel(cfg, tokens, fused, launches=20):
+    """The dominant kernel alone, back to back on resident buffers, at [tokens, hidden]: ms per launch."""
+    import ctypes
+    H, M = cfg.hidden, cfg.mlp
+    rows = 3 * H + 2 * M if fused else 2 * M
     a = fluxhip.DevBuf.from_array(normal_bf16((tokens, H), 5, 1))
-    w = fluxhip.DevBuf.from_array(normal_bf16((2 * M, H), 5, 2, 0.0, 0.02))
+    w = fluxhip.DevBuf.from_array(normal_bf16((rows, H), 5, 2, 0.0, 0.02))
     out = fluxhip.DevBuf(tokens * M * 2)
+    qkv = fluxhip.DevBuf(tokens * 3 * H * 2) if fused else None
     L = fluxhip.lib()
-    part = [(a.ptr, w.ptr, out.ptr, None, tokens)]
-    for _ in range(3):
-        fluxhip.linear(fluxhip.EPI_SWIGLU, part, 2 * M, H, H, H, M, 0, M)
+    L.flux_hip_linear_qkv_swiglu.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 8
+
+    def run():
+        if fused:
+            fluxhip.check(L.flux_hip_linear_qkv_swiglu(a.ptr, w.ptr, qkv.ptr, out.ptr, tokens, 3 * H, M, H, H, H, 3 * H, M), "flux_hip_linear_qkv_swiglu")
+        else:
+            fluxhip.linear(fluxhip.EPI_SWIGLU, [(a.ptr, w.ptr, out.ptr, None, tokens)], 2 * M, H, H, H, M, 0, M)
+
+    for _ in range(5):
+        run()
     fluxhip.sync()
     L.flux_hip_timer_start()
     for _ in range(launches):
-        fluxhip.linear(fluxhip.EPI_SWIGLU, part, 2 * M, H, H, H, M, 0, M)
+        run()
     ms = L.flux_hip_timer_stop() / launches
-    flops = 2.0 * tokens * H * 2 * M
-    for b in (a, w, out):
-        b.free()
-    return ms, flops
+    for b in (a, w, out, qkv):
+        if b is not None:
+            b.free()
+    return ms
 
 
 def cpu_baseline(cfg, wl, forwards):
@@ -360,6 +384,74 @@ def bench_attention(args):
         "cpu_baseline": None}))
 
 
+BW_WORKLOADS = {"bw_c3": 1536, "bw_c4": 4608}
+
+
+def bench_bandwidth(args):
+    """The bandwidth-bound kernels of a block at a workload's token count, each alone on resident buffers: LayerNorm +
+    modulation (flux_hip_adaln_norm: fp32 [tokens, 3072] in, bf16 out), K/V preparation (flux_hip_kv_prepare: K and V
+    of 24 heads in, normalised + rotated K and transposed V out) and, as the yardstick for what a trivial streaming
+    kernel reaches at this size, the fp32 -> bf16 conversion over the same element count. Every kernel is timed twice:
+    launches over the same buffers (operands stay in the 256 MB memory-side cache) and over four buffer sets in turn
+    (every launch finds its operands in HBM). One "step" is one launch of each kernel on rotating buffers."""
+    n, heads, H = BW_WORKLOADS[args.workload], KLEIN_4B.heads, KLEIN_4B.hidden
+    fluxhip.init()
+    L = fluxhip.lib()
+    NB = 4
+    launches = max(args.steps, 1)
+
+    def timed(fn):
+        for i in range(max(args.warmup, 1) * NB):
+            fn(i)
+        fluxhip.sync()
+        L.flux_hip_timer_start()
+        for i in range(launches):
+            fn(i)
+        return L.flux_hip_timer_stop() / launches
+
+    x = [fluxhip.DevBuf.from_array(normal_f32((n, H), 7, i)) for i in range(NB)]
+    o = [fluxhip.DevBuf(n * H * 2) for _ in range(NB)]
+    sh, sc = fluxhip.DevBuf.from_array(normal_f32((H,), 7, 20)), fluxhip.DevBuf.from_array(normal_f32((H,), 7, 21))
+    qkv = [fluxhip.DevBuf.from_array(normal_bf16((n, 3 * H), 5, i)) for i in range(NB)]
+    w = fluxhip.DevBuf.from_array(np.ones(128, np.float32))
+    ang = normal_f32((n, 128), 5, 2)
+    cos, sin = fluxhip.DevBuf.from_array(np.cos(ang)), fluxhip.DevBuf.from_array(np.sin(ang))
+    ldvt = (n + 63) // 64 * 64
+    kn, vt = [fluxhip.DevBuf(n * H * 2) for _ in range(NB)], [fluxhip.DevBuf(H * ldvt * 2) for _ in range(NB)]
+
+    def adaln(j):
+        fluxhip.check(L.flux_hip_adaln_norm(o[j].ptr, H, x[j].ptr, n, H, 512, sh.ptr, sc.ptr, sh.ptr, sc.ptr, 1e-6))
+
+    def prep(j):
+        fluxhip.check(L.flux_hip_kv_prepare(kn[j].ptr, vt[j].ptr, ldvt, qkv[j].ptr, 3 * H, H, 2 * H, n, heads, 512, w.ptr, w.ptr, cos.ptr, sin.ptr, 1e-6))
+
+    def conv(j):
+        fluxhip.check(L.flux_hip_f32_to_bf16(o[j].ptr, x[j].ptr, n * H))
+
+    kernels = {"adaln_kernel": (adaln, 6.0 * n * H, "fp32 row in, bf16 row out: 6 bytes per element"),
+               "kv_prepare_kernel": (prep, 8.0 * n * H, "bf16 K and V in, bf16 K and V^T out: 8 bytes per element of K"),
+               "f32_to_bf16_kernel": (conv, 6.0 * n * H, "yardstick: same bytes as adaln_kernel, no reduction")}
+    table = {}
+    t0 = time.perf_counter()
+    for name, (fn, nbytes, what) in kernels.items():
+        warm = timed(lambda i: fn(0))
+        cold = timed(lambda i: fn(i % NB))
+        table[name] = {"bytes_per_launch": nbytes, "what": what,
+                       "same_buffers": {"us": round(warm * 1e3, 2), "GBps": round(nbytes / warm / 1e6, 1), "frac_of_hbm_peak": round(nbytes / warm / 1e6 / PEAK_HBM_GBPS, 4)},
+                       "four_buffer_sets_in_turn": {"us": round(cold * 1e3, 2), "GBps": round(nbytes / cold / 1e6, 1),
+                                                    "frac_of_hbm_peak": round(nbytes / cold / 1e6 / PEAK_HBM_GBPS, 4)}}
+    wall = time.perf_counter() - t0
+    a = table["adaln_kernel"]["four_buffer_sets_in_turn"]
+    print(json.dumps({
+        "metric": f"launches/s of the bandwidth-bound kernels ({n} tokens, 1 GPU)", "value": round(6 * launches / wall, 1), "unit": "launches/s",
+        "n_gpus": 1, "steps": launches, "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: adaln_kernel, kv_prepare_kernel and the fp32->bf16 yardstick at [{n}, {H}], N(0,1) inputs"},
+        "roofline": {"bound": "hbm", "achieved": a["GBps"], "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": a["frac_of_hbm_peak"], "traffic": None,
+                     "kernel": "adaln_kernel, operands in HBM (four buffer sets in turn)"},
+        "kernels": table, "cpu_baseline": None}))
+
+
 def bf16_to_f32_host(a):
     return (a.astype(np.uint32) << 16).view(np.float32)
 
@@ -403,7 +495,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=8)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + sorted(VAE_WORKLOADS) + sorted(ATT_WORKLOADS) + ["qwen3", "mfma_peak"])
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + sorted(VAE_WORKLOADS) + sorted(ATT_WORKLOADS) + sorted(BW_WORKLOADS) + ["qwen3", "mfma_peak"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     ap.add_argument("--tile-mask", type=lambda v: int(v, 0), default=0,
@@ -431,6 +523,8 @@ def main():
         return bench_mfma_peak(args)
     if args.workload in ATT_WORKLOADS:
         return bench_attention(args)
+    if args.workload in BW_WORKLOADS:
+        return bench_bandwidth(args)
     cfg = KLEIN_4B
     wl = WORKLOADS[args.workload]
     if args.calibrate:
@@ -443,15 +537,17 @@ def main():
             fluxhip.check(fluxhip.lib().flux_hip_f32_to_bf16(dst.ptr, src.ptr, n))
         fluxhip.sync()
         tokens = wl["h"] * wl["w"] + sum(rh * rw for rh, rw, _ in wl["refs"]) + wl["txt"]
-        ms, fl = time_dominant_kernel(cfg, tokens, launches=5)
-        print(json.dumps({"calibration_copy": {"read_MiB": 256, "write_MiB": 128},
-                          "gemm_ms": ms, "gemm_tflops": fl / ms / 1e9}))
+        ms = time_dominant_kernel(cfg, tokens, bool(args.fused_qkv_mlp), launches=5)
+        fl, by = dominant_kernel_cost(cfg, tokens, bool(args.fused_qkv_mlp))
+        print(json.dumps({"calibration_copy": {"read_MiB": 256, "write_MiB": 128}, "gemm_ms": ms, "gemm_tflops": fl / ms / 1e9,
+                          "gemm_algorithmic_bytes": by}))
         return
     K, Wm = args.steps, args.warmup
     h, w, nt = wl["h"], wl["w"], wl["txt"]
     n_target = h * w
     n_img = n_target + sum(rh * rw for rh, rw, _ in wl["refs"])
     forwards = 2 if wl["cfg"] else 1
+    fused = bool(args.fused_qkv_mlp)
 
     fluxhip.init()
     if args.tile_mask:
@@ -473,7 +569,7 @@ def main():
     fluxhip.sync()
     L = fluxhip.lib()
     if not args.no_kernel_timing:
-        L.flux_hip_linear_probe(fluxhip.EPI_SWIGLU)   # events around the dominant kernel's launches
+        L.flux_hip_linear_probe(EPI_QKV_SWIGLU if fused else fluxhip.EPI_SWIGLU)   # events around the dominant kernel's launches
     t0 = time.perf_counter()
     L.flux_hip_timer_start()
     for i in range(Wm, Wm + K):
@@ -483,11 +579,12 @@ def main():
     wall = time.perf_counter() - t0
     import ctypes
     k_n, k_ms = ctypes.c_int(0), ctypes.c_float(0.0)
-    # the gate/up projection runs under more than one tile shape in a step (single-stream blocks
-    # and two-part double-stream blocks); the dominant kernel is the shape with the most time
-    TILE_NAMES = {0: "gemm_kernel<64,128,2,2,SWIGLU>", 1: "gemm_kernel<128,128,2,2,SWIGLU>", 2: "gemm4w_kernel<8,8,SWIGLU> (256x256 tile)",
-                  3: "gemm_kernel<64,64,2,2,SWIGLU>", 4: "gemm_kernel<256,256,2,4,SWIGLU>", 5: "gemm4w_kernel<9,6,SWIGLU> (288x192 tile)", 6: "gemm4w_kernel<6,6,SWIGLU> (192x192 tile)",
-                  7: "gemm4w_kernel<8,6,SWIGLU> (256x192 tile)"}
+    # one projection runs under more than one tile shape in a step when it is launched at several sizes (the
+    # two-part launches of the double-stream blocks); the dominant kernel is the shape with the most time
+    epi_name = "QKV_SWIGLU" if fused else "SWIGLU"
+    TILE_NAMES = {0: f"gemm_kernel<64,128,2,2,{epi_name}>", 1: f"gemm_kernel<128,128,2,2,{epi_name}>", 2: f"gemm4w_kernel<8,8,{epi_name}> (256x256 tile)",
+                  3: f"gemm_kernel<64,64,2,2,{epi_name}>", 4: f"gemm_kernel<256,256,2,4,{epi_name}>", 5: f"gemm4w_kernel<9,6,{epi_name}> (288x192 tile)",
+                  6: f"gemm4w_kernel<6,6,{epi_name}> (192x192 tile)", 7: f"gemm4w_kernel<8,6,{epi_name}> (256x192 tile)"}
     k_tile = -1
     for tile in TILE_NAMES:
         n_t, ms_t = ctypes.c_int(0), ctypes.c_float(0.0)
@@ -515,16 +612,24 @@ def main():
 
     roof = None
     if not args.no_kernel_timing and k_n.value > 0:
-        # every launch of the gate/up projection in a step has the same cost: [tokens, H] x [2*mlp, H]^T
+        # fused: only the single-stream blocks launch this kernel, all at [image + text tokens, H]; not fused: every
+        # gate/up launch of the step, which all have that cost too
         per_ms = k_ms.value / k_n.value
-        k_flops = 2.0 * (n_img + nt) * cfg.hidden * 2 * cfg.mlp
+        k_flops, k_bytes = dominant_kernel_cost(cfg, n_img + nt, fused)
         ach = k_flops / (per_ms * 1e-3) / 1e12
-        alone_ms, _ = time_dominant_kernel(cfg, n_img + nt)
-        roof = {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES.get(args.workload),
-                "kernel": TILE_NAMES[k_tile] + ": gate/up projection + SiLU*up",
-                "launches_timed": k_n.value, "ms_per_launch": round(per_ms, 4), "flops_per_launch": k_flops,
-                "ms_per_launch_back_to_back": round(alone_ms, 4)}
+        gbps = k_bytes / (per_ms * 1e-3) / 1e9
+        alone_ms = time_dominant_kernel(cfg, n_img + nt, fused)
+        what = "[Q|K|V|gate|up] projection of a single-stream block, bf16 store + SiLU(gate)*up" if fused else "gate/up projection + SiLU*up"
+        # the launch is bound by whichever of the two it needs longer for at the datasheet rates
+        if k_flops / (PEAK_BF16_TFLOPS * 1e12) >= k_bytes / (PEAK_HBM_GBPS * 1e9):
+            roof = {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES.get((args.workload, fused))}
+        else:
+            roof = {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                    "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": TRAFFIC_BYTES.get((args.workload, fused))}
+        roof.update({"kernel": TILE_NAMES[k_tile] + ": " + what, "launches_timed": k_n.value, "ms_per_launch": round(per_ms, 4),
+                     "flops_per_launch": k_flops, "bytes_per_launch": k_bytes, "tflops": round(ach, 1), "GBps": round(gbps, 1),
+                     "ms_per_launch_back_to_back": round(alone_ms, 4)})
     model.close()
 
     cpu = None

@@ -21,46 +21,58 @@ __device__ __forceinline__ float wave_sum(float v) {
  * --------------------------------------------------------------------------------------- */
 #define ADALN_MAX_V4 16 /* float4 per lane: rows up to 64*4*16 = 4096 columns */
 
+/* A wave takes R rows and requests all of them before it reduces the first: with one row per wave a launch over
+ * 4608 rows needs more workgroups than the GPU holds at a time, and its last few run alone. NV = float4 per lane
+ * the registers are laid out for (hidden <= 256 NV; EXACT: hidden = 256 NV, no guards around the loads). */
+template <int R, int NV, bool EXACT>
 __global__ __launch_bounds__(256) void adaln_kernel(bf16 *__restrict__ out, int ldo, const float *__restrict__ x,
                                                     int rows, int hidden, int split,
                                                     const float *__restrict__ shift0, const float *__restrict__ scale0,
                                                     const float *__restrict__ shift1, const float *__restrict__ scale1,
                                                     float eps) {
-    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (row >= rows) return;
+    const int row0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * R;
+    if (row0 >= rows) return;
     const int lane = threadIdx.x & 63;
-    const int nv = hidden >> 8; /* float4 per lane */
-    const float *xr = x + (size_t)row * hidden;
-    f32x4 v[ADALN_MAX_V4];
-    float s = 0.0f;
+    const int nv = EXACT ? NV : hidden >> 8; /* float4 per lane */
+    f32x4 v[R][NV];
 #pragma unroll
-    for (int i = 0; i < ADALN_MAX_V4; i++)
-        if (i < nv) {
-            v[i] = *(const f32x4 *)(xr + (i * 64 + lane) * 4);
-            s += (v[i][0] + v[i][1]) + (v[i][2] + v[i][3]);
-        }
-    const float mean = wave_sum(s) / (float)hidden;
-    float q = 0.0f;
+    for (int r = 0; r < R; r++) {
+        const float *xr = x + (size_t)min(row0 + r, rows - 1) * hidden;
 #pragma unroll
-    for (int i = 0; i < ADALN_MAX_V4; i++)
-        if (i < nv) {
+        for (int i = 0; i < NV; i++)
+            if (i < nv) v[r][i] = *(const f32x4 *)(xr + (i * 64 + lane) * 4);
+    }
 #pragma unroll
-            for (int e = 0; e < 4; e++) { float d = v[i][e] - mean; q += d * d; }
-        }
-    const float inv = 1.0f / sqrtf(wave_sum(q) / (float)hidden + eps);
-    const float *shift = row < split ? shift0 : shift1;
-    const float *scale = row < split ? scale0 : scale1;
-    bf16 *o = out + (size_t)row * ldo;
+    for (int r = 0; r < R; r++) {
+        const int row = row0 + r;
+        if (row >= rows) break;
+        float s = 0.0f;
 #pragma unroll
-    for (int i = 0; i < ADALN_MAX_V4; i++)
-        if (i < nv) {
-            const int c = (i * 64 + lane) * 4;
-            f32x4 sh = *(const f32x4 *)(shift + c), sc = *(const f32x4 *)(scale + c);
-            bf16x4 r;
+        for (int i = 0; i < NV; i++)
+            if (i < nv) s += (v[r][i][0] + v[r][i][1]) + (v[r][i][2] + v[r][i][3]);
+        const float mean = wave_sum(s) / (float)hidden;
+        float q = 0.0f;
 #pragma unroll
-            for (int e = 0; e < 4; e++) r[e] = (bf16)((1.0f + sc[e]) * ((v[i][e] - mean) * inv) + sh[e]);
-            *(bf16x4 *)(o + c) = r;
-        }
+        for (int i = 0; i < NV; i++)
+            if (i < nv) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) { float d = v[r][i][e] - mean; q += d * d; }
+            }
+        const float inv = 1.0f / sqrtf(wave_sum(q) / (float)hidden + eps);
+        const float *shift = row < split ? shift0 : shift1;
+        const float *scale = row < split ? scale0 : scale1;
+        bf16 *o = out + (size_t)row * ldo;
+#pragma unroll
+        for (int i = 0; i < NV; i++)
+            if (i < nv) {
+                const int c = (i * 64 + lane) * 4;
+                f32x4 sh = *(const f32x4 *)(shift + c), sc = *(const f32x4 *)(scale + c);
+                bf16x4 rr;
+#pragma unroll
+                for (int e = 0; e < 4; e++) rr[e] = (bf16)((1.0f + sc[e]) * ((v[r][i][e] - mean) * inv) + sh[e]);
+                *(bf16x4 *)(o + c) = rr;
+            }
+    }
 }
 
 extern "C" int flux_hip_adaln_norm(void *out_bf16, int ldo, const float *x, int rows, int hidden, int split,
@@ -72,8 +84,13 @@ extern "C" int flux_hip_adaln_norm(void *out_bf16, int ldo, const float *x, int 
     if (!out_bf16 || !x || !shift0 || !scale0) return flux_hip_fail("flux_hip_adaln_norm: NULL argument");
     if (split < rows && (!shift1 || !scale1)) return flux_hip_fail("flux_hip_adaln_norm: second modulation missing");
     if (ldo < hidden || (ldo & 3)) return flux_hip_fail("flux_hip_adaln_norm: bad ldo=%d", ldo);
-    hipLaunchKernelGGL(adaln_kernel, dim3((rows + 3) / 4), dim3(256), 0, flux_hip_stream_handle(),
-                       (bf16 *)out_bf16, ldo, x, rows, hidden, split, shift0, scale0, shift1, scale1, eps);
+    hipStream_t st = flux_hip_stream_handle();
+    if (hidden == 256 * 12)
+        hipLaunchKernelGGL((adaln_kernel<2, 12, true>), dim3((rows + 7) / 8), dim3(256), 0, st, (bf16 *)out_bf16, ldo, x, rows, hidden, split, shift0,
+                           scale0, shift1, scale1, eps);
+    else
+        hipLaunchKernelGGL((adaln_kernel<1, ADALN_MAX_V4, false>), dim3((rows + 3) / 4), dim3(256), 0, st, (bf16 *)out_bf16, ldo, x, rows, hidden, split,
+                           shift0, scale0, shift1, scale1, eps);
     HIP_OK(hipGetLastError());
     return 1;
 }
