@@ -266,7 +266,7 @@ __device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f
     }
 }
 
-template <int BM, int BN, int WGM, int WGN, int EPI>
+template <int BM, int BN, int WGM, int WGN, int EPI, int NS = 2>
 __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
     constexpr int T = WGM * WGN * 64;
     constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 16, TN = WN / 16;
@@ -320,7 +320,11 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
     };
     const int kt_begin = ks * g.kt_per;
     const int KT = min(g.K >> 6, kt_begin + g.kt_per) - kt_begin;
-    issue(kt_begin, 0);
+    /* NS - 1 stages are requested ahead: with few rows (M <= BM, weights streamed once, hardly any arithmetic) a
+     * workgroup is only as fast as the bytes it keeps in flight, and the ring then takes the whole LDS */
+#pragma unroll
+    for (int s = 0; s < NS - 1; s++)
+        if (s < KT) issue(kt_begin + s, s);
 
     f32x4 acc[TN][TM];
 #pragma unroll
@@ -335,13 +339,21 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
     const int a_frag = (wm * WM + l15) * 128;
     const int b_frag = BM * 128 + (wn * WN + l15) * 128;
 
+    int cur = 0;
     for (int kt = 0; kt < KT; kt++) {
-        const int cur = kt & 1;
-        /* stage `cur` has landed for this wave; after the barrier it has for all, and everyone
-         * is done reading the other stage, which can then be refilled */
-        WAIT_VMCNT0();
-        __syncthreads();
-        if (kt + 1 < KT) issue(kt_begin + kt + 1, cur ^ 1);
+        /* stage `cur` has landed for this wave (the NS - 2 stages requested after it may still be on their way);
+         * after the barrier it has for all, and everyone is done reading the stage before it, which is refilled */
+        if constexpr (NS > 2) {
+            /* __syncthreads() would wait for every load in flight (its fence counts the global->LDS loads); here the
+             * wait names what must have landed, and this wave's own LDS reads of the stage that is refilled next */
+            if (kt + NS - 2 < KT) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((NS - 2) * (PA + PB)) : "memory");
+            else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        } else {
+            WAIT_VMCNT0();
+            __syncthreads();
+        }
+        const int refill = cur == 0 ? NS - 1 : cur - 1;
+        if (kt + NS - 1 < KT) issue(kt_begin + kt + NS - 1, refill);
         const char *st = smem + cur * STAGE;
 #pragma unroll
         for (int kk = 0; kk < 2; kk++) {
@@ -357,6 +369,7 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
                 for (int j = 0; j < TM; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[i], fa[j], acc[i][j], 0, 0, 0);
         }
+        cur = cur == NS - 1 ? 0 : cur + 1;
     }
 
     store_tile<BN, WM, WN, EPI>(g, t, acc, m0, M, wm, wn, l15, lq, t.tm * WGM + wm);
@@ -563,12 +576,13 @@ static void set_row_tiles(GemmArgs &g, int BM) {
     g.mtiles = end;
 }
 
-template <int BM, int BN, int WGM, int WGN, int EPI>
+template <int BM, int BN, int WGM, int WGN, int EPI, int NS = 2>
 static int launch_cfg(GemmArgs &g) {
     constexpr int T = WGM * WGN * 64;
-    constexpr int LDS = 2 * (BM + BN) * 128;
+    constexpr int LDS = NS * (BM + BN) * 128;
+    static_assert(LDS <= 160 * 1024 && (NS - 2) * ((BM + BN) * 8 / T) < 64, "the ring fits the LDS, the loads in flight the wait counter");
     static bool attr_done = false;
-    auto kern = gemm_kernel<BM, BN, WGM, WGN, EPI>;
+    auto kern = gemm_kernel<BM, BN, WGM, WGN, EPI, NS>;
     if (!attr_done) {
         HIP_OK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
         attr_done = true;
@@ -619,6 +633,8 @@ static int launch_epi(GemmArgs &g, int tile) {
         case 4: return launch_4w<8, 4, EPI, 2, 4>(g); /* 8 waves, two per SIMD, on the 256x256 tile */
         case 1: return launch_cfg<128, 128, 2, 2, EPI>(g);
         case 3: return launch_cfg<64, 64, 2, 2, EPI>(g);
+        case 8: return launch_cfg<64, 128, 2, 2, EPI, 6>(g);  /* few rows: the same tiles with a ring that fills the LDS */
+        case 9: return launch_cfg<128, 128, 2, 2, EPI, 5>(g);
         default: return launch_cfg<64, 128, 2, 2, EPI>(g);
     }
 }
@@ -863,10 +879,10 @@ extern "C" void flux_hip_linear_release(void) {
 }
 
 static int g_force_tile = -1;
-static unsigned g_tile_mask = 0xEF; /* tiles the automatic choice may use: all but the 8-wave form of 256 x 256 */
+static unsigned g_tile_mask = 0x3EF; /* tiles the automatic choice may use: all but the 8-wave form of 256 x 256 */
 static int g_splitk_enabled = 1;
 extern "C" void flux_hip_linear_force_tile(int tile) { g_force_tile = tile; }
-extern "C" void flux_hip_linear_tile_mask(unsigned mask) { g_tile_mask = mask ? mask : 0xEF; }
+extern "C" void flux_hip_linear_tile_mask(unsigned mask) { g_tile_mask = mask ? mask : 0x3EF; }
 extern "C" void flux_hip_linear_enable_splitk(int on) { g_splitk_enabled = on; }
 
 /* Launch probe: HIP events around every launch with one chosen epilogue, so a benchmark can
@@ -936,10 +952,12 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
      * fixed prologue/epilogue cost; the launch cannot beat the time to stream its operands,
      * which depends on how many bytes the resident workgroups keep in flight. */
     /* tile ids: 0..3 the small tiles and 256 x 256, 4 = the 8-wave form of 256 x 256 (only when
-     * forced, for comparison runs), 5 = 288 x 192, 6 = 192 x 192, 7 = 256 x 192 */
-    constexpr int NT = 8;
-    static const int bm[NT] = {64, 128, 256, 64, 256, 288, 192, 256}, bn[NT] = {128, 128, 256, 64, 256, 192, 192, 192}, occ[NT] = {3, 2, 1, 4, 1, 1, 1, 1};
-    static const double rate[NT] = {2.0e12, 2.9e12, 5.3e12, 1.5e12, 4.6e12, 5.0e12, 4.0e12, 4.9e12}; /* FLOP/s of one CU running this tile */
+     * forced, for comparison runs), 5 = 288 x 192, 6 = 192 x 192, 7 = 256 x 192, 8 and 9 = 64 x 128 and 128 x 128
+     * with a ring of 6 and 5 stages instead of 2 (one workgroup per compute unit; for parts of at most that many rows) */
+    constexpr int NT = 10;
+    static const int bm[NT] = {64, 128, 256, 64, 256, 288, 192, 256, 64, 128}, bn[NT] = {128, 128, 256, 64, 256, 192, 192, 192, 128, 128};
+    static const int occ[NT] = {3, 2, 1, 4, 1, 1, 1, 1, 1, 1}, ahead[NT] = {1, 1, 1, 1, 1, 1, 1, 1, 5, 4}; /* stages a workgroup keeps in flight */
+    static const double rate[NT] = {2.0e12, 2.9e12, 5.3e12, 1.5e12, 4.6e12, 5.0e12, 4.0e12, 4.9e12, 1.6e12, 3.0e12}; /* FLOP/s of one CU running this tile */
     const int kt_total = g.K >> 6;
     int tile = -1, best_split = 1;
     {
@@ -956,6 +974,11 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
         for (int t = 0; t < NT; t++) {
             if (N % bn[t] || g.nq_cols % bn[t]) continue;
             if (!((allowed >> t) & 1)) continue;
+            if (ahead[t] > 1) { /* the deep rings stream the weights once: every part in one row tile */
+                bool fits = true;
+                for (int i = 0; i < np; i++) fits = fits && g.M[i] <= bm[t];
+                if (!fits) continue;
+            }
             long tiles = 0;
             for (int i = 0; i < np; i++) tiles += (g.M[i] + bm[t] - 1) / bm[t];
             tiles *= N / bn[t];
@@ -972,7 +995,7 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
                 const double t_block = 2.0 * bm[t] * bn[t] * 64.0 * per / (rate[t] / per_cu) + 2.5e-6;
                 double t_compute = rounds * t_block;
                 const double bytes = (rows + N) * (double)K * 2.0;
-                double bw = 5.5e12 * (double)(resident * (bm[t] + bn[t]) * 128) / 12.0e6;
+                double bw = 5.5e12 * (double)(resident * ahead[t] * (bm[t] + bn[t]) * 128) / 12.0e6;
                 if (bw > 5.5e12) bw = 5.5e12;
                 double est = t_compute > bytes / bw ? t_compute : bytes / bw;
                 if (sp > 1) est += 3.0e-6 + (sp + 2.0) * rows * N * 4.0 / 4.0e12;
@@ -1070,7 +1093,7 @@ static int linear_impl(int epilogue, int nparts, const flux_hip_linear_part *par
     g.N = N; g.K = K; g.lda = lda; g.ldw = ldw; g.ldc = ldc; g.w_row0 = w_row0; g.w_row1 = w_row1;
     a.ldo = N;
     a.eps = eps;
-    return gemm_dispatch(g, np, epilogue, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0xFFu, nullptr, norm ? &a : nullptr, fused,
+    return gemm_dispatch(g, np, epilogue, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0x3FFu, nullptr, norm ? &a : nullptr, fused,
                          fixed_ws, fixed_ws_bytes);
 }
 
@@ -1098,7 +1121,7 @@ extern "C" int flux_hip_linear_qkv_swiglu(const void *A, const void *W, void *qk
     int tile = -1;
     const int saved = g_splitk_enabled;
     g_splitk_enabled = 0;
-    const int ok = gemm_dispatch(g, 1, EPI_QKV_SWIGLU, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0xFFu, &tile);
+    const int ok = gemm_dispatch(g, 1, EPI_QKV_SWIGLU, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0x3FFu, &tile);
     g_splitk_enabled = saved;
     return ok;
 }

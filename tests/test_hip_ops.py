@@ -334,6 +334,61 @@ def test_linear_qkv_swiglu_one_launch(hip, oracle_mod, tile, M):
     assert not got_q[:, qc:].any() and not got_m[:, :64].any() and not got_m[:, 64 + mlp:].any()
 
 
+@pytest.mark.parametrize("tile,M", [(8, 1), (8, 37), (8, 64), (9, 80), (9, 128)])
+@pytest.mark.parametrize("K", [64, 192, 320, 448, 1024])
+def test_linear_deep_ring_tiles(hip, oracle_mod, tile, M, K):
+    """Tiles 8 and 9: the 64 x 128 and 128 x 128 tiles with a ring of 6 and 5 LDS stages for parts of few rows.
+    K steps from one (fewer than the ring holds) to sixteen (the ring wraps several times); bf16, fp32, gated
+    residual over two parts, SwiGLU and the fused [Q|K|V|gate|up] launch; bit for bit what the two-stage form of the
+    same tile gives (same MFMA order), and right against the oracle. The launch probe confirms which tile ran."""
+    import ctypes
+    L = hip.lib()
+    L.flux_hip_linear_qkv_swiglu.argtypes = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 8
+    N, mlp = 512, 256
+    x = q(normal_f32((M, K), 71, 1))
+    x2 = q(normal_f32((M // 2 + 1, K), 71, 2))
+    W = q(normal_f32((N + 2 * mlp, K), 71, 3, 0.0, 0.1))
+    gate = normal_f32((N,), 71, 4)
+    res = [normal_f32((M, N), 71, 5), normal_f32((M // 2 + 1, N), 71, 6)]
+    dx, dx2, dW, dg = dev_bf16(hip, x), dev_bf16(hip, x2), dev_bf16(hip, W), hip.DevBuf.from_array(gate)
+    outs = {}
+    L.flux_hip_linear_enable_splitk(0)
+    try:
+        for t in (tile, tile - 8):            # tile 0 = 64 x 128 and tile 1 = 128 x 128 with two stages
+            L.flux_hip_linear_force_tile(t)
+            L.flux_hip_linear_probe(hip.EPI_BF16)
+            o16, o32 = hip.DevBuf(M * N * 2), hip.DevBuf(M * N * 4)
+            hip.linear(hip.EPI_BF16, [(dx.ptr, dW.ptr, o16.ptr, None, M)], N, K, K, K, N)
+            tiles, ms = np.zeros(4, np.int32), np.zeros(4, np.float32)
+            assert L.flux_hip_linear_probe_read_launches(4, tiles.ctypes.data, ms.ctypes.data) == 1 and tiles[0] == t
+            L.flux_hip_linear_probe(-1)
+            hip.linear(hip.EPI_F32, [(dx.ptr, dW.ptr, o32.ptr, None, M)], N, K, K, K, N)
+            r = [hip.DevBuf.from_array(a) for a in res]
+            hip.linear(hip.EPI_RESID, [(dx.ptr, dW.ptr, r[0].ptr, dg.ptr, M), (dx2.ptr, dW.at(64 * K * 2), r[1].ptr, dg.ptr, M // 2 + 1)], N, K, K, K, N)
+            sw = hip.DevBuf(M * mlp * 2)
+            hip.linear(hip.EPI_SWIGLU, [(dx.ptr, dW.ptr, sw.ptr, None, M)], 2 * mlp, K, K, K, mlp, N, N + mlp)
+            fq, fm = hip.DevBuf(M * N * 2), hip.DevBuf(M * mlp * 2)
+            hip.check(L.flux_hip_linear_qkv_swiglu(dx.ptr, dW.ptr, fq.ptr, fm.ptr, M, N, mlp, K, K, K, N, mlp), "flux_hip_linear_qkv_swiglu")
+            outs[t] = [o16.to_array(np.uint16, (M, N)), o32.to_array(np.float32, (M, N)), r[0].to_array(np.float32, (M, N)),
+                       r[1].to_array(np.float32, (M // 2 + 1, N)), sw.to_array(np.uint16, (M, mlp)), fq.to_array(np.uint16, (M, N)),
+                       fm.to_array(np.uint16, (M, mlp))]
+    finally:
+        L.flux_hip_linear_enable_splitk(1)
+        L.flux_hip_linear_force_tile(-1)
+        L.flux_hip_linear_probe(-1)
+    for a, b in zip(outs[tile], outs[tile - 8]):
+        np.testing.assert_array_equal(a, b)
+    lin = oracle_mod.linear(x, W)
+    o16, o32, r0, r1, sw, fq, fm = outs[tile]
+    assert rel_l2(o32, lin[:, :N]) < 2e-6 and rel_l2(bf16_to_f32(o16), lin[:, :N]) < 4e-3
+    assert rel_l2(r0, res[0] + gate * lin[:, :N]) < 2e-6
+    assert rel_l2(r1, res[1] + gate * oracle_mod.linear(x2, W[64:64 + N])) < 2e-6
+    want_sw = oracle_mod.silu(lin[:, N:N + mlp]) * lin[:, N + mlp:]
+    assert rel_l2(bf16_to_f32(sw), want_sw) < 4e-3
+    np.testing.assert_array_equal(fq, o16)
+    np.testing.assert_array_equal(fm, sw)
+
+
 def test_linear_rejects_bad_shapes(hip):
     d = hip.DevBuf(1024)
     with pytest.raises(hip.FluxHipError):
