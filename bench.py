@@ -504,6 +504,7 @@ def main():
                     help="run the two forwards of a CFG step one after the other instead of as one batch (A/B runs)")
     ap.add_argument("--fused-qkv-mlp", type=int, default=1, choices=[0, 1],
                     help="single-stream blocks: 1 = QKV and gate/up projections as one launch (default), 0 = as two (A/B runs)")
+    ap.add_argument("--ring", type=int, default=1, help="GEMM operand rings (flux_hip_linear_ring), for A/B runs")
     ap.add_argument("--attention-variant", type=int, default=-1,
                     help="attention kernel variant (flux_hip_attention_force_variant; -1 = the backend's choice), for A/B runs")
     ap.add_argument("--calibrate", action="store_true",
@@ -555,6 +556,7 @@ def main():
     if args.sequential_cfg:
         fluxhip.lib().flux_hip_set_batched_cfg(0)
     fluxhip.lib().flux_hip_set_fused_qkv_mlp(args.fused_qkv_mlp)
+    fluxhip.lib().flux_hip_linear_ring(args.ring)
     fluxhip.lib().flux_hip_attention_force_variant(args.attention_variant)
     model = load_model(cfg)
     z = normal_f32((cfg.channels, h, w), 123, 1)

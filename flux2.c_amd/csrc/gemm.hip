@@ -554,6 +554,160 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm4w_kernel(GemmArgs g) {
     }
 }
 
+/* The same tiles with deeper operand rings, for the transformer's epilogues. gemm4w_kernel holds two stages and
+ * waits at its barrier for every load it has in flight (requested one to two half-steps earlier); operands that
+ * come from HBM rather than from a cache arrive later than that now and then, and a wave that waits holds the
+ * other three up at the barrier. Here the activation tile and the weight tile have rings of their own, NSA and NSW
+ * slots of one K step (128-byte rows, the layout of gemm4w_kernel) each, as many as the 160 KB of LDS hold: the
+ * operand with three slots is requested a whole K step earlier, and the barrier waits with a count (the loads of
+ * the two-slot operand are issued first in a step, so that "all but the last L" is exactly what must have landed)
+ * instead of a fence. The MFMA order is that of gemm4w_kernel: bit-identical results. */
+template <int TM, int TN, int EPI, int NSA, int NSW>
+__global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
+    constexpr int WGM = 2, WGN = 2;
+    constexpr int WM = 16 * TM, WN = 16 * TN, BM = WGM * WM, BN = WGN * WN;
+    constexpr int RPP = 32; /* tile rows one pass of the workgroup's loads covers: 8 per wave instruction */
+    static_assert(BM % RPP == 0 && BN % RPP == 0, "tile rows must divide evenly over the waves' loads");
+    constexpr int LA = BM / RPP, LB = BN / RPP, NL = LA + LB;
+    constexpr int NF = TM + TN, NM = TM * TN, RD = NM / NF;
+    constexpr int ASZ = BM * 128, WSZ = BN * 128;
+    constexpr int AHEAD = (NSA == 3 ? LA : 0) + (NSW == 3 ? LB : 0); /* loads that may be in flight past the barrier */
+    static_assert((NSA == 2 || NSA == 3) && (NSW == 2 || NSW == 3) && NSA * ASZ + NSW * WSZ <= 160 * 1024, "rings of two or three slots within the LDS");
+    static_assert((EPI != FLUX_HIP_EPI_SWIGLU && EPI != EPI_QKV_SWIGLU) || (TN % 2 == 0), "swiglu pairs 16-column blocks");
+    static_assert(RD >= 2 && RD * (NF - 1) + 1 < NM, "reads and loads must fit between the MFMAs");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6) & 3;
+    const int wm = wave / WGN, wn = wave % WGN;
+    const int lrow = tid >> 3, lchunk = tid & 7;
+    const int l15 = lane & 15, lq = lane >> 4;
+    const int swzl = lds_swz(l15);
+    const int coff0 = (lq ^ swzl) << 4, coff1 = ((4 + lq) ^ swzl) << 4;
+    const unsigned a_frag = (wm * WM + l15) * 128, w_frag = NSA * ASZ + (wn * WN + l15) * 128;
+
+    int vb = blockIdx.x;
+    TileId t;
+    if (!decode_tile(g, vb, t)) return;
+
+    unsigned voff[NL];
+    const char *baseA, *baseW;
+    auto set_sources = [&](const TileId &tt) {
+        const int M = g.M[tt.prob], m0 = tt.tml * BM;
+        const int chunk = (lchunk ^ lds_swz(lrow)) << 3;
+        baseA = (const char *)(g.A[tt.prob] + tt.ks * g.kt_per * 64);
+        baseW = (const char *)(g.W[tt.prob] + tt.ks * g.kt_per * 64);
+#pragma unroll
+        for (int i = 0; i < LA; i++) voff[i] = ((unsigned)min(m0 + lrow + i * RPP, M - 1) * (unsigned)g.lda + chunk) * 2u;
+#pragma unroll
+        for (int i = 0; i < LB; i++) voff[LA + i] = ((unsigned)weight_row<BN, WN, EPI>(g, tt.tn, lrow + i * RPP) * (unsigned)g.ldw + chunk) * 2u;
+    };
+    /* load i of K step kt: activation rows for i < LA (into slot sa of their ring), weight rows after (slot sw) */
+    auto issue1 = [&](int kt, int sa, int sw, int i) {
+        const char *base = (i < LA ? baseA : baseW) + (ptrdiff_t)kt * 128;
+        const int dst = i < LA ? sa * ASZ + (wave * 8 + i * RPP) * 128 : NSA * ASZ + sw * WSZ + (wave * 8 + (i - LA) * RPP) * 128;
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(base + voff[i]), LDS_PTR(smem + dst), 16, 0, 0);
+    };
+    /* the order in which a step issues its loads: the operand with the two-slot ring first (see the file comment) */
+    auto nth = [](int n) { return NSA < NSW ? n : (n < LB ? LA + n : n - LB); };
+    set_sources(t);
+#pragma unroll
+    for (int n = 0; n < NL; n++) issue1(0, 0, 0, nth(n));
+
+    for (;;) {
+        const int kt_begin = t.ks * g.kt_per;
+        const int KT = min(g.K >> 6, kt_begin + g.kt_per) - kt_begin;
+
+        f32x4 acc[TN][TM];
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+#pragma unroll
+            for (int j = 0; j < TM; j++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[i][j][e] = 0.0f;
+        acc_fence<TM, TN>(acc); /* the zeroes are written, and a few cycles pass, before the first MFMA reads them */
+        asm volatile("s_nop 7" ::: "memory");
+
+        bf16x8 f0[NF], f1[NF];
+        int ca = 0, cw = 0;                   /* ring slots of the step being multiplied */
+        unsigned va = a_frag, vw = w_frag;    /* this lane's fragment rows in those slots */
+        auto frag = [&](unsigned xa, unsigned xw, int coff, int q) -> bf16x8 {
+            return q < TN ? *(const bf16x8 *)(smem + xw + coff + q * 2048) : *(const bf16x8 *)(smem + xa + coff + (q - TN) * 2048);
+        };
+
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); /* step 0 is in LDS */
+        if (KT > 1) {
+#pragma unroll
+            for (int n = 0; n < NL; n++) issue1(1, 1, 1, nth(n));
+        }
+        if (KT > 2) {
+#pragma unroll
+            for (int n = 0; n < NL; n++) {
+                const int i = nth(n);
+                if (i < LA ? NSA == 3 : NSW == 3) issue1(2, 2, 2, i);
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < NF; q++) f0[q] = frag(va, vw, coff0, q);
+
+        auto serp = [](int b) { return ((b / TN) & 1) ? TN - 1 - b % TN : b % TN; };
+        /* steady: steps kt + 1 .. kt + 3 all exist, so every load below is issued and the wait count is exact; the last
+         * steps of a tile run with tests and wait for everything */
+        auto step = [&](int kt, auto steady_c) {
+            constexpr bool steady = decltype(steady_c)::value;
+            auto &accr = acc;
+            const bool more = steady || kt + 1 < KT;
+            const int na = ca == NSA - 1 ? 0 : ca + 1, nw = cw == NSW - 1 ? 0 : cw + 1;
+            const unsigned van = a_frag + na * ASZ, vwn = w_frag + nw * WSZ;
+#pragma unroll
+            for (int b = 0; b < NM; b++) {
+                MFMA_AGPR(accr[serp(b)][b / TN], f0[serp(b)], f0[TN + b / TN]);
+                if (b % RD == 0 && b / RD < NF) f1[b / RD] = frag(va, vw, coff1, b / RD);
+            }
+            if (more) {
+                /* step kt + 1 has landed for this wave and its reads of step kt are complete; past the barrier both
+                 * hold for all, and the slots of step kt are refilled below */
+                if (steady) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(AHEAD) : "memory");
+                else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            }
+#pragma unroll
+            for (int b = 0; b < NM; b++) {
+                MFMA_AGPR(accr[serp(b)][b / TN], f1[serp(b)], f1[TN + b / TN]);
+                if (more && b % RD == 0 && b / RD < NF) f0[b / RD] = frag(van, vwn, coff0, b / RD);
+                if (b % RD == 1 && b / RD < NL) {
+                    const int i = nth(b / RD);
+                    const int ahead = i < LA ? NSA : NSW;
+                    if (steady || kt + ahead < KT) issue1(kt + ahead, ca, cw, i);
+                }
+            }
+            ca = na;
+            cw = nw;
+            va = van;
+            vw = vwn;
+        };
+        int kt = 0;
+        for (; kt < KT - 3; kt++) step(kt, BoolC<true>{});
+        for (; kt < KT; kt++) step(kt, BoolC<false>{});
+
+        /* The next tile's first stage is requested before this tile is stored: every wave has taken
+         * its last fragments out of LDS once it is past this barrier. */
+        const TileId done = t;
+        vb += gridDim.x;
+        const bool again = vb < g.vgrid && decode_tile(g, vb, t);
+        if (again) {
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            set_sources(t);
+#pragma unroll
+            for (int n = 0; n < NL; n++) issue1(0, 0, 0, nth(n));
+        }
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); /* the last MFMA results retire before they are read */
+        acc_fence<TM, TN>(acc);
+
+        store_tile<BN, WM, WN, EPI>(g, done, acc, done.tml * BM, g.M[done.prob], wm, wn, l15, lq, done.tm * WGM + wm);
+        if (!again) break;
+    }
+}
+
 /* ------------------------------------------------------------------ host side */
 
 static int g_persistent = 1;
@@ -623,8 +777,47 @@ static int launch_4w(GemmArgs &g) {
     return 1;
 }
 
+static int g_ring = 1;
+extern "C" void flux_hip_linear_ring(int on) { g_ring = on; }
+
+/* The deep-ring form of the 4-wave tiles: one workgroup per compute unit at most, each walks its share of the tiles. */
+template <int TM, int TN, int EPI, int NSA, int NSW>
+static int launch_4d(GemmArgs &g) {
+    constexpr int BM = 32 * TM, BN = 32 * TN, LDS = (NSA * BM + NSW * BN) * 128;
+    static bool attr_done = false;
+    auto kern = gemm4d_kernel<TM, TN, EPI, NSA, NSW>;
+    if (!attr_done) {
+        HIP_OK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+        attr_done = true;
+    }
+    set_row_tiles(g, BM);
+    g.ntiles = g.N / BN;
+    g.nq_tiles = g.nq_cols / BN;
+    g.total_tiles = g.mtiles * g.ntiles;
+    size_t span = ((size_t)max(max(g.w_row0, g.w_row1), g.w_row2) + g.N) * g.ldw * 2;
+    for (int i = 0; i < GEMM_MAX_PARTS; i++) span = max(span, (size_t)g.M[i] * g.lda * 2);
+    if (span >= ((size_t)1 << 32)) return g.N % 128 == 0 ? launch_cfg<128, 128, 2, 2, EPI>(g) : launch_cfg<64, 64, 2, 2, EPI>(g);
+    g.vgrid = (g.total_tiles * g.ksplit + 7) & ~7;
+    const int grid = min(g.vgrid, compute_units() & ~7);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), LDS, flux_hip_stream_handle(), g);
+    HIP_OK(hipGetLastError());
+    return 1;
+}
+
 template <int EPI>
 static int launch_epi(GemmArgs &g, int tile) {
+    if (g_ring && g_persistent) {
+        /* three weight slots, two activation slots: in a denoising step the weights always come from HBM, the
+         * activations mostly from the memory-side cache (measured per kernel in a step, this split beat the other
+         * one by 0 - 10 %); the 192 x 192 tile has room for three of each */
+        switch (tile) {
+            case 2: return launch_4d<8, 8, EPI, 2, 3>(g);
+            case 5: return launch_4d<9, 6, EPI, 2, 3>(g);
+            case 6: return launch_4d<6, 6, EPI, 3, 3>(g);
+            case 7: return launch_4d<8, 6, EPI, 2, 3>(g);
+            default: break;
+        }
+    }
     switch (tile) {
         case 2: return launch_4w<8, 8, EPI>(g);
         case 5: return launch_4w<9, 6, EPI>(g);

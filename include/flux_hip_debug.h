@@ -16,18 +16,23 @@ extern "C" {
 #endif
 
 /* force_tile: 0/1/2/3/5/6/7 pins the GEMM tile of flux_hip_linear (64x128, 128x128, 256x256, 64x64,
- * 288x192, 192x192, 256x192; 4 = 256x256 in its 8-wave form, never chosen automatically), -1 restores
+ * 288x192, 192x192, 256x192; 4 = 256x256 in its 8-wave form, never chosen automatically; 8 / 9 = 64x128 / 128x128
+ * with a ring of 6 / 5 LDS stages, only for row ranges of at most 64 / 128 rows), -1 restores
  * the automatic choice (a tile whose width does not divide N is skipped; if none is left the 128x128
  * tile runs). */
 void flux_hip_linear_force_tile(int tile);
-/* bit t set = the automatic choice may use tile t (default 0xEF: all but tile 4; 0 restores it) */
+/* bit t set = the automatic choice may use tile t (default 0x3EF: all but tile 4; 0 restores it) */
 void flux_hip_linear_tile_mask(unsigned mask);
 /* 0 turns the split-K path off (default 1) */
 void flux_hip_linear_enable_splitk(int on);
 /* 1 (default): the 4-wave GEMM launches at most one workgroup per compute unit and each walks several
  * tiles; 0: one workgroup per tile */
 void flux_hip_linear_persistent(int on);
-/* 0 = 128-query workgroups, 1 = 256-query workgroups, -1 = automatic (default) */
+/* 1 (default): the 4-wave tiles run as gemm4d_kernel (operand rings of two or three LDS slots, count-based waits at
+ * the barrier); 0: as gemm4w_kernel (two stages, everything in flight awaited at the barrier). Bit-identical results. */
+void flux_hip_linear_ring(int on);
+/* attention kernel: -1 = automatic (default: 64-query waves, block lengths chosen per sequence length); 0 / 1 = the
+ * 32-query-per-wave kernel with 128 / 256 queries per workgroup; 11..14 = 16, 32, 48, 64 queries per wave throughout */
 void flux_hip_attention_force_variant(int v);
 /* 1 (default): a CFG step runs its two forwards as one batch of two sequences; 0: one after the other.
  * Takes effect at the next flux_hip_session_begin. */

@@ -43,6 +43,7 @@ def _default_switches(request):
         L.flux_hip_linear_tile_mask(0)
         L.flux_hip_linear_enable_splitk(1)
         L.flux_hip_linear_persistent(1)
+        L.flux_hip_linear_ring(1)
         L.flux_hip_attention_force_variant(-1)
         L.flux_hip_set_batched_cfg(1)
         L.flux_hip_set_fused_qkv_mlp(1)

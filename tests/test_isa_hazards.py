@@ -118,7 +118,7 @@ def lint(body):
 
 
 @pytest.mark.parametrize("src,extra,pattern", [("attention.hip", ["-fno-honor-nans"], "attention_wide_kernel"),
-                                               ("gemm.hip", [], "gemm4w_kernel")])
+                                               ("gemm.hip", [], "gemm4w_kernel"), ("gemm.hip", [], "gemm4d_kernel")])
 def test_inline_asm_mfma_hazards(src, extra, pattern, tmp_path):
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
