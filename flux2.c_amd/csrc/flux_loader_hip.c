@@ -353,6 +353,13 @@ static flux_transformer_t *load_from_handle(void *p) {
 
 flux_transformer_t *flux_transformer_load_safetensors(void *sf) { return load_from_handle(sf); }
 
+flux_transformer_t *flux_transformer_load(void *f) {
+    (void)f;
+    flux_hip_fail("flux_transformer_load: the binary weight format is not read by this backend; load the safetensors file "
+                  "(flux_transformer_load_safetensors)");
+    return NULL;
+}
+
 flux_transformer_t *flux_transformer_load_safetensors_mmap(void *sf) {
     /* Weights are device resident after loading, so the mapping is not needed afterwards; the
      * handle is still owned and closed on free, as callers of the reference expect

@@ -610,13 +610,29 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
     };
     /* the order in which a step issues its loads: the operand with the two-slot ring first (see the file comment) */
     auto nth = [](int n) { return NSA < NSW ? n : (n < LB ? LA + n : n - LB); };
-    set_sources(t);
+    /* The first K steps of a tile, as many as the rings hold beside the step that is multiplied first: requested
+     * before the previous tile is stored, so that they arrive while its results go out */
+    auto prime = [&](int KTn) {
 #pragma unroll
-    for (int n = 0; n < NL; n++) issue1(0, 0, 0, nth(n));
+        for (int n = 0; n < NL; n++) issue1(0, 0, 0, nth(n));
+        if (KTn > 1) {
+#pragma unroll
+            for (int n = 0; n < NL; n++) issue1(1, 1, 1, nth(n));
+        }
+        if (KTn > 2) {
+#pragma unroll
+            for (int n = 0; n < NL; n++) {
+                const int i = nth(n);
+                if (i < LA ? NSA == 3 : NSW == 3) issue1(2, 2, 2, i);
+            }
+        }
+    };
+    auto k_steps = [&](const TileId &tt) { return min(g.K >> 6, tt.ks * g.kt_per + g.kt_per) - tt.ks * g.kt_per; };
+    set_sources(t);
+    prime(k_steps(t));
 
     for (;;) {
-        const int kt_begin = t.ks * g.kt_per;
-        const int KT = min(g.K >> 6, kt_begin + g.kt_per) - kt_begin;
+        const int KT = k_steps(t);
 
         f32x4 acc[TN][TM];
 #pragma unroll
@@ -635,18 +651,8 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
             return q < TN ? *(const bf16x8 *)(smem + xw + coff + q * 2048) : *(const bf16x8 *)(smem + xa + coff + (q - TN) * 2048);
         };
 
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); /* step 0 is in LDS */
-        if (KT > 1) {
-#pragma unroll
-            for (int n = 0; n < NL; n++) issue1(1, 1, 1, nth(n));
-        }
-        if (KT > 2) {
-#pragma unroll
-            for (int n = 0; n < NL; n++) {
-                const int i = nth(n);
-                if (i < LA ? NSA == 3 : NSW == 3) issue1(2, 2, 2, i);
-            }
-        }
+        /* the tile's first steps are in LDS (they, and the previous tile's stores, were issued long ago) */
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
         for (int q = 0; q < NF; q++) f0[q] = frag(va, vw, coff0, q);
 
@@ -697,8 +703,7 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
         if (again) {
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
             set_sources(t);
-#pragma unroll
-            for (int n = 0; n < NL; n++) issue1(0, 0, 0, nth(n));
+            prime(k_steps(t));
         }
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); /* the last MFMA results retire before they are read */
         acc_fence<TM, TN>(acc);

@@ -249,6 +249,10 @@ flux_transformer_t *flux_hip_transformer_load_file(const char *path, const flux_
 struct safetensors_file;
 flux_transformer_t *flux_transformer_load_safetensors(void *sf);
 flux_transformer_t *flux_transformer_load_safetensors_mmap(void *sf);
+/* The reference's loader for its own binary weight format (flux_transformer.c:4059, declared at flux.c:45 and
+ * called from nowhere in its pipeline). Exported so that every flux_transformer_load* name of the reference
+ * resolves; the format is not read here: returns NULL and sets the error text. `f` is a FILE*. */
+flux_transformer_t *flux_transformer_load(void *f);
 void flux_transformer_free(flux_transformer_t *tf);
 
 typedef struct {
