@@ -42,7 +42,7 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA peak (datasheet)
 # `bench.py --calibrate` (profiles/gemm_qkv_swiglu_c4_traffic.txt, profiles/gemm_swiglu_c4_traffic.txt), scaled by
 # the same counters on a streaming kernel of known size.
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E peak (datasheet)
-TRAFFIC_BYTES = {("c4", True): 1_551_000_000, ("c4", False): 878_000_000}   # keyed by (workload, fused [Q|K|V|gate|up] launch)
+TRAFFIC_BYTES = {("c4", True): 1_361_000_000, ("c4", False): 878_000_000}   # keyed by (workload, fused [Q|K|V|gate|up] launch)
 
 # (latent h, w, text tokens, reference-image latents [(h, w, t_offset)], cfg, schedule steps)
 WORKLOADS = {
@@ -618,10 +618,12 @@ def main():
         # fused: only the single-stream blocks launch this kernel, all at [image + text tokens, H]; not fused: every
         # gate/up launch of the step, which all have that cost too
         per_ms = k_ms.value / k_n.value
-        k_flops, k_bytes = dominant_kernel_cost(cfg, n_img + nt, fused)
+        # a CFG step runs its two sequences as one batch: the launch then covers the rows of both
+        seqs = forwards if (fused and not args.sequential_cfg) else 1
+        k_flops, k_bytes = dominant_kernel_cost(cfg, seqs * (n_img + nt), fused)
         ach = k_flops / (per_ms * 1e-3) / 1e12
         gbps = k_bytes / (per_ms * 1e-3) / 1e9
-        alone_ms = time_dominant_kernel(cfg, n_img + nt, fused)
+        alone_ms = time_dominant_kernel(cfg, seqs * (n_img + nt), fused)
         what = "[Q|K|V|gate|up] projection of a single-stream block, bf16 store + SiLU(gate)*up" if fused else "gate/up projection + SiLU*up"
         # the launch is bound by whichever of the two it needs longer for at the datasheet rates
         if k_flops / (PEAK_BF16_TFLOPS * 1e12) >= k_bytes / (PEAK_HBM_GBPS * 1e9):
