@@ -598,8 +598,9 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
     /* The loop is software-pipelined inside each wave, because with one wave per SIMD nothing else overlaps the
      * softmax with the matrix pipe. The unit is a chunk of 32 keys (half a tile): while chunk u is exponentiated
      * and multiplied into O, the scores of chunk u + 1 are already being computed:
-     *   phase 1: S(u+1) = K Q^T - m   (8 NQ MFMAs)  with  P(u) = 2^S(u) -> bf16 (12 NQ vector instructions)
-     *   phase 2: row sums and O += V^T P(u)^T (9 NQ MFMAs), the requests for the next fragments and loads
+     *   phase 1: S(u+1) = K Q^T - m   (8 NQ MFMAs)  with  the conversion of 2^S(u) to bf16 P(u) (4 NQ vector instructions)
+     *   phase 2: row sums and O += V^T P(u)^T (9 NQ MFMAs)  with  2^S(u+1) (8 NQ exponentials), the requests for the
+     *            next fragments and the loads
      * Vector instructions sit one or two behind each MFMA; sched_barrier keeps them there. Two score buffers
      * alternate, so one trip of the loop is one tile: an "even" step (second chunk's scores, first chunk's
      * product) and an "odd" step (next tile's first chunk's scores, second chunk's product). One barrier per
@@ -607,6 +608,8 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
      * V(t+2); everything read before the next barrier landed before this one (three slots per ring), so
      * fragments are requested from LDS a phase ahead of their MFMAs, across the barrier too.
      * The reference maxima are fixed on the first chunk, see first_reference. */
+    constexpr int EXP0 = NQ < 2 ? 4 : 0; /* with 16 queries per wave the score phase is so short that the first exponentials wait four MFMAs */
+    constexpr int CVT0 = NQ; /* the conversions start NQ MFMAs into the score phase: the product phase's last readers of P have long issued */
     f32x4 s_a[2][NQ], s_b[2][NQ];
     bf16x8 kf[4][2];  /* K fragments of a chunk: [32-dim step of the head dim][key block of the chunk] */
     bf16x8 vf[2][4];  /* V^T fragments: [half of the head dim][16-row block] */
@@ -625,20 +628,23 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
     };
     /* The vector instructions of the loop are inline assembly as well: an ordinary expression the compiler may
      * sink to its use in the next phase, and then nothing overlaps.
-     * One instruction of the exponentiation of a chunk: k = 0 .. 12 NQ - 1, per query block eight exponentials and
-     * then four conversions of pairs (a conversion reads exponentials issued at least four instructions earlier). */
-    auto exp_op = [&](f32x4 (&sc)[2][NQ], int k) {
-        const int j = k / 12, r = k % 12;
-        if (r < 8) {
-            float x = sc[r >> 2][j][r & 3];
-            asm volatile("v_exp_f32_e32 %0, %0" : "+v"(x));
-            sc[r >> 2][j][r & 3] = x;
-        } else {
-            const int hh = r - 8, i = hh >> 1, e = 2 * (hh & 1);
-            unsigned w;
-            asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(w) : "v"(sc[i][j][e]), "v"(sc[i][j][e + 1]));
-            pf[j][hh] = w;
-        }
+     * The exponentiation of a chunk is 8 NQ exponentials (16 cycles of the transcendental unit each) and 4 NQ
+     * conversions of pairs. The exponentials run behind the MFMAs of the product phase BEFORE (the chunk's scores are
+     * complete by then: the MFMA that finishes query block j, key block i is the (2 NQ - i NQ - j)-th from the end
+     * of the score phase, and its eight exponentials come 8 j + 4 i MFMAs into the product phase, behind the NQ
+     * row-sum MFMAs), the conversions behind the first MFMAs of the chunk's own score phase: that way both phases
+     * carry about as much vector work as matrix work, instead of all of it sitting in the score phase. */
+    auto exp1 = [&](f32x4 (&sc)[2][NQ], int n) { /* n = 0 .. 8 NQ - 1: query block n / 8, its eight scores in turn */
+        const int j = n >> 3, r = n & 7;
+        float x = sc[r >> 2][j][r & 3];
+        asm volatile("v_exp_f32_e32 %0, %0" : "+v"(x));
+        sc[r >> 2][j][r & 3] = x;
+    };
+    auto cvt1 = [&](f32x4 (&sc)[2][NQ], int n) { /* n = 0 .. 4 NQ - 1: query block n / 4, its four pairs in turn */
+        const int j = n >> 2, hh = n & 3, i = hh >> 1, e = 2 * (hh & 1);
+        unsigned w;
+        asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(w) : "v"(sc[i][j][e]), "v"(sc[i][j][e + 1]));
+        pf[j][hh] = w;
     };
     /* lane-wise maximum of a chunk's scores, one instruction at a time: 4 per query block (three-operand maxima
      * over the block's 8 values), the query blocks taking turns so that dependent instructions lie NQ apart */
@@ -747,6 +753,8 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
     for (int k = 0; k < 4 * NQ; k++) max_op(s_a, k);
     first_reference(s_a);
 #pragma unroll
+    for (int n = 0; n < 8 * NQ; n++) exp1(s_a, n);
+#pragma unroll
     for (int x = 0; x < 8; x++) kfrag1(0, 1, x);
 
     /* Even step of tile t (slot sl = t % 3): scores of its second chunk into s_b, product of its first chunk.
@@ -754,13 +762,15 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
     auto even_step = [&](int t, int sl, int sn, auto guard_c) {
         s_phase(s_b, [&](int m) {
             if (m < 8) vfrag1(sl, 0, m);
-#pragma unroll
-            for (int k = (m * 3) / 2; k < ((m + 1) * 3) / 2; k++) exp_op(s_a, k);
+            if (m >= CVT0 && m < CVT0 + 4 * NQ) cvt1(s_a, m - CVT0);
         }, guard_c);
         mask_chunk(s_b, 2 * t + 1);
         pv_phase([&](int m) {
             if (m < 8 && t + 1 < ntiles) kfrag1(sn, 0, m);
+            if (m >= EXP0) exp1(s_b, m - EXP0);
         }, guard_c);
+#pragma unroll
+        for (int n = 8 * NQ - EXP0; n < 8 * NQ; n++) exp1(s_b, n);
     };
     /* Odd step of tile t: the barrier, the loads of K(t+3) and V(t+2), scores of tile t+1's first chunk into s_a,
      * product of tile t's second chunk. sp = (t + 2) % 3 is the slot V(t+2) goes to. */
@@ -769,25 +779,27 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
         __syncthreads();
         s_phase(s_a, [&](int m) {
             if (m < 8) vfrag1(sl, 1, m);
-#pragma unroll
-            for (int k = (m * 3) / 2; k < ((m + 1) * 3) / 2; k++) exp_op(s_b, k);
+            if (m >= CVT0 && m < CVT0 + 4 * NQ) cvt1(s_b, m - CVT0);
         }, AttFlag<false>{});
         mask_chunk(s_a, 2 * t + 2);
         pv_phase([&](int m) {
             if (m < 8) kfrag1(sn, 1, m);
+            if (m >= EXP0) exp1(s_a, m - EXP0);
             if (m >= 8 * NQ - 2 * LP) { /* the tile's eight loads behind the last eight MFMAs */
                 const int i = m - (8 * NQ - 2 * LP);
                 if (i & 1) issue_v1(sp, min(t + 2, ntiles - 1), i >> 1);
                 else issue_k1(sl, min(t + 3, ntiles - 1), i >> 1);
             }
         }, AttFlag<false>{});
+#pragma unroll
+        for (int n = 8 * NQ - EXP0; n < 8 * NQ; n++) exp1(s_a, n);
     };
     /* the last chunk: nothing left to overlap */
     auto last_step = [&](int sl) {
 #pragma unroll
         for (int x = 0; x < 8; x++) vfrag1(sl, 1, x);
 #pragma unroll
-        for (int k = 0; k < 12 * NQ; k++) exp_op(s_b, k);
+        for (int n = 0; n < 4 * NQ; n++) cvt1(s_b, n);
         __builtin_amdgcn_sched_barrier(0);
         pv_phase(nothing, AttFlag<true>{});
     };
