@@ -320,7 +320,7 @@ def bench_qwen3(args):
         "tflops": round(flops * K / wall / 1e12, 1), "flops_per_step": flops, "roofline": roof, "cpu_baseline": cpu}))
 
 
-ATT_WORKLOADS = {"att_c2": 768, "att_c3": 1536, "att_c4": 4608, "att_c5": 2560}
+ATT_WORKLOADS = {"att_c1": 80, "att_c2": 768, "att_c3": 1536, "att_c4": 4608, "att_c5": 2560}   # tokens (text first: 64 at c1, else 512)
 
 
 def bench_attention(args):
@@ -329,6 +329,7 @@ def bench_attention(args):
     block runs them. The roofline object is the attention kernel by itself (HIP events around runs of it)."""
     n, heads = ATT_WORKLOADS[args.workload], KLEIN_4B.heads
     H = heads * 128
+    split = 64 if n < 512 else 512
     fluxhip.init()
     L = fluxhip.lib()
     L.flux_hip_attention_force_variant(args.attention_variant)
@@ -340,10 +341,10 @@ def bench_attention(args):
     kn, vt, out = fluxhip.DevBuf(n * H * 2), fluxhip.DevBuf(H * ldvt * 2), fluxhip.DevBuf(n * H * 2)
 
     def prep():
-        fluxhip.check(L.flux_hip_kv_prepare(kn.ptr, vt.ptr, ldvt, qkv.ptr, 3 * H, H, 2 * H, n, heads, 512, w.ptr, w.ptr, cos.ptr, sin.ptr, 1e-6))
+        fluxhip.check(L.flux_hip_kv_prepare(kn.ptr, vt.ptr, ldvt, qkv.ptr, 3 * H, H, 2 * H, n, heads, split, w.ptr, w.ptr, cos.ptr, sin.ptr, 1e-6))
 
     def att():
-        fluxhip.check(L.flux_hip_attention(out.ptr, H, qkv.ptr, 3 * H, kn.ptr, vt.ptr, ldvt, n, n, heads, 512, w.ptr, w.ptr, cos.ptr, sin.ptr, 1e-6))
+        fluxhip.check(L.flux_hip_attention(out.ptr, H, qkv.ptr, 3 * H, kn.ptr, vt.ptr, ldvt, n, n, heads, split, w.ptr, w.ptr, cos.ptr, sin.ptr, 1e-6))
 
     for _ in range(max(args.warmup, 1)):
         prep(); att()
@@ -372,7 +373,7 @@ def bench_attention(args):
         "metric": f"attention calls/s ({n} tokens, {heads} heads, 1 GPU)", "value": round(args.steps / wall, 2), "unit": "calls/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1000.0 / args.steps, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: K/V preparation + joint attention over {n} tokens (512 text), {heads} heads x 128, N(0,1) bf16 "
+        "config": {"workload": f"{args.workload}: K/V preparation + joint attention over {n} tokens ({split} text), {heads} heads x 128, N(0,1) bf16 "
                                f"q/k/v, unit QK-norm weights, random RoPE angles; variant {args.attention_variant}"},
         "device_ms_per_step_events": round(ev_ms / args.steps, 4),
         "roofline": {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4),

@@ -50,6 +50,18 @@
  * per SIMD) on the 256 x 256 tile it runs at the speed of the 4-wave form and is kept for comparison
  * runs (tile id 4).
  *
+ * Three kernels, then: gemm_kernel (small tiles; with NS > 2 a ring of NS LDS stages for row ranges of few
+ * rows, where a launch only streams weights), gemm4w_kernel (large tiles, two LDS stages; convolutions, and the
+ * comparison form of the next one) and gemm4d_kernel (large tiles with an LDS ring per operand, the form the
+ * transformer's projections run). What separates the last two is the barrier: __syncthreads() carries a fence
+ * that waits for every global->LDS load in flight, so a two-stage loop can never have more than the next stage
+ * on its way, requested one to two half-steps earlier; operands that come from HBM arrive later than that now and
+ * then, and a wave that waits holds its three neighbours up at the barrier (measured: the same launch takes
+ * 232-241 us when its operands are reused from the memory-side cache and 272-277 us when they rotate through
+ * six buffer sets; a copy without the barrier does not care). gemm4d_kernel waits with a count instead
+ * (s_waitcnt vmcnt(n) + s_barrier in one asm statement): everything but the last n loads, which belong to the
+ * operand whose ring has a third slot and are needed a whole K step later.
+ *
  * LDS rows are 128 bytes (64 bf16); the 16-byte chunk index is XOR-swizzled with a function of
  * the row so that the 16 rows a fragment read touches spread over all banks. A direct-to-LDS
  * load writes lane i's 16 bytes at (wave base + 16 i), so the swizzle is applied on the global
