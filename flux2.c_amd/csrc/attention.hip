@@ -618,13 +618,27 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
     /* Fragments are requested from LDS a whole phase before the MFMAs that read them (the chunk's eight K
      * fragments during the product phase before, its eight V^T fragments during the score phase before), one
      * read behind each of the phase's first eight MFMAs: no MFMA waits for LDS. */
-    auto kfrag1 = [&](int slot, int cp, int x) { /* x = 0..7: key block 2cp + x%2 of the tile, head dims 32 (x/2) .. +31 */
+    /* Per-lane LDS addresses of the fragments in the slots that are read next, kept in registers and moved on by one
+     * slot per tile (recomputed from the slot number they cost a vector add per read): the K fragments of head-dim
+     * step kk, key block 0 of chunk 0 (the others lie 4096 (2 cp + i) further), and the V^T fragments of chunk cp,
+     * head-dim block 0 (block x lies 2048 x further). */
+    unsigned ka[4], va[2];
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) ka[kk] = l15 * 256 + (((kk * 4 + lq) ^ l15) << 4);
+#pragma unroll
+    for (int cp = 0; cp < 2; cp++) va[cp] = 3 * 16384 + l15 * 128 + (((4 * cp + lq) ^ vt_swz(l15)) << 4);
+    auto kfrag1 = [&](int cp, int x) { /* x = 0..7: key block 2cp + x%2 of the tile, head dims 32 (x/2) .. +31 */
         const int kk = x >> 1, i = x & 1;
-        kf[kk][i] = *(const bf16x8 *)(smem + slot * 16384 + ((2 * cp + i) * 16 + l15) * 256 + (((kk * 4 + lq) ^ l15) << 4));
+        kf[kk][i] = *(const bf16x8 *)(smem + ka[kk] + (2 * cp + i) * 4096);
     };
-    auto vfrag1 = [&](int slot, int cp, int x) { /* x = 0..7: head-dim block x, keys of 32-key chunk cp */
-        const int d = x * 16 + l15;
-        vf[x >> 2][x & 3] = *(const bf16x8 *)(smem + 3 * 16384 + slot * 16384 + d * 128 + (((4 * cp + lq) ^ vt_swz(d)) << 4));
+    auto vfrag1 = [&](int cp, int x) { /* x = 0..7: head-dim block x, keys of 32-key chunk cp */
+        vf[x >> 2][x & 3] = *(const bf16x8 *)(smem + va[cp] + x * 2048);
+    };
+    auto move_slots = [&](int dk, int dv) { /* byte distances to the next K slot and the next V^T slot */
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) ka[kk] += dk;
+#pragma unroll
+        for (int cp = 0; cp < 2; cp++) va[cp] += dv;
     };
     /* The vector instructions of the loop are inline assembly as well: an ordinary expression the compiler may
      * sink to its use in the next phase, and then nothing overlaps.
@@ -745,7 +759,7 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads(); /* K(0), V(0), K(1), V(1), K(2) are in LDS */
 #pragma unroll
-    for (int x = 0; x < 8; x++) kfrag1(0, 0, x);
+    for (int x = 0; x < 8; x++) kfrag1(0, x);
     s_phase(s_a, nothing, AttFlag<true>{});
     fence_scores(s_a);
     mask_chunk(s_a, 0);
@@ -755,18 +769,19 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
 #pragma unroll
     for (int n = 0; n < 8 * NQ; n++) exp1(s_a, n);
 #pragma unroll
-    for (int x = 0; x < 8; x++) kfrag1(0, 1, x);
+    for (int x = 0; x < 8; x++) kfrag1(1, x);
+    move_slots(16384, 0); /* K fragments now come from tile 1's slot, V^T fragments from tile 0's */
 
     /* Even step of tile t (slot sl = t % 3): scores of its second chunk into s_b, product of its first chunk.
      * The first K fragments of the odd step's chunk (first chunk of tile t + 1, slot sn) are requested meanwhile. */
     auto even_step = [&](int t, int sl, int sn, auto guard_c) {
         s_phase(s_b, [&](int m) {
-            if (m < 8) vfrag1(sl, 0, m);
+            if (m < 8) vfrag1(0, m);
             if (m >= CVT0 && m < CVT0 + 4 * NQ) cvt1(s_a, m - CVT0);
         }, guard_c);
         mask_chunk(s_b, 2 * t + 1);
         pv_phase([&](int m) {
-            if (m < 8 && t + 1 < ntiles) kfrag1(sn, 0, m);
+            if (m < 8 && t + 1 < ntiles) kfrag1(0, m);
             if (m >= EXP0) exp1(s_b, m - EXP0);
         }, guard_c);
 #pragma unroll
@@ -778,12 +793,12 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
         __builtin_amdgcn_s_waitcnt(0x0F70); /* this wave's parts of K(t+2) and V(t+1) are in LDS */
         __syncthreads();
         s_phase(s_a, [&](int m) {
-            if (m < 8) vfrag1(sl, 1, m);
+            if (m < 8) vfrag1(1, m);
             if (m >= CVT0 && m < CVT0 + 4 * NQ) cvt1(s_b, m - CVT0);
         }, AttFlag<false>{});
         mask_chunk(s_a, 2 * t + 2);
         pv_phase([&](int m) {
-            if (m < 8) kfrag1(sn, 1, m);
+            if (m < 8) kfrag1(1, m);
             if (m >= EXP0) exp1(s_a, m - EXP0);
             if (m >= 8 * NQ - 2 * LP) { /* the tile's eight loads behind the last eight MFMAs */
                 const int i = m - (8 * NQ - 2 * LP);
@@ -797,7 +812,7 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
     /* the last chunk: nothing left to overlap */
     auto last_step = [&](int sl) {
 #pragma unroll
-        for (int x = 0; x < 8; x++) vfrag1(sl, 1, x);
+        for (int x = 0; x < 8; x++) vfrag1(1, x);
 #pragma unroll
         for (int n = 0; n < 4 * NQ; n++) cvt1(s_b, n);
         __builtin_amdgcn_sched_barrier(0);
@@ -808,6 +823,7 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
         for (int t = 0; t < ntiles - 1; t++) {
             even_step(t, sl, sn, AttFlag<false>{});
             odd_step(t, sl, sn, sp);
+            move_slots((sp - sn) * 16384, (sn - sl) * 16384);
             const int r = sl; sl = sn; sn = sp; sp = r;
         }
         even_step(ntiles - 1, sl, sn, AttFlag<true>{});
