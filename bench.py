@@ -466,7 +466,7 @@ def bench_gemm_vs_library(args):
     fluxhip.init()
     L = fluxhip.lib()
     L.flux_hip_linear_enable_splitk(0)
-    NB, launches = 4, max(args.steps, 4)
+    NB, launches, warm = 4, max(args.steps, 4), 40
     rows = {}
     t0 = time.perf_counter()
     for name, (M, N, K) in GEMM_SHAPES.items():
@@ -479,8 +479,15 @@ def bench_gemm_vs_library(args):
         def mine(j):
             fluxhip.linear(fluxhip.EPI_BF16, [(a[j].ptr, w[j].ptr, c.ptr, None, M)], N, K, K, K, N)
 
+        ta = [torch.from_numpy(x.view(np.int16)).cuda().view(torch.bfloat16) for x in a_h]
+        tw = [torch.from_numpy(x.view(np.int16)).cuda().view(torch.bfloat16) for x in w_h]
+        out = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+
+        def lib(j):
+            torch.matmul(ta[j], tw[j].t(), out=out)
+
         def timed_mine(rot):
-            for i in range(3 * NB):
+            for i in range(warm):
                 mine(i % NB if rot else 0)
             fluxhip.sync()
             L.flux_hip_timer_start()
@@ -488,29 +495,30 @@ def bench_gemm_vs_library(args):
                 mine(i % NB if rot else 0)
             return L.flux_hip_timer_stop() / launches
 
-        m_same, m_rot = timed_mine(False), timed_mine(True)
-        ta = [torch.from_numpy(x.view(np.int16)).cuda().view(torch.bfloat16) for x in a_h]
-        tw = [torch.from_numpy(x.view(np.int16)).cuda().view(torch.bfloat16) for x in w_h]
-        out = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
-
         def timed_lib(rot):
-            for i in range(3 * NB):
-                torch.matmul(ta[i % NB if rot else 0], tw[i % NB if rot else 0].t(), out=out)
+            for i in range(warm):
+                lib(i % NB if rot else 0)
             torch.cuda.synchronize()
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             for i in range(launches):
-                torch.matmul(ta[i % NB if rot else 0], tw[i % NB if rot else 0].t(), out=out)
+                lib(i % NB if rot else 0)
             e1.record()
             torch.cuda.synchronize()
             return e0.elapsed_time(e1) / launches
 
-        l_same, l_rot = timed_lib(False), timed_lib(True)
+        # the clocks take a second to settle after the uploads, and they drift with what ran before: the four
+        # measurements take turns, three rounds, and each reports its best round
+        m_same = m_rot = l_same = l_rot = 1e9
+        for _ in range(3):
+            m_same = min(m_same, timed_mine(False))
+            l_same = min(l_same, timed_lib(False))
+            m_rot = min(m_rot, timed_mine(True))
+            l_rot = min(l_rot, timed_lib(True))
         mine(0)
         fluxhip.sync()
         got = bf16_to_f32_host(c.to_array(np.uint16, (M, N))[:64])
-        ref = out[:64].float().cpu().numpy() if False else None
-        torch.matmul(ta[0], tw[0].t(), out=out)
+        lib(0)
         ref = out[:64].float().cpu().numpy()
         err = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
         assert err < 1e-2, (name, err)
@@ -530,7 +538,7 @@ def bench_gemm_vs_library(args):
     k = rows["fused_qkv_gate_up"]["flux_hip_linear"]
     print(json.dumps({
         "metric": "bf16 GEMM TFLOP/s on the step's projection shapes, this backend against the vendor library (1 GPU)",
-        "value": k["rotating_tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": launches, "warmup": 3 * NB, "ms_per_step": None,
+        "value": k["rotating_tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": launches, "warmup": warm, "ms_per_step": None,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "gemm_vs_lib: C = A W^T, bf16 in and out, fp32 accumulation; value = flux_hip_linear at [4608,3072] x [27648,3072]^T "
                                f"with operands from HBM; library = torch {torch.__version__} matmul"},
