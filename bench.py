@@ -549,6 +549,37 @@ def bench_gemm_vs_library(args):
         "cpu_baseline": None}))
 
 
+def bench_mfma_issue(args):
+    """What another instruction costs a lone wave when it sits between that wave's MFMAs (flux_hip_mfma_issue_cost:
+    one workgroup of four waves per compute unit, 16 independent accumulator blocks per wave, one instruction of the
+    given kind behind every n-th MFMA): clock cycles per MFMA, 16 = the matrix pipe never waits. The GEMM and
+    attention kernels run one wave per SIMD, so these are the costs their loops pay."""
+    import ctypes
+    fluxhip.init()
+    L = fluxhip.lib()
+    L.flux_hip_mfma_issue_cost.argtypes = [ctypes.c_int] * 3 + [ctypes.POINTER(ctypes.c_float)] * 2
+    kinds = {0: "nothing", 1: "global_load_lds_dwordx4", 2: "ds_read_b128", 3: "v_exp_f32", 4: "3 x v_fma_f32",
+             5: "global_load_dwordx4 + ds_write_b128"}
+    iters = 4000
+    table = []
+    for mode, name in kinds.items():
+        for every in ((4,) if mode == 0 else (16, 8, 4, 2, 1)):
+            c, g = ctypes.c_float(0.0), ctypes.c_float(0.0)
+            fluxhip.check(L.flux_hip_mfma_issue_cost(mode, every, iters, ctypes.byref(c), ctypes.byref(g)), "flux_hip_mfma_issue_cost")
+            table.append({"between_the_mfmas": name, "one_per_mfmas": every, "cycles_per_mfma": round(c.value, 2), "core_ghz": round(g.value, 2)})
+    base = table[0]["cycles_per_mfma"]
+    for r in table[1:]:
+        r["cycles_per_instruction_beyond_the_loop_alone"] = round((r["cycles_per_mfma"] - base) * r["one_per_mfmas"], 1)
+    dma8 = next(r for r in table if r["between_the_mfmas"] == "global_load_lds_dwordx4" and r["one_per_mfmas"] == 8)
+    print(json.dumps({
+        "metric": "matrix-pipe cycles per MFMA of a lone wave with one global->LDS load behind every 8th MFMA (16 = no loss, 1 GPU)",
+        "value": dma8["cycles_per_mfma"], "unit": "cycles", "n_gpus": 1, "steps": 2, "warmup": 1, "ms_per_step": None,
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"mfma_issue: {iters} x 16 v_mfma_f32_16x16x32_bf16 per wave, four waves per compute unit, one other instruction "
+                               "behind every n-th MFMA"},
+        "table": table, "roofline": None, "cpu_baseline": None}))
+
+
 def bf16_to_f32_host(a):
     return (a.astype(np.uint32) << 16).view(np.float32)
 
@@ -592,7 +623,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=8)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + sorted(VAE_WORKLOADS) + sorted(ATT_WORKLOADS) + sorted(BW_WORKLOADS) + ["qwen3", "mfma_peak", "gemm_vs_lib"])
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + sorted(VAE_WORKLOADS) + sorted(ATT_WORKLOADS) + sorted(BW_WORKLOADS) + ["qwen3", "mfma_peak", "mfma_issue", "gemm_vs_lib"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     ap.add_argument("--tile-mask", type=lambda v: int(v, 0), default=0,
@@ -625,6 +656,8 @@ def main():
         return bench_bandwidth(args)
     if args.workload == "gemm_vs_lib":
         return bench_gemm_vs_library(args)
+    if args.workload == "mfma_issue":
+        return bench_mfma_issue(args)
     cfg = KLEIN_4B
     wl = WORKLOADS[args.workload]
     if args.calibrate:

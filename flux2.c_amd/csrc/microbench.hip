@@ -10,7 +10,12 @@
  * from one MFMA to the next, as in the GEMM kernel. The MFMAs are written as inline assembly: left
  * to the compiler's builtin, a loop with one wave per SIMD moves accumulators between the two
  * register files between the MFMAs and measures that instead.
+ *
+ * A second loop (mfma_issue_kernel) measures what another instruction costs a lone wave when it sits between
+ * that wave's MFMAs: the GEMM and attention kernels run one wave per SIMD, so whatever such an instruction keeps
+ * the wave's issue slot for beyond the 16 cycles of the MFMA before it is time the matrix pipe idles.
  */
+#include <stdlib.h>
 #include "common.h"
 #include "../../include/flux_hip.h"
 #include "../../include/flux_hip_debug.h"
@@ -130,5 +135,143 @@ extern "C" int flux_hip_mfma_peak(int shape, int pattern, int waves_per_simd, in
     if (!ok) return flux_hip_fail("flux_hip_mfma_peak: launch or timing failed: %s", hipGetErrorString(hipGetLastError()));
     const double flops = (double)cus * (threads / 64) * (double)iters * 16.0 * (shape == 0 ? 16384.0 : 32768.0);
     *tflops = (float)(flops / (best * 1e-3) / 1e12);
+    return 1;
+}
+
+/* ---------------------------------------------------------------------------------------
+ * Cost of an instruction between a lone wave's MFMAs. Every wave runs `iters` x 16 independent MFMAs
+ * (16 accumulator blocks) and behind every EVERY-th MFMA one instruction of kind MODE:
+ *   0 nothing, 1 global_load_lds_dwordx4 (1 KB per wave from the workgroup's own 64 KB of a buffer, into its own LDS
+ *   region), 2 ds_read_b128, 3 v_exp_f32, 4 three v_fma_f32, 5 global_load_dwordx4 followed a round later by ds_write_b128
+ * and reports its cycle count (clock64 around the loop). One workgroup of four waves per compute unit.
+ * --------------------------------------------------------------------------------------- */
+#define MB_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
+#define MB_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
+template <int MODE, int EVERY>
+__global__ __launch_bounds__(256) void mfma_issue_kernel(const char *buf, int iters, long long *cyc, float *sink) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    f32x4 acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) acc[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    bf16x8 a = operand(1, threadIdx.x), b = operand(1, threadIdx.x + 4096u);
+    const char *src = buf + (size_t)blockIdx.x * 65536 + wave * 1024; /* this wave's KB of each 4 KB step */
+    const unsigned voff = lane * 16;
+    const char *base = src + voff;
+    const unsigned lds = wave * 16384 + lane * 16;
+    u32x4 r[4] = {};
+    u32x4 rd = {};
+    float x[4] = {0.5f, 0.25f, 0.125f, 0.75f}, y[3] = {1.0f, 2.0f, 3.0f};
+    unsigned pos = 0;
+    asm volatile("s_nop 7" ::: "memory");
+    const long long t0 = clock64();
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int m = 0; m < 16; m++) {
+            asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[m]) : "v"(a), "v"(b));
+            if (m % EVERY == 0) {
+                const int n = m / EVERY;
+                if (MODE == 1) __builtin_amdgcn_global_load_lds(MB_GLOBAL_PTR(base + pos), MB_LDS_PTR(smem + wave * 16384 + (n & 7) * 1024), 16, 0, 0);
+                if (MODE == 2) asm volatile("ds_read_b128 %0, %1" : "=v"(rd) : "v"(lds + (n & 7) * 1024) : "memory");
+                if (MODE == 3) asm volatile("v_exp_f32_e32 %0, %0" : "+v"(x[n & 3]));
+                if (MODE == 4) {
+#pragma unroll
+                    for (int e = 0; e < 3; e++) asm volatile("v_fma_f32 %0, %0, %1, %1" : "+v"(y[e]) : "v"(x[0]));
+                }
+                if (MODE == 5) {
+                    asm volatile("s_waitcnt vmcnt(3)\n\tds_write_b128 %0, %1" ::"v"(lds + (n & 7) * 1024), "v"(r[n & 3]) : "memory");
+                    /* the load as assembly as well: the wait for it is the one written above, a round later */
+                    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(r[n & 3]) : "v"(voff), "s"(src + pos) : "memory");
+                }
+                pos = (pos + 4096u) & 0xFFFFu;
+            }
+        }
+        if (MODE == 2) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+    const long long t1 = clock64();
+    float s = x[0] + x[1] + x[2] + x[3] + y[0] + y[1] + y[2] + (float)rd[0];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        asm volatile("" : "+a"(acc[i]));
+        s += acc[i][0];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) s += (float)r[j][0];
+    if (lane == 0) cyc[blockIdx.x * 4 + wave] = t1 - t0;
+    if (s == 12345.678f) sink[0] = s;
+}
+
+template <int MODE>
+static int issue_launch(int every, int cus, hipStream_t st, const char *buf, int iters, long long *cyc, float *sink) {
+#define MB_CASE(E) \
+    case E: { \
+        auto kern = mfma_issue_kernel<MODE, E>; \
+        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 65536) != hipSuccess) return 0; \
+        hipLaunchKernelGGL(kern, dim3(cus), dim3(256), 65536, st, buf, iters, cyc, sink); \
+        return hipGetLastError() == hipSuccess; \
+    }
+    switch (every) {
+        MB_CASE(1) MB_CASE(2) MB_CASE(4) MB_CASE(8) MB_CASE(16)
+        default: return 0;
+    }
+#undef MB_CASE
+}
+
+/*
+ * mode as above (0..5), every = 1, 2, 4, 8 or 16 MFMAs per interleaved instruction. Returns the average number of
+ * clock cycles per MFMA over all waves in *cycles_per_mfma (16 = the matrix pipe never waits) and the core clock
+ * during the run in *ghz (cycle counter against the launch's duration).
+ */
+extern "C" int flux_hip_mfma_issue_cost(int mode, int every, int iters, float *cycles_per_mfma, float *ghz) {
+    if (!flux_hip_available()) return 0;
+    if (mode < 0 || mode > 5 || iters < 1 || iters > (1 << 20) || !cycles_per_mfma || !ghz) return flux_hip_fail("flux_hip_mfma_issue_cost: bad argument");
+    int dev = 0, cus = 0;
+    HIP_OK(hipGetDevice(&dev));
+    HIP_OK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    char *buf = nullptr;
+    long long *cyc = nullptr;
+    float *sink = nullptr;
+    const size_t bytes = (size_t)(cus + 1) * 65536;
+    HIP_OK(hipMalloc((void **)&buf, bytes));
+    HIP_OK(hipMalloc((void **)&cyc, (size_t)cus * 4 * sizeof(long long)));
+    HIP_OK(hipMalloc((void **)&sink, sizeof(float)));
+    hipStream_t st = flux_hip_stream_handle();
+    hipEvent_t e0, e1;
+    HIP_OK(hipEventCreate(&e0));
+    HIP_OK(hipEventCreate(&e1));
+    int ok = hipMemsetAsync(buf, 1, bytes, st) == hipSuccess;
+    float best = 1e30f;
+    for (int l = 0; l < 3 && ok; l++) { /* the first launch is a warm-up */
+        ok = hipEventRecord(e0, st) == hipSuccess;
+        switch (mode) {
+            case 0: ok = ok && issue_launch<0>(every, cus, st, buf, iters, cyc, sink); break;
+            case 1: ok = ok && issue_launch<1>(every, cus, st, buf, iters, cyc, sink); break;
+            case 2: ok = ok && issue_launch<2>(every, cus, st, buf, iters, cyc, sink); break;
+            case 3: ok = ok && issue_launch<3>(every, cus, st, buf, iters, cyc, sink); break;
+            case 4: ok = ok && issue_launch<4>(every, cus, st, buf, iters, cyc, sink); break;
+            default: ok = ok && issue_launch<5>(every, cus, st, buf, iters, cyc, sink); break;
+        }
+        ok = ok && hipEventRecord(e1, st) == hipSuccess && hipEventSynchronize(e1) == hipSuccess;
+        float ms = 0.0f;
+        ok = ok && hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+        if (ok && l > 0 && ms < best) best = ms;
+    }
+    double avg = 0.0;
+    if (ok) {
+        long long *h = (long long *)malloc((size_t)cus * 4 * sizeof(long long));
+        ok = h && hipMemcpy(h, cyc, (size_t)cus * 4 * sizeof(long long), hipMemcpyDeviceToHost) == hipSuccess;
+        for (int i = 0; ok && i < cus * 4; i++) avg += (double)h[i];
+        free(h);
+        avg /= (double)cus * 4;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(buf);
+    (void)hipFree(cyc);
+    (void)hipFree(sink);
+    if (!ok) return flux_hip_fail("flux_hip_mfma_issue_cost: launch or timing failed (every must be 1, 2, 4, 8 or 16): %s", hipGetErrorString(hipGetLastError()));
+    *cycles_per_mfma = (float)(avg / ((double)iters * 16.0));
+    *ghz = (float)(avg / (best * 1e-3) / 1e9);
     return 1;
 }

@@ -59,6 +59,11 @@ int flux_hip_linear_probe_read_launches(int max, int *tiles, float *ms);
  * v_mfma_f32_16x16x32_bf16, 1 = v_mfma_f32_32x32x16_bf16; pattern 0 = all-zero operands, 1 = values in
  * [1, 2) with a random low byte, 2 = random bit patterns. `bench.py --workload mfma_peak` prints the table. */
 int flux_hip_mfma_peak(int shape, int pattern, int waves_per_simd, int iters, int launches, float *tflops);
+/* What an instruction between a lone wave's MFMAs costs the matrix pipe (csrc/microbench.hip): mode 0 nothing,
+ * 1 global_load_lds_dwordx4, 2 ds_read_b128, 3 v_exp_f32, 4 three v_fma_f32, 5 global_load_dwordx4 + ds_write_b128; one
+ * such instruction behind every `every`-th MFMA (1, 2, 4, 8, 16). Returns clock cycles per MFMA (16 = no loss) and
+ * the core clock of the run. */
+int flux_hip_mfma_issue_cost(int mode, int every, int iters, float *cycles_per_mfma, float *ghz);
 
 #ifdef __cplusplus
 }
