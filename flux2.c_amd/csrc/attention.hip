@@ -57,7 +57,10 @@ __global__ __launch_bounds__(256) void kv_prepare_kernel(bf16 *__restrict__ k_ou
         if (row >= rows)
 #pragma unroll
             for (int e = 0; e < 8; e++) vv[e] = (bf16)0.0f;
-        *(bf16x8 *)(&vt_tile[r][c * 8]) = vv;
+        /* token r of the block goes to LDS row 8 (r % 8) + r / 8: the transposing reads below then take their eight
+         * tokens from rows that lie 8 apart and their eight lanes (token groups) from consecutive rows, whose 272-byte
+         * stride spreads them over the banks (token-major rows put all eight lanes on one bank) */
+        *(bf16x8 *)(&vt_tile[(r & 7) * 8 + (r >> 3)][c * 8]) = vv;
 
         /* K chunk: norm + rope */
         bf16x8 kv = *(const bf16x8 *)(qkv + (size_t)rowc * ld + k_col + h * HD + c * 8);
@@ -92,7 +95,7 @@ __global__ __launch_bounds__(256) void kv_prepare_kernel(bf16 *__restrict__ k_ou
         const int tg = tid & 7, d = (tid >> 3) + i * 32;
         bf16x8 o;
 #pragma unroll
-        for (int e = 0; e < 8; e++) o[e] = vt_tile[tg * 8 + e][d];
+        for (int e = 0; e < 8; e++) o[e] = vt_tile[e * 8 + tg][d];
         *(bf16x8 *)(vt_out + (size_t)(h * HD + d) * ld_vt + r0 + tg * 8) = o;
     }
 }
