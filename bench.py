@@ -9,8 +9,8 @@ FLUX.2-klein-4B architecture with random-init bf16 weights ~N(0, 0.02) and N(0,1
 region; the host only queues kernels. Prints ONE JSON line.
 
 Also measured in the same run:
-  roofline      the dominant kernel (gate/up projection GEMM with the SiLU*up epilogue) launched
-                alone at the workload's shape and timed with HIP events on the backend's stream
+  roofline      the dominant kernel (the fused [Q|K|V|gate|up] projection of the single-stream blocks): HIP events on
+                the backend's stream around every launch of it inside the timed region; also launched alone
   cpu_baseline  the CPU oracle (fp32, BLAS when available) on a bounded sample of the same
                 workload: one whole forward at full shape after a small warm-up forward
 
@@ -20,8 +20,11 @@ vae_enc_c4 the VAE encoder on a picture of those sizes (the input of image-to-im
 --workload qwen3 measures the step before the loop: one forward of the text encoder over 512 tokens.
 --workload att_c2 | att_c3 | att_c4 | att_c5 measures the attention operator alone (K/V preparation + attention) at
 that workload's sequence length.
+--workload att_c1 ... att_c5 also exist for the other sequence lengths; bw_c3 | bw_c4 time the bandwidth-bound kernels
+(AdaLN, K/V preparation) against a streaming yardstick.
 --workload mfma_peak measures no part of the model: what the matrix pipes sustain on their own (the measured
-peak beside the datasheet's 2.5 PFLOP/s).
+peak beside the datasheet's 2.5 PFLOP/s); mfma_issue what another instruction between a lone wave's MFMAs costs them;
+gemm_vs_lib the step's projection shapes as plain GEMMs against the vendor library behind torch.matmul.
 """
 import argparse
 import json
