@@ -722,7 +722,8 @@ def main():
     TILE_NAMES = {0: f"gemm_kernel<64,128,2,2,{epi_name}>", 1: f"gemm_kernel<128,128,2,2,{epi_name}>", 2: f"gemm4d_kernel<8,8,{epi_name}> (256x256 tile)",
                   3: f"gemm_kernel<64,64,2,2,{epi_name}>", 4: f"gemm_kernel<256,256,2,4,{epi_name}>", 5: f"gemm4d_kernel<9,6,{epi_name}> (288x192 tile)",
                   6: f"gemm4d_kernel<6,6,{epi_name}> (192x192 tile)", 7: f"gemm4d_kernel<8,6,{epi_name}> (256x192 tile)",
-                  8: f"gemm_kernel<64,128,2,2,{epi_name},6> (ring of 6 stages)", 9: f"gemm_kernel<128,128,2,2,{epi_name},5> (ring of 5 stages)"}
+                  8: f"gemm_kernel<64,128,2,2,{epi_name},6> (ring of 6 stages)", 9: f"gemm_kernel<128,128,2,2,{epi_name},5> (ring of 5 stages)",
+                  10: f"gemm_kernel<96,128,2,2,{epi_name},5> (ring of 5 stages)"}
     k_tile = -1
     for tile in TILE_NAMES:
         n_t, ms_t = ctypes.c_int(0), ctypes.c_float(0.0)

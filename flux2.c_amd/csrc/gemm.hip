@@ -845,6 +845,7 @@ static int launch_epi(GemmArgs &g, int tile) {
         case 3: return launch_cfg<64, 64, 2, 2, EPI>(g);
         case 8: return launch_cfg<64, 128, 2, 2, EPI, 6>(g);  /* few rows: the same tiles with a ring that fills the LDS */
         case 9: return launch_cfg<128, 128, 2, 2, EPI, 5>(g);
+        case 10: return launch_cfg<96, 128, 2, 2, EPI, 5>(g);
         default: return launch_cfg<64, 128, 2, 2, EPI>(g);
     }
 }
@@ -1089,10 +1090,10 @@ extern "C" void flux_hip_linear_release(void) {
 }
 
 static int g_force_tile = -1;
-static unsigned g_tile_mask = 0x3EF; /* tiles the automatic choice may use: all but the 8-wave form of 256 x 256 */
+static unsigned g_tile_mask = 0x7EF; /* tiles the automatic choice may use: all but the 8-wave form of 256 x 256 */
 static int g_splitk_enabled = 1;
 extern "C" void flux_hip_linear_force_tile(int tile) { g_force_tile = tile; }
-extern "C" void flux_hip_linear_tile_mask(unsigned mask) { g_tile_mask = mask ? mask : 0x3EF; }
+extern "C" void flux_hip_linear_tile_mask(unsigned mask) { g_tile_mask = mask ? mask : 0x7EF; }
 extern "C" void flux_hip_linear_enable_splitk(int on) { g_splitk_enabled = on; }
 
 /* Launch probe: HIP events around every launch with one chosen epilogue, so a benchmark can
@@ -1162,12 +1163,13 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
      * fixed prologue/epilogue cost; the launch cannot beat the time to stream its operands,
      * which depends on how many bytes the resident workgroups keep in flight. */
     /* tile ids: 0..3 the small tiles and 256 x 256, 4 = the 8-wave form of 256 x 256 (only when
-     * forced, for comparison runs), 5 = 288 x 192, 6 = 192 x 192, 7 = 256 x 192, 8 and 9 = 64 x 128 and 128 x 128
-     * with a ring of 6 and 5 stages instead of 2 (one workgroup per compute unit; for parts of at most that many rows) */
-    constexpr int NT = 10;
-    static const int bm[NT] = {64, 128, 256, 64, 256, 288, 192, 256, 64, 128}, bn[NT] = {128, 128, 256, 64, 256, 192, 192, 192, 128, 128};
-    static const int occ[NT] = {3, 2, 1, 4, 1, 1, 1, 1, 1, 1}, ahead[NT] = {1, 1, 1, 1, 1, 1, 1, 1, 5, 4}; /* stages a workgroup keeps in flight */
-    static const double rate[NT] = {2.0e12, 2.9e12, 5.3e12, 1.5e12, 4.6e12, 5.45e12, 5.1e12, 5.55e12, 1.6e12, 3.0e12}; /* FLOP/s of one CU running this tile */
+     * forced, for comparison runs), 5 = 288 x 192, 6 = 192 x 192, 7 = 256 x 192, 8, 9 and 10 = 64 x 128, 128 x 128 and
+     * 96 x 128 with a ring of 6, 5 and 5 stages instead of 2 (one workgroup per compute unit; for parts of at most that
+     * many rows) */
+    constexpr int NT = 11;
+    static const int bm[NT] = {64, 128, 256, 64, 256, 288, 192, 256, 64, 128, 96}, bn[NT] = {128, 128, 256, 64, 256, 192, 192, 192, 128, 128, 128};
+    static const int occ[NT] = {3, 2, 1, 4, 1, 1, 1, 1, 1, 1, 1}, ahead[NT] = {1, 1, 1, 1, 1, 1, 1, 1, 5, 4, 4}; /* stages a workgroup keeps in flight */
+    static const double rate[NT] = {2.0e12, 2.9e12, 5.3e12, 1.5e12, 4.6e12, 5.45e12, 5.1e12, 5.55e12, 1.6e12, 3.0e12, 2.4e12}; /* FLOP/s of one CU running this tile */
     const int kt_total = g.K >> 6;
     int tile = -1, best_split = 1;
     {
@@ -1205,8 +1207,11 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
                 const double t_block = 2.0 * bm[t] * bn[t] * 64.0 * per / (rate[t] / per_cu) + 2.5e-6;
                 double t_compute = rounds * t_block;
                 const double bytes = (rows + N) * (double)K * 2.0;
+                /* what a launch that only streams its operands has been seen to reach: 3.2-3.5 TB/s with two LDS stages
+                 * (every step waits for the loads it has just requested), 4.3-5.2 TB/s with a deep ring */
+                const double bw_cap = ahead[t] > 1 ? 4.6e12 : 3.4e12;
                 double bw = 5.5e12 * (double)(resident * ahead[t] * (bm[t] + bn[t]) * 128) / 12.0e6;
-                if (bw > 5.5e12) bw = 5.5e12;
+                if (bw > bw_cap) bw = bw_cap;
                 double est = t_compute > bytes / bw ? t_compute : bytes / bw;
                 if (sp > 1) est += 3.0e-6 + (sp + 2.0) * rows * N * 4.0 / 4.0e12;
                 if (est < best) { best = est; tile = t; best_split = sp; }
@@ -1303,7 +1308,7 @@ static int linear_impl(int epilogue, int nparts, const flux_hip_linear_part *par
     g.N = N; g.K = K; g.lda = lda; g.ldw = ldw; g.ldc = ldc; g.w_row0 = w_row0; g.w_row1 = w_row1;
     a.ldo = N;
     a.eps = eps;
-    return gemm_dispatch(g, np, epilogue, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0x3FFu, nullptr, norm ? &a : nullptr, fused,
+    return gemm_dispatch(g, np, epilogue, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0x7FFu, nullptr, norm ? &a : nullptr, fused,
                          fixed_ws, fixed_ws_bytes);
 }
 
@@ -1331,7 +1336,7 @@ extern "C" int flux_hip_linear_qkv_swiglu(const void *A, const void *W, void *qk
     int tile = -1;
     const int saved = g_splitk_enabled;
     g_splitk_enabled = 0;
-    const int ok = gemm_dispatch(g, 1, EPI_QKV_SWIGLU, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0x3FFu, &tile);
+    const int ok = gemm_dispatch(g, 1, EPI_QKV_SWIGLU, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0x7FFu, &tile);
     g_splitk_enabled = saved;
     return ok;
 }

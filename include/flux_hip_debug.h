@@ -16,12 +16,12 @@ extern "C" {
 #endif
 
 /* force_tile: 0/1/2/3/5/6/7 pins the GEMM tile of flux_hip_linear (64x128, 128x128, 256x256, 64x64,
- * 288x192, 192x192, 256x192; 4 = 256x256 in its 8-wave form, never chosen automatically; 8 / 9 = 64x128 / 128x128
- * with a ring of 6 / 5 LDS stages, only for row ranges of at most 64 / 128 rows), -1 restores
+ * 288x192, 192x192, 256x192; 4 = 256x256 in its 8-wave form, never chosen automatically; 8 / 9 / 10 = 64x128 / 128x128 / 96x128
+ * with a ring of 6 / 5 / 5 LDS stages, only for row ranges of at most 64 / 128 / 96 rows), -1 restores
  * the automatic choice (a tile whose width does not divide N is skipped; if none is left the 128x128
  * tile runs). */
 void flux_hip_linear_force_tile(int tile);
-/* bit t set = the automatic choice may use tile t (default 0x3EF: all but tile 4; 0 restores it) */
+/* bit t set = the automatic choice may use tile t (default 0x7EF: all but tile 4; 0 restores it) */
 void flux_hip_linear_tile_mask(unsigned mask);
 /* 0 turns the split-K path off (default 1) */
 void flux_hip_linear_enable_splitk(int on);
