@@ -18,10 +18,10 @@ Also measured in the same run:
 one VAE decode of a 16/32/64-wide latent to a 256/512/1024-pixel image; vae_enc_c2 | vae_enc_c3 |
 vae_enc_c4 the VAE encoder on a picture of those sizes (the input of image-to-image generation).
 --workload qwen3 measures the step before the loop: one forward of the text encoder over 512 tokens.
---workload att_c2 | att_c3 | att_c4 | att_c5 measures the attention operator alone (K/V preparation + attention) at
+--workload att_c2 | att_c3 | att_c4 | att_c5 measures the attention operator alone (Q/K preparation + attention) at
 that workload's sequence length.
 --workload att_c1 ... att_c5 also exist for the other sequence lengths; bw_c3 | bw_c4 time the bandwidth-bound kernels
-(AdaLN, K/V preparation) against a streaming yardstick.
+(AdaLN, Q/K preparation) against a streaming yardstick.
 --workload mfma_peak measures no part of the model: what the matrix pipes sustain on their own (the measured
 peak beside the datasheet's 2.5 PFLOP/s); mfma_issue what another instruction between a lone wave's MFMAs costs them;
 gemm_vs_lib the step's projection shapes as plain GEMMs against the vendor library behind torch.matmul.
@@ -328,7 +328,7 @@ ATT_WORKLOADS = {"att_c1": 80, "att_c2": 768, "att_c3": 1536, "att_c4": 4608, "a
 
 def bench_attention(args):
     """The attention operator alone at a workload's sequence length (24 heads of 128, text split at 512): one "step"
-    is one flux_hip_kv_prepare + flux_hip_attention pair, back to back on resident buffers, as a single-stream
+    is one flux_hip_qk_prepare + flux_hip_attention pair, back to back on resident buffers, as a single-stream
     block runs them. The roofline object is the attention kernel by itself (HIP events around runs of it)."""
     n, heads = ATT_WORKLOADS[args.workload], KLEIN_4B.heads
     H = heads * 128
@@ -340,14 +340,14 @@ def bench_attention(args):
     w = fluxhip.DevBuf.from_array(np.ones(128, np.float32))
     ang = normal_f32((n, 128), 5, 2)
     cos, sin = fluxhip.DevBuf.from_array(np.cos(ang)), fluxhip.DevBuf.from_array(np.sin(ang))
-    ldvt = (n + 63) // 64 * 64
-    kn, vt, out = fluxhip.DevBuf(n * H * 2), fluxhip.DevBuf(H * ldvt * 2), fluxhip.DevBuf(n * H * 2)
+    kn, out = fluxhip.DevBuf(n * H * 2), fluxhip.DevBuf(n * H * 2)
 
     def prep():
-        fluxhip.check(L.flux_hip_kv_prepare(kn.ptr, vt.ptr, ldvt, qkv.ptr, 3 * H, H, 2 * H, n, heads, split, w.ptr, w.ptr, cos.ptr, sin.ptr, 1e-6))
+        # Q is prepared in place: every pass normalises the Q columns again (finite, and the timing does not depend on the values)
+        fluxhip.check(L.flux_hip_qk_prepare(kn.ptr, qkv.ptr, 3 * H, 0, H, n, heads, split, w.ptr, w.ptr, w.ptr, w.ptr, cos.ptr, sin.ptr, 1e-6))
 
     def att():
-        fluxhip.check(L.flux_hip_attention(out.ptr, H, qkv.ptr, 3 * H, kn.ptr, vt.ptr, ldvt, n, n, heads, split, w.ptr, w.ptr, cos.ptr, sin.ptr, 1e-6))
+        fluxhip.check(L.flux_hip_attention(out.ptr, H, qkv.ptr, 3 * H, kn.ptr, qkv.at(2 * H * 2), 3 * H, n, n, heads))
 
     for _ in range(max(args.warmup, 1)):
         prep(); att()
@@ -376,13 +376,13 @@ def bench_attention(args):
         "metric": f"attention calls/s ({n} tokens, {heads} heads, 1 GPU)", "value": round(args.steps / wall, 2), "unit": "calls/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1000.0 / args.steps, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: K/V preparation + joint attention over {n} tokens ({split} text), {heads} heads x 128, N(0,1) bf16 "
+        "config": {"workload": f"{args.workload}: Q/K preparation + joint attention over {n} tokens ({split} text), {heads} heads x 128, N(0,1) bf16 "
                                f"q/k/v, unit QK-norm weights, random RoPE angles; variant {args.attention_variant}"},
         "device_ms_per_step_events": round(ev_ms / args.steps, 4),
         "roofline": {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4),
                      "traffic": None, "kernel": "attention_wide_kernel (+ its empty second pass): softmax(q k^T / sqrt(128)) v, 4 n^2 H FLOP",
                      "ms_per_launch": round(att_ms, 4), "flops_per_launch": flops},
-        "kv_prepare": {"bound": "hbm", "ms_per_launch": round(prep_ms, 4), "bytes_per_launch": prep_bytes,
+        "qk_prepare": {"bound": "hbm", "ms_per_launch": round(prep_ms, 4), "bytes_per_launch": prep_bytes,
                        "achieved_GBps": round(prep_bytes / (prep_ms * 1e-3) / 1e9, 1), "peak_GBps": 8000.0,
                        "frac": round(prep_bytes / (prep_ms * 1e-3) / 8e12, 4)},
         "cpu_baseline": None}))
@@ -393,8 +393,8 @@ BW_WORKLOADS = {"bw_c3": 1536, "bw_c4": 4608}
 
 def bench_bandwidth(args):
     """The bandwidth-bound kernels of a block at a workload's token count, each alone on resident buffers: LayerNorm +
-    modulation (flux_hip_adaln_norm: fp32 [tokens, 3072] in, bf16 out), K/V preparation (flux_hip_kv_prepare: K and V
-    of 24 heads in, normalised + rotated K and transposed V out) and, as the yardstick for what a trivial streaming
+    modulation (flux_hip_adaln_norm: fp32 [tokens, 3072] in, bf16 out), Q/K preparation (flux_hip_qk_prepare: Q and K
+    of 24 heads in, normalised + rotated Q (in place) and K out) and, as the yardstick for what a trivial streaming
     kernel reaches at this size, the fp32 -> bf16 conversion over the same element count. Every kernel is timed twice:
     launches over the same buffers (operands stay in the 256 MB memory-side cache) and over four buffer sets in turn
     (every launch finds its operands in HBM). One "step" is one launch of each kernel on rotating buffers."""
@@ -420,20 +420,20 @@ def bench_bandwidth(args):
     w = fluxhip.DevBuf.from_array(np.ones(128, np.float32))
     ang = normal_f32((n, 128), 5, 2)
     cos, sin = fluxhip.DevBuf.from_array(np.cos(ang)), fluxhip.DevBuf.from_array(np.sin(ang))
-    ldvt = (n + 63) // 64 * 64
-    kn, vt = [fluxhip.DevBuf(n * H * 2) for _ in range(NB)], [fluxhip.DevBuf(H * ldvt * 2) for _ in range(NB)]
+    kn = [fluxhip.DevBuf(n * H * 2) for _ in range(NB)]
 
     def adaln(j):
         fluxhip.check(L.flux_hip_adaln_norm(o[j].ptr, H, x[j].ptr, n, H, 512, sh.ptr, sc.ptr, sh.ptr, sc.ptr, 1e-6))
 
     def prep(j):
-        fluxhip.check(L.flux_hip_kv_prepare(kn[j].ptr, vt[j].ptr, ldvt, qkv[j].ptr, 3 * H, H, 2 * H, n, heads, 512, w.ptr, w.ptr, cos.ptr, sin.ptr, 1e-6))
+        fluxhip.check(L.flux_hip_qk_prepare(kn[j].ptr, qkv[j].ptr, 3 * H, 0, H, n, heads, 512, w.ptr, w.ptr, w.ptr, w.ptr, cos.ptr, sin.ptr, 1e-6))
 
     def conv(j):
         fluxhip.check(L.flux_hip_f32_to_bf16(o[j].ptr, x[j].ptr, n * H))
 
     kernels = {"adaln_kernel": (adaln, 6.0 * n * H, "fp32 row in, bf16 row out: 6 bytes per element"),
-               "kv_prepare_kernel": (prep, 8.0 * n * H, "bf16 K and V in, bf16 K and V^T out: 8 bytes per element of K"),
+               "qk_prepare_kernel": (prep, 8.0 * n * H, "bf16 Q and K in, bf16 Q and K out: 8 bytes per element of K (the cos/sin rows, 1 KB per token, "
+                                                            "which every head reads again from L2, not counted)"),
                "f32_to_bf16_kernel": (conv, 6.0 * n * H, "yardstick: same bytes as adaln_kernel, no reduction")}
     table = {}
     t0 = time.perf_counter()
@@ -450,7 +450,7 @@ def bench_bandwidth(args):
         "metric": f"launches/s of the bandwidth-bound kernels ({n} tokens, 1 GPU)", "value": round(6 * launches / wall, 1), "unit": "launches/s",
         "n_gpus": 1, "steps": launches, "warmup": args.warmup, "ms_per_step": None, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"{args.workload}: adaln_kernel, kv_prepare_kernel and the fp32->bf16 yardstick at [{n}, {H}], N(0,1) inputs"},
+        "config": {"workload": f"{args.workload}: adaln_kernel, qk_prepare_kernel and the fp32->bf16 yardstick at [{n}, {H}], N(0,1) inputs"},
         "roofline": {"bound": "hbm", "achieved": a["GBps"], "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": a["frac_of_hbm_peak"], "traffic": None,
                      "kernel": "adaln_kernel, operands in HBM (four buffer sets in turn)"},
         "kernels": table, "cpu_baseline": None}))

@@ -1,5 +1,5 @@
 /*
- * attention.hip - joint text+image attention for gfx950: a K/V preparation pass and a
+ * attention.hip - joint text+image attention for gfx950: a K preparation pass and a
  * flash-style MFMA kernel with online softmax that never stores the score matrix.
  *
  * Reference semantics: joint_attention / mha_forward (flux_transformer.c:1249-1460):
@@ -14,7 +14,9 @@
  * lane exchanges, and the rescale of O is a per-lane scalar. The accumulator of S^T
  * also already has the register layout the "B" operand of the second product needs, up to a
  * permutation of keys inside each group of 32, which is applied for free when the K tile is
- * loaded (the loader picks which key goes to which LDS row).
+ * loaded (the loader picks which key goes to which LDS row). V is taken row-major, straight from
+ * the projection's output: the "A" operand V^T of the second product is read from the LDS tile with
+ * transposing reads (ds_read_b64_tr_b16), so no transposed copy of V is ever written.
  */
 #include "common.h"
 #include "../../include/flux_hip.h"
@@ -29,91 +31,96 @@ __device__ __forceinline__ float wave16_sum(float v) {
 }
 
 /* ---------------------------------------------------------------------------------------
- * K/V preparation. One workgroup handles 64 tokens of one head.
- *   K: RMSNorm over the 128 dims * weight, then rotation of pairs (d, d+1) by the token's
- *      cos/sin row; written token-major.
- *   V: written transposed, vt[head*128 + d][token], columns beyond `rows` zero-filled up to
- *      the next multiple of 64 so that the attention kernel can read whole key tiles.
+ * Q/K preparation. One workgroup handles 64 tokens of one head, Q and K: RMSNorm over the 128 dims *
+ * weight, then rotation of pairs (d, d+1) by the token's cos/sin row.
+ * K is written token-major to k_out. Q is written back in place, already multiplied by
+ * 1/sqrt(128) and log2(e), so that the attention kernel's scores are base-2 logits and its Q
+ * fragments are plain loads. (The same arithmetic inside the attention kernel, where a lane owns a
+ * query row, read the cos/sin rows 16 bytes per lane and row: a fifth of a workgroup's time at 4608
+ * tokens went into those loads. Here 16 lanes share a row.) V needs no preparation: the attention
+ * kernel reads it where the projection wrote it.
  * --------------------------------------------------------------------------------------- */
-__global__ __launch_bounds__(256) void kv_prepare_kernel(bf16 *__restrict__ k_out, bf16 *__restrict__ vt_out, int ld_vt,
-                                                         const bf16 *__restrict__ qkv, int ld, int k_col, int v_col,
+#define Q_FOLD (0.08838834764831845f * 1.44269504088896341f)
+/* norm * weight, RoPE and scale of one 8-dim chunk whose squared sum over the row's 16 lanes is already in ss */
+__device__ __forceinline__ bf16x8 qk_prepare_chunk(const float (&x)[8], float ss, float eps, const float *__restrict__ w, const float (&cv)[8],
+                                                   const float (&sv)[8], float scale) {
+    const float inv = 1.0f / sqrtf(ss * (1.0f / HD) + eps);
+    f32x4 wa = *(const f32x4 *)w, wb = *(const f32x4 *)(w + 4);
+    float wv[8] = {wa[0], wa[1], wa[2], wa[3], wb[0], wb[1], wb[2], wb[3]};
+    bf16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; e += 2) {
+        float a = x[e] * inv * wv[e], b = x[e + 1] * inv * wv[e + 1];
+        o[e] = (bf16)((a * cv[e] - b * sv[e]) * scale);
+        o[e + 1] = (bf16)((b * cv[e] + a * sv[e]) * scale);
+    }
+    return o;
+}
+__global__ __launch_bounds__(256) void qk_prepare_kernel(bf16 *__restrict__ k_out, bf16 *qkv, int ld, int q_col, int k_col,
                                                          int rows, int heads, int split,
+                                                         const float *__restrict__ q_w0, const float *__restrict__ q_w1,
                                                          const float *__restrict__ k_w0, const float *__restrict__ k_w1,
                                                          const float *__restrict__ rope_cos,
                                                          const float *__restrict__ rope_sin, float eps) {
-    __shared__ __attribute__((aligned(16))) bf16 vt_tile[64][HD + 8];
     const int r0 = blockIdx.x * 64, h = blockIdx.y;
     const int tid = threadIdx.x;
     const int c = tid & 15; /* 16-byte chunk of the 128-dim head row */
+    bf16 *qp = qkv + q_col + h * HD + c * 8;
+    const bf16 *kp = qkv + k_col + h * HD + c * 8;
+    bf16 *ko = k_out + h * HD + c * 8;
     const int H = heads * HD;
-
+    int rowc[4];
+    bf16x8 qv[4], kv[4];
+    /* all rows of a thread are requested before the first is used; a row's cos/sin chunk serves its Q and its K */
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        const int r = (tid >> 4) + i * 16;
-        const int row = r0 + r;
-        const int rowc = min(row, rows - 1);
-        /* V chunk into the LDS tile */
-        bf16x8 vv = *(const bf16x8 *)(qkv + (size_t)rowc * ld + v_col + h * HD + c * 8);
-        if (row >= rows)
+        rowc[i] = min(r0 + (tid >> 4) + i * 16, rows - 1);
+        qv[i] = *(const bf16x8 *)(qp + (size_t)rowc[i] * ld);
+        kv[i] = *(const bf16x8 *)(kp + (size_t)rowc[i] * ld);
+    }
 #pragma unroll
-            for (int e = 0; e < 8; e++) vv[e] = (bf16)0.0f;
-        /* token r of the block goes to LDS row 8 (r % 8) + r / 8: the transposing reads below then take their eight
-         * tokens from rows that lie 8 apart and their eight lanes (token groups) from consecutive rows, whose 272-byte
-         * stride spreads them over the banks (token-major rows put all eight lanes on one bank) */
-        *(bf16x8 *)(&vt_tile[(r & 7) * 8 + (r >> 3)][c * 8]) = vv;
-
-        /* K chunk: norm + rope */
-        bf16x8 kv = *(const bf16x8 *)(qkv + (size_t)rowc * ld + k_col + h * HD + c * 8);
-        float x[8];
-        float ss = 0.0f;
-#pragma unroll
-        for (int e = 0; e < 8; e++) { x[e] = (float)kv[e]; ss += x[e] * x[e]; }
-        ss = wave16_sum(ss);
-        const float inv = 1.0f / sqrtf(ss * (1.0f / HD) + eps);
-        const float *w = (rowc < split ? k_w0 : k_w1) + c * 8;
-        const float *cs = rope_cos + (size_t)rowc * HD + c * 8;
-        const float *sn = rope_sin + (size_t)rowc * HD + c * 8;
-        f32x4 w0 = *(const f32x4 *)w, w1 = *(const f32x4 *)(w + 4);
+    for (int i = 0; i < 4; i++) {
+        const int row = r0 + (tid >> 4) + i * 16;
+        const float *cs = rope_cos + (size_t)rowc[i] * HD + c * 8;
+        const float *sn = rope_sin + (size_t)rowc[i] * HD + c * 8;
         f32x4 c0 = *(const f32x4 *)cs, c1 = *(const f32x4 *)(cs + 4);
         f32x4 s0 = *(const f32x4 *)sn, s1 = *(const f32x4 *)(sn + 4);
-        float wv[8] = {w0[0], w0[1], w0[2], w0[3], w1[0], w1[1], w1[2], w1[3]};
         float cv[8] = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
         float sv[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
-        bf16x8 o;
+        float xq[8], xk[8];
+        float sq = 0.0f, sk = 0.0f;
 #pragma unroll
-        for (int e = 0; e < 8; e += 2) {
-            float a = x[e] * inv * wv[e], b = x[e + 1] * inv * wv[e + 1];
-            o[e] = (bf16)(a * cv[e] - b * sv[e]);
-            o[e + 1] = (bf16)(b * cv[e] + a * sv[e]);
+        for (int e = 0; e < 8; e++) {
+            xq[e] = (float)qv[i][e]; sq += xq[e] * xq[e];
+            xk[e] = (float)kv[i][e]; sk += xk[e] * xk[e];
         }
-        if (row < rows) *(bf16x8 *)(k_out + (size_t)row * H + h * HD + c * 8) = o;
-    }
-    __syncthreads();
-    /* transposed write: thread -> (d, group of 8 tokens) */
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int tg = tid & 7, d = (tid >> 3) + i * 32;
-        bf16x8 o;
-#pragma unroll
-        for (int e = 0; e < 8; e++) o[e] = vt_tile[e * 8 + tg][d];
-        *(bf16x8 *)(vt_out + (size_t)(h * HD + d) * ld_vt + r0 + tg * 8) = o;
+        sq = wave16_sum(sq);
+        sk = wave16_sum(sk);
+        const bool first = rowc[i] < split;
+        const bf16x8 oq = qk_prepare_chunk(xq, sq, eps, (first ? q_w0 : q_w1) + c * 8, cv, sv, Q_FOLD);
+        const bf16x8 ok = qk_prepare_chunk(xk, sk, eps, (first ? k_w0 : k_w1) + c * 8, cv, sv, 1.0f);
+        if (row < rows) {
+            *(bf16x8 *)(qp + (size_t)row * ld) = oq;
+            *(bf16x8 *)(ko + (size_t)row * H) = ok;
+        }
     }
 }
 
-extern "C" int flux_hip_kv_prepare(void *k_out, void *vt_out, int ld_vt, const void *qkv, int ld, int k_col, int v_col,
-                                   int rows, int heads, int split, const float *k_w0, const float *k_w1,
+extern "C" int flux_hip_qk_prepare(void *k_out, void *qkv, int ld, int q_col, int k_col, int rows, int heads, int split,
+                                   const float *q_w0, const float *q_w1, const float *k_w0, const float *k_w1,
                                    const float *rope_cos, const float *rope_sin, float eps) {
     if (rows <= 0) return 1;
-    if (!k_out || !vt_out || !qkv || !k_w0 || !rope_cos || !rope_sin) return flux_hip_fail("flux_hip_kv_prepare: NULL argument");
-    if (split < rows && !k_w1) return flux_hip_fail("flux_hip_kv_prepare: second weight missing");
-    const int padded = (rows + 63) / 64 * 64;
-    if (ld_vt < padded || (ld_vt & 7)) return flux_hip_fail("flux_hip_kv_prepare: ld_vt=%d must be >= %d and a multiple of 8", ld_vt, padded);
-    if ((ld & 7) || (k_col & 7) || (v_col & 7)) return flux_hip_fail("flux_hip_kv_prepare: ld/k_col/v_col must be multiples of 8");
-    if (((uintptr_t)k_out | (uintptr_t)vt_out | (uintptr_t)qkv | (uintptr_t)k_w0 | (uintptr_t)k_w1 | (uintptr_t)rope_cos | (uintptr_t)rope_sin) & 15)
-        return flux_hip_fail("flux_hip_kv_prepare: operands must be 16-byte aligned");
-    hipLaunchKernelGGL(kv_prepare_kernel, dim3(padded / 64, heads), dim3(256), 0, flux_hip_stream_handle(),
-                       (bf16 *)k_out, (bf16 *)vt_out, ld_vt, (const bf16 *)qkv, ld, k_col, v_col, rows, heads, split,
-                       k_w0, k_w1 ? k_w1 : k_w0, rope_cos, rope_sin, eps);
+    if (!k_out || !qkv || !q_w0 || !k_w0 || !rope_cos || !rope_sin) return flux_hip_fail("flux_hip_qk_prepare: NULL argument");
+    if (split < rows && (!q_w1 || !k_w1)) return flux_hip_fail("flux_hip_qk_prepare: second weight missing");
+    if ((ld & 7) || (q_col & 7) || (k_col & 7)) return flux_hip_fail("flux_hip_qk_prepare: ld, q_col and k_col must be multiples of 8");
+    if (q_col + heads * HD > ld || k_col + heads * HD > ld || (q_col < k_col + heads * HD && k_col < q_col + heads * HD))
+        return flux_hip_fail("flux_hip_qk_prepare: Q and K columns (%d, %d; %d wide) do not fit ld=%d or overlap", q_col, k_col, heads * HD, ld);
+    if (((uintptr_t)k_out | (uintptr_t)qkv | (uintptr_t)q_w0 | (uintptr_t)q_w1 | (uintptr_t)k_w0 | (uintptr_t)k_w1 | (uintptr_t)rope_cos |
+         (uintptr_t)rope_sin) & 15)
+        return flux_hip_fail("flux_hip_qk_prepare: operands must be 16-byte aligned");
+    hipLaunchKernelGGL(qk_prepare_kernel, dim3((rows + 63) / 64, heads), dim3(256), 0, flux_hip_stream_handle(),
+                       (bf16 *)k_out, (bf16 *)qkv, ld, q_col, k_col, rows, heads, split, q_w0, q_w1 ? q_w1 : q_w0, k_w0, k_w1 ? k_w1 : k_w0,
+                       rope_cos, rope_sin, eps);
     HIP_OK(hipGetLastError());
     return 1;
 }
@@ -123,20 +130,43 @@ extern "C" int flux_hip_kv_prepare(void *k_out, void *vt_out, int ld_vt, const v
  * queries (two 16-query MFMA columns) and the full head dimension. Keys are walked in tiles of 64
  * through two LDS stages filled by direct global->LDS loads (no register staging).
  *   LDS stage: K tile [64 keys][128 d] (256-byte rows, 16-byte chunks XOR-swizzled by key%16)
- *              V^T tile [128 d][64 keys] (128-byte rows, 16-byte chunks swizzled by (d/2)%8)
+ *              V tile [64 keys][128 d] (256-byte rows, 16-byte chunk c of key r at position c ^ 2 (r%4))
  * MFMA: v_mfma_f32_16x16x32_bf16 (the form that sustains the most under the power limit).
  *   S^T[key][q]: A = K fragment (lane: key l%16, dims 8(l/16)..+8 of a 32-dim chunk),
  *                B = Q fragment (lane: query l%16, same dims); accumulator lane: query l%16,
  *                keys 4(l/16)..+4 of the 16-key block.
  *   O^T[d][q]:   B = P^T fragment for 32 keys = the accumulators of two 16-row score blocks;
  *                the K rows are permuted when the tile is loaded so that these are 8
- *                consecutive keys per lane, and A = V^T fragment is one 16-byte LDS read.
+ *                consecutive keys per lane, and A = V^T fragment (lane: dim l%16 of a 16-dim block,
+ *                keys 8(l/16)..+8 of the chunk) is two transposing LDS reads of four keys each.
+ * A transposing read works in groups of 16 lanes: lane 4 e + t of the group points at four
+ * consecutive dims (quad t of a 16-dim block) of key e of four keys, and lane j of the group receives
+ * dim j of the block for those four keys. The four keys' rows lie 256 bytes apart, i.e. on the same
+ * banks; the swizzle moves each row's 32-byte piece of a block to a different bank group.
  * --------------------------------------------------------------------------------------- */
-#define ATT_STAGE (64 * 256 + 128 * 128)
-#define ATT_WIDE_LDS (6 * 16384) /* attention_wide_kernel: three K and three V^T slots */
-__device__ __forceinline__ int vt_swz(int d) { return ((d >> 1) & 7) ^ ((d & 1) << 2); }
+#define ATT_STAGE (64 * 256 + 64 * 256)
+#define ATT_WIDE_LDS (8 * 16384) /* attention_wide_kernel: four K and four V slots */
 #define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
 #define LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+/* Half a V^T fragment: one transposing read, four keys of this lane's dim. */
+__device__ __forceinline__ s16x4 v_half_fragment(const char *p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)LDS_PTR(p));
+}
+/* The same from an LDS byte address (what a pointer into LDS is, as a number). */
+__device__ __forceinline__ s16x4 v_half_fragment_at(unsigned lds_addr) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(uintptr_t)lds_addr);
+}
+__device__ __forceinline__ bf16x8 lds_read_bf16x8(unsigned lds_addr) {
+    return *(const __attribute__((address_space(3))) bf16x8 *)(uintptr_t)lds_addr;
+}
+__device__ __forceinline__ bf16x8 v_join(s16x4 lo, s16x4 hi) {
+    const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, both);
+}
+/* The V^T fragment of eight keys from two transposing reads 1024 bytes (four key rows) apart. */
+__device__ __forceinline__ bf16x8 v_fragment(const char *p) { return v_join(v_half_fragment(p), v_half_fragment(p + 1024)); }
 
 template <bool V> struct AttFlag { static constexpr bool value = V; };
 template <int V> struct AttInt { static constexpr int value = V; };
@@ -144,18 +174,15 @@ template <int V> struct AttInt { static constexpr int value = V; };
 template <int NW>
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf16 *__restrict__ out, int ldo,
                                                            const bf16 *__restrict__ q, int ldq,
-                                                           const bf16 *__restrict__ k, const bf16 *__restrict__ vt, int ld_vt,
-                                                           int seq_q, int seq_k, int heads, int split,
-                                                           const float *__restrict__ q_w0, const float *__restrict__ q_w1,
-                                                           const float *__restrict__ rope_cos,
-                                                           const float *__restrict__ rope_sin, float eps, int *redo) {
+                                                           const bf16 *__restrict__ k, const bf16 *__restrict__ v, int ldv,
+                                                           int seq_q, int seq_k, int heads, int *redo) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     /* Workgroups are dealt round-robin to the 8 XCDs, each with its own L2. Give every XCD a
      * contiguous run of (head, query block) pairs, so that all query blocks of a head run on one
-     * XCD and its K / V^T (2.4 MB at 4608 tokens) are fetched from HBM once and then served from
+     * XCD and its K / V (2.4 MB at 4608 tokens) are fetched from HBM once and then served from
      * that L2, instead of by all eight. */
     constexpr int BQ = NW * 32;  /* queries per workgroup */
-    constexpr int LP = 16 / NW;  /* wave-wide load instructions per wave and tile, for K and for V^T */
+    constexpr int LP = 16 / NW;  /* wave-wide load instructions per wave and tile, for K and for V */
     const int nqb = (seq_q + BQ - 1) / BQ;
     const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
     if (logical >= nqb * heads) return;
@@ -176,7 +203,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
     const int ntiles = (seq_k + 63) >> 6;
     const bf16 *k_src[LP];
     const bf16 *v_src[LP];
-    int k_dst[LP], v_dst[LP], k_row[LP];
+    int k_dst[LP], k_row[LP];
 #pragma unroll
     for (int i = 0; i < LP; i++) {
         /* K: one wave instruction covers 4 rows of 256 bytes */
@@ -189,12 +216,10 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
         }
         k_src[i] = k + h * HD + (((lane & 15) ^ (r & 15)) << 3);
         k_dst[i] = (wave * 4 + i * (NW * 4)) * 256;
-        /* V^T: one wave instruction covers 8 rows of 128 bytes */
-        int d = wave * 8 + i * (NW * 8) + (lane >> 3);
-        v_src[i] = vt + (size_t)(h * HD + d) * ld_vt + (((lane & 7) ^ vt_swz(d)) << 3);
-        v_dst[i] = (wave * 8 + i * (NW * 8)) * 128;
+        /* V: the same four rows, keys in their natural order (LDS row r = key r of the tile) */
+        v_src[i] = v + h * HD + (((lane & 15) ^ (2 * (r & 3))) << 3);
     }
-    /* LDS: K ring = 2 slots of 16 KB at 0 and 16 KB; V^T ring = 2 slots of 16 KB at 32 and 48 KB */
+    /* LDS: K ring = 2 slots of 16 KB at 0 and 16 KB; V ring = 2 slots of 16 KB at 32 and 48 KB */
     auto issue_k = [&](int t) {
         char *base = smem + (t & 1) * (64 * 256);
         const int key0 = t * 64;
@@ -205,54 +230,26 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
         }
     };
     auto issue_v = [&](int t) {
-        char *base = smem + 2 * (64 * 256) + (t & 1) * (128 * 128);
+        char *base = smem + 2 * (64 * 256) + (t & 1) * (64 * 256);
         const int key0 = t * 64;
 #pragma unroll
-        for (int i = 0; i < LP; i++)
-            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(v_src[i] + key0), LDS_PTR(base + v_dst[i]), 16, 0, 0);
+        for (int i = 0; i < LP; i++) {
+            int r = min(key0 + wave * 4 + i * (NW * 4) + (lane >> 4), seq_k - 1); /* beyond the end: any finite row (its probabilities are 0) */
+            __builtin_amdgcn_global_load_lds(GLOBAL_PTR(v_src[i] + (size_t)r * ldv), LDS_PTR(base + k_dst[i]), 16, 0, 0);
+        }
     };
     issue_k(0);
     issue_v(0);
 
-    /* ---- Q fragments (B operand), with RMSNorm * weight, RoPE and the softmax scale ---- */
+    /* ---- Q fragments (B operand): prepared by qk_prepare_kernel (norm, RoPE, softmax scale), loaded as they are ---- */
     bf16x8 qf[2][4];
     int qrow[2];
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         qrow[t] = qb * BQ + wave * 32 + t * 16 + l15;
-        const int qrc = min(qrow[t], seq_q - 1);
-        const bf16 *qp = q + (size_t)qrc * ldq + h * HD + lq * 8;
-        float x[4][8];
-        float ss = 0.0f;
+        const bf16 *qp = q + (size_t)min(qrow[t], seq_q - 1) * ldq + h * HD + lq * 8;
 #pragma unroll
-        for (int kk = 0; kk < 4; kk++) {
-            bf16x8 v = *(const bf16x8 *)(qp + kk * 32);
-#pragma unroll
-            for (int e = 0; e < 8; e++) { x[kk][e] = (float)v[e]; ss += x[kk][e] * x[kk][e]; }
-        }
-        ss += __shfl_xor(ss, 16, 64);
-        ss += __shfl_xor(ss, 32, 64);
-        const float inv = 1.0f / sqrtf(ss * (1.0f / HD) + eps);
-        /* 1/sqrt(128) and log2(e) folded into q: scores come out as base-2 logits */
-        const float fold = 0.08838834764831845f * 1.44269504088896341f;
-        const float *w = (qrc < split ? q_w0 : q_w1) + lq * 8;
-        const float *cs = rope_cos + (size_t)qrc * HD + lq * 8;
-        const float *sn = rope_sin + (size_t)qrc * HD + lq * 8;
-#pragma unroll
-        for (int kk = 0; kk < 4; kk++) {
-            f32x4 w0 = *(const f32x4 *)(w + kk * 32), w1 = *(const f32x4 *)(w + kk * 32 + 4);
-            f32x4 c0 = *(const f32x4 *)(cs + kk * 32), c1 = *(const f32x4 *)(cs + kk * 32 + 4);
-            f32x4 s0 = *(const f32x4 *)(sn + kk * 32), s1 = *(const f32x4 *)(sn + kk * 32 + 4);
-            float wv[8] = {w0[0], w0[1], w0[2], w0[3], w1[0], w1[1], w1[2], w1[3]};
-            float cv[8] = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
-            float sv[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
-#pragma unroll
-            for (int e = 0; e < 8; e += 2) {
-                float a = x[kk][e] * inv * wv[e], b = x[kk][e + 1] * inv * wv[e + 1];
-                qf[t][kk][e] = (bf16)((a * cv[e] - b * sv[e]) * fold);
-                qf[t][kk][e + 1] = (bf16)((b * cv[e] + a * sv[e]) * fold);
-            }
-        }
+        for (int kk = 0; kk < 4; kk++) qf[t][kk] = *(const bf16x8 *)(qp + kk * 32);
     }
 
     f32x4 o_acc[8][2];
@@ -280,7 +277,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
         for (int e = 0; e < 4; e++) l_acc[u][e] = 0.0f;
 
     /* One key tile: S^T = K Q^T - m_run (32 MFMAs), online softmax, O^T += V^T P^T (32 MFMAs).
-     * K(t) and V^T(t) sit in slot t%2 of their rings; the loads of tile t+1 are issued at the
+     * K(t) and V(t) sit in slot t%2 of their rings; the loads of tile t+1 are issued at the
      * top of the step and awaited at the top of the next one. Fragments are read from LDS one
      * block of four (8 MFMAs) ahead of their use; the first V^T block is requested before the
      * softmax so that its latency hides behind the exponentials. */
@@ -293,17 +290,15 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
             issue_v(t + 1);
         }
         const char *kt = smem + (t & 1) * (64 * 256);
-        const char *vtile = smem + 2 * (64 * 256) + (t & 1) * (128 * 128);
+        const char *vtile = smem + 2 * (64 * 256) + (t & 1) * (64 * 256);
         auto kread = [&](int kk, bf16x8 (&dst)[4]) { /* 32 head dims, key blocks 0..3 */
 #pragma unroll
             for (int i = 0; i < 4; i++) dst[i] = *(const bf16x8 *)(kt + (i * 16 + l15) * 256 + (((kk * 4 + lq) ^ l15) << 4));
         };
         auto vread = [&](int b, bf16x8 (&dst)[4]) { /* 32-key chunk b/2, head-dim blocks 4(b%2) .. +3 */
 #pragma unroll
-            for (int f = 0; f < 4; f++) {
-                const int d = ((b & 1) * 4 + f) * 16 + l15;
-                dst[f] = *(const bf16x8 *)(vtile + d * 128 + (((4 * (b >> 1) + lq) ^ vt_swz(d)) << 4));
-            }
+            for (int f = 0; f < 4; f++) /* this lane points at key 32 (b/2) + 8 lq + l15/4 (+4), dims 4 (l15%4) .. +3 of block f */
+                dst[f] = v_fragment(vtile + (32 * (b >> 1) + 8 * lq + (l15 >> 2)) * 256 + ((f ^ (l15 >> 2)) << 5) + (l15 & 3) * 8 + (b & 1) * 128);
         };
         bf16x8 fa[4], fb[4];
         {
@@ -486,93 +481,79 @@ __device__ __forceinline__ void mfma_results_fence_a(f32x4 (&acc)[8][N]) {
 template <int NQ>
 __device__ __forceinline__ void attention_wide_body(char *smem, const int h, const int q0, bf16 *__restrict__ out, int ldo,
                                                     const bf16 *__restrict__ q, int ldq, const bf16 *__restrict__ k,
-                                                    const bf16 *__restrict__ vt, int ld_vt, int seq_q, int seq_k, int heads, int split,
-                                                    const float *__restrict__ q_w0, const float *__restrict__ q_w1,
-                                                    const float *__restrict__ rope_cos, const float *__restrict__ rope_sin, float eps,
-                                                    int *redo) {
+                                                    const bf16 *__restrict__ v, int ldv, int seq_q, int seq_k, int heads, int *redo) {
     constexpr int NW = 4, WQ = 16 * NQ, LP = 16 / NW;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l15 = lane & 15, lq = lane >> 4;
     const int H = heads * HD;
 
+    /* ---- Q fragments (B operand): prepared by qk_prepare_kernel (norm, RoPE, softmax scale). Requested before the
+     * tile loads: loads return in order, and behind 28 tile loads these would arrive last ---- */
+    bf16x8 qf[NQ][4];
+#pragma unroll
+    for (int t = 0; t < NQ; t++) {
+        const bf16 *qp = q + (size_t)min(q0 + wave * WQ + t * 16 + l15, seq_q - 1) * ldq + h * HD + lq * 8;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) qf[t][kk] = *(const bf16x8 *)(qp + kk * 32);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
     /* ---- tile loader: LDS layout and key permutation as in attention_kernel<4>; the global sources are a
-     * uniform base (scalar arithmetic per tile) plus one 32-bit byte offset per lane and load ---- */
+     * uniform base plus one running 32-bit byte offset per lane and load ---- */
     const int ntiles = (seq_k + 63) >> 6;
     const char *k_base = (const char *)(k + h * HD);
-    const char *v_base = (const char *)(vt + (size_t)h * HD * ld_vt);
+    const char *v_base = (const char *)(v + h * HD);
     int k_row[LP];       /* key of the tile that this lane fetches with load i */
-    unsigned v_off[LP];  /* byte offset of this lane's V^T chunk for load i */
     const unsigned k_chunk = (unsigned)(((lane & 15) ^ ((wave * 4 + (lane >> 4)) & 15)) << 4);
+    /* V: LDS row = key of the tile, 16-byte chunk c of row r at position c ^ 2 (r % 4) */
+    const unsigned v_chunk = (unsigned)(((lane & 15) ^ (2 * (lane >> 4))) << 4);
 #pragma unroll
     for (int i = 0; i < LP; i++) {
         const int r = wave * 4 + i * (NW * 4) + (lane >> 4); /* LDS row; (r & 15) is the same for every i */
         const int ib = r >> 4, jj = (r >> 2) & 3, ee = r & 3;
         k_row[i] = 32 * (ib >> 1) + 8 * jj + 4 * (ib & 1) + ee;
-        const int d = wave * 8 + i * (NW * 8) + (lane >> 3);
-        v_off[i] = ((unsigned)d * (unsigned)ld_vt + (unsigned)(((lane & 7) ^ vt_swz(d)) << 3)) * 2u;
     }
-    /* LDS: three K slots of 16 KB, then three V^T slots of 16 KB; tile x lives in slot x % 3 of its ring.
-     * load i of tile `src` goes into slot `slot` (src is the tile the slot is for, except beyond the last tile,
-     * where the last one is fetched again into a slot nobody reads any more: no branches in the loop) */
-    auto issue_k1 = [&](int slot, int src, int i) {
-        const unsigned off = (unsigned)min(src * 64 + k_row[i], seq_k - 1) * (unsigned)(H * 2) + k_chunk;
-        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(k_base + off), LDS_PTR(smem + slot * 16384 + (wave * 4 + i * (NW * 4)) * 256), 16, 0, 0);
+    /* LDS: four K slots of 16 KB, then four V slots of 16 KB; tile x lives in slot x % 4 of its ring.
+     * Each load of a lane moves its offset on by 64 rows and stops at the last row (a multiply per load in the loop
+     * costs as much as four other vector instructions), so the tile is implied by the order of the calls: one per
+     * tile and load. Beyond the last tile the last row is fetched again, into a slot nobody reads any more: no
+     * branches in the loop. */
+    unsigned k_cur[LP], v_cur[LP];
+    const unsigned k_last = (unsigned)(seq_k - 1) * (unsigned)(H * 2) + k_chunk, k_step = 64u * (unsigned)(H * 2);
+    const unsigned v_last = (unsigned)(seq_k - 1) * (unsigned)(ldv * 2) + v_chunk, v_step = 64u * (unsigned)(ldv * 2);
+#pragma unroll
+    for (int i = 0; i < LP; i++) {
+        k_cur[i] = min((unsigned)k_row[i] * (unsigned)(H * 2) + k_chunk, k_last);
+        v_cur[i] = min((unsigned)(wave * 4 + i * (NW * 4) + (lane >> 4)) * (unsigned)(ldv * 2) + v_chunk, v_last);
+    }
+    auto load_k1 = [&](int slot, int i) {
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(k_base + k_cur[i]), LDS_PTR(smem + slot * 16384 + (wave * 4 + i * (NW * 4)) * 256), 16, 0, 0);
     };
-    auto issue_v1 = [&](int slot, int src, int i) {
-        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(v_base + src * 128 + v_off[i]),
-                                         LDS_PTR(smem + 3 * 16384 + slot * 16384 + (wave * 8 + i * (NW * 8)) * 128), 16, 0, 0);
+    /* (assembly, so that the two instructions stay behind the MFMA they are written behind) */
+    auto next_k1 = [&](int i) { asm volatile("v_add_u32 %0, %1, %0\n\tv_min_u32 %0, %0, %2" : "+v"(k_cur[i]) : "s"(k_step), "v"(k_last)); };
+    auto load_v1 = [&](int slot, int i) {
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(v_base + v_cur[i]), LDS_PTR(smem + 4 * 16384 + slot * 16384 + (wave * 4 + i * (NW * 4)) * 256), 16, 0, 0);
     };
-    /* before the loop: K(0), V(0), K(1), V(1), K(2) */
+    auto next_v1 = [&](int i) { asm volatile("v_add_u32 %0, %1, %0\n\tv_min_u32 %0, %0, %2" : "+v"(v_cur[i]) : "s"(v_step), "v"(v_last)); };
+    auto issue_k1 = [&](int slot, int i) { load_k1(slot, i); next_k1(i); };
+    auto issue_v1 = [&](int slot, int i) { load_v1(slot, i); next_v1(i); };
+    /* before the loop, in this order: K(0), V(0), K(1), V(1), K(2), V(2), K(3) */
 #pragma unroll
-    for (int x = 0; x < 3; x++) {
-        const int src = min(x, ntiles - 1);
+    for (int x = 0; x < 4; x++) {
 #pragma unroll
-        for (int i = 0; i < LP; i++) issue_k1(x, src, i);
-        if (x < 2) {
+        for (int i = 0; i < LP; i++) issue_k1(x, i);
+        if (x < 3) {
 #pragma unroll
-            for (int i = 0; i < LP; i++) issue_v1(x, src, i);
+            for (int i = 0; i < LP; i++) issue_v1(x, i);
         }
     }
 
-    /* ---- Q fragments (B operand) with RMSNorm * weight, RoPE and the softmax scale; they live in AGPRs ---- */
-    bf16x8 qf[NQ][4];
+    /* the Q fragments arrive first (requested before the tile loads) and live in AGPRs */
 #pragma unroll
-    for (int t = 0; t < NQ; t++) {
-        const int qrc = min(q0 + wave * WQ + t * 16 + l15, seq_q - 1);
-        const bf16 *qp = q + (size_t)qrc * ldq + h * HD + lq * 8;
-        float x[4][8];
-        float ss = 0.0f;
+    for (int t = 0; t < NQ; t++)
 #pragma unroll
-        for (int kk = 0; kk < 4; kk++) {
-            bf16x8 v = *(const bf16x8 *)(qp + kk * 32);
-#pragma unroll
-            for (int e = 0; e < 8; e++) { x[kk][e] = (float)v[e]; ss += x[kk][e] * x[kk][e]; }
-        }
-        ss += __shfl_xor(ss, 16, 64);
-        ss += __shfl_xor(ss, 32, 64);
-        const float inv = 1.0f / sqrtf(ss * (1.0f / HD) + eps);
-        const float fold = 0.08838834764831845f * 1.44269504088896341f; /* 1/sqrt(128) and log2(e): scores are base-2 logits */
-        const float *w = (qrc < split ? q_w0 : q_w1) + lq * 8;
-        const float *cs = rope_cos + (size_t)qrc * HD + lq * 8;
-        const float *sn = rope_sin + (size_t)qrc * HD + lq * 8;
-#pragma unroll
-        for (int kk = 0; kk < 4; kk++) {
-            f32x4 w0 = *(const f32x4 *)(w + kk * 32), w1 = *(const f32x4 *)(w + kk * 32 + 4);
-            f32x4 c0 = *(const f32x4 *)(cs + kk * 32), c1 = *(const f32x4 *)(cs + kk * 32 + 4);
-            f32x4 s0 = *(const f32x4 *)(sn + kk * 32), s1 = *(const f32x4 *)(sn + kk * 32 + 4);
-            float wv[8] = {w0[0], w0[1], w0[2], w0[3], w1[0], w1[1], w1[2], w1[3]};
-            float cv[8] = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
-            float sv[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
-#pragma unroll
-            for (int e = 0; e < 8; e += 2) {
-                float a = x[kk][e] * inv * wv[e], b = x[kk][e + 1] * inv * wv[e + 1];
-                qf[t][kk][e] = (bf16)((a * cv[e] - b * sv[e]) * fold);
-                qf[t][kk][e + 1] = (bf16)((b * cv[e] + a * sv[e]) * fold);
-            }
-            asm volatile("" : "+a"(qf[t][kk])); /* one aligned AGPR quad per fragment from here on */
-        }
-    }
+        for (int kk = 0; kk < 4; kk++) asm volatile("" : "+a"(qf[t][kk])); /* one aligned AGPR quad per fragment from here on */
 
     f32x4 o_acc[8][NQ]; /* AGPRs */
 #pragma unroll
@@ -607,41 +588,71 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
      * Vector instructions sit one or two behind each MFMA; sched_barrier keeps them there. Two score buffers
      * alternate, so one trip of the loop is one tile: an "even" step (second chunk's scores, first chunk's
      * product) and an "odd" step (next tile's first chunk's scores, second chunk's product). One barrier per
-     * tile, at the start of the odd step: behind it K(t)'s and V(t-1)'s slots are free and take K(t+3) and
-     * V(t+2); everything read before the next barrier landed before this one (three slots per ring), so
-     * fragments are requested from LDS a phase ahead of their MFMAs, across the barrier too.
+     * tile, at the start of the odd step: behind it K(t)'s and V(t-1)'s slots are free and take K(t+4) and
+     * V(t+3), whose eight loads are spread over the 34 NQ MFMAs up to the next barrier (a direct global->LDS load
+     * costs the matrix pipe some 12 cycles when it stands alone and 30 in a run of eight). With four slots per
+     * ring those loads are not needed before the barrier after the next, so a barrier waits for all but the newest
+     * eight loads (a count, not "all": the compiler's own barrier would wait for every load in flight).
+     * Everything read before the next barrier landed before this one, so fragments are requested from LDS a phase
+     * ahead of their MFMAs, across the barrier too.
      * The reference maxima are fixed on the first chunk, see first_reference. */
     constexpr int EXP0 = NQ < 2 ? 4 : 0; /* with 16 queries per wave the score phase is so short that the first exponentials wait four MFMAs */
     constexpr int CVT0 = NQ; /* the conversions start NQ MFMAs into the score phase: the product phase's last readers of P have long issued */
     f32x4 s_a[2][NQ], s_b[2][NQ];
     bf16x8 kf[4][2];  /* K fragments of a chunk: [32-dim step of the head dim][key block of the chunk] */
-    bf16x8 vf[2][4];  /* V^T fragments: [half of the head dim][16-row block] */
+    s16x4 vh[8][2];   /* V^T fragments: [16-row block of the head dim][first / second four keys of the lane's eight] */
     u32x4 pf[NQ];     /* P^T of the chunk as MFMA B fragments (8 bf16), per query block */
 
     /* Fragments are requested from LDS a whole phase before the MFMAs that read them (the chunk's eight K
-     * fragments during the product phase before, its eight V^T fragments during the score phase before), one
-     * read behind each of the phase's first eight MFMAs: no MFMA waits for LDS. */
+     * fragments during the product phase before, its sixteen V^T half fragments during the score phase before),
+     * spread over the phase in the order of their use (reads in a run cost the matrix pipe 4-5 cycles each, a read
+     * every few MFMAs next to nothing): no MFMA waits for LDS. */
     /* Per-lane LDS addresses of the fragments in the slots that are read next, kept in registers and moved on by one
      * slot per tile (recomputed from the slot number they cost a vector add per read): the K fragments of head-dim
-     * step kk, key block 0 of chunk 0 (the others lie 4096 (2 cp + i) further), and the V^T fragments of chunk cp,
-     * head-dim block 0 (block x lies 2048 x further). */
-    unsigned ka[4], va[2];
+     * step kk, key block 0 of chunk 0 (the others lie 4096 (2 cp + i) further), and the V^T fragments of chunk 0 for
+     * the head-dim blocks x with x % 4 = w, as this lane of a transposing read sees them (see v_fragment: the swizzle
+     * moves a block by the lane's key; chunk 1 lies 8192 further, blocks 4 .. 7 128). */
+    const unsigned lds0 = (unsigned)(uintptr_t)LDS_PTR(smem); /* folded into the addresses once, not added at every read */
+    unsigned ka[4], va[4];
 #pragma unroll
-    for (int kk = 0; kk < 4; kk++) ka[kk] = l15 * 256 + (((kk * 4 + lq) ^ l15) << 4);
+    for (int kk = 0; kk < 4; kk++) ka[kk] = lds0 + l15 * 256 + (((kk * 4 + lq) ^ l15) << 4);
 #pragma unroll
-    for (int cp = 0; cp < 2; cp++) va[cp] = 3 * 16384 + l15 * 128 + (((4 * cp + lq) ^ vt_swz(l15)) << 4);
+    for (int w = 0; w < 4; w++) va[w] = lds0 + 4 * 16384 + (8 * lq + (l15 >> 2)) * 256 + ((w ^ (l15 >> 2)) << 5) + (l15 & 3) * 8;
     auto kfrag1 = [&](int cp, int x) { /* x = 0..7: key block 2cp + x%2 of the tile, head dims 32 (x/2) .. +31 */
         const int kk = x >> 1, i = x & 1;
-        kf[kk][i] = *(const bf16x8 *)(smem + ka[kk] + (2 * cp + i) * 4096);
+        kf[kk][i] = lds_read_bf16x8(ka[kk] + (2 * cp + i) * 4096);
     };
-    auto vfrag1 = [&](int cp, int x) { /* x = 0..7: head-dim block x, keys of 32-key chunk cp */
-        vf[x >> 2][x & 3] = *(const bf16x8 *)(smem + va[cp] + x * 2048);
+    auto vhalf1 = [&](int cp, int y) { /* y = 0..15: head-dim block y / 2, keys 8 lq + 4 (y % 2) .. +3 of 32-key chunk cp */
+        const int x = y >> 1;
+        vh[x][y & 1] = v_half_fragment_at(va[x & 3] + cp * 8192 + (x >> 2) * 128 + (y & 1) * 1024);
     };
-    auto move_slots = [&](int dk, int dv) { /* byte distances to the next K slot and the next V^T slot */
+    /* what a phase of 8 NQ MFMAs requests behind MFMA m: K fragment x behind MFMA x NQ, V^T half fragment y behind
+     * MFMA y NQ / 2 */
+    auto k_reads_at = [&](int cp, int m) {
+#pragma unroll
+        for (int x = 0; x < 8; x++)
+            if (x * NQ == m) kfrag1(cp, x);
+    };
+    auto v_reads_at = [&](int cp, int m) {
+#pragma unroll
+        for (int y = 0; y < 16; y++)
+            if (y * NQ / 2 == m) vhalf1(cp, y);
+    };
+    auto move_slots = [&](int dk, int dv) { /* byte distances to the next K slot and the next V slot */
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) ka[kk] += dk;
 #pragma unroll
-        for (int cp = 0; cp < 2; cp++) va[cp] += dv;
+        for (int w = 0; w < 4; w++) va[w] += dv;
+    };
+    /* The same one register at a time behind the MFMAs of an odd step's product phase: the V addresses (last used in
+     * the score phase before) behind MFMAs 1, 2, 3, 5, the K addresses behind the last K read (at 7 NQ) */
+    auto move_slots_at = [&](int dk, int dv, int m) {
+#pragma unroll
+        for (int w = 0; w < 4; w++)
+            if (m == (NQ > 1 ? w + 1 + (w == 3) : 2 * w + 1)) va[w] += dv;
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++)
+            if (m == (NQ > 1 ? 8 * NQ - 4 + kk : 7)) ka[kk] += dk;
     };
     /* The vector instructions of the loop are inline assembly as well: an ordinary expression the compiler may
      * sink to its use in the next phase, and then nothing overlaps.
@@ -694,8 +705,8 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
                 }
         }
     };
-    /* row sums and O^T += V^T P^T for one chunk; vf[0] and vf[1] must already hold (or be receiving) the chunk's
-     * fragments. between(m) runs behind PV MFMA m (m = 0 .. 8 NQ - 1). */
+    /* row sums and O^T += V^T P^T for one chunk; vh must already hold (or be receiving) the chunk's fragments.
+     * between(m) runs behind PV MFMA m (m = 0 .. 8 NQ - 1). */
     auto pv_phase = [&](auto &&between, auto guard_c) {
         constexpr bool GUARD = decltype(guard_c)::value;
         /* the row sums are the first readers of each probability fragment */
@@ -708,8 +719,9 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
             for (int f = 0; f < 4; f++)
 #pragma unroll
                 for (int j = 0; j < NQ; j++) {
-                    if (GUARD) MFMA_ACC_A_GUARDED(o_acc[g * 4 + f][j], vf[g][f], pf[j]);
-                    else MFMA_ACC_A(o_acc[g * 4 + f][j], vf[g][f], pf[j]);
+                    const bf16x8 vf = v_join(vh[g * 4 + f][0], vh[g * 4 + f][1]);
+                    if (GUARD) MFMA_ACC_A_GUARDED(o_acc[g * 4 + f][j], vf, pf[j]);
+                    else MFMA_ACC_A(o_acc[g * 4 + f][j], vf, pf[j]);
                     between((g * 4 + f) * NQ + j);
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -759,8 +771,7 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
     };
     auto nothing = [](int) {};
     /* ---- first chunk, not pipelined: S(0) and its exact maxima ---- */
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads(); /* K(0), V(0), K(1), V(1), K(2) are in LDS */
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(6 * LP) : "memory"); /* K(0) is in LDS, the other six tiles on their way */
 #pragma unroll
     for (int x = 0; x < 8; x++) kfrag1(0, x);
     s_phase(s_a, nothing, AttFlag<true>{});
@@ -774,64 +785,87 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
 #pragma unroll
     for (int x = 0; x < 8; x++) kfrag1(1, x);
     move_slots(16384, 0); /* K fragments now come from tile 1's slot, V^T fragments from tile 0's */
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(4 * LP) : "memory"); /* V(0), K(1) are in LDS; V(1), K(2), V(2), K(3) on their way */
 
-    /* Even step of tile t (slot sl = t % 3): scores of its second chunk into s_b, product of its first chunk.
-     * The first K fragments of the odd step's chunk (first chunk of tile t + 1, slot sn) are requested meanwhile. */
-    auto even_step = [&](int t, int sl, int sn, auto guard_c) {
+    /* The tile's eight loads, K(t+4) and V(t+3): the four of K in the last eight gaps of the odd step's score phase, the
+     * four of V in those of the next even step's (gaps that carry little else): a load behind an even MFMA, the step of
+     * its offset behind the next. */
+    auto k_loads_at = [&](int slot, int m) {
+#pragma unroll
+        for (int i = 0; i < LP; i++) {
+            if (m == 8 * NQ - 8 + 2 * i) load_k1(slot, i);
+            if (m == 8 * NQ - 7 + 2 * i) next_k1(i);
+        }
+    };
+    auto v_loads_at = [&](int slot, int m) {
+#pragma unroll
+        for (int i = 0; i < LP; i++) {
+            if (m == 8 * NQ - 8 + 2 * i) load_v1(slot, i);
+            if (m == 8 * NQ - 7 + 2 * i) next_v1(i);
+        }
+    };
+    /* Even step of tile t: scores of its second chunk into s_b, product of its first chunk. The K fragments of the
+     * odd step's chunk (first chunk of tile t + 1) are requested meanwhile. Only the last tile can be ragged:
+     * the check for keys beyond the end (a branch: 30 cycles with nothing to hide it) is compiled into the copies
+     * of the steps that can meet it, not into the loop. */
+    auto even_step = [&](int t, auto loads_c, auto last_c, auto guard_c) {
+        constexpr bool LOADS = decltype(loads_c)::value, LAST = decltype(last_c)::value;
         s_phase(s_b, [&](int m) {
-            if (m < 8) vfrag1(0, m);
+            v_reads_at(0, m);
             if (m >= CVT0 && m < CVT0 + 4 * NQ) cvt1(s_a, m - CVT0);
+            if (LOADS) v_loads_at((t + 2) & 3, m);
         }, guard_c);
-        mask_chunk(s_b, 2 * t + 1);
+        if (LAST) mask_chunk(s_b, 2 * t + 1);
         pv_phase([&](int m) {
-            if (m < 8 && t + 1 < ntiles) kfrag1(0, m);
+            if (!LAST) k_reads_at(0, m);
             if (m >= EXP0) exp1(s_b, m - EXP0);
         }, guard_c);
 #pragma unroll
         for (int n = 8 * NQ - EXP0; n < 8 * NQ; n++) exp1(s_b, n);
     };
-    /* Odd step of tile t: the barrier, the loads of K(t+3) and V(t+2), scores of tile t+1's first chunk into s_a,
-     * product of tile t's second chunk. sp = (t + 2) % 3 is the slot V(t+2) goes to. */
-    auto odd_step = [&](int t, int sl, int sn, int sp) {
-        __builtin_amdgcn_s_waitcnt(0x0F70); /* this wave's parts of K(t+2) and V(t+1) are in LDS */
-        __syncthreads();
+    /* Odd step of tile t: the barrier, scores of tile t+1's first chunk into s_a, product of tile t's second chunk. */
+    auto odd_step = [&](int t, auto ragged_c, auto guard_c) {
+        /* to the slots of the next tile (K fragments then come from tile t + 2's slot, V^T fragments from tile t + 1's):
+         * one slot on, or three back */
+        const int dk = ((t + 2) & 3) ? 16384 : -3 * 16384, dv = ((t + 1) & 3) ? 16384 : -3 * 16384;
+        /* this wave's parts of K(t+2) and V(t+1) are in LDS: everything but the eight loads issued since the last barrier */
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * LP) : "memory");
         s_phase(s_a, [&](int m) {
-            if (m < 8) vfrag1(1, m);
+            v_reads_at(1, m);
             if (m >= CVT0 && m < CVT0 + 4 * NQ) cvt1(s_b, m - CVT0);
-        }, AttFlag<false>{});
-        mask_chunk(s_a, 2 * t + 2);
+            k_loads_at(t & 3, m);
+        }, guard_c);
+        if (decltype(ragged_c)::value) mask_chunk(s_a, 2 * t + 2);
         pv_phase([&](int m) {
-            if (m < 8) kfrag1(1, m);
+            k_reads_at(1, m);
             if (m >= EXP0) exp1(s_a, m - EXP0);
-            if (m >= 8 * NQ - 2 * LP) { /* the tile's eight loads behind the last eight MFMAs */
-                const int i = m - (8 * NQ - 2 * LP);
-                if (i & 1) issue_v1(sp, min(t + 2, ntiles - 1), i >> 1);
-                else issue_k1(sl, min(t + 3, ntiles - 1), i >> 1);
-            }
-        }, AttFlag<false>{});
+            move_slots_at(dk, dv, m);
+        }, guard_c);
 #pragma unroll
         for (int n = 8 * NQ - EXP0; n < 8 * NQ; n++) exp1(s_a, n);
     };
     /* the last chunk: nothing left to overlap */
-    auto last_step = [&](int sl) {
+    auto last_step = [&]() {
 #pragma unroll
-        for (int x = 0; x < 8; x++) vfrag1(1, x);
+        for (int y = 0; y < 16; y++) vhalf1(1, y);
 #pragma unroll
         for (int n = 0; n < 4 * NQ; n++) cvt1(s_b, n);
         __builtin_amdgcn_sched_barrier(0);
         pv_phase(nothing, AttFlag<true>{});
     };
-    {
-        int sl = 0, sn = 1, sp = 2; /* slots of tiles t, t + 1, t + 2 */
-        for (int t = 0; t < ntiles - 1; t++) {
-            even_step(t, sl, sn, AttFlag<false>{});
-            odd_step(t, sl, sn, sp);
-            move_slots((sp - sn) * 16384, (sn - sl) * 16384);
-            const int r = sl; sl = sn; sn = sp; sp = r;
+    /* (outside the loop every MFMA carries its guard, see s_phase) */
+    if (ntiles == 1) {
+        even_step(0, AttFlag<false>{}, AttFlag<true>{}, AttFlag<true>{});
+    } else {
+        even_step(0, AttFlag<false>{}, AttFlag<false>{}, AttFlag<true>{});
+        for (int t = 0; t < ntiles - 2; t++) {
+            odd_step(t, AttFlag<false>{}, AttFlag<false>{});
+            even_step(t + 1, AttFlag<true>{}, AttFlag<false>{}, AttFlag<false>{});
         }
-        even_step(ntiles - 1, sl, sn, AttFlag<true>{});
-        last_step(sl);
+        odd_step(ntiles - 2, AttFlag<true>{}, AttFlag<true>{});
+        even_step(ntiles - 1, AttFlag<false>{}, AttFlag<true>{}, AttFlag<true>{});
     }
+    last_step();
     __builtin_amdgcn_s_waitcnt(0x0F70); /* no load into LDS is left in flight */
 
     mfma_results_fence_a<NQ>(o_acc);
@@ -880,26 +914,22 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
  * (NQB = NQA - 1): a launch whose workgroups are all alike leaves compute units idle in its last round (18 blocks
  * of 256 queries per head, 24 heads: 432 workgroups, 1.69 rounds over 256 units, paid as 2), and with shorter
  * blocks at the end the last round is a short one. Each XCD takes a contiguous run of heads, so that a head's K and
- * V^T are fetched into one L2 only, and within its run the long blocks of all its heads come first (workgroups are
+ * V are fetched into one L2 only, and within its run the long blocks of all its heads come first (workgroups are
  * dealt to the XCDs round-robin and started in order). */
 template <int NQA, int NQB>
 __global__ __launch_bounds__(256, 1) void attention_wide_kernel(bf16 *__restrict__ out, int ldo, const bf16 *__restrict__ q, int ldq,
-                                                                const bf16 *__restrict__ k, const bf16 *__restrict__ vt, int ld_vt,
-                                                                int seq_q, int seq_k, int heads, int split,
-                                                                const float *__restrict__ q_w0, const float *__restrict__ q_w1,
-                                                                const float *__restrict__ rope_cos, const float *__restrict__ rope_sin,
-                                                                float eps, int *redo, int na, int nb) {
+                                                                const bf16 *__restrict__ k, const bf16 *__restrict__ v, int ldv,
+                                                                int seq_q, int seq_k, int heads, int *redo, int na, int nb) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int xcd = blockIdx.x & 7, hx0 = xcd * heads / 8, nh = (xcd + 1) * heads / 8 - hx0;
     int item = blockIdx.x >> 3;
     if (item >= nh * (na + nb)) return;
     if (item < nh * na) {
-        attention_wide_body<NQA>(smem, hx0 + item / na, (item % na) * 64 * NQA, out, ldo, q, ldq, k, vt, ld_vt, seq_q, seq_k, heads, split,
-                                 q_w0, q_w1, rope_cos, rope_sin, eps, redo);
+        attention_wide_body<NQA>(smem, hx0 + item / na, (item % na) * 64 * NQA, out, ldo, q, ldq, k, v, ldv, seq_q, seq_k, heads, redo);
     } else {
         item -= nh * na;
-        attention_wide_body<NQB>(smem, hx0 + item / nb, na * 64 * NQA + (item % nb) * 64 * NQB, out, ldo, q, ldq, k, vt, ld_vt, seq_q,
-                                 seq_k, heads, split, q_w0, q_w1, rope_cos, rope_sin, eps, redo);
+        attention_wide_body<NQB>(smem, hx0 + item / nb, na * 64 * NQA + (item % nb) * 64 * NQB, out, ldo, q, ldq, k, v, ldv, seq_q,
+                                 seq_k, heads, redo);
     }
 }
 
@@ -962,18 +992,18 @@ static WidePlan wide_plan(int seq_q, int heads) {
 static int g_att_force = -1;
 extern "C" void flux_hip_attention_force_variant(int v) { g_att_force = v; }
 
-extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ldq, const void *k, const void *vt,
-                                  int ld_vt, int seq_q, int seq_k, int heads, int split, const float *q_w0,
-                                  const float *q_w1, const float *rope_cos, const float *rope_sin, float eps) {
+extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ldq, const void *k, const void *v,
+                                  int ldv, int seq_q, int seq_k, int heads) {
     if (seq_q <= 0) return 1;
     if (seq_k <= 0) return flux_hip_fail("flux_hip_attention: seq_k=%d", seq_k);
-    if (!out_bf16 || !q || !k || !vt || !q_w0 || !rope_cos || !rope_sin) return flux_hip_fail("flux_hip_attention: NULL argument");
-    if (split < seq_q && !q_w1) return flux_hip_fail("flux_hip_attention: second weight missing");
-    if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)vt | (uintptr_t)q_w0 | (uintptr_t)q_w1 | (uintptr_t)rope_cos | (uintptr_t)rope_sin) & 15) ||
-        ((uintptr_t)out_bf16 & 7))
+    if (!out_bf16 || !q || !k || !v) return flux_hip_fail("flux_hip_attention: NULL argument");
+    if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) || ((uintptr_t)out_bf16 & 7))
         return flux_hip_fail("flux_hip_attention: operands must be 16-byte aligned (output 8-byte)");
-    if ((ldo & 3) || (ldq & 7) || (ld_vt & 7) || ld_vt < (seq_k + 63) / 64 * 64)
-        return flux_hip_fail("flux_hip_attention: bad leading dimensions (ldo=%d ldq=%d ld_vt=%d)", ldo, ldq, ld_vt);
+    if ((ldo & 3) || (ldq & 7) || (ldv & 7) || ldv < heads * HD)
+        return flux_hip_fail("flux_hip_attention: bad leading dimensions (ldo=%d ldq=%d ldv=%d)", ldo, ldq, ldv);
+    /* the tile loaders address K and V rows with 32-bit byte offsets that run up to 64 rows past the end */
+    if ((double)(seq_k + 64) * ldv * 2.0 >= 4294967296.0 || (double)(seq_k + 64) * heads * HD * 2.0 >= 4294967296.0)
+        return flux_hip_fail("flux_hip_attention: %d keys of %d-element rows exceed 32-bit offsets", seq_k, ldv);
     /* Variants: 0 / 1 = attention_kernel with 128 / 256 queries per workgroup; 11 .. 14 = attention_wide_kernel with
      * 16 NQ queries per wave throughout (NQ = 1 .. 4); -1 (default) and 15 = attention_wide_kernel with the mix of
      * block lengths that wide_plan() finds. */
@@ -990,8 +1020,8 @@ extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ld
     if (variant == 0 || variant == 1) {
         const int bq = variant ? 256 : 128, blocks = ((seq_q + bq - 1) / bq) * heads;
         hipLaunchKernelGGL(variant ? attention_kernel<8> : attention_kernel<4>, dim3((blocks + 7) & ~7), dim3(variant ? 512 : 256), 2 * ATT_STAGE,
-                           flux_hip_stream_handle(), (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt,
-                           seq_q, seq_k, heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps, (int *)nullptr);
+                           flux_hip_stream_handle(), (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)v, ldv,
+                           seq_q, seq_k, heads, (int *)nullptr);
         HIP_OK(hipGetLastError());
         return 1;
     }
@@ -1011,12 +1041,10 @@ extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ld
     const dim3 grid(8 * max_nh * (plan.na + plan.nb));
     auto kern = plan.nqa == 4 ? attention_wide_kernel<4, 3> : plan.nqa == 3 ? attention_wide_kernel<3, 2> : attention_wide_kernel<2, 1>;
     hipLaunchKernelGGL(kern, grid, dim3(256), ATT_WIDE_LDS, flux_hip_stream_handle(), (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq,
-                       (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k, heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps,
-                       redo, plan.na, plan.nb);
+                       (const bf16 *)k, (const bf16 *)v, ldv, seq_q, seq_k, heads, redo, plan.na, plan.nb);
     /* second pass: the blocks of 128 queries the first one marked (normally none: every workgroup leaves at once) */
     hipLaunchKernelGGL(attention_kernel<4>, dim3((blocks128 + 7) & ~7), dim3(256), 2 * ATT_STAGE, flux_hip_stream_handle(),
-                       (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)vt, ld_vt, seq_q, seq_k,
-                       heads, split, q_w0, q_w1 ? q_w1 : q_w0, rope_cos, rope_sin, eps, redo);
+                       (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)v, ldv, seq_q, seq_k, heads, redo);
     HIP_OK(hipGetLastError());
     return 1;
 }

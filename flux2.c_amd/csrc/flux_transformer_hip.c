@@ -158,8 +158,8 @@ int fh_model_complete(flux_transformer_t *tf) {
 
 static void free_ws(flux_transformer_t *tf) {
     flux_hip_free(tf->x); flux_hip_free(tf->xn); flux_hip_free(tf->qkv); flux_hip_free(tf->kn);
-    flux_hip_free(tf->vt); flux_hip_free(tf->cat); flux_hip_free(tf->tok);
-    tf->x = NULL; tf->xn = tf->qkv = tf->kn = tf->vt = tf->cat = tf->tok = NULL;
+    flux_hip_free(tf->cat); flux_hip_free(tf->tok);
+    tf->x = NULL; tf->xn = tf->qkv = tf->kn = tf->cat = tf->tok = NULL;
     tf->cap_tokens = 0;
 }
 
@@ -196,15 +196,14 @@ int fh_ensure_workspace(flux_transformer_t *tf, int tokens) {
     if (tokens <= tf->cap_tokens) return 1;
     flux_hip_sync();
     free_ws(tf);
-    const size_t H = tf->c.hidden, M = tf->c.mlp, n = tokens, npad = (n + 63) / 64 * 64;
+    const size_t H = tf->c.hidden, M = tf->c.mlp, n = tokens;
     tf->x = (float *)flux_hip_malloc(n * H * 4);
     tf->xn = flux_hip_malloc(n * H * 2);
     tf->qkv = flux_hip_malloc(n * 3 * H * 2);
     tf->kn = flux_hip_malloc(n * H * 2);
-    tf->vt = flux_hip_malloc(H * (npad + 64) * 2); /* two sequences pad their key counts to 64 separately */
     tf->cat = flux_hip_malloc(n * (H + M) * 2);
     tf->tok = flux_hip_malloc(n * tf->c.channels * 2);
-    if (!tf->x || !tf->xn || !tf->qkv || !tf->kn || !tf->vt || !tf->cat || !tf->tok) {
+    if (!tf->x || !tf->xn || !tf->qkv || !tf->kn || !tf->cat || !tf->tok) {
         free_ws(tf);
         return flux_hip_fail("cannot allocate work buffers for %d tokens", tokens);
     }
@@ -349,7 +348,7 @@ static int linear1(int epi, const void *A, const void *W, void *C, const float *
  * [text ; target ; refs], so every GEMM of the single-stream blocks sees all rows of both
  * sequences as one matrix (each weight matrix is streamed once per step instead of twice, and the
  * launch has twice the tiles), the double-stream GEMMs run as 2 nb row ranges, and only attention
- * and its K/V preparation run per sequence.
+ * and its Q/K preparation run per sequence.
  *   z_dev      fp32 [channels, img_h*img_w] target latent
  *   txt_dev[b] bf16 [txt_seq_b, text_dim]
  *   tf->tok rows [n_target, n_img) must already hold the reference tokens (bf16)
@@ -363,18 +362,15 @@ int fh_forward_device_n(flux_transformer_t *tf, int nb, const fh_rope *const *rp
     const int ldcat = H + M;
     const float eps = 1e-6f;
     if (nb < 1 || nb > 2) return flux_hip_fail("forward: %d sequences (1 or 2)", nb);
-    int R[2] = {0, 0}, Nt[2] = {0, 0}, N[2] = {0, 0}, ldvt[2] = {0, 0}, Ntot = 0;
-    size_t vt_off[2] = {0, 0};
+    int R[2] = {0, 0}, Nt[2] = {0, 0}, N[2] = {0, 0}, Ntot = 0;
     const int Ni = rp[0]->n_img;
     for (int b = 0; b < nb; b++) {
         if (rp[b]->n_img != Ni) return flux_hip_fail("forward: sequences differ in image tokens");
         R[b] = Ntot; Nt[b] = rp[b]->txt_seq; N[b] = rp[b]->n;
-        ldvt[b] = (N[b] + 63) / 64 * 64;
-        vt_off[b] = b ? vt_off[b - 1] + (size_t)H * ldvt[b - 1] * 2 : 0;
         Ntot += N[b];
     }
     if (Ntot > tf->cap_tokens) return flux_hip_fail("forward: work buffers hold %d tokens, %d needed", tf->cap_tokens, Ntot);
-    char *xn = (char *)tf->xn, *qkv = (char *)tf->qkv, *cat = (char *)tf->cat, *kn = (char *)tf->kn, *vt = (char *)tf->vt;
+    char *xn = (char *)tf->xn, *qkv = (char *)tf->qkv, *cat = (char *)tf->cat, *kn = (char *)tf->kn;
     float *x = tf->x;
     const float *mt = mod_ptr(tf, 0, step), *mi = mod_ptr(tf, 1, step), *ms = mod_ptr(tf, 2, step), *mf = mod_ptr(tf, 3, step);
     flux_hip_linear_part p[4];
@@ -402,11 +398,11 @@ int fh_forward_device_n(flux_transformer_t *tf, int nb, const fh_rope *const *rp
         }
         if (!flux_hip_linear(FLUX_HIP_EPI_BF16, 2 * nb, p, 3 * H, H, H, H, 3 * H, 0, 0)) return 0;
         for (int b = 0; b < nb; b++) {
-            const char *q_b = qkv + (size_t)R[b] * 3 * H * 2;
-            if (!flux_hip_kv_prepare(kn + (size_t)R[b] * H * 2, vt + vt_off[b], ldvt[b], q_b, 3 * H, H, 2 * H, N[b], heads, Nt[b], blk->norm_k[0],
-                                     blk->norm_k[1], rp[b]->cos, rp[b]->sin, eps)) return 0;
-            if (!flux_hip_attention(cat + (size_t)R[b] * ldcat * 2, ldcat, q_b, 3 * H, kn + (size_t)R[b] * H * 2, vt + vt_off[b], ldvt[b], N[b], N[b],
-                                    heads, Nt[b], blk->norm_q[0], blk->norm_q[1], rp[b]->cos, rp[b]->sin, eps)) return 0;
+            char *q_b = qkv + (size_t)R[b] * 3 * H * 2;
+            if (!flux_hip_qk_prepare(kn + (size_t)R[b] * H * 2, q_b, 3 * H, 0, H, N[b], heads, Nt[b], blk->norm_q[0], blk->norm_q[1],
+                                     blk->norm_k[0], blk->norm_k[1], rp[b]->cos, rp[b]->sin, eps)) return 0;
+            if (!flux_hip_attention(cat + (size_t)R[b] * ldcat * 2, ldcat, q_b, 3 * H, kn + (size_t)R[b] * H * 2, q_b + (size_t)2 * H * 2, 3 * H,
+                                    N[b], N[b], heads)) return 0;
         }
         for (int b = 0; b < nb; b++) {
             p[2 * b] = (flux_hip_linear_part){cat + (size_t)R[b] * ldcat * 2, blk->proj[0], x + (size_t)R[b] * H, mt + 2 * H, Nt[b]};
@@ -451,11 +447,11 @@ int fh_forward_device_n(flux_transformer_t *tf, int nb, const fh_rope *const *rp
             if (!linear1(FLUX_HIP_EPI_SWIGLU, xn, blk->qkv_mlp, cat + (size_t)H * 2, NULL, Ntot, 2 * M, H, H, H, ldcat, 3 * H, 3 * H + M)) return 0;
         }
         for (int b = 0; b < nb; b++) {
-            const char *q_b = qkv + (size_t)R[b] * 3 * H * 2;
-            if (!flux_hip_kv_prepare(kn + (size_t)R[b] * H * 2, vt + vt_off[b], ldvt[b], q_b, 3 * H, H, 2 * H, N[b], heads, N[b], blk->norm_k, NULL,
+            char *q_b = qkv + (size_t)R[b] * 3 * H * 2;
+            if (!flux_hip_qk_prepare(kn + (size_t)R[b] * H * 2, q_b, 3 * H, 0, H, N[b], heads, N[b], blk->norm_q, NULL, blk->norm_k, NULL,
                                      rp[b]->cos, rp[b]->sin, eps)) return 0;
-            if (!flux_hip_attention(cat + (size_t)R[b] * ldcat * 2, ldcat, q_b, 3 * H, kn + (size_t)R[b] * H * 2, vt + vt_off[b], ldvt[b], N[b], N[b],
-                                    heads, N[b], blk->norm_q, NULL, rp[b]->cos, rp[b]->sin, eps)) return 0;
+            if (!flux_hip_attention(cat + (size_t)R[b] * ldcat * 2, ldcat, q_b, 3 * H, kn + (size_t)R[b] * H * 2, q_b + (size_t)2 * H * 2, 3 * H,
+                                    N[b], N[b], heads)) return 0;
         }
         p[0] = (flux_hip_linear_part){cat, blk->out, x, ms + 2 * H, Ntot};
         an[0] = (flux_hip_adaln_part){xn, ms, ms + H};

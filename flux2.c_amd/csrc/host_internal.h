@@ -45,7 +45,7 @@ struct flux_transformer {
     /* work buffers for cap_tokens tokens */
     int cap_tokens;
     float *x;                      /* f32 [n, H] residual stream */
-    void *xn, *qkv, *kn, *vt, *cat, *tok;
+    void *xn, *qkv, *kn, *cat, *tok;
     fh_rope rope[FH_ROPE_SLOTS];
     int rope_next;
     /* per-schedule modulation */

@@ -77,8 +77,8 @@ def lib():
     L.flux_hip_linear_probe_read_tile.argtypes = [c_i, ctypes.POINTER(c_i), ctypes.POINTER(c_f)]
     L.flux_hip_linear_probe_read_launches.argtypes = [c_i, vp, vp]
     L.flux_hip_adaln_norm.argtypes = [vp, c_i, vp, c_i, c_i, c_i, vp, vp, vp, vp, c_f]
-    L.flux_hip_kv_prepare.argtypes = [vp, vp, c_i, vp, c_i, c_i, c_i, c_i, c_i, c_i, vp, vp, vp, vp, c_f]
-    L.flux_hip_attention.argtypes = [vp, c_i, vp, c_i, vp, vp, c_i, c_i, c_i, c_i, c_i, vp, vp, vp, vp, c_f]
+    L.flux_hip_qk_prepare.argtypes = [vp, vp, c_i, c_i, c_i, c_i, c_i, c_i, vp, vp, vp, vp, vp, vp, c_f]
+    L.flux_hip_attention.argtypes = [vp, c_i, vp, c_i, vp, vp, c_i, c_i, c_i, c_i]
     L.flux_hip_gemv.argtypes = [vp, vp, vp, c_i, c_i, c_i, c_i]
     L.flux_hip_latent_to_tokens.argtypes = [vp, vp, c_i, c_i]
     L.flux_hip_f32_to_bf16.argtypes = [vp, vp, c_sz]

@@ -181,28 +181,30 @@ int flux_hip_adaln_norm(void *out_bf16, int ldo, const float *x, int rows, int h
                         const float *shift1, const float *scale1, float eps);
 
 /*
- * Prepares K and V of one attention call from the fused qkv buffer (bf16 [rows, ld] with
- * K at column k_col and V at column v_col): K gets per-head RMSNorm * weight then RoPE and is
- * written to k_out [rows, heads*128]; V is written transposed to vt_out [heads*128, ld_vt].
- * Rows [0, split) use k_w0, the rest k_w1. Replaces the K half of apply_qk_norm
- * (flux_transformer.c:1052-1106) and apply_rope_2d (flux_transformer.c:719-741), and the
- * head transposes (flux_transformer.c:1117-1138).
+ * Prepares Q and K of one attention call in the fused qkv buffer (bf16 [rows, ld] with Q at column
+ * q_col and K at column k_col): per-head RMSNorm * weight, then RoPE. K is written to k_out
+ * [rows, heads*128]; Q is written back in place, already multiplied by 1/sqrt(128) and log2(e) (the
+ * attention kernel works on base-2 logits). Rows [0, split) use q_w0 / k_w0, the rest q_w1 / k_w1.
+ * Replaces apply_qk_norm (flux_transformer.c:1052-1106) and apply_rope_2d
+ * (flux_transformer.c:719-741). The reference's head transposes (flux_transformer.c:1117-1138)
+ * have no counterpart: the attention kernel reads V where the projection wrote it and transposes
+ * tiles of it on the way into the matrix unit.
  */
-int flux_hip_kv_prepare(void *k_out, void *vt_out, int ld_vt, const void *qkv, int ld, int k_col, int v_col,
-                        int rows, int heads, int split, const float *k_w0, const float *k_w1,
+int flux_hip_qk_prepare(void *k_out, void *qkv, int ld, int q_col, int k_col, int rows, int heads, int split,
+                        const float *q_w0, const float *q_w1, const float *k_w0, const float *k_w1,
                         const float *rope_cos, const float *rope_sin, float eps);
 
 /*
- * Multi-head attention, no mask: out = softmax(q k^T / sqrt(128)) v per head, online softmax,
- * scores never stored. q is read raw from the qkv buffer and gets per-head RMSNorm * weight and
- * RoPE inside the kernel; k and vt come from flux_hip_kv_prepare. head_dim is 128.
+ * Multi-head attention, no mask: out = softmax(q k^T) v per head with base-2 exponentials, online
+ * softmax, scores never stored. q (prepared in place by flux_hip_qk_prepare) and v are read from
+ * the qkv buffer (row strides ldq and ldv, the pointers already at their first column); k
+ * [seq_k, heads*128] comes from flux_hip_qk_prepare. head_dim is 128. The queries may be a row
+ * range of the sequence (q and out at its first row). (seq_k + 64) * ldv * 2 must stay below 2^32.
  * Replaces joint_attention / mha_forward (flux_transformer.c:1249-1460), flux_flash_attention
- * (flux_kernels.c:877), flux_softmax (flux_kernels.c:596) and the Q half of apply_qk_norm /
- * apply_rope_2d.
+ * (flux_kernels.c:877) and flux_softmax (flux_kernels.c:596).
  */
-int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ldq, const void *k, const void *vt, int ld_vt,
-                       int seq_q, int seq_k, int heads, int split, const float *q_w0, const float *q_w1,
-                       const float *rope_cos, const float *rope_sin, float eps);
+int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ldq, const void *k, const void *v, int ldv,
+                       int seq_q, int seq_k, int heads);
 
 /* y[m, n] = sum_k f(x[m, k]) * W[n, k], x f32 [M, K] (M small), W bf16, y f32; f = SiLU when
  * silu_input. The modulation and time-embedding projections (flux_transformer.c:956-969,

@@ -429,7 +429,7 @@ def test_gemv(hip, oracle_mod, silu):
 
 
 def _attention_case(hip, oracle_mod, n, split, heads, seed, qk_scale=1.0, qkv=None, w=None):
-    """qkv buffer -> kv_prepare -> attention, against qk_norm + rope + attention of the oracle."""
+    """qkv buffer -> qk_prepare -> attention, against qk_norm + rope + attention of the oracle."""
     H = heads * 128
     if qkv is None:
         qkv = q(normal_f32((n, 3 * H), seed, 1))
@@ -450,20 +450,19 @@ def _attention_case(hip, oracle_mod, n, split, heads, seed, qk_scale=1.0, qkv=No
     dqkv = dev_bf16(hip, qkv)
     dw = [hip.DevBuf.from_array(v.astype(np.float32)) for v in w]
     dcos, dsin = hip.DevBuf.from_array(cos), hip.DevBuf.from_array(sin)
-    ldvt = (n + 63) // 64 * 64
-    kn, vt = hip.DevBuf(n * H * 2), hip.DevBuf(H * ldvt * 2)
+    kn = hip.DevBuf(n * H * 2)
     ldo = H + 64
     out = hip.DevBuf.from_array(np.zeros((n, ldo), np.uint16))
     L = hip.lib()
-    hip.check(L.flux_hip_kv_prepare(kn.ptr, vt.ptr, ldvt, dqkv.ptr, 3 * H, H, 2 * H, n, heads, split,
-                                    dw[2].ptr, dw[3].ptr, dcos.ptr, dsin.ptr, 1e-6))
-    hip.check(L.flux_hip_attention(out.ptr, ldo, dqkv.ptr, 3 * H, kn.ptr, vt.ptr, ldvt, n, n, heads, split,
-                                   dw[0].ptr, dw[1].ptr, dcos.ptr, dsin.ptr, 1e-6))
-    # prepared K and V^T
+    hip.check(L.flux_hip_qk_prepare(kn.ptr, dqkv.ptr, 3 * H, 0, H, n, heads, split, dw[0].ptr, dw[1].ptr, dw[2].ptr, dw[3].ptr,
+                                    dcos.ptr, dsin.ptr, 1e-6))
+    hip.check(L.flux_hip_attention(out.ptr, ldo, dqkv.ptr, 3 * H, kn.ptr, dqkv.at(2 * H * 2), 3 * H, n, n, heads))
+    # prepared K; prepared Q in place, scaled by 1/sqrt(128) and log2(e); V untouched
     kn_h = bf16_to_f32(kn.to_array(np.uint16, (n, H)))
     assert rel_l2(kn_h, K) < 4e-3
-    vt_h = bf16_to_f32(vt.to_array(np.uint16, (H, ldvt)))
-    assert np.array_equal(vt_h[:, :n], V.T) and not vt_h[:, n:].any()
+    after = bf16_to_f32(dqkv.to_array(np.uint16, (n, 3 * H)))
+    assert rel_l2(after[:, :H], Q * np.float32(0.08838834764831845 * 1.4426950408889634)) < 4e-3
+    assert np.array_equal(after[:, H:], qkv[:, H:])
     got = bf16_to_f32(out.to_array(np.uint16, (n, ldo)))
     assert not got[:, H:].any()
     return got[:, :H], want
@@ -499,8 +498,8 @@ def test_attention_full_shape_sharp(hip, oracle_mod, n, split):
 @pytest.mark.parametrize("variant", [0, 1])
 def test_attention_query_subrange(hip, oracle_mod, variant):
     """seq_q != seq_k: queries are a row range of the sequence (the reference's joint attention asks for the image and
-    the text queries separately against all keys, flux_transformer.c:1335-1460). The q, RoPE and output pointers move
-    to the range's first row and `split` is counted from there. The rows agree with those of the full call up to bf16
+    the text queries separately against all keys, flux_transformer.c:1335-1460). Q and K are prepared once for the whole
+    sequence; the q and output pointers move to the range's first row. The rows agree with those of the full call up to bf16
     rounding (which queries share a wave decides when the running maximum is re-based, so not bit for bit)."""
     L = hip.lib()
     L.flux_hip_attention_force_variant(variant)
@@ -515,13 +514,11 @@ def test_attention_query_subrange(hip, oracle_mod, variant):
         dqkv = dev_bf16(hip, qkv)
         dw = [hip.DevBuf.from_array(v) for v in w]
         dcos, dsin = hip.DevBuf.from_array(cos), hip.DevBuf.from_array(sin)
-        ldvt = (n + 63) // 64 * 64
-        kn, vt = hip.DevBuf(n * H * 2), hip.DevBuf(H * ldvt * 2)
-        hip.check(L.flux_hip_kv_prepare(kn.ptr, vt.ptr, ldvt, dqkv.ptr, 3 * H, H, 2 * H, n, heads, split,
-                                        dw[2].ptr, dw[3].ptr, dcos.ptr, dsin.ptr, 1e-6))
+        kn, dv = hip.DevBuf(n * H * 2), dqkv.at(2 * H * 2)
+        hip.check(L.flux_hip_qk_prepare(kn.ptr, dqkv.ptr, 3 * H, 0, H, n, heads, split, dw[0].ptr, dw[1].ptr, dw[2].ptr, dw[3].ptr,
+                                        dcos.ptr, dsin.ptr, 1e-6))
         full = hip.DevBuf(n * H * 2)
-        hip.check(L.flux_hip_attention(full.ptr, H, dqkv.ptr, 3 * H, kn.ptr, vt.ptr, ldvt, n, n, heads, split,
-                                       dw[0].ptr, dw[1].ptr, dcos.ptr, dsin.ptr, 1e-6))
+        hip.check(L.flux_hip_attention(full.ptr, H, dqkv.ptr, 3 * H, kn.ptr, dv, 3 * H, n, n, heads))
         full_h = full.to_array(np.uint16, (n, H))
         Q, K, V = qkv[:, :H].copy(), qkv[:, H:2 * H].copy(), qkv[:, 2 * H:].copy()
         for lo, hi, qw, kw in ((0, split, w[0], w[2]), (split, n, w[1], w[3])):
@@ -531,8 +528,7 @@ def test_attention_query_subrange(hip, oracle_mod, variant):
         # text queries only, image queries only, a range that starts inside the text and is not a multiple of anything
         for a, b in ((0, split), (split, n), (137, 431), (699, 700)):
             part = hip.DevBuf.from_array(np.full((b - a, H), 0x7fc0, np.uint16))
-            hip.check(L.flux_hip_attention(part.ptr, H, dqkv.at(a * 3 * H * 2), 3 * H, kn.ptr, vt.ptr, ldvt, b - a, n, heads,
-                                           max(split - a, 0), dw[0].ptr, dw[1].ptr, dcos.at(a * 128 * 4), dsin.at(a * 128 * 4), 1e-6))
+            hip.check(L.flux_hip_attention(part.ptr, H, dqkv.at(a * 3 * H * 2), 3 * H, kn.ptr, dv, 3 * H, b - a, n, heads))
             got = bf16_to_f32(part.to_array(np.uint16, (b - a, H)))
             assert np.isfinite(got).all()
             assert rel_l2(got, bf16_to_f32(full_h[a:b])) < 4e-3, (a, b)
