@@ -130,7 +130,7 @@ extern "C" int flux_hip_qk_prepare(void *k_out, void *qkv, int ld, int q_col, in
  * queries (two 16-query MFMA columns) and the full head dimension. Keys are walked in tiles of 64
  * through two LDS stages filled by direct global->LDS loads (no register staging).
  *   LDS stage: K tile [64 keys][128 d] (256-byte rows, 16-byte chunks XOR-swizzled by key%16)
- *              V tile [64 keys][128 d] (256-byte rows, 16-byte chunk c of key r at position c ^ 2 (r%4))
+ *              V tile [64 keys][128 d] (256-byte rows, 16-byte chunk c of key r at position c ^ 2 (r%4) ^ (r&8))
  * MFMA: v_mfma_f32_16x16x32_bf16 (the form that sustains the most under the power limit).
  *   S^T[key][q]: A = K fragment (lane: key l%16, dims 8(l/16)..+8 of a 32-dim chunk),
  *                B = Q fragment (lane: query l%16, same dims); accumulator lane: query l%16,
@@ -142,7 +142,9 @@ extern "C" int flux_hip_qk_prepare(void *k_out, void *qkv, int ld, int q_col, in
  * A transposing read works in groups of 16 lanes: lane 4 e + t of the group points at four
  * consecutive dims (quad t of a 16-dim block) of key e of four keys, and lane j of the group receives
  * dim j of the block for those four keys. The four keys' rows lie 256 bytes apart, i.e. on the same
- * banks; the swizzle moves each row's 32-byte piece of a block to a different bank group.
+ * banks; the swizzle moves each row's 32-byte piece of a block to a different bank group, and the
+ * pieces of the rows eight further on (the next group of 16 lanes, served in the same cycle) to
+ * the other half of the 256 bytes.
  * --------------------------------------------------------------------------------------- */
 #define ATT_STAGE (64 * 256 + 64 * 256)
 #define ATT_WIDE_LDS (8 * 16384) /* attention_wide_kernel: four K and four V slots */
@@ -217,7 +219,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
         k_src[i] = k + h * HD + (((lane & 15) ^ (r & 15)) << 3);
         k_dst[i] = (wave * 4 + i * (NW * 4)) * 256;
         /* V: the same four rows, keys in their natural order (LDS row r = key r of the tile) */
-        v_src[i] = v + h * HD + (((lane & 15) ^ (2 * (r & 3))) << 3);
+        v_src[i] = v + h * HD + (((lane & 15) ^ (2 * (r & 3)) ^ (r & 8)) << 3);
     }
     /* LDS: K ring = 2 slots of 16 KB at 0 and 16 KB; V ring = 2 slots of 16 KB at 32 and 48 KB */
     auto issue_k = [&](int t) {
@@ -298,7 +300,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
         auto vread = [&](int b, bf16x8 (&dst)[4]) { /* 32-key chunk b/2, head-dim blocks 4(b%2) .. +3 */
 #pragma unroll
             for (int f = 0; f < 4; f++) /* this lane points at key 32 (b/2) + 8 lq + l15/4 (+4), dims 4 (l15%4) .. +3 of block f */
-                dst[f] = v_fragment(vtile + (32 * (b >> 1) + 8 * lq + (l15 >> 2)) * 256 + ((f ^ (l15 >> 2)) << 5) + (l15 & 3) * 8 + (b & 1) * 128);
+                dst[f] = v_fragment(vtile + (32 * (b >> 1) + 8 * lq + (l15 >> 2)) * 256 + ((f ^ (l15 >> 2)) << 5) + (l15 & 3) * 8 + (((b ^ lq) & 1) << 7));
         };
         bf16x8 fa[4], fb[4];
         {
@@ -506,8 +508,8 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
     const char *v_base = (const char *)(v + h * HD);
     int k_row[LP];       /* key of the tile that this lane fetches with load i */
     const unsigned k_chunk = (unsigned)(((lane & 15) ^ ((wave * 4 + (lane >> 4)) & 15)) << 4);
-    /* V: LDS row = key of the tile, 16-byte chunk c of row r at position c ^ 2 (r % 4) */
-    const unsigned v_chunk = (unsigned)(((lane & 15) ^ (2 * (lane >> 4))) << 4);
+    /* V: LDS row = key of the tile, 16-byte chunk c of row r at position c ^ 2 (r % 4) ^ (r & 8) */
+    const unsigned v_chunk = (unsigned)(((lane & 15) ^ (2 * (lane >> 4)) ^ ((wave & 2) << 2)) << 4);
 #pragma unroll
     for (int i = 0; i < LP; i++) {
         const int r = wave * 4 + i * (NW * 4) + (lane >> 4); /* LDS row; (r & 15) is the same for every i */
@@ -610,21 +612,21 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
     /* Per-lane LDS addresses of the fragments in the slots that are read next, kept in registers and moved on by one
      * slot per tile (recomputed from the slot number they cost a vector add per read): the K fragments of head-dim
      * step kk, key block 0 of chunk 0 (the others lie 4096 (2 cp + i) further), and the V^T fragments of chunk 0 for
-     * the head-dim blocks x with x % 4 = w, as this lane of a transposing read sees them (see v_fragment: the swizzle
-     * moves a block by the lane's key; chunk 1 lies 8192 further, blocks 4 .. 7 128). */
+     * head-dim block x, as this lane of a transposing read sees them (the swizzle moves a block by the lane's key;
+     * chunk 1 lies 8192 further). */
     const unsigned lds0 = (unsigned)(uintptr_t)LDS_PTR(smem); /* folded into the addresses once, not added at every read */
-    unsigned ka[4], va[4];
+    unsigned ka[4], va[8];
 #pragma unroll
     for (int kk = 0; kk < 4; kk++) ka[kk] = lds0 + l15 * 256 + (((kk * 4 + lq) ^ l15) << 4);
 #pragma unroll
-    for (int w = 0; w < 4; w++) va[w] = lds0 + 4 * 16384 + (8 * lq + (l15 >> 2)) * 256 + ((w ^ (l15 >> 2)) << 5) + (l15 & 3) * 8;
+    for (int x = 0; x < 8; x++) va[x] = lds0 + 4 * 16384 + (8 * lq + (l15 >> 2)) * 256 + ((x ^ (l15 >> 2) ^ ((lq & 1) << 2)) << 5) + (l15 & 3) * 8;
     auto kfrag1 = [&](int cp, int x) { /* x = 0..7: key block 2cp + x%2 of the tile, head dims 32 (x/2) .. +31 */
         const int kk = x >> 1, i = x & 1;
         kf[kk][i] = lds_read_bf16x8(ka[kk] + (2 * cp + i) * 4096);
     };
     auto vhalf1 = [&](int cp, int y) { /* y = 0..15: head-dim block y / 2, keys 8 lq + 4 (y % 2) .. +3 of 32-key chunk cp */
         const int x = y >> 1;
-        vh[x][y & 1] = v_half_fragment_at(va[x & 3] + cp * 8192 + (x >> 2) * 128 + (y & 1) * 1024);
+        vh[x][y & 1] = v_half_fragment_at(va[x] + cp * 8192 + (y & 1) * 1024);
     };
     /* what a phase of 8 NQ MFMAs requests behind MFMA m: K fragment x behind MFMA x NQ, V^T half fragment y behind
      * MFMA y NQ / 2 */
@@ -642,17 +644,20 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) ka[kk] += dk;
 #pragma unroll
-        for (int w = 0; w < 4; w++) va[w] += dv;
+        for (int x = 0; x < 8; x++) va[x] += dv;
     };
-    /* The same one register at a time behind the MFMAs of an odd step's product phase: the V addresses (last used in
-     * the score phase before) behind MFMAs 1, 2, 3, 5, the K addresses behind the last K read (at 7 NQ) */
-    auto move_slots_at = [&](int dk, int dv, int m) {
+    /* The same a few registers at a time behind the row-sum MFMAs (the only MFMAs of the loop that carry no other
+     * vector instruction; next to an exponential an addition costs the matrix pipe some nine cycles): the V addresses
+     * in the odd step, whose score phase was their last user, the K addresses in the even step after it. */
+    auto move_v_slots_at = [&](int dv, int j) {
 #pragma unroll
-        for (int w = 0; w < 4; w++)
-            if (m == (NQ > 1 ? w + 1 + (w == 3) : 2 * w + 1)) va[w] += dv;
+        for (int x = 0; x < 8; x++)
+            if (x * NQ / 8 == j) asm volatile("v_add_u32 %0, %1, %0" : "+v"(va[x]) : "s"(dv));
+    };
+    auto move_k_slots_at = [&](int dk, int j) {
 #pragma unroll
         for (int kk = 0; kk < 4; kk++)
-            if (m == (NQ > 1 ? 8 * NQ - 4 + kk : 7)) ka[kk] += dk;
+            if (kk * NQ / 4 == j) asm volatile("v_add_u32 %0, %1, %0" : "+v"(ka[kk]) : "s"(dk));
     };
     /* The vector instructions of the loop are inline assembly as well: an ordinary expression the compiler may
      * sink to its use in the next phase, and then nothing overlaps.
@@ -706,12 +711,16 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
         }
     };
     /* row sums and O^T += V^T P^T for one chunk; vh must already hold (or be receiving) the chunk's fragments.
-     * between(m) runs behind PV MFMA m (m = 0 .. 8 NQ - 1). */
-    auto pv_phase = [&](auto &&between, auto guard_c) {
+     * head(j) runs behind row-sum MFMA j (j = 0 .. NQ - 1), between(m) behind PV MFMA m (m = 0 .. 8 NQ - 1). */
+    auto pv_phase = [&](auto &&head, auto &&between, auto guard_c) {
         constexpr bool GUARD = decltype(guard_c)::value;
         /* the row sums are the first readers of each probability fragment */
 #pragma unroll
-        for (int j = 0; j < NQ; j++) MFMA_ACC_A_ONES_GUARDED(l_acc[j], ones, pf[j]);
+        for (int j = 0; j < NQ; j++) {
+            MFMA_ACC_A_ONES_GUARDED(l_acc[j], ones, pf[j]);
+            head(j);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int g = 0; g < 2; g++)
@@ -816,7 +825,10 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
             if (LOADS) v_loads_at((t + 2) & 3, m);
         }, guard_c);
         if (LAST) mask_chunk(s_b, 2 * t + 1);
-        pv_phase([&](int m) {
+        const int dk = ((t + 1) & 3) ? 16384 : -3 * 16384; /* K fragments from tile t + 1's slot now: one slot on, or three back */
+        pv_phase([&](int j) {
+            if (LOADS) move_k_slots_at(dk, j);
+        }, [&](int m) {
             if (!LAST) k_reads_at(0, m);
             if (m >= EXP0) exp1(s_b, m - EXP0);
         }, guard_c);
@@ -825,9 +837,7 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
     };
     /* Odd step of tile t: the barrier, scores of tile t+1's first chunk into s_a, product of tile t's second chunk. */
     auto odd_step = [&](int t, auto ragged_c, auto guard_c) {
-        /* to the slots of the next tile (K fragments then come from tile t + 2's slot, V^T fragments from tile t + 1's):
-         * one slot on, or three back */
-        const int dk = ((t + 2) & 3) ? 16384 : -3 * 16384, dv = ((t + 1) & 3) ? 16384 : -3 * 16384;
+        const int dv = ((t + 1) & 3) ? 16384 : -3 * 16384; /* V^T fragments from tile t + 1's slot after this step */
         /* this wave's parts of K(t+2) and V(t+1) are in LDS: everything but the eight loads issued since the last barrier */
         asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * LP) : "memory");
         s_phase(s_a, [&](int m) {
@@ -836,10 +846,9 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
             k_loads_at(t & 3, m);
         }, guard_c);
         if (decltype(ragged_c)::value) mask_chunk(s_a, 2 * t + 2);
-        pv_phase([&](int m) {
+        pv_phase([&](int j) { move_v_slots_at(dv, j); }, [&](int m) {
             k_reads_at(1, m);
             if (m >= EXP0) exp1(s_a, m - EXP0);
-            move_slots_at(dk, dv, m);
         }, guard_c);
 #pragma unroll
         for (int n = 8 * NQ - EXP0; n < 8 * NQ; n++) exp1(s_a, n);
@@ -851,7 +860,7 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
 #pragma unroll
         for (int n = 0; n < 4 * NQ; n++) cvt1(s_b, n);
         __builtin_amdgcn_sched_barrier(0);
-        pv_phase(nothing, AttFlag<true>{});
+        pv_phase(nothing, nothing, AttFlag<true>{});
     };
     /* (outside the loop every MFMA carries its guard, see s_phase) */
     if (ntiles == 1) {
