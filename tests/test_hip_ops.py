@@ -587,13 +587,15 @@ def test_layout_edges_and_updates(hip, oracle_mod):
     np.testing.assert_allclose(dz.to_array(np.float32, (999,)), want, rtol=0, atol=2e-6)
 
 
-@pytest.mark.parametrize("variant", [-1, 0, 1, 11, 12, 13, 14])
+@pytest.mark.parametrize("variant", [-1, 0, 1, 11, 12, 13, 14, 15])
 def test_attention_workgroup_variants(hip, oracle_mod, variant):
     """Every kernel variant (32 queries per wave in workgroups of 128 and 256 queries; 16, 32, 48 and 64 queries
-    per wave in workgroups of four waves) gives the same answer on ragged lengths, from a single key tile up."""
+    per wave in workgroups of four waves; 15: their automatic mix also below 129 keys, where -1 takes the older kernel)
+    gives the same answer on ragged lengths, from a single key tile up (one, two and three tiles take their own paths
+    through the four-slot rings of the wide kernel)."""
     hip.lib().flux_hip_attention_force_variant(variant)
     try:
-        for n, split, heads in ((300, 100, 2), (513, 512, 1), (40, 16, 2), (64, 64, 1), (130, 0, 3), (1000, 77, 2)):
+        for n, split, heads in ((300, 100, 2), (513, 512, 1), (40, 16, 2), (64, 64, 1), (100, 30, 2), (128, 0, 1), (130, 0, 3), (1000, 77, 2)):
             got, want = _attention_case(hip, oracle_mod, n, split, heads, 30 + variant)
             assert rel_l2(got, want) < 1e-2, (n, rel_l2(got, want))
         got, want = _attention_case(hip, oracle_mod, 700, 130, 2, 60 + variant, qk_scale=3.0)     # sharp logits: the maximum moves
