@@ -968,7 +968,7 @@ static WidePlan wide_plan(int seq_q, int heads) {
     static int c_seq = -1, c_heads = -1;
     static WidePlan c_plan;
     if (seq_q == c_seq && heads == c_heads) return c_plan;
-    static const double cost[5] = {0.0, 0.43, 0.54, 0.70, 1.0};
+    static const double cost[5] = {0.0, 0.44, 0.62, 0.81, 1.0};
     int cus = 256, dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 8) cus = 256;
     const int per_xcd = cus / 8, nh = (heads + 7) / 8;
