@@ -380,7 +380,7 @@ def bench_attention(args):
                                f"q/k/v, unit QK-norm weights, random RoPE angles; variant {args.attention_variant}"},
         "device_ms_per_step_events": round(ev_ms / args.steps, 4),
         "roofline": {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(ach / PEAK_BF16_TFLOPS, 4),
-                     "traffic": None, "kernel": "attention_wide_kernel (+ its empty second pass): softmax(q k^T / sqrt(128)) v, 4 n^2 H FLOP",
+                     "traffic": None, "kernel": "attention_wide_kernel: softmax(q k^T / sqrt(128)) v, 4 n^2 H FLOP",
                      "ms_per_launch": round(att_ms, 4), "flops_per_launch": flops},
         "qk_prepare": {"bound": "hbm", "ms_per_launch": round(prep_ms, 4), "bytes_per_launch": prep_bytes,
                        "achieved_GBps": round(prep_bytes / (prep_ms * 1e-3) / 1e9, 1), "peak_GBps": 8000.0,

@@ -173,30 +173,13 @@ __device__ __forceinline__ bf16x8 v_fragment(const char *p) { return v_join(v_ha
 template <bool V> struct AttFlag { static constexpr bool value = V; };
 template <int V> struct AttInt { static constexpr int value = V; };
 
+/* One workgroup's work: the queries [q_begin, q_end) of head h, at most 32 NW of them. All NW waves must call it. */
 template <int NW>
-__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf16 *__restrict__ out, int ldo,
-                                                           const bf16 *__restrict__ q, int ldq,
-                                                           const bf16 *__restrict__ k, const bf16 *__restrict__ v, int ldv,
-                                                           int seq_q, int seq_k, int heads, int *redo) {
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-    /* Workgroups are dealt round-robin to the 8 XCDs, each with its own L2. Give every XCD a
-     * contiguous run of (head, query block) pairs, so that all query blocks of a head run on one
-     * XCD and its K / V (2.4 MB at 4608 tokens) are fetched from HBM once and then served from
-     * that L2, instead of by all eight. */
-    constexpr int BQ = NW * 32;  /* queries per workgroup */
+__device__ __forceinline__ void attention_block(char *smem, const int h, const int q_begin, const int q_end, bf16 *__restrict__ out, int ldo,
+                                const bf16 *__restrict__ q, int ldq, const bf16 *__restrict__ k, const bf16 *__restrict__ v, int ldv,
+                                int seq_k, int heads) {
     constexpr int LP = 16 / NW;  /* wave-wide load instructions per wave and tile, for K and for V */
-    const int nqb = (seq_q + BQ - 1) / BQ;
-    const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
-    if (logical >= nqb * heads) return;
-    const int h = logical / nqb, qb = logical - h * nqb;
     const int tid = threadIdx.x, lane = tid & 63;
-    if (redo) {
-        /* second pass behind attention_wide_kernel: only the query blocks it has marked are computed (again) here */
-        const int marked = redo[h * nqb + qb];
-        __syncthreads();
-        if (!marked) return;
-        if (tid == 0) redo[h * nqb + qb] = 0;
-    }
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l15 = lane & 15, lq = lane >> 4;
     const int H = heads * HD;
@@ -248,8 +231,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
     int qrow[2];
 #pragma unroll
     for (int t = 0; t < 2; t++) {
-        qrow[t] = qb * BQ + wave * 32 + t * 16 + l15;
-        const bf16 *qp = q + (size_t)min(qrow[t], seq_q - 1) * ldq + h * HD + lq * 8;
+        qrow[t] = q_begin + wave * 32 + t * 16 + l15;
+        const bf16 *qp = q + (size_t)min(qrow[t], q_end - 1) * ldq + h * HD + lq * 8;
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) qf[t][kk] = *(const bf16x8 *)(qp + kk * 32);
     }
@@ -419,7 +402,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
 #pragma unroll
     for (int u = 0; u < 2; u++) {
         const float inv_l = 1.0f / l_acc[u][0];
-        if (qrow[u] < seq_q) {
+        if (qrow[u] < q_end) {
             bf16 *op = out + (size_t)qrow[u] * ldo + h * HD + lq * 4;
 #pragma unroll
             for (int dt = 0; dt < 8; dt++) {
@@ -429,6 +412,35 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
                 *(bf16x4 *)(op + dt * 16) = r;
             }
         }
+    }
+}
+
+
+template <int NW>
+__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf16 *__restrict__ out, int ldo,
+                                                           const bf16 *__restrict__ q, int ldq,
+                                                           const bf16 *__restrict__ k, const bf16 *__restrict__ v, int ldv,
+                                                           int seq_q, int seq_k, int heads) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    /* Workgroups are dealt round-robin to the 8 XCDs, each with its own L2. Give every XCD a
+     * contiguous run of (head, query block) pairs, so that all query blocks of a head run on one
+     * XCD and its K / V (2.4 MB at 4608 tokens) are fetched from HBM once and then served from
+     * that L2, instead of by all eight. */
+    constexpr int BQ = NW * 32;  /* queries per workgroup */
+    const int nqb = (seq_q + BQ - 1) / BQ;
+    const int logical = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    if (logical >= nqb * heads) return;
+    const int h = logical / nqb, qb = logical - h * nqb;
+    attention_block<NW>(smem, h, qb * BQ, min(qb * BQ + BQ, seq_q), out, ldo, q, ldq, k, v, ldv, seq_k, heads);
+}
+
+/* The wide kernel's way out for a workgroup whose softmax references did not hold (see first_reference): the same
+ * queries once more with moving references, 128 at a time. One copy for all instances of the wide kernel. */
+__device__ __attribute__((noinline)) void attention_redo(char *smem, int h, int q_begin, int q_end, bf16 *out, int ldo, const bf16 *q, int ldq,
+                                                         const bf16 *k, const bf16 *v, int ldv, int seq_k, int heads) {
+    for (int qs = q_begin; qs < q_end; qs += 128) {
+        attention_block<4>(smem, h, qs, min(qs + 128, q_end), out, ldo, q, ldq, k, v, ldv, seq_k, heads);
+        __syncthreads(); /* the next block's first loads go to LDS slots this one may still be reading */
     }
 }
 
@@ -483,7 +495,7 @@ __device__ __forceinline__ void mfma_results_fence_a(f32x4 (&acc)[8][N]) {
 template <int NQ>
 __device__ __forceinline__ void attention_wide_body(char *smem, const int h, const int q0, bf16 *__restrict__ out, int ldo,
                                                     const bf16 *__restrict__ q, int ldq, const bf16 *__restrict__ k,
-                                                    const bf16 *__restrict__ v, int ldv, int seq_q, int seq_k, int heads, int *redo) {
+                                                    const bf16 *__restrict__ v, int ldv, int seq_q, int seq_k, int heads) {
     constexpr int NW = 4, WQ = 16 * NQ, LP = 16 / NW;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -760,9 +772,8 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
      * probabilities of one row) before anything leaves the range of fp32. The loop never looks at the scores'
      * size again and never moves the references: maxima cost a vector instruction per two scores, and rescaling
      * O with vector instructions inside the loop makes the register allocator carry O through VGPRs on every
-     * trip. Should a row overflow all the same, its sums show it at the end: the wave then marks its query blocks
-     * in `redo` instead of writing output, and attention_kernel<4>, launched behind this kernel, computes the
-     * marked blocks with its moving references. */
+     * trip. Should a row overflow all the same, its sums show it at the end: the workgroup then writes no output
+     * and computes its queries once more with moving references (attention_redo). */
     auto first_reference = [&](f32x4 (&sc)[2][NQ]) {
 #pragma unroll
         for (int j = 0; j < NQ; j++) {
@@ -893,13 +904,9 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
 #pragma unroll
             for (int e = 0; e < 4; e++) worst = max(worst, __float_as_uint(o_acc[i][j][e]) & 0x7fffffffu);
     }
-    if (__any(worst >= 0x71800000u)) {
-        /* attention_kernel<4> works on blocks of 128 queries: mark those this wave's queries lie in */
-        const int qw0 = q0 + wave * WQ, qw1 = min(qw0 + WQ, seq_q) - 1;
-        if (lane == 0 && qw0 < seq_q) {
-            const int nqb128 = (seq_q + 127) >> 7;
-            for (int b128 = qw0 >> 7; b128 <= qw1 >> 7; b128++) redo[h * nqb128 + b128] = 1;
-        }
+    /* the workgroup decides as one: the way out needs all four waves */
+    if (__syncthreads_or(worst >= 0x71800000u)) {
+        attention_redo(smem, h, q0, min(q0 + NW * WQ, seq_q), out, ldo, q, ldq, k, v, ldv, seq_k, heads);
         return;
     }
 #pragma unroll
@@ -928,34 +935,18 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
 template <int NQA, int NQB>
 __global__ __launch_bounds__(256, 1) void attention_wide_kernel(bf16 *__restrict__ out, int ldo, const bf16 *__restrict__ q, int ldq,
                                                                 const bf16 *__restrict__ k, const bf16 *__restrict__ v, int ldv,
-                                                                int seq_q, int seq_k, int heads, int *redo, int na, int nb) {
+                                                                int seq_q, int seq_k, int heads, int na, int nb) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int xcd = blockIdx.x & 7, hx0 = xcd * heads / 8, nh = (xcd + 1) * heads / 8 - hx0;
     int item = blockIdx.x >> 3;
     if (item >= nh * (na + nb)) return;
     if (item < nh * na) {
-        attention_wide_body<NQA>(smem, hx0 + item / na, (item % na) * 64 * NQA, out, ldo, q, ldq, k, v, ldv, seq_q, seq_k, heads, redo);
+        attention_wide_body<NQA>(smem, hx0 + item / na, (item % na) * 64 * NQA, out, ldo, q, ldq, k, v, ldv, seq_q, seq_k, heads);
     } else {
         item -= nh * na;
         attention_wide_body<NQB>(smem, hx0 + item / nb, na * 64 * NQA + (item % nb) * 64 * NQB, out, ldo, q, ldq, k, v, ldv, seq_q,
-                                 seq_k, heads, redo);
+                                 seq_k, heads);
     }
-}
-
-/* Marks of attention_wide_kernel for the second pass, one per (head, block of 128 queries); all zero between
- * calls (the second pass clears what it finds). A static device array: attention allocates nothing. */
-#define ATT_REDO_MAX (1 << 16)
-static __device__ int g_att_redo[ATT_REDO_MAX];
-static int *g_att_redo_ptr[64];
-static int *att_redo_for_current_device() {
-    int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
-    if (!g_att_redo_ptr[dev]) {
-        int *p = nullptr;
-        if (hipGetSymbolAddress((void **)&p, HIP_SYMBOL(g_att_redo)) != hipSuccess) return nullptr;
-        g_att_redo_ptr[dev] = p;
-    }
-    return g_att_redo_ptr[dev];
 }
 
 /* How a head's queries are cut into blocks: na blocks of 64 nqa queries, then nb blocks of 64 (nqa - 1). The choice
@@ -1025,14 +1016,12 @@ extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ld
         HIP_OK(hipFuncSetAttribute((const void *)attention_wide_kernel<2, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, ATT_WIDE_LDS));
         attr_done = true;
     }
-    /* Up to two key tiles the kernel with moving references alone is as fast as the wide kernel, and it needs no second
-     * launch (4.6 us that nothing hides at such sizes). */
-    const int variant = g_att_force == -1 && seq_k <= 128 ? 0 : g_att_force;
+    const int variant = g_att_force;
     if (variant == 0 || variant == 1) {
         const int bq = variant ? 256 : 128, blocks = ((seq_q + bq - 1) / bq) * heads;
         hipLaunchKernelGGL(variant ? attention_kernel<8> : attention_kernel<4>, dim3((blocks + 7) & ~7), dim3(variant ? 512 : 256), 2 * ATT_STAGE,
                            flux_hip_stream_handle(), (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)v, ldv,
-                           seq_q, seq_k, heads, (int *)nullptr);
+                           seq_q, seq_k, heads);
         HIP_OK(hipGetLastError());
         return 1;
     }
@@ -1045,17 +1034,11 @@ extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ld
     } else {
         plan = wide_plan(seq_q, heads);
     }
-    const int blocks128 = ((seq_q + 127) / 128) * heads;
-    int *redo = att_redo_for_current_device();
-    if (!redo || blocks128 > ATT_REDO_MAX) return flux_hip_fail("flux_hip_attention: no room for the second-pass marks");
     const int max_nh = (heads + 7) / 8; /* the most heads one XCD takes */
     const dim3 grid(8 * max_nh * (plan.na + plan.nb));
     auto kern = plan.nqa == 4 ? attention_wide_kernel<4, 3> : plan.nqa == 3 ? attention_wide_kernel<3, 2> : attention_wide_kernel<2, 1>;
     hipLaunchKernelGGL(kern, grid, dim3(256), ATT_WIDE_LDS, flux_hip_stream_handle(), (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq,
-                       (const bf16 *)k, (const bf16 *)v, ldv, seq_q, seq_k, heads, redo, plan.na, plan.nb);
-    /* second pass: the blocks of 128 queries the first one marked (normally none: every workgroup leaves at once) */
-    hipLaunchKernelGGL(attention_kernel<4>, dim3((blocks128 + 7) & ~7), dim3(256), 2 * ATT_STAGE, flux_hip_stream_handle(),
-                       (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)v, ldv, seq_q, seq_k, heads, redo);
+                       (const bf16 *)k, (const bf16 *)v, ldv, seq_q, seq_k, heads, plan.na, plan.nb);
     HIP_OK(hipGetLastError());
     return 1;
 }

@@ -31,9 +31,9 @@ void flux_hip_linear_persistent(int on);
 /* 1 (default): the 4-wave tiles run as gemm4d_kernel (operand rings of two or three LDS slots, count-based waits at
  * the barrier); 0: as gemm4w_kernel (two stages, everything in flight awaited at the barrier). Bit-identical results. */
 void flux_hip_linear_ring(int on);
-/* attention kernel: -1 = automatic (default: 64-query waves, block lengths chosen per sequence length; the 32-query-
- * per-wave kernel alone up to 128 keys); 0 / 1 = the 32-query-per-wave kernel with 128 / 256 queries per workgroup;
- * 11..14 = 16, 32, 48, 64 queries per wave throughout; 15 = the automatic mix of block lengths at every size */
+/* attention kernel: -1 and 15 = automatic (default: 64-query waves, block lengths chosen per sequence length);
+ * 0 / 1 = the 32-query-per-wave kernel with 128 / 256 queries per workgroup; 11..14 = 16, 32, 48, 64 queries per wave
+ * throughout */
 void flux_hip_attention_force_variant(int v);
 /* 1 (default): a CFG step runs its two forwards as one batch of two sequences; 0: one after the other.
  * Takes effect at the next flux_hip_session_begin. */

@@ -543,7 +543,8 @@ def test_attention_first_key_tile_far_below_the_rest(hip, oracle_mod, variant):
     all queries and carry a norm weight of 10. The running maximum then starts far below zero; re-basing it must not
     scale the still empty accumulators by 2^1000 (0 * inf). The later keys have logits of order three. The kernels
     with 16 NQ queries per wave fix their references on the first 32 keys and cannot represent the later ones:
-    they hand every query block to the second pass, which must leave the same answer."""
+    their workgroups notice at the end and compute their queries again with moving references, which must leave the same
+    answer."""
     n, split, heads = 192, 64, 1
     u = np.zeros(128, np.float32)
     u[:96] = normal_f32((96,), 46, 1)                 # dims of the RoPE axes that do not turn for text tokens
@@ -556,7 +557,7 @@ def test_attention_first_key_tile_far_below_the_rest(hip, oracle_mod, variant):
         got, want = _attention_case(hip, oracle_mod, n, split, heads, 46, qkv=q(qkv), w=w)
         assert np.isfinite(got).all()
         assert rel_l2(got, want) < 2.5e-2, rel_l2(got, want)
-        # and an ordinary call right afterwards: the second pass has cleared its marks
+        # and an ordinary call right afterwards
         got, want = _attention_case(hip, oracle_mod, 200, 72, 2, 47)
         assert rel_l2(got, want) < 1e-2, rel_l2(got, want)
     finally:
@@ -590,8 +591,7 @@ def test_layout_edges_and_updates(hip, oracle_mod):
 @pytest.mark.parametrize("variant", [-1, 0, 1, 11, 12, 13, 14, 15])
 def test_attention_workgroup_variants(hip, oracle_mod, variant):
     """Every kernel variant (32 queries per wave in workgroups of 128 and 256 queries; 16, 32, 48 and 64 queries
-    per wave in workgroups of four waves; 15: their automatic mix also below 129 keys, where -1 takes the older kernel)
-    gives the same answer on ragged lengths, from a single key tile up (one, two and three tiles take their own paths
+    per wave in workgroups of four waves; 15: their automatic mix, as -1) gives the same answer on ragged lengths, from a single key tile up (one, two and three tiles take their own paths
     through the four-slot rings of the wide kernel)."""
     hip.lib().flux_hip_attention_force_variant(variant)
     try:
