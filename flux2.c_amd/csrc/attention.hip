@@ -932,18 +932,38 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
  * blocks at the end the last round is a short one. Each XCD takes a contiguous run of heads, so that a head's K and
  * V are fetched into one L2 only, and within its run the long blocks of all its heads come first (workgroups are
  * dealt to the XCDs round-robin and started in order). */
+/* One or two sequences per launch (the two forwards of a classifier-free-guidance step attend separately but can
+ * share a launch: more workgroups per round, one launch less per layer). */
+struct AttSeq { bf16 *out; const bf16 *q, *k, *v; int seq_q, seq_k, na, nb; };
+struct AttSeqs { AttSeq s[2]; int nseq; };
+
 template <int NQA, int NQB>
-__global__ __launch_bounds__(256, 1) void attention_wide_kernel(bf16 *__restrict__ out, int ldo, const bf16 *__restrict__ q, int ldq,
-                                                                const bf16 *__restrict__ k, const bf16 *__restrict__ v, int ldv,
-                                                                int seq_q, int seq_k, int heads, int na, int nb) {
+__global__ __launch_bounds__(256, 1) void attention_wide_kernel(AttSeqs p, int ldo, int ldq, int ldv, int heads) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int xcd = blockIdx.x & 7, hx0 = xcd * heads / 8, nh = (xcd + 1) * heads / 8 - hx0;
     int item = blockIdx.x >> 3;
-    if (item >= nh * (na + nb)) return;
-    if (item < nh * na) {
+    /* within an XCD's run: the long blocks of the first sequence, of the second, then the short blocks likewise */
+    const int la0 = nh * p.s[0].na, la1 = p.nseq > 1 ? nh * p.s[1].na : 0;
+    const int lb0 = nh * p.s[0].nb, lb1 = p.nseq > 1 ? nh * p.s[1].nb : 0;
+    const bool is_long = item < la0 + la1;
+    bool second;
+    if (is_long) {
+        second = item >= la0;
+        if (second) item -= la0;
+    } else {
+        item -= la0 + la1;
+        if (item >= lb0 + lb1) return;
+        second = item >= lb0;
+        if (second) item -= lb0;
+    }
+    /* (fields picked one by one: an index into the argument structure would send it through scratch memory) */
+    bf16 *out = second ? p.s[1].out : p.s[0].out;
+    const bf16 *q = second ? p.s[1].q : p.s[0].q, *k = second ? p.s[1].k : p.s[0].k, *v = second ? p.s[1].v : p.s[0].v;
+    const int seq_q = second ? p.s[1].seq_q : p.s[0].seq_q, seq_k = second ? p.s[1].seq_k : p.s[0].seq_k;
+    const int na = second ? p.s[1].na : p.s[0].na, nb = second ? p.s[1].nb : p.s[0].nb;
+    if (is_long) {
         attention_wide_body<NQA>(smem, hx0 + item / na, (item % na) * 64 * NQA, out, ldo, q, ldq, k, v, ldv, seq_q, seq_k, heads);
     } else {
-        item -= nh * na;
         attention_wide_body<NQB>(smem, hx0 + item / nb, na * 64 * NQA + (item % nb) * 64 * NQB, out, ldo, q, ldq, k, v, ldv, seq_q,
                                  seq_k, heads);
     }
@@ -992,9 +1012,7 @@ static WidePlan wide_plan(int seq_q, int heads) {
 static int g_att_force = -1;
 extern "C" void flux_hip_attention_force_variant(int v) { g_att_force = v; }
 
-extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ldq, const void *k, const void *v,
-                                  int ldv, int seq_q, int seq_k, int heads) {
-    if (seq_q <= 0) return 1;
+static int attention_check(const void *out_bf16, int ldo, const void *q, int ldq, const void *k, const void *v, int ldv, int seq_k, int heads) {
     if (seq_k <= 0) return flux_hip_fail("flux_hip_attention: seq_k=%d", seq_k);
     if (!out_bf16 || !q || !k || !v) return flux_hip_fail("flux_hip_attention: NULL argument");
     if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) || ((uintptr_t)out_bf16 & 7))
@@ -1004,6 +1022,28 @@ extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ld
     /* the tile loaders address K and V rows with 32-bit byte offsets that run up to 64 rows past the end */
     if ((double)(seq_k + 64) * ldv * 2.0 >= 4294967296.0 || (double)(seq_k + 64) * heads * HD * 2.0 >= 4294967296.0)
         return flux_hip_fail("flux_hip_attention: %d keys of %d-element rows exceed 32-bit offsets", seq_k, ldv);
+    return 1;
+}
+
+static WidePlan attention_plan(int variant, int seq_q, int heads) {
+    WidePlan plan;
+    if (variant >= 11 && variant <= 14) {
+        const int nq = variant - 10;
+        plan.nqa = nq > 1 ? nq : 2;
+        plan.na = nq > 1 ? (seq_q + 64 * nq - 1) / (64 * nq) : 0;
+        plan.nb = nq > 1 ? 0 : (seq_q + 63) / 64;
+    } else {
+        plan = wide_plan(seq_q, heads);
+    }
+    return plan;
+}
+
+extern "C" int flux_hip_attention_batch(int nseq, void *const *out_bf16, int ldo, const void *const *q, int ldq, const void *const *k,
+                                        const void *const *v, int ldv, const int *seq_q, const int *seq_k, int heads) {
+    if (nseq <= 0) return 1;
+    if (!out_bf16 || !q || !k || !v || !seq_q || !seq_k) return flux_hip_fail("flux_hip_attention_batch: NULL argument");
+    for (int i = 0; i < nseq; i++)
+        if (seq_q[i] > 0 && !attention_check(out_bf16[i], ldo, q[i], ldq, k[i], v[i], ldv, seq_k[i], heads)) return 0;
     /* Variants: 0 / 1 = attention_kernel with 128 / 256 queries per workgroup; 11 .. 14 = attention_wide_kernel with
      * 16 NQ queries per wave throughout (NQ = 1 .. 4); -1 (default) and 15 = attention_wide_kernel with the mix of
      * block lengths that wide_plan() finds. */
@@ -1017,28 +1057,41 @@ extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ld
         attr_done = true;
     }
     const int variant = g_att_force;
-    if (variant == 0 || variant == 1) {
-        const int bq = variant ? 256 : 128, blocks = ((seq_q + bq - 1) / bq) * heads;
-        hipLaunchKernelGGL(variant ? attention_kernel<8> : attention_kernel<4>, dim3((blocks + 7) & ~7), dim3(variant ? 512 : 256), 2 * ATT_STAGE,
-                           flux_hip_stream_handle(), (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq, (const bf16 *)k, (const bf16 *)v, ldv,
-                           seq_q, seq_k, heads);
-        HIP_OK(hipGetLastError());
-        return 1;
-    }
-    WidePlan plan;
-    if (variant >= 11 && variant <= 14) {
-        const int nq = variant - 10;
-        plan.nqa = nq > 1 ? nq : 2;
-        plan.na = nq > 1 ? (seq_q + 64 * nq - 1) / (64 * nq) : 0;
-        plan.nb = nq > 1 ? 0 : (seq_q + 63) / 64;
-    } else {
-        plan = wide_plan(seq_q, heads);
-    }
     const int max_nh = (heads + 7) / 8; /* the most heads one XCD takes */
-    const dim3 grid(8 * max_nh * (plan.na + plan.nb));
-    auto kern = plan.nqa == 4 ? attention_wide_kernel<4, 3> : plan.nqa == 3 ? attention_wide_kernel<3, 2> : attention_wide_kernel<2, 1>;
-    hipLaunchKernelGGL(kern, grid, dim3(256), ATT_WIDE_LDS, flux_hip_stream_handle(), (bf16 *)out_bf16, ldo, (const bf16 *)q, ldq,
-                       (const bf16 *)k, (const bf16 *)v, ldv, seq_q, seq_k, heads, plan.na, plan.nb);
+    for (int i = 0; i < nseq;) {
+        if (seq_q[i] <= 0) { i++; continue; }
+        if (variant == 0 || variant == 1) {
+            const int bq = variant ? 256 : 128, blocks = ((seq_q[i] + bq - 1) / bq) * heads;
+            hipLaunchKernelGGL(variant ? attention_kernel<8> : attention_kernel<4>, dim3((blocks + 7) & ~7), dim3(variant ? 512 : 256), 2 * ATT_STAGE,
+                               flux_hip_stream_handle(), (bf16 *)out_bf16[i], ldo, (const bf16 *)q[i], ldq, (const bf16 *)k[i], (const bf16 *)v[i],
+                               ldv, seq_q[i], seq_k[i], heads);
+            i++;
+            continue;
+        }
+        /* two sequences share a launch when their blocks have the same lengths */
+        AttSeqs p = {};
+        const WidePlan plan = attention_plan(variant, seq_q[i], heads);
+        p.s[0] = {(bf16 *)out_bf16[i], (const bf16 *)q[i], (const bf16 *)k[i], (const bf16 *)v[i], seq_q[i], seq_k[i], plan.na, plan.nb};
+        p.nseq = 1;
+        int blocks = plan.na + plan.nb;
+        if (i + 1 < nseq && seq_q[i + 1] > 0) {
+            const WidePlan plan1 = attention_plan(variant, seq_q[i + 1], heads);
+            if (plan1.nqa == plan.nqa) {
+                p.s[1] = {(bf16 *)out_bf16[i + 1], (const bf16 *)q[i + 1], (const bf16 *)k[i + 1], (const bf16 *)v[i + 1], seq_q[i + 1], seq_k[i + 1],
+                          plan1.na, plan1.nb};
+                p.nseq = 2;
+                blocks += plan1.na + plan1.nb;
+            }
+        }
+        auto kern = plan.nqa == 4 ? attention_wide_kernel<4, 3> : plan.nqa == 3 ? attention_wide_kernel<3, 2> : attention_wide_kernel<2, 1>;
+        hipLaunchKernelGGL(kern, dim3(8 * max_nh * blocks), dim3(256), ATT_WIDE_LDS, flux_hip_stream_handle(), p, ldo, ldq, ldv, heads);
+        i += p.nseq;
+    }
     HIP_OK(hipGetLastError());
     return 1;
+}
+
+extern "C" int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ldq, const void *k, const void *v,
+                                  int ldv, int seq_q, int seq_k, int heads) {
+    return flux_hip_attention_batch(1, &out_bf16, ldo, &q, ldq, &k, &v, ldv, &seq_q, &seq_k, heads);
 }

@@ -340,6 +340,20 @@ static int linear1(int epi, const void *A, const void *W, void *C, const float *
     return flux_hip_linear(epi, 1, &p, N, K, lda, ldw, ldc, r0, r1);
 }
 
+/* Attention of every sequence of the batch (rows R[b] .. R[b] + N[b] of the qkv, K and output buffers): one call, so that
+ * two sequences can share a launch. */
+static int attention_of_all(int nb, char *cat, int ldcat, char *qkv, char *kn, const int *R, const int *N, int H, int heads) {
+    void *out[2];
+    const void *q[2], *k[2], *v[2];
+    for (int b = 0; b < nb; b++) {
+        out[b] = cat + (size_t)R[b] * ldcat * 2;
+        q[b] = qkv + (size_t)R[b] * 3 * H * 2;
+        k[b] = kn + (size_t)R[b] * H * 2;
+        v[b] = qkv + (size_t)R[b] * 3 * H * 2 + (size_t)2 * H * 2;
+    }
+    return flux_hip_attention_batch(nb, out, ldcat, q, 3 * H, k, v, 3 * H, N, N, heads);
+}
+
 /*
  * One velocity prediction per sequence, entirely on the device, for nb = 1 or 2 sequences that
  * share the target latent, the reference tokens and the timestep (the unconditional and the
@@ -347,8 +361,8 @@ static int linear1(int epi, const void *A, const void *W, void *C, const float *
  * flux_sample.c:485-493). Rows are laid out sequence after sequence, each as
  * [text ; target ; refs], so every GEMM of the single-stream blocks sees all rows of both
  * sequences as one matrix (each weight matrix is streamed once per step instead of twice, and the
- * launch has twice the tiles), the double-stream GEMMs run as 2 nb row ranges, and only attention
- * and its Q/K preparation run per sequence.
+ * launch has twice the tiles), the double-stream GEMMs run as 2 nb row ranges; attention attends per
+ * sequence (in one launch for both when their block lengths agree), its Q/K preparation runs per sequence.
  *   z_dev      fp32 [channels, img_h*img_w] target latent
  *   txt_dev[b] bf16 [txt_seq_b, text_dim]
  *   tf->tok rows [n_target, n_img) must already hold the reference tokens (bf16)
@@ -401,9 +415,8 @@ int fh_forward_device_n(flux_transformer_t *tf, int nb, const fh_rope *const *rp
             char *q_b = qkv + (size_t)R[b] * 3 * H * 2;
             if (!flux_hip_qk_prepare(kn + (size_t)R[b] * H * 2, q_b, 3 * H, 0, H, N[b], heads, Nt[b], blk->norm_q[0], blk->norm_q[1],
                                      blk->norm_k[0], blk->norm_k[1], rp[b]->cos, rp[b]->sin, eps)) return 0;
-            if (!flux_hip_attention(cat + (size_t)R[b] * ldcat * 2, ldcat, q_b, 3 * H, kn + (size_t)R[b] * H * 2, q_b + (size_t)2 * H * 2, 3 * H,
-                                    N[b], N[b], heads)) return 0;
         }
+        if (!attention_of_all(nb, cat, ldcat, qkv, kn, R, N, H, heads)) return 0;
         for (int b = 0; b < nb; b++) {
             p[2 * b] = (flux_hip_linear_part){cat + (size_t)R[b] * ldcat * 2, blk->proj[0], x + (size_t)R[b] * H, mt + 2 * H, Nt[b]};
             p[2 * b + 1] = (flux_hip_linear_part){cat + (size_t)(R[b] + Nt[b]) * ldcat * 2, blk->proj[1], x + (size_t)(R[b] + Nt[b]) * H, mi + 2 * H, Ni};
@@ -450,9 +463,8 @@ int fh_forward_device_n(flux_transformer_t *tf, int nb, const fh_rope *const *rp
             char *q_b = qkv + (size_t)R[b] * 3 * H * 2;
             if (!flux_hip_qk_prepare(kn + (size_t)R[b] * H * 2, q_b, 3 * H, 0, H, N[b], heads, N[b], blk->norm_q, NULL, blk->norm_k, NULL,
                                      rp[b]->cos, rp[b]->sin, eps)) return 0;
-            if (!flux_hip_attention(cat + (size_t)R[b] * ldcat * 2, ldcat, q_b, 3 * H, kn + (size_t)R[b] * H * 2, q_b + (size_t)2 * H * 2, 3 * H,
-                                    N[b], N[b], heads)) return 0;
         }
+        if (!attention_of_all(nb, cat, ldcat, qkv, kn, R, N, H, heads)) return 0;
         p[0] = (flux_hip_linear_part){cat, blk->out, x, ms + 2 * H, Ntot};
         an[0] = (flux_hip_adaln_part){xn, ms, ms + H};
         if (!flux_hip_linear_resid_adaln(1, p, H, H + M, ldcat, H + M, H, i + 1 < c->n_single ? an : NULL, eps, &normed)) return 0;

@@ -79,6 +79,7 @@ def lib():
     L.flux_hip_adaln_norm.argtypes = [vp, c_i, vp, c_i, c_i, c_i, vp, vp, vp, vp, c_f]
     L.flux_hip_qk_prepare.argtypes = [vp, vp, c_i, c_i, c_i, c_i, c_i, c_i, vp, vp, vp, vp, vp, vp, c_f]
     L.flux_hip_attention.argtypes = [vp, c_i, vp, c_i, vp, vp, c_i, c_i, c_i, c_i]
+    L.flux_hip_attention_batch.argtypes = [c_i, vp, c_i, vp, c_i, vp, vp, c_i, vp, vp, c_i]
     L.flux_hip_gemv.argtypes = [vp, vp, vp, c_i, c_i, c_i, c_i]
     L.flux_hip_latent_to_tokens.argtypes = [vp, vp, c_i, c_i]
     L.flux_hip_f32_to_bf16.argtypes = [vp, vp, c_sz]

@@ -205,6 +205,11 @@ int flux_hip_qk_prepare(void *k_out, void *qkv, int ld, int q_col, int k_col, in
  */
 int flux_hip_attention(void *out_bf16, int ldo, const void *q, int ldq, const void *k, const void *v, int ldv,
                        int seq_q, int seq_k, int heads);
+/* The same for nseq independent sequences (arrays of nseq pointers and lengths; leading dimensions and heads in
+ * common): sequences whose query blocks have the same lengths share a launch, two at a time. For the two forwards of
+ * a classifier-free-guidance step (flux_sample.c:485-493), which attend separately. */
+int flux_hip_attention_batch(int nseq, void *const *out_bf16, int ldo, const void *const *q, int ldq, const void *const *k,
+                             const void *const *v, int ldv, const int *seq_q, const int *seq_k, int heads);
 
 /* y[m, n] = sum_k f(x[m, k]) * W[n, k], x f32 [M, K] (M small), W bf16, y f32; f = SiLU when
  * silu_input. The modulation and time-embedding projections (flux_transformer.c:956-969,

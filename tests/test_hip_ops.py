@@ -564,6 +564,39 @@ def test_attention_first_key_tile_far_below_the_rest(hip, oracle_mod, variant):
         hip.lib().flux_hip_attention_force_variant(-1)
 
 
+@pytest.mark.parametrize("lens", [((700, 700), (700, 700)), ((640, 640), (600, 600)), ((300, 300), (2000, 2000)), ((200, 700), (130, 130))])
+def test_attention_two_sequences_in_one_launch(hip, lens):
+    """flux_hip_attention_batch with two sequences (the two forwards of a CFG step) against one flux_hip_attention call per
+    sequence, bit for bit: equal lengths, unequal lengths with the same block plan, lengths whose block plans differ (then
+    the batch falls back to a launch per sequence), and a query sub-range in one of them."""
+    import ctypes
+    L = hip.lib()
+    heads = 3
+    H = heads * 128
+    bufs = []
+    for i, (nq, nk) in enumerate(lens):
+        qkv = q(normal_f32((nk, 3 * H), 70 + i, 1))
+        dqkv = dev_bf16(hip, qkv)
+        w = hip.DevBuf.from_array(np.ones(128, np.float32))
+        ang = normal_f32((nk, 128), 70 + i, 2)
+        dcos, dsin = hip.DevBuf.from_array(np.cos(ang)), hip.DevBuf.from_array(np.sin(ang))
+        kn = hip.DevBuf(nk * H * 2)
+        hip.check(L.flux_hip_qk_prepare(kn.ptr, dqkv.ptr, 3 * H, 0, H, nk, heads, nk, w.ptr, w.ptr, w.ptr, w.ptr, dcos.ptr, dsin.ptr, 1e-6))
+        one = hip.DevBuf.from_array(np.zeros((nq, H), np.uint16))
+        hip.check(L.flux_hip_attention(one.ptr, H, dqkv.ptr, 3 * H, kn.ptr, dqkv.at(2 * H * 2), 3 * H, nq, nk, heads))
+        both = hip.DevBuf.from_array(np.full((nq, H), 0x7fc0, np.uint16))
+        bufs.append((dqkv, kn, one, both, nq, nk, w, dcos, dsin))
+    vp2, i2 = ctypes.c_void_p * 2, ctypes.c_int * 2
+    out = vp2(*[b[3].ptr for b in bufs])
+    qs = vp2(*[b[0].ptr for b in bufs])
+    ks = vp2(*[b[1].ptr for b in bufs])
+    vs = vp2(*[b[0].at(2 * H * 2) for b in bufs])
+    nqs, nks = i2(*[b[4] for b in bufs]), i2(*[b[5] for b in bufs])
+    hip.check(L.flux_hip_attention_batch(2, out, H, qs, 3 * H, ks, vs, 3 * H, nqs, nks, heads))
+    for dqkv, kn, one, both, nq, nk, *_ in bufs:
+        assert np.array_equal(one.to_array(np.uint16, (nq, H)), both.to_array(np.uint16, (nq, H)))
+
+
 def test_layout_edges_and_updates(hip, oracle_mod):
     C, n = 128, 45
     lat = normal_f32((C, n), 10, 1)
