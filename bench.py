@@ -13,6 +13,8 @@ Also measured in the same run:
                 the backend's stream around every launch of it inside the timed region; also launched alone
   cpu_baseline  the CPU oracle (fp32, BLAS when available) on a bounded sample of the same
                 workload: one whole forward at full shape after a small warm-up forward
+  box           what this machine's matrix pipes sustain on their own (a register-resident MFMA loop on random bit
+                patterns, right after the timed steps), and the step's TFLOP/s over it: boxes differ by several per cent
 
 --workload vae_c2 | vae_c3 | vae_c4 measures the step after the sampling loop instead: one "step" is
 one VAE decode of a 16/32/64-wide latent to a 256/512/1024-pixel image; vae_enc_c2 | vae_enc_c3 |
@@ -773,6 +775,18 @@ def main():
                      "ms_per_launch_back_to_back": round(alone_ms, 4)})
     model.close()
 
+    # What this box's matrix pipes sustain on their own (register-resident v_mfma_f32_16x16x32_bf16 on random bit patterns, two
+    # waves per SIMD, best of three 5 ms launches): boxes differ by several per cent under the power limit, and the step follows.
+    box = None
+    if not args.no_kernel_timing:
+        import ctypes
+        Lb = fluxhip.lib()
+        Lb.flux_hip_mfma_peak.argtypes = [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_float)]
+        t = ctypes.c_float(0.0)
+        fluxhip.check(Lb.flux_hip_mfma_peak(0, 2, 2, 12000, 1, ctypes.byref(t)), "flux_hip_mfma_peak")
+        fluxhip.check(Lb.flux_hip_mfma_peak(0, 2, 2, 12000, 3, ctypes.byref(t)), "flux_hip_mfma_peak")
+        box = {"mfma_only_tflops_random_bits": round(t.value, 1), "step_tflops_over_it": round(tflops / t.value, 4)}
+
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(cfg, wl, forwards)
@@ -791,7 +805,7 @@ def main():
                             "steps_per_s": round(n_run / host_run_ms * 1000.0, 3)},
         "stage_ms_per_step": {"double": round(stages[0] / (K + Wm), 3), "single": round(stages[1] / (K + Wm), 3),
                               "final": round(stages[2] / (K + Wm), 3)},
-        "roofline": roof, "cpu_baseline": cpu,
+        "roofline": roof, "cpu_baseline": cpu, "box": box,
     }
     print(json.dumps(out))
 
