@@ -596,15 +596,17 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
     /* The loop is software-pipelined inside each wave, because with one wave per SIMD nothing else overlaps the
      * softmax with the matrix pipe. The unit is a chunk of 32 keys (half a tile): while chunk u is exponentiated
      * and multiplied into O, the scores of chunk u + 1 are already being computed:
-     *   phase 1: S(u+1) = K Q^T - m   (8 NQ MFMAs)  with  the conversion of 2^S(u) to bf16 P(u) (4 NQ vector instructions)
-     *   phase 2: row sums and O += V^T P(u)^T (9 NQ MFMAs)  with  2^S(u+1) (8 NQ exponentials), the requests for the
-     *            next fragments and the loads
+     *   phase 1: S(u+1) = K Q^T - m   (8 NQ MFMAs)  with  the conversion of 2^S(u) to bf16 P(u) (4 NQ vector instructions),
+     *            the requests for chunk u's V^T fragments and, in its last eight gaps, four tile loads
+     *   phase 2: row sums and O += V^T P(u)^T (9 NQ MFMAs)  with  2^S(u+1) (8 NQ exponentials) and the requests for
+     *            chunk u+2's K fragments
      * Vector instructions sit one or two behind each MFMA; sched_barrier keeps them there. Two score buffers
      * alternate, so one trip of the loop is one tile: an "even" step (second chunk's scores, first chunk's
      * product) and an "odd" step (next tile's first chunk's scores, second chunk's product). One barrier per
      * tile, at the start of the odd step: behind it K(t)'s and V(t-1)'s slots are free and take K(t+4) and
-     * V(t+3), whose eight loads are spread over the 34 NQ MFMAs up to the next barrier (a direct global->LDS load
-     * costs the matrix pipe some 12 cycles when it stands alone and 30 in a run of eight). With four slots per
+     * V(t+3), whose eight loads go behind MFMAs of the two score phases up to the next barrier that carry little else
+     * (in a run of eight behind MFMAs that also carry an exponential a direct global->LDS load cost the matrix pipe 30
+     * cycles; alone behind its MFMA nothing that can be measured). With four slots per
      * ring those loads are not needed before the barrier after the next, so a barrier waits for all but the newest
      * eight loads (a count, not "all": the compiler's own barrier would wait for every load in flight).
      * Everything read before the next barrier landed before this one, so fragments are requested from LDS a phase
