@@ -172,11 +172,13 @@ __device__ __forceinline__ int weight_row(const GemmArgs &g, int tn, int v) {
 
 /* Accumulator element e of block (i, j): feature n = 4*(lane/16) + e of the 16-column block,
  * token m = lane%16 of the 16-row block. */
-template <int BN, int WM, int WN, int EPI>
-__device__ __forceinline__ void store_tile_to(const GemmArgs &g, const TileId &t, f32x4 (&acc)[WN / 16][WM / 16], int m0, int M,
+template <int BN, int WM, int WN, int EPI, bool HERE = false>
+__device__ __forceinline__ void store_tile_to(const GemmArgs &g, const TileId &t, f32x4 (&acc_in)[WN / 16][WM / 16], int m0, int M,
                                               int wm, int wn, int l15, int lq, int prow, void *Cp, const int ldc, const int tn) {
     constexpr int TM = WM / 16, TN = WN / 16;
     const int prob = t.prob, n0 = tn * BN, ks = t.ks;
+    f32x4 acc_here[HERE ? TN : 1][HERE ? TM : 1];
+    auto &acc = [&]() -> auto & { if constexpr (HERE) return acc_here; else return acc_in; }();
     float st_s[TN], st_q[TN]; /* convolutions with statistics: this lane's sums per 16-column block */
 #pragma unroll
     for (int i = 0; i < TN; i++) st_s[i] = st_q[i] = 0.0f;
@@ -184,6 +186,13 @@ __device__ __forceinline__ void store_tile_to(const GemmArgs &g, const TileId &t
     for (int j = 0; j < TM; j++) {
         const int m = m0 + wm * WM + j * 16 + l15;
         if (m >= M) continue;
+        if constexpr (HERE) {
+#pragma unroll
+            for (int i = 0; i < TN; i++) {
+                acc[i][j] = acc_in[i][j];
+                asm volatile("" : "+v"(acc[i][j]));
+            }
+        }
         bool inside = true; /* convolutions: border positions of the image are written as zeros */
         if (IsConv<EPI>::value && g.conv_wp > 0) {
             const int y = m / g.conv_wp, x = m - y * g.conv_wp;
@@ -271,8 +280,12 @@ template <int BN, int WM, int WN, int EPI>
 __device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f32x4 (&acc)[WN / 16][WM / 16], int m0, int M,
                                            int wm, int wn, int l15, int lq, int prow) {
     if constexpr (EPI == EPI_QKV_SWIGLU) {
-        if (t.tn < g.nq_tiles) store_tile_to<BN, WM, WN, FLUX_HIP_EPI_BF16>(g, t, acc, m0, M, wm, wn, l15, lq, prow, g.C[0], g.ldc, t.tn);
-        else store_tile_to<BN, WM, WN, FLUX_HIP_EPI_SWIGLU>(g, t, acc, m0, M, wm, wn, l15, lq, prow, g.C2, g.ldc2, t.tn - g.nq_tiles);
+        /* HERE = true: each side reads the accumulators through an empty asm statement, row by row. The conversions
+         * are then work of that side; left to itself the compiler converted the whole tile to bf16 in front of the
+         * branch, for both sides, and kept the hundred results in registers next to the other side's work, past
+         * what the register file holds beside the fragments. */
+        if (t.tn < g.nq_tiles) store_tile_to<BN, WM, WN, FLUX_HIP_EPI_BF16, true>(g, t, acc, m0, M, wm, wn, l15, lq, prow, g.C[0], g.ldc, t.tn);
+        else store_tile_to<BN, WM, WN, FLUX_HIP_EPI_SWIGLU, true>(g, t, acc, m0, M, wm, wn, l15, lq, prow, g.C2, g.ldc2, t.tn - g.nq_tiles);
     } else {
         store_tile_to<BN, WM, WN, EPI>(g, t, acc, m0, M, wm, wn, l15, lq, prow, g.C[t.prob], g.ldc, t.tn);
     }
@@ -477,6 +490,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm4w_kernel(GemmArgs g) {
     /* (convolutions never split K, so for them kt below is the absolute K step) */
     auto issue1 = [&](int kt, int stage, int i) {
         const char *base = i < LA ? baseA + (ptrdiff_t)a_step_offset<EPI>(g, kt) * 2 : baseW + kt * 128;
+        asm volatile("" : "+v"(voff[i])); /* keeps the load in its scalar base + 32-bit lane offset form, see gemm4d_kernel */
         __builtin_amdgcn_global_load_lds(GLOBAL_PTR(base + voff[i]), LDS_PTR(smem + stage * STAGE + (wave * 8 + i * RPP) * 128), 16, 0, 0);
     };
     set_sources(t);
@@ -561,7 +575,13 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm4w_kernel(GemmArgs g) {
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); /* the last MFMA results retire before they are read */
         acc_fence<TM, TN>(acc);
 
-        store_tile<BN, WM, WN, EPI>(g, done, acc, done.tml * BM, g.M[done.prob], wm, wn, l15, lq, done.tm * WGM + wm);
+        /* The lane's position enters the epilogue through an empty asm statement: what the epilogue derives from it
+         * (row and column offsets of every store, for the fused projection those of both store bodies) is then computed
+         * per tile. Left visible, the compiler computes all of it once before the first tile and keeps it in registers
+         * across the K loops, beyond what the register file holds beside the accumulators and fragments. */
+        int l15e = l15, lqe = lq;
+        asm volatile("" : "+v"(l15e), "+v"(lqe));
+        store_tile<BN, WM, WN, EPI>(g, done, acc, done.tml * BM, g.M[done.prob], wm, wn, l15e, lqe, done.tm * WGM + wm);
         if (!again) break;
     }
 }
@@ -606,18 +626,28 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
     const char *baseA, *baseW;
     auto set_sources = [&](const TileId &tt) {
         const int M = g.M[tt.prob], m0 = tt.tml * BM;
-        const int chunk = (lchunk ^ lds_swz(lrow)) << 3;
+        /* the lane's row enters through an empty asm statement, so that the per-load row numbers derived from it (two
+         * sets of weight rows for the fused projection) are computed here, per tile, and not once before the first
+         * tile, from where they would have to be kept in registers across every K loop */
+        int lr = lrow;
+        asm volatile("" : "+v"(lr));
+        const int chunk = (lchunk ^ lds_swz(lr)) << 3;
         baseA = (const char *)(g.A[tt.prob] + tt.ks * g.kt_per * 64);
         baseW = (const char *)(g.W[tt.prob] + tt.ks * g.kt_per * 64);
 #pragma unroll
-        for (int i = 0; i < LA; i++) voff[i] = ((unsigned)min(m0 + lrow + i * RPP, M - 1) * (unsigned)g.lda + chunk) * 2u;
+        for (int i = 0; i < LA; i++) voff[i] = ((unsigned)min(m0 + lr + i * RPP, M - 1) * (unsigned)g.lda + chunk) * 2u;
 #pragma unroll
-        for (int i = 0; i < LB; i++) voff[LA + i] = ((unsigned)weight_row<BN, WN, EPI>(g, tt.tn, lrow + i * RPP) * (unsigned)g.ldw + chunk) * 2u;
+        for (int i = 0; i < LB; i++) voff[LA + i] = ((unsigned)weight_row<BN, WN, EPI>(g, tt.tn, lr + i * RPP) * (unsigned)g.ldw + chunk) * 2u;
     };
     /* load i of K step kt: activation rows for i < LA (into slot sa of their ring), weight rows after (slot sw) */
     auto issue1 = [&](int kt, int sa, int sw, int i) {
         const char *base = (i < LA ? baseA : baseW) + (ptrdiff_t)kt * 128;
         const int dst = i < LA ? sa * ASZ + (wave * 8 + i * RPP) * 128 : NSA * ASZ + sw * WSZ + (wave * 8 + (i - LA) * RPP) * 128;
+        /* The offset passes through an empty asm statement where it is used: the load is then selected in its
+         * "scalar base + 32-bit lane offset" form. Without it the compiler widens every offset to 64 bits once, outside
+         * the K loop, keeps NL register pairs instead of NL registers, and adds the base with a 64-bit vector addition
+         * in front of every load. */
+        asm volatile("" : "+v"(voff[i]));
         __builtin_amdgcn_global_load_lds(GLOBAL_PTR(base + voff[i]), LDS_PTR(smem + dst), 16, 0, 0);
     };
     /* the order in which a step issues its loads: the operand with the two-slot ring first (see the file comment) */
@@ -720,7 +750,13 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); /* the last MFMA results retire before they are read */
         acc_fence<TM, TN>(acc);
 
-        store_tile<BN, WM, WN, EPI>(g, done, acc, done.tml * BM, g.M[done.prob], wm, wn, l15, lq, done.tm * WGM + wm);
+        /* The lane's position enters the epilogue through an empty asm statement: what the epilogue derives from it
+         * (row and column offsets of every store, for the fused projection those of both store bodies) is then computed
+         * per tile. Left visible, the compiler computes all of it once before the first tile and keeps it in registers
+         * across the K loops, beyond what the register file holds beside the accumulators and fragments. */
+        int l15e = l15, lqe = lq;
+        asm volatile("" : "+v"(l15e), "+v"(lqe));
+        store_tile<BN, WM, WN, EPI>(g, done, acc, done.tml * BM, g.M[done.prob], wm, wn, l15e, lqe, done.tm * WGM + wm);
         if (!again) break;
     }
 }

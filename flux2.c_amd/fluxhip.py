@@ -43,7 +43,8 @@ _lib = None
 
 
 def lib_path():
-    return os.path.join(_HERE, "libflux_hip.so")
+    """libflux_hip.so next to this file, or the file FLUX_HIP_LIBRARY names (another build of the same ABI)."""
+    return os.environ.get("FLUX_HIP_LIBRARY") or os.path.join(_HERE, "libflux_hip.so")
 
 
 def lib():

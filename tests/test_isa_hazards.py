@@ -22,8 +22,31 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(ROOT, "flux2.c_amd", "csrc")
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-         "--cuda-device-only", "-S"]
+MAKEFILE = os.path.join(ROOT, "flux2.c_amd", "Makefile")
+
+
+def makefile_flags(src):
+    """The device-side compile flags the Makefile uses for csrc/<src>: HIPFLAGS with $(ARCH) expanded, plus the
+    file's own FLAGS_<name> if it has one. Read from the Makefile so that this test compiles what ships."""
+    text = open(MAKEFILE).read()
+
+    def var(name):
+        m = re.search(r"^%s\s*\??=\s*(.*)$" % re.escape(name), text, flags=re.M)
+        return m.group(1).strip() if m else ""
+
+    flags = var("HIPFLAGS").replace("$(ARCH)", var("ARCH")).split()
+    assert any(f.startswith("--offload-arch=gfx") for f in flags) and "-packed-fp32-ops" in flags, flags
+    return flags + var("FLAGS_" + os.path.splitext(src)[0]).split()
+
+
+def compile_device(src, out, extra):
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc is not installed")
+    r = subprocess.run([hipcc] + makefile_flags(src) + ["--cuda-device-only"] + extra + [os.path.join(CSRC, src), "-o", str(out)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
+    return r
 
 VALU_TO_MFMA_SLOTS = 2
 TRANS = ("v_exp_", "v_log_", "v_rcp_", "v_rsq_", "v_sqrt_", "v_sin_", "v_cos_")
@@ -117,16 +140,20 @@ def lint(body):
     return problems
 
 
-@pytest.mark.parametrize("src,extra,pattern", [("attention.hip", ["-fno-honor-nans"], "attention_wide_kernel"),
-                                               ("gemm.hip", [], "gemm4w_kernel"), ("gemm.hip", [], "gemm4d_kernel")])
-def test_inline_asm_mfma_hazards(src, extra, pattern, tmp_path):
-    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    if not os.path.exists(hipcc):
-        pytest.skip("hipcc is not installed")
-    out = tmp_path / (src + ".s")
-    r = subprocess.run([hipcc] + FLAGS + extra + [os.path.join(CSRC, src), "-o", str(out)], capture_output=True, text=True)
-    assert r.returncode == 0, r.stderr[-2000:]
-    kernels = {k: v for k, v in kernel_bodies(out.read_text()).items() if pattern in k}
+@pytest.fixture(scope="module")
+def assembly(tmp_path_factory):
+    """Assembly text and resource-usage remarks of gemm.hip and attention.hip, compiled once per test run."""
+    out = {}
+    for src in ("gemm.hip", "attention.hip"):
+        path = tmp_path_factory.mktemp("asm") / (src + ".s")
+        r = compile_device(src, path, ["-S", "-Rpass-analysis=kernel-resource-usage"])
+        out[src] = (path.read_text(), r.stderr)
+    return out
+
+
+@pytest.mark.parametrize("src,pattern", [("attention.hip", "attention_wide_kernel"), ("gemm.hip", "gemm4w_kernel"), ("gemm.hip", "gemm4d_kernel")])
+def test_inline_asm_mfma_hazards(src, pattern, assembly):
+    kernels = {k: v for k, v in kernel_bodies(assembly[src][0]).items() if pattern in k}
     assert kernels, f"no kernel named *{pattern}* in {src}"
     report = []
     for name, body in sorted(kernels.items()):
@@ -146,3 +173,48 @@ def test_the_lint_sees_a_planted_hazard():
     clean = ["\tv_mov_b32_e32 v5, v9", "\ts_nop 1", "\tv_mfma_f32_16x16x32_bf16 v[0:3], v[4:7], v[8:11], v[0:3]", "\ts_nop 7",
              "\tv_add_f32_e32 v20, v1, v1", "\ts_endpgm"]
     assert not lint(clean)
+
+
+def resource_usage(remarks):
+    """{mangled kernel name: {field: int}} from the compiler's -Rpass-analysis=kernel-resource-usage remarks."""
+    out, name = {}, None
+    for line in remarks.splitlines():
+        m = re.search(r"remark:\s+Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+            out[name] = {}
+            continue
+        m = re.search(r"remark:\s+([A-Za-z ]+?)(?: \[[^\]]*\])?: (\d+) \[-Rpass", line)
+        if m and name:
+            out[name][m.group(1).strip()] = int(m.group(2))
+    return out
+
+
+def test_gemm_kernels_fit_the_register_file(assembly):
+    """No GEMM kernel may spill: a spilled register is a scratch store next to the next tile's primed loads (the
+    compiler waits for all of them first), and the fused [Q|K|V|gate|up] epilogue went over the ceiling that way
+    before its two store bodies were kept apart. Every kernel of gemm.hip: no scratch frame, no spilled VGPR or SGPR;
+    the 4-wave kernels keep their accumulators in AGPRs and nothing else (AGPRs == 16 TM TN / 4 means that no
+    vector register was parked there either)."""
+    usage = resource_usage(assembly["gemm.hip"][1])
+    big = {k: v for k, v in usage.items() if "gemm4d_kernel" in k or "gemm4w_kernel" in k}
+    assert len(big) >= 60 and len(usage) >= 100, (len(big), len(usage))
+    bad = []
+    for name, u in sorted(usage.items()):
+        if u["ScratchSize"] or u["VGPRs Spill"] or u["SGPRs Spill"]:
+            bad.append((name, u))
+    assert not bad, bad
+    for name, u in sorted(big.items()):
+        tm, tn, epi = map(int, re.search(r"kernelILi(\d+)ELi(\d+)ELi(\d+)E", name).groups())
+        assert u["AGPRs"] == 4 * tm * tn, (name, u)
+        if epi not in (6, 7):                    # the transformer's epilogues (the convolution ones sit at 252-256, unspilled)
+            assert u["VGPRs"] <= 200, (name, u)  # room to spare: 180 at most when this was written
+
+
+def test_the_remark_parser_reads_the_fields_the_test_uses():
+    text = ("x.hip:1:1: remark: Function Name: _Z1kv [-Rpass-analysis=kernel-resource-usage]\n"
+            "x.hip:1:1: remark:     VGPRs: 12 [-Rpass-analysis=kernel-resource-usage]\n"
+            "x.hip:1:1: remark:     AGPRs: 4 [-Rpass-analysis=kernel-resource-usage]\n"
+            "x.hip:1:1: remark:     ScratchSize [bytes/lane]: 8 [-Rpass-analysis=kernel-resource-usage]\n"
+            "x.hip:1:1: remark:     VGPRs Spill: 1 [-Rpass-analysis=kernel-resource-usage]\n")
+    assert resource_usage(text) == {"_Z1kv": {"VGPRs": 12, "AGPRs": 4, "ScratchSize": 8, "VGPRs Spill": 1}}
