@@ -429,6 +429,7 @@ __device__ __forceinline__ void acc_fence(f32x4 (&acc)[TN][TM]) {
 }
 
 template <bool V> struct BoolC { static constexpr bool value = V; };
+template <int V> struct IntC { static constexpr int value = V; };
 /* whether a workgroup of gemm4w_kernel goes on to further tiles (the 4-wave form of the transformer's epilogues;
  * with the convolution epilogues the values kept across tiles would spill) */
 template <int EPI, int WAVES> struct Walks4w { static constexpr bool value = !IsConv<EPI>::value && WAVES == 4; };
@@ -590,10 +591,29 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm4w_kernel(GemmArgs g) {
  * waits at its barrier for every load it has in flight (requested one to two half-steps earlier); operands that
  * come from HBM rather than from a cache arrive later than that now and then, and a wave that waits holds the
  * other three up at the barrier. Here the activation tile and the weight tile have rings of their own, NSA and NSW
- * slots of one K step (128-byte rows, the layout of gemm4w_kernel) each, as many as the 160 KB of LDS hold: the
- * operand with three slots is requested a whole K step earlier, and the barrier waits with a count (the loads of
- * the two-slot operand are issued first in a step, so that "all but the last L" is exactly what must have landed)
- * instead of a fence. The MFMA order is that of gemm4w_kernel: bit-identical results. */
+ * slots of one K step (128-byte rows, the layout of gemm4w_kernel) each, as many as the 160 KB of LDS hold, and
+ * the barrier waits with a count instead of a fence. The MFMA order is that of gemm4w_kernel: bit-identical results.
+ *
+ * Loads of a K step kt are spread over both of its halves (one load costs a lone wave 12 cycles of matrix-pipe
+ * time at one load per eight MFMAs and 19 at one per four). The "first" operand - the one with three slots,
+ * activations if both have three - is requested in the first half for step kt + 2, into the slot that step kt - 1
+ * left at the last barrier; the "second" operand in the second half for step kt + NS2 (its ring's depth), into
+ * the slot whose last reads completed at this step's barrier. The barrier in the middle of step kt needs step
+ * kt + 1 in LDS: everything but the loads issued after it, which is a count (vector memory operations of a wave
+ * complete in the order of their issue).
+ *
+ * Tiles follow each other without a gap in that pipeline: the last steps of a tile request the first steps of the
+ * workgroup's next tile where they would request steps beyond their own K range, the last step reads the next
+ * tile's first fragments, and the ring positions carry over. The finished tile is stored between the two K
+ * loops, and nothing waits for those stores there: the first barrier of the next tile allows them (and the
+ * loads behind them) to be in flight, the second one needs loads that were issued after them. Before that, a
+ * tile began by waiting for every store of its predecessor to be acknowledged and for its own first steps,
+ * requested only then, with the matrix pipes idle: 12 % of a 288 x 192 x 3072 tile's time. */
+template <int EPI, int TM, int TN>
+struct EpilogueOps { /* vector memory instructions a wave issues in the epilogue of a tile whose rows are all valid */
+    static constexpr int value = EPI == FLUX_HIP_EPI_SWIGLU || EPI == EPI_QKV_SWIGLU ? TM * TN / 2 : EPI == FLUX_HIP_EPI_F32_T ? 4 * TM * TN : TM * TN;
+};
+
 template <int TM, int TN, int EPI, int NSA, int NSW>
 __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
     constexpr int WGM = 2, WGN = 2;
@@ -603,10 +623,18 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
     constexpr int LA = BM / RPP, LB = BN / RPP, NL = LA + LB;
     constexpr int NF = TM + TN, NM = TM * TN, RD = NM / NF;
     constexpr int ASZ = BM * 128, WSZ = BN * 128;
-    constexpr int AHEAD = (NSA == 3 ? LA : 0) + (NSW == 3 ? LB : 0); /* loads that may be in flight past the barrier */
-    static_assert((NSA == 2 || NSA == 3) && (NSW == 2 || NSW == 3) && NSA * ASZ + NSW * WSZ <= 160 * 1024, "rings of two or three slots within the LDS");
+    static_assert((NSA == 2 || NSA == 3) && (NSW == 2 || NSW == 3) && (NSA == 3 || NSW == 3) && NSA * ASZ + NSW * WSZ <= 160 * 1024,
+                  "rings of two or three slots within the LDS, one of them with three");
     static_assert((EPI != FLUX_HIP_EPI_SWIGLU && EPI != EPI_QKV_SWIGLU) || (TN % 2 == 0), "swiglu pairs 16-column blocks");
-    static_assert(RD >= 2 && RD * (NF - 1) + 1 < NM, "reads and loads must fit between the MFMAs");
+    static_assert(RD >= 2 && RD * (NF - 1) + 1 < NM, "reads must fit between the MFMAs");
+    constexpr bool FIRST_A = NSA == 3;
+    constexpr int LF = FIRST_A ? LA : LB, LS = FIRST_A ? LB : LA, NS2 = FIRST_A ? NSW : NSA;
+    constexpr int SF = (NM / LF) / RD * RD, SS = (NM / LS) / RD * RD; /* MFMAs between two loads of a half: a multiple of RD */
+    static_assert(SF >= RD && SS >= RD && 1 + SF * (LF - 1) < NM && 1 + SS * (LS - 1) < NM, "the loads of a half fit between its MFMAs");
+    constexpr int AHEAD = LF + (NS2 == 3 ? LS : 0); /* loads that may be in flight past the barrier */
+    /* first barrier of a tile that follows another: also the stored tile's memory operations may be in flight (the wait
+     * counter holds 63) */
+    constexpr int AHEAD_STORES = AHEAD + EpilogueOps<EPI, TM, TN>::value < 63 ? AHEAD + EpilogueOps<EPI, TM, TN>::value : 63;
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -622,9 +650,15 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
     TileId t;
     if (!decode_tile(g, vb, t)) return;
 
-    unsigned voff[NL];
-    const char *baseA, *baseW;
-    auto set_sources = [&](const TileId &tt) {
+    /* Sources of a tile's loads: a uniform base per operand (the tile's matrix + this workgroup's K slice) and a 32-bit
+     * byte offset per lane and load, so that stepping along K is scalar work. Two sets: the tile being multiplied and
+     * the workgroup's next one. */
+    struct Src {
+        unsigned voff[NL];
+        const char *baseA, *baseW;
+    };
+    Src cur, nxt;
+    auto set_sources = [&](Src &sc, const TileId &tt) {
         const int M = g.M[tt.prob], m0 = tt.tml * BM;
         /* the lane's row enters through an empty asm statement, so that the per-load row numbers derived from it (two
          * sets of weight rows for the fused projection) are computed here, per tile, and not once before the first
@@ -632,49 +666,57 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
         int lr = lrow;
         asm volatile("" : "+v"(lr));
         const int chunk = (lchunk ^ lds_swz(lr)) << 3;
-        baseA = (const char *)(g.A[tt.prob] + tt.ks * g.kt_per * 64);
-        baseW = (const char *)(g.W[tt.prob] + tt.ks * g.kt_per * 64);
+        sc.baseA = (const char *)(g.A[tt.prob] + tt.ks * g.kt_per * 64);
+        sc.baseW = (const char *)(g.W[tt.prob] + tt.ks * g.kt_per * 64);
 #pragma unroll
-        for (int i = 0; i < LA; i++) voff[i] = ((unsigned)min(m0 + lr + i * RPP, M - 1) * (unsigned)g.lda + chunk) * 2u;
+        for (int i = 0; i < LA; i++) sc.voff[i] = ((unsigned)min(m0 + lr + i * RPP, M - 1) * (unsigned)g.lda + chunk) * 2u;
 #pragma unroll
-        for (int i = 0; i < LB; i++) voff[LA + i] = ((unsigned)weight_row<BN, WN, EPI>(g, tt.tn, lr + i * RPP) * (unsigned)g.ldw + chunk) * 2u;
+        for (int i = 0; i < LB; i++) sc.voff[LA + i] = ((unsigned)weight_row<BN, WN, EPI>(g, tt.tn, lr + i * RPP) * (unsigned)g.ldw + chunk) * 2u;
     };
-    /* load i of K step kt: activation rows for i < LA (into slot sa of their ring), weight rows after (slot sw) */
-    auto issue1 = [&](int kt, int sa, int sw, int i) {
+    /* load i of K step kt of the tile whose sources are (baseA, baseW, vo): activation rows for i < LA (into slot sa
+     * of their ring), weight rows after (slot sw). The offset passes through an empty asm statement where it is used: the
+     * load is then selected in its "scalar base + 32-bit lane offset" form. Without it the compiler widens every offset
+     * to 64 bits once, outside the K loop, keeps NL register pairs instead of NL registers, and adds the base with a
+     * 64-bit vector addition in front of every load. */
+    auto issue1 = [&](const char *baseA, const char *baseW, unsigned &vo, int kt, int sa, int sw, int i) {
         const char *base = (i < LA ? baseA : baseW) + (ptrdiff_t)kt * 128;
         const int dst = i < LA ? sa * ASZ + (wave * 8 + i * RPP) * 128 : NSA * ASZ + sw * WSZ + (wave * 8 + (i - LA) * RPP) * 128;
-        /* The offset passes through an empty asm statement where it is used: the load is then selected in its
-         * "scalar base + 32-bit lane offset" form. Without it the compiler widens every offset to 64 bits once, outside
-         * the K loop, keeps NL register pairs instead of NL registers, and adds the base with a 64-bit vector addition
-         * in front of every load. */
-        asm volatile("" : "+v"(voff[i]));
-        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(base + voff[i]), LDS_PTR(smem + dst), 16, 0, 0);
-    };
-    /* the order in which a step issues its loads: the operand with the two-slot ring first (see the file comment) */
-    auto nth = [](int n) { return NSA < NSW ? n : (n < LB ? LA + n : n - LB); };
-    /* The first K steps of a tile, as many as the rings hold beside the step that is multiplied first: requested
-     * before the previous tile is stored, so that they arrive while its results go out */
-    auto prime = [&](int KTn) {
-#pragma unroll
-        for (int n = 0; n < NL; n++) issue1(0, 0, 0, nth(n));
-        if (KTn > 1) {
-#pragma unroll
-            for (int n = 0; n < NL; n++) issue1(1, 1, 1, nth(n));
-        }
-        if (KTn > 2) {
-#pragma unroll
-            for (int n = 0; n < NL; n++) {
-                const int i = nth(n);
-                if (i < LA ? NSA == 3 : NSW == 3) issue1(2, 2, 2, i);
-            }
-        }
+        asm volatile("" : "+v"(vo));
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(base + vo), LDS_PTR(smem + dst), 16, 0, 0);
     };
     auto k_steps = [&](const TileId &tt) { return min(g.K >> 6, tt.ks * g.kt_per + g.kt_per) - tt.ks * g.kt_per; };
-    set_sources(t);
-    prime(k_steps(t));
+    /* The first K steps of a tile that no predecessor requested, into slots 0, 1 (and 2): what the pipeline below has
+     * in flight when it enters a tile's step 0, oldest first */
+    auto prime = [&](Src &sc, int KTn) {
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            if (s < KTn) {
+#pragma unroll
+                for (int i = 0; i < NL; i++) issue1(sc.baseA, sc.baseW, sc.voff[i], s, s, s, i);
+            }
+        }
+        if (NS2 == 3 && KTn > 2) {
+#pragma unroll
+            for (int n = 0; n < LS; n++) issue1(sc.baseA, sc.baseW, sc.voff[(FIRST_A ? LA : 0) + n], 2, 2, 2, (FIRST_A ? LA : 0) + n);
+        }
+    };
+
+    bf16x8 f0[NF], f1[NF];
+    int ca = 0, cw = 0;                   /* ring slots of the step being multiplied */
+    unsigned va = a_frag, vw = w_frag;    /* this lane's fragment rows in those slots */
+    auto frag = [&](unsigned xa, unsigned xw, int coff, int q) -> bf16x8 {
+        return q < TN ? *(const bf16x8 *)(smem + xw + coff + q * 2048) : *(const bf16x8 *)(smem + xa + coff + (q - TN) * 2048);
+    };
+    /* the first tile: its first steps are requested here, and everything has landed before its step 0 */
+    set_sources(cur, t);
+    prime(cur, k_steps(t));
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+    for (int q = 0; q < NF; q++) f0[q] = frag(va, vw, coff0, q);
+    bool strict = false; /* the first barrier of the tile must not count on the stored tile's operations */
 
     for (;;) {
-        const int KT = k_steps(t);
+        const int KT = k_steps(t); /* at least 4: the host sends shorter K ranges to gemm4w_kernel */
 
         f32x4 acc[TN][TM];
 #pragma unroll
@@ -686,67 +728,66 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
         acc_fence<TM, TN>(acc); /* the zeroes are written, and a few cycles pass, before the first MFMA reads them */
         asm volatile("s_nop 7" ::: "memory");
 
-        bf16x8 f0[NF], f1[NF];
-        int ca = 0, cw = 0;                   /* ring slots of the step being multiplied */
-        unsigned va = a_frag, vw = w_frag;    /* this lane's fragment rows in those slots */
-        auto frag = [&](unsigned xa, unsigned xw, int coff, int q) -> bf16x8 {
-            return q < TN ? *(const bf16x8 *)(smem + xw + coff + q * 2048) : *(const bf16x8 *)(smem + xa + coff + (q - TN) * 2048);
-        };
-
-        /* the tile's first steps are in LDS (they, and the previous tile's stores, were issued long ago) */
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-#pragma unroll
-        for (int q = 0; q < NF; q++) f0[q] = frag(va, vw, coff0, q);
-
         auto serp = [](int b) { return ((b / TN) & 1) ? TN - 1 - b % TN : b % TN; };
-        /* steady: steps kt + 1 .. kt + 3 all exist, so every load below is issued and the wait count is exact; the last
-         * steps of a tile run with tests and wait for everything */
-        auto step = [&](int kt, auto steady_c) {
-            constexpr bool steady = decltype(steady_c)::value;
+        /* TAIL = false: steps kt + 1 .. kt + 3 belong to this tile. TAIL = true: one of the last three steps of a tile;
+         * loads for steps beyond its K range request the first steps of the tile in nxt instead (every load is issued,
+         * so the wait counts stay exact). WAIT: what may be in flight at the barrier. */
+        auto step = [&](int kt, auto tail_c, auto wait_c) {
+            constexpr bool TAIL = decltype(tail_c)::value;
+            constexpr int WAIT = decltype(wait_c)::value;
             auto &accr = acc;
-            const bool more = steady || kt + 1 < KT;
             const int na = ca == NSA - 1 ? 0 : ca + 1, nw = cw == NSW - 1 ? 0 : cw + 1;
             const unsigned van = a_frag + na * ASZ, vwn = w_frag + nw * WSZ;
+            auto load = [&](int ks, int sa, int sw, int i) {
+                if (!TAIL) {
+                    issue1(cur.baseA, cur.baseW, cur.voff[i], ks, sa, sw, i);
+                } else {
+                    const bool over = ks >= KT;
+                    unsigned vo = over ? nxt.voff[i] : cur.voff[i];
+                    issue1(over ? nxt.baseA : cur.baseA, over ? nxt.baseW : cur.baseW, vo, over ? ks - KT : ks, sa, sw, i);
+                }
+            };
 #pragma unroll
             for (int b = 0; b < NM; b++) {
                 MFMA_AGPR(accr[serp(b)][b / TN], f0[serp(b)], f0[TN + b / TN]);
                 if (b % RD == 0 && b / RD < NF) f1[b / RD] = frag(va, vw, coff1, b / RD);
+                /* step kt + 2 of the first operand, into the slot that step kt - 1 left */
+                if (b % SF == 1 && b / SF < LF) load(kt + 2, ca == 0 ? 2 : ca - 1, cw == 0 ? 2 : cw - 1, (FIRST_A ? 0 : LA) + b / SF);
             }
-            if (more) {
-                /* step kt + 1 has landed for this wave and its reads of step kt are complete; past the barrier both
-                 * hold for all, and the slots of step kt are refilled below */
-                if (steady) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(AHEAD) : "memory");
-                else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            }
+            /* step kt + 1 has landed for this wave and its reads of step kt are complete; past the barrier both hold
+             * for all */
+            if (WAIT != AHEAD && strict) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AHEAD) : "memory");
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(WAIT) : "memory");
 #pragma unroll
             for (int b = 0; b < NM; b++) {
                 MFMA_AGPR(accr[serp(b)][b / TN], f1[serp(b)], f1[TN + b / TN]);
-                if (more && b % RD == 0 && b / RD < NF) f0[b / RD] = frag(van, vwn, coff0, b / RD);
-                if (b % RD == 1 && b / RD < NL) {
-                    const int i = nth(b / RD);
-                    const int ahead = i < LA ? NSA : NSW;
-                    if (steady || kt + ahead < KT) issue1(kt + ahead, ca, cw, i);
-                }
+                if (b % RD == 0 && b / RD < NF) f0[b / RD] = frag(van, vwn, coff0, b / RD);
+                /* step kt + NS2 of the second operand, into the slot of step kt */
+                if (b % SS == 1 && b / SS < LS) load(kt + NS2, ca, cw, (FIRST_A ? LA : 0) + b / SS);
             }
             ca = na;
             cw = nw;
             va = van;
             vw = vwn;
         };
-        int kt = 0;
-        for (; kt < KT - 3; kt++) step(kt, BoolC<true>{});
-        for (; kt < KT; kt++) step(kt, BoolC<false>{});
+        /* step 0: the stored tile's memory operations are older than anything its barrier needs (for the first tile
+         * everything has landed already) */
+        step(0, BoolC<false>{}, IntC<AHEAD_STORES>{});
+        int kt = 1;
+#ifdef GEMM_ABL_RELAX
+        for (; kt < KT - 3 && kt < 6; kt++) step(kt, BoolC<false>{}, IntC<40>{});
+#endif
+        for (; kt < KT - 3; kt++) step(kt, BoolC<false>{}, IntC<AHEAD>{});
 
-        /* The next tile's first stage is requested before this tile is stored: every wave has taken
-         * its last fragments out of LDS once it is past this barrier. */
+        /* the workgroup's next tile: its first steps are requested by this tile's last ones. After the last tile they
+         * request this tile's first steps once more, into slots that nobody reads again. */
         const TileId done = t;
         vb += gridDim.x;
         const bool again = vb < g.vgrid && decode_tile(g, vb, t);
-        if (again) {
-            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            set_sources(t);
-            prime(k_steps(t));
-        }
+        if (again) set_sources(nxt, t);
+        else nxt = cur;
+        for (; kt < KT; kt++) step(kt, BoolC<true>{}, IntC<AHEAD>{});
+
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); /* the last MFMA results retire before they are read */
         acc_fence<TM, TN>(acc);
 
@@ -756,9 +797,19 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
          * across the K loops, beyond what the register file holds beside the accumulators and fragments. */
         int l15e = l15, lqe = lq;
         asm volatile("" : "+v"(l15e), "+v"(lqe));
+#if defined(GEMM_ABL_STORE_SAME)
+        { TileId d2 = done; d2.tn = g.nq_tiles && done.tn >= g.nq_tiles ? g.nq_tiles : 0; d2.tm = 0; d2.tml = 0; d2.prob = 0;
+          store_tile<BN, WM, WN, EPI>(g, d2, acc, 0, g.M[0], wm, wn, l15e, lqe, wm); }
+#elif !defined(GEMM_ABL_NOSTORE)
         store_tile<BN, WM, WN, EPI>(g, done, acc, done.tml * BM, g.M[done.prob], wm, wn, l15e, lqe, done.tm * WGM + wm);
+#endif
         if (!again) break;
+        /* not every row of this wave's part of the stored tile was valid: it issued fewer than EpilogueOps operations */
+        strict = done.tml * BM + wm * WM + WM > g.M[done.prob];
+        cur = nxt;
     }
+    /* the requests made in place of a next tile's land in this workgroup's LDS: not after it has gone */
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 /* ------------------------------------------------------------------ host side */
@@ -859,7 +910,10 @@ static int launch_4d(GemmArgs &g) {
 
 template <int EPI>
 static int launch_epi(GemmArgs &g, int tile) {
-    if (g_ring && g_persistent) {
+    /* the ring kernel runs its tiles as one pipeline and wants at least four K steps in every K slice (the last slice
+     * may be shorter than the others); shorter ones go to the two-stage kernel */
+    const int kt_total = g.K >> 6, kt_last = kt_total - (g.ksplit - 1) * g.kt_per;
+    if (g_ring && g_persistent && g.kt_per >= 4 && kt_last >= 4) {
         /* three weight slots, two activation slots: in a denoising step the weights always come from HBM, the
          * activations mostly from the memory-side cache (measured per kernel in a step, this split beat the other
          * one by 0 - 10 %); the 192 x 192 tile has room for three of each */
