@@ -623,6 +623,98 @@ def bench_mfma_peak(args):
         "table": table, "roofline": None, "cpu_baseline": None}))
 
 
+def measure_workload(model, cfg, name, K, Wm, fused, args, headline):
+    """Wm untimed + K timed denoising steps of workload `name` through the session API on the resident model: inputs,
+    text and every step's modulation are in HBM before the timed region, which is bracketed by stream synchronisation
+    (wall clock) and by HIP events on the backend's stream; HIP events around every launch of the dominant kernel."""
+    import ctypes
+    wl = WORKLOADS[name]
+    h, w, nt = wl["h"], wl["w"], wl["txt"]
+    n_target = h * w
+    n_img = n_target + sum(rh * rw for rh, rw, _ in wl["refs"])
+    forwards = 2 if wl["cfg"] else 1
+    z = normal_f32((cfg.channels, h, w), 123, 1)
+    txt = normal_f32((nt, cfg.text_dim), 123, 2)
+    txt_u = normal_f32((nt, cfg.text_dim), 123, 3) if wl["cfg"] else None
+    refs = [(normal_f32((cfg.channels, rh, rw), 123, 10 + i), rh, rw, t) for i, (rh, rw, t) in enumerate(wl["refs"])]
+    sched = fluxhip.schedule("official", K + Wm, n_target)
+    sess = fluxhip.Session(model, z, h, w, txt, sched, refs=refs, txt_uncond=txt_u, guidance=4.0)
+
+    for i in range(Wm):
+        sess.step(i)
+    fluxhip.sync()
+    L = fluxhip.lib()
+    if not args.no_kernel_timing:
+        L.flux_hip_linear_probe(EPI_QKV_SWIGLU if fused else fluxhip.EPI_SWIGLU)   # events around the dominant kernel's launches
+    t0 = time.perf_counter()
+    L.flux_hip_timer_start()
+    for i in range(Wm, Wm + K):
+        sess.step(i)
+    ev_ms = L.flux_hip_timer_stop()      # waits for the last kernel
+    fluxhip.sync()
+    wall = time.perf_counter() - t0
+    k_n, k_ms = ctypes.c_int(0), ctypes.c_float(0.0)
+    # one projection runs under more than one tile shape in a step when it is launched at several sizes (the
+    # two-part launches of the double-stream blocks); the dominant kernel is the shape with the most time
+    epi_name = "QKV_SWIGLU" if fused else "SWIGLU"
+    TILE_NAMES = {0: f"gemm_kernel<64,128,2,2,{epi_name}>", 1: f"gemm_kernel<128,128,2,2,{epi_name}>", 2: f"gemm4d_kernel<8,8,{epi_name}> (256x256 tile)",
+                  3: f"gemm_kernel<64,64,2,2,{epi_name}>", 4: f"gemm_kernel<256,256,2,4,{epi_name}>", 5: f"gemm4d_kernel<9,6,{epi_name}> (288x192 tile)",
+                  6: f"gemm4d_kernel<6,6,{epi_name}> (192x192 tile)", 7: f"gemm4d_kernel<8,6,{epi_name}> (256x192 tile)",
+                  8: f"gemm_kernel<64,128,2,2,{epi_name},6> (ring of 6 stages)", 9: f"gemm_kernel<128,128,2,2,{epi_name},5> (ring of 5 stages)",
+                  10: f"gemm_kernel<96,128,2,2,{epi_name},5> (ring of 5 stages)"}
+    k_tile = -1
+    for tile in TILE_NAMES:
+        n_t, ms_t = ctypes.c_int(0), ctypes.c_float(0.0)
+        L.flux_hip_linear_probe_read_tile(tile, ctypes.byref(n_t), ctypes.byref(ms_t))
+        if ms_t.value > k_ms.value:
+            k_tile, k_n, k_ms = tile, n_t, ms_t
+    L.flux_hip_linear_probe(-1)
+    zf = sess.latent()
+    assert np.isfinite(zf).all(), "latent is not finite"
+    stages = fluxhip.stage_timing()
+    sess.close()
+
+    # The drop-in sampler entry point on host buffers (upload of latent and text, modulation for
+    # the schedule, 4 steps, download): the PCIe-inclusive figure, reported beside `value`, never as it.
+    n_run, host_run_ms = 4, None
+    if headline:
+        s4 = fluxhip.schedule("official", n_run, n_target)
+        model.sample(z, h, w, txt, s4, refs=refs, txt_uncond=txt_u, guidance=4.0)
+        t1 = time.perf_counter()
+        model.sample(z, h, w, txt, s4, refs=refs, txt_uncond=txt_u, guidance=4.0)
+        host_run_ms = (time.perf_counter() - t1) * 1000.0
+
+    ms_per_step = wall * 1000.0 / K
+    flops_step = forwards * flops_per_forward(cfg, n_img, nt, n_target)
+    tflops = flops_step / (wall / K) / 1e12
+
+    roof = None
+    if not args.no_kernel_timing and k_n.value > 0:
+        # fused: only the single-stream blocks launch this kernel, all at [image + text tokens, H]; not fused: every
+        # gate/up launch of the step, which all have that cost too
+        per_ms = k_ms.value / k_n.value
+        # a CFG step runs its two sequences as one batch: the launch then covers the rows of both
+        seqs = forwards if (fused and not args.sequential_cfg) else 1
+        k_flops, k_bytes = dominant_kernel_cost(cfg, seqs * (n_img + nt), fused)
+        ach = k_flops / (per_ms * 1e-3) / 1e12
+        gbps = k_bytes / (per_ms * 1e-3) / 1e9
+        what = "[Q|K|V|gate|up] projection of a single-stream block, bf16 store + SiLU(gate)*up" if fused else "gate/up projection + SiLU*up"
+        # the launch is bound by whichever of the two it needs longer for at the datasheet rates
+        if k_flops / (PEAK_BF16_TFLOPS * 1e12) >= k_bytes / (PEAK_HBM_GBPS * 1e9):
+            roof = {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES.get((name, fused))}
+        else:
+            roof = {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                    "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": TRAFFIC_BYTES.get((name, fused))}
+        roof.update({"kernel": TILE_NAMES[k_tile] + ": " + what, "launches_timed": k_n.value, "ms_per_launch": round(per_ms, 4),
+                     "flops_per_launch": k_flops, "bytes_per_launch": k_bytes, "tflops": round(ach, 1), "GBps": round(gbps, 1)})
+        if headline:
+            roof["ms_per_launch_back_to_back"] = round(time_dominant_kernel(cfg, seqs * (n_img + nt), fused), 4)
+    return {"ms_per_step": ms_per_step, "tflops": tflops, "flops_per_step": flops_step, "forwards": forwards, "roofline": roof,
+            "stages": [x / (K + Wm) for x in stages], "ev_ms": ev_ms, "host_run_ms": host_run_ms, "host_run_steps": n_run, "steps": K,
+            "tokens": n_img + nt}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -631,6 +723,8 @@ def main():
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + sorted(VAE_WORKLOADS) + sorted(ATT_WORKLOADS) + sorted(BW_WORKLOADS) + ["qwen3", "mfma_peak", "mfma_issue", "gemm_vs_lib"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="c4 only: leave out the short runs of c1, c2, c3 and c5 that follow the headline on the same weights")
     ap.add_argument("--tile-mask", type=lambda v: int(v, 0), default=0,
                     help="restrict the GEMM tiles the backend may choose (bit t = tile id t), for A/B runs")
     ap.add_argument("--sequential-cfg", action="store_true",
@@ -681,10 +775,6 @@ def main():
                           "gemm_algorithmic_bytes": by}))
         return
     K, Wm = args.steps, args.warmup
-    h, w, nt = wl["h"], wl["w"], wl["txt"]
-    n_target = h * w
-    n_img = n_target + sum(rh * rw for rh, rw, _ in wl["refs"])
-    forwards = 2 if wl["cfg"] else 1
     fused = bool(args.fused_qkv_mlp)
 
     fluxhip.init()
@@ -696,83 +786,20 @@ def main():
     fluxhip.lib().flux_hip_linear_ring(args.ring)
     fluxhip.lib().flux_hip_attention_force_variant(args.attention_variant)
     model = load_model(cfg)
-    z = normal_f32((cfg.channels, h, w), 123, 1)
-    txt = normal_f32((nt, cfg.text_dim), 123, 2)
-    txt_u = normal_f32((nt, cfg.text_dim), 123, 3) if wl["cfg"] else None
-    refs = [(normal_f32((cfg.channels, rh, rw), 123, 10 + i), rh, rw, t) for i, (rh, rw, t) in enumerate(wl["refs"])]
-    sched = fluxhip.schedule("official", K + Wm, n_target)
-    sess = fluxhip.Session(model, z, h, w, txt, sched, refs=refs, txt_uncond=txt_u, guidance=4.0)
+    head = measure_workload(model, cfg, args.workload, K, Wm, fused, args, headline=True)
+    ms_per_step, tflops, flops_step, forwards = head["ms_per_step"], head["tflops"], head["flops_per_step"], head["forwards"]
+    roof, stages, ev_ms, host_run_ms, n_run = head["roofline"], head["stages"], head["ev_ms"], head["host_run_ms"], head["host_run_steps"]
 
-    for i in range(Wm):
-        sess.step(i)
-    fluxhip.sync()
-    L = fluxhip.lib()
-    if not args.no_kernel_timing:
-        L.flux_hip_linear_probe(EPI_QKV_SWIGLU if fused else fluxhip.EPI_SWIGLU)   # events around the dominant kernel's launches
-    t0 = time.perf_counter()
-    L.flux_hip_timer_start()
-    for i in range(Wm, Wm + K):
-        sess.step(i)
-    ev_ms = L.flux_hip_timer_stop()      # waits for the last kernel
-    fluxhip.sync()
-    wall = time.perf_counter() - t0
-    import ctypes
-    k_n, k_ms = ctypes.c_int(0), ctypes.c_float(0.0)
-    # one projection runs under more than one tile shape in a step when it is launched at several sizes (the
-    # two-part launches of the double-stream blocks); the dominant kernel is the shape with the most time
-    epi_name = "QKV_SWIGLU" if fused else "SWIGLU"
-    TILE_NAMES = {0: f"gemm_kernel<64,128,2,2,{epi_name}>", 1: f"gemm_kernel<128,128,2,2,{epi_name}>", 2: f"gemm4d_kernel<8,8,{epi_name}> (256x256 tile)",
-                  3: f"gemm_kernel<64,64,2,2,{epi_name}>", 4: f"gemm_kernel<256,256,2,4,{epi_name}>", 5: f"gemm4d_kernel<9,6,{epi_name}> (288x192 tile)",
-                  6: f"gemm4d_kernel<6,6,{epi_name}> (192x192 tile)", 7: f"gemm4d_kernel<8,6,{epi_name}> (256x192 tile)",
-                  8: f"gemm_kernel<64,128,2,2,{epi_name},6> (ring of 6 stages)", 9: f"gemm_kernel<128,128,2,2,{epi_name},5> (ring of 5 stages)",
-                  10: f"gemm_kernel<96,128,2,2,{epi_name},5> (ring of 5 stages)"}
-    k_tile = -1
-    for tile in TILE_NAMES:
-        n_t, ms_t = ctypes.c_int(0), ctypes.c_float(0.0)
-        L.flux_hip_linear_probe_read_tile(tile, ctypes.byref(n_t), ctypes.byref(ms_t))
-        if ms_t.value > k_ms.value:
-            k_tile, k_n, k_ms = tile, n_t, ms_t
-    L.flux_hip_linear_probe(-1)
-    zf = sess.latent()
-    assert np.isfinite(zf).all(), "latent is not finite"
-    stages = fluxhip.stage_timing()
-    sess.close()
-
-    # The drop-in sampler entry point on host buffers (upload of latent and text, modulation for
-    # the schedule, 4 steps, download): the PCIe-inclusive figure, reported beside `value`, never as it.
-    n_run = 4
-    s4 = fluxhip.schedule("official", n_run, n_target)
-    model.sample(z, h, w, txt, s4, refs=refs, txt_uncond=txt_u, guidance=4.0)
-    t1 = time.perf_counter()
-    model.sample(z, h, w, txt, s4, refs=refs, txt_uncond=txt_u, guidance=4.0)
-    host_run_ms = (time.perf_counter() - t1) * 1000.0
-
-    ms_per_step = wall * 1000.0 / K
-    flops_step = forwards * flops_per_forward(cfg, n_img, nt, n_target)
-    tflops = flops_step / (wall / K) / 1e12
-
-    roof = None
-    if not args.no_kernel_timing and k_n.value > 0:
-        # fused: only the single-stream blocks launch this kernel, all at [image + text tokens, H]; not fused: every
-        # gate/up launch of the step, which all have that cost too
-        per_ms = k_ms.value / k_n.value
-        # a CFG step runs its two sequences as one batch: the launch then covers the rows of both
-        seqs = forwards if (fused and not args.sequential_cfg) else 1
-        k_flops, k_bytes = dominant_kernel_cost(cfg, seqs * (n_img + nt), fused)
-        ach = k_flops / (per_ms * 1e-3) / 1e12
-        gbps = k_bytes / (per_ms * 1e-3) / 1e9
-        alone_ms = time_dominant_kernel(cfg, seqs * (n_img + nt), fused)
-        what = "[Q|K|V|gate|up] projection of a single-stream block, bf16 store + SiLU(gate)*up" if fused else "gate/up projection + SiLU*up"
-        # the launch is bound by whichever of the two it needs longer for at the datasheet rates
-        if k_flops / (PEAK_BF16_TFLOPS * 1e12) >= k_bytes / (PEAK_HBM_GBPS * 1e9):
-            roof = {"bound": "mfma", "achieved": round(ach, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                    "frac": round(ach / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES.get((args.workload, fused))}
-        else:
-            roof = {"bound": "hbm", "achieved": round(gbps, 1), "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                    "frac": round(gbps / PEAK_HBM_GBPS, 4), "traffic": TRAFFIC_BYTES.get((args.workload, fused))}
-        roof.update({"kernel": TILE_NAMES[k_tile] + ": " + what, "launches_timed": k_n.value, "ms_per_launch": round(per_ms, 4),
-                     "flops_per_launch": k_flops, "bytes_per_launch": k_bytes, "tflops": round(ach, 1), "GBps": round(gbps, 1),
-                     "ms_per_launch_back_to_back": round(alone_ms, 4)})
+    # The other configurations of the benchmark on the same resident weights, so that one line carries all five: a short
+    # run each (same timing brackets, same probe on the dominant kernel), no CPU baseline of their own.
+    others = None
+    if args.workload == "c4" and not args.no_other_configs:
+        others = {}
+        for name in ("c1", "c2", "c3", "c5"):
+            r = measure_workload(model, cfg, name, max(4, min(K, 8)), 2, fused, args, headline=False)
+            others[name] = {"workload": WORKLOADS[name]["desc"], "ms_per_step": round(r["ms_per_step"], 3), "steps_per_s": round(1000.0 / r["ms_per_step"], 3),
+                            "steps": r["steps"], "tflops": round(r["tflops"], 1), "frac_of_bf16_peak": round(r["tflops"] / PEAK_BF16_TFLOPS, 4),
+                            "forwards_per_step": r["forwards"], "roofline": r["roofline"]}
     model.close()
 
     # What this box's matrix pipes sustain on their own (register-resident v_mfma_f32_16x16x32_bf16 on random bit patterns, two
@@ -803,9 +830,8 @@ def main():
         "flops_per_step": flops_step, "device_ms_per_step_events": round(ev_ms / K, 3),
         "host_buffer_run": {"steps": n_run, "ms": round(host_run_ms, 2),
                             "steps_per_s": round(n_run / host_run_ms * 1000.0, 3)},
-        "stage_ms_per_step": {"double": round(stages[0] / (K + Wm), 3), "single": round(stages[1] / (K + Wm), 3),
-                              "final": round(stages[2] / (K + Wm), 3)},
-        "roofline": roof, "cpu_baseline": cpu, "box": box,
+        "stage_ms_per_step": {"double": round(stages[0], 3), "single": round(stages[1], 3), "final": round(stages[2], 3)},
+        "roofline": roof, "cpu_baseline": cpu, "box": box, "other_configs": others,
     }
     print(json.dumps(out))
 

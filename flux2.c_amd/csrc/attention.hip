@@ -118,6 +118,11 @@ extern "C" int flux_hip_qk_prepare(void *k_out, void *qkv, int ld, int q_col, in
     if (((uintptr_t)k_out | (uintptr_t)qkv | (uintptr_t)q_w0 | (uintptr_t)q_w1 | (uintptr_t)k_w0 | (uintptr_t)k_w1 | (uintptr_t)rope_cos |
          (uintptr_t)rope_sin) & 15)
         return flux_hip_fail("flux_hip_qk_prepare: operands must be 16-byte aligned");
+    {
+        /* K goes to k_out while the same launch still reads and rewrites qkv: the two must not overlap */
+        const uintptr_t a0 = (uintptr_t)qkv, a1 = a0 + (size_t)rows * ld * 2, b0 = (uintptr_t)k_out, b1 = b0 + (size_t)rows * heads * HD * 2;
+        if (a0 < b1 && b0 < a1) return flux_hip_fail("flux_hip_qk_prepare: k_out overlaps the qkv buffer");
+    }
     hipLaunchKernelGGL(qk_prepare_kernel, dim3((rows + 63) / 64, heads), dim3(256), 0, flux_hip_stream_handle(),
                        (bf16 *)k_out, (bf16 *)qkv, ld, q_col, k_col, rows, heads, split, q_w0, q_w1 ? q_w1 : q_w0, k_w0, k_w1 ? k_w1 : k_w0,
                        rope_cos, rope_sin, eps);
@@ -978,12 +983,16 @@ __global__ __launch_bounds__(256, 1) void attention_wide_kernel(AttSeqs p, int l
  * blocks dearer per query). */
 struct WidePlan { int nqa, na, nb; };
 static WidePlan wide_plan(int seq_q, int heads) {
-    static int c_seq = -1, c_heads = -1;
-    static WidePlan c_plan;
-    if (seq_q == c_seq && heads == c_heads) return c_plan;
+    /* the search below is some 1e5 operations at 4608 queries: its last results are kept, keyed by everything it
+     * depends on (two alternating query lengths, or two devices, would otherwise repeat it on every call) */
+    struct Entry { int seq, heads, cus; WidePlan plan; };
+    static Entry cache[8];
+    static int n_cached = 0, next = 0;
     static const double cost[5] = {0.0, 0.44, 0.62, 0.81, 1.0};
     int cus = 256, dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 8) cus = 256;
+    for (int i = 0; i < n_cached; i++)
+        if (cache[i].seq == seq_q && cache[i].heads == heads && cache[i].cus == cus) return cache[i].plan;
     const int per_xcd = cus / 8, nh = (heads + 7) / 8;
     WidePlan best = {2, 0, (seq_q + 63) / 64};
     double best_t = 1e30;
@@ -1007,7 +1016,9 @@ static WidePlan wide_plan(int seq_q, int heads) {
             if (t < best_t) { best_t = t; best = {nqa, na, nb}; }
         }
     }
-    c_seq = seq_q; c_heads = heads; c_plan = best;
+    cache[next] = {seq_q, heads, cus, best};
+    next = (next + 1) % 8;
+    if (n_cached < 8) n_cached++;
     return best;
 }
 
@@ -1016,11 +1027,13 @@ extern "C" void flux_hip_attention_force_variant(int v) { g_att_force = v; }
 
 static int attention_check(const void *out_bf16, int ldo, const void *q, int ldq, const void *k, const void *v, int ldv, int seq_k, int heads) {
     if (seq_k <= 0) return flux_hip_fail("flux_hip_attention: seq_k=%d", seq_k);
+    if (heads <= 0) return flux_hip_fail("flux_hip_attention: heads=%d", heads);
     if (!out_bf16 || !q || !k || !v) return flux_hip_fail("flux_hip_attention: NULL argument");
     if ((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v) & 15) || ((uintptr_t)out_bf16 & 7))
         return flux_hip_fail("flux_hip_attention: operands must be 16-byte aligned (output 8-byte)");
-    if ((ldo & 3) || (ldq & 7) || (ldv & 7) || ldv < heads * HD)
-        return flux_hip_fail("flux_hip_attention: bad leading dimensions (ldo=%d ldq=%d ldv=%d)", ldo, ldq, ldv);
+    if ((ldo & 3) || (ldq & 7) || (ldv & 7) || ldv < heads * HD || ldq < heads * HD || ldo < heads * HD)
+        return flux_hip_fail("flux_hip_attention: bad leading dimensions (ldo=%d ldq=%d ldv=%d; each at least heads * %d = %d)", ldo, ldq, ldv, HD,
+                             heads * HD);
     /* the tile loaders address K and V rows with 32-bit byte offsets that run up to 64 rows past the end */
     if ((double)(seq_k + 64) * ldv * 2.0 >= 4294967296.0 || (double)(seq_k + 64) * heads * HD * 2.0 >= 4294967296.0)
         return flux_hip_fail("flux_hip_attention: %d keys of %d-element rows exceed 32-bit offsets", seq_k, ldv);

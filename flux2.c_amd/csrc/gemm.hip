@@ -1185,6 +1185,8 @@ static int g_splitk_enabled = 1;
 extern "C" void flux_hip_linear_force_tile(int tile) { g_force_tile = tile; }
 extern "C" void flux_hip_linear_tile_mask(unsigned mask) { g_tile_mask = mask ? mask : 0x7EF; }
 extern "C" void flux_hip_linear_enable_splitk(int on) { g_splitk_enabled = on; }
+static int g_force_split = 0; /* > 1: every projection that can run as K slices runs as this many (comparison runs and tests) */
+extern "C" void flux_hip_linear_force_split(int slices) { g_force_split = slices > 1 ? slices : 0; }
 
 /* Launch probe: HIP events around every launch with one chosen epilogue, so a benchmark can
  * read that kernel's average duration inside its timed region. */
@@ -1287,7 +1289,15 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
             for (int si = 0; si < 10; si++) {
                 const int sp = splits[si];
                 if (sp > 1 && (!can_split || kt_total / sp < 4)) break;
-                if (sp > 1 && fixed_ws && (double)sp * rows * N * sizeof(float) > (double)fixed_ws_bytes) break; /* the slices must fit the given workspace */
+                if (g_force_split && can_split && sp != g_force_split && kt_total / g_force_split >= 4) continue;
+                if (sp > 1 && fixed_ws && (double)sp * rows * N * sizeof(float) > (double)fixed_ws_bytes) {
+                    /* the slices must fit the given workspace: fewer slices then, down to none - unless this number
+                     * of slices was demanded, which is the one request the fixed workspace refuses */
+                    if (sp == g_force_split)
+                        return flux_hip_fail("flux_hip_linear_static: %d K slices of %.0f rows x %d columns need %.1f MiB of partial sums, beyond the maximum "
+                                             "of %zu MiB of the static workspace", sp, rows, N, sp * rows * N * 4.0 / 1048576.0, fixed_ws_bytes >> 20);
+                    break;
+                }
                 const int per = (kt_total + sp - 1) / sp;
                 const long blocks = tiles * ((kt_total + per - 1) / per);
                 const long slots = 256L * occ[t];
@@ -1328,7 +1338,8 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
     }
 
     if (tile_out) *tile_out = tile;
-    const int slot = probe_slot(epilogue);
+    /* the launch probe creates events: never on the path that promises to allocate nothing */
+    const int slot = fixed_ws ? -1 : probe_slot(epilogue);
     if (slot >= 0) g_probe_tile[slot] = (unsigned char)tile;
     if (slot >= 0) (void)hipEventRecord(g_probe_ev[slot][0], flux_hip_stream_handle());
     int ok;
@@ -1356,14 +1367,15 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
 }
 
 static int linear_impl(int epilogue, int nparts, const flux_hip_linear_part *parts, int N, int K, int lda, int ldw, int ldc, int w_row0,
-                       int w_row1, const flux_hip_adaln_part *norm, float eps, int *fused, float *fixed_ws = nullptr, size_t fixed_ws_bytes = 0) {
-    if (epilogue < FLUX_HIP_EPI_BF16 || epilogue > FLUX_HIP_EPI_SWIGLU) return flux_hip_fail("flux_hip_linear: unknown epilogue %d", epilogue);
-    if (nparts < 1 || nparts > GEMM_MAX_PARTS) return flux_hip_fail("flux_hip_linear: nparts=%d (1 to %d)", nparts, GEMM_MAX_PARTS);
-    if (K <= 0 || (K & 63)) return flux_hip_fail("flux_hip_linear: K=%d must be a positive multiple of 64", K);
-    if (N <= 0 || (N & 127)) return flux_hip_fail("flux_hip_linear: N=%d must be a positive multiple of 128", N);
+                       int w_row1, const flux_hip_adaln_part *norm, float eps, int *fused, float *fixed_ws = nullptr, size_t fixed_ws_bytes = 0,
+                       const char *who = "flux_hip_linear") {
+    if (epilogue < FLUX_HIP_EPI_BF16 || epilogue > FLUX_HIP_EPI_SWIGLU) return flux_hip_fail("%s: unknown epilogue %d", who, epilogue);
+    if (nparts < 1 || nparts > GEMM_MAX_PARTS) return flux_hip_fail("%s: nparts=%d (1 to %d)", who, nparts, GEMM_MAX_PARTS);
+    if (K <= 0 || (K & 63)) return flux_hip_fail("%s: K=%d must be a positive multiple of 64", who, K);
+    if (N <= 0 || (N & 127)) return flux_hip_fail("%s: N=%d must be a positive multiple of 128", who, N);
     if (lda < K || ldw < K || (lda & 7) || (ldw & 7))
-        return flux_hip_fail("flux_hip_linear: lda=%d ldw=%d must be >= K and multiples of 8", lda, ldw);
-    if (epilogue != FLUX_HIP_EPI_F32_T && (ldc & 3)) return flux_hip_fail("flux_hip_linear: ldc=%d must be a multiple of 4", ldc);
+        return flux_hip_fail("%s: lda=%d ldw=%d must be >= K and multiples of 8", who, lda, ldw);
+    if (epilogue != FLUX_HIP_EPI_F32_T && (ldc & 3)) return flux_hip_fail("%s: ldc=%d must be a multiple of 4", who, ldc);
     GemmArgs g = {};
     AdalnArgs a = {};
     int maxm = 0;
@@ -1438,16 +1450,10 @@ extern "C" int flux_hip_linear_qkv_swiglu(const void *A, const void *W, void *qk
  * streams, two host threads) would share it and race. */
 extern "C" int flux_hip_linear_static(int epilogue, int nparts, const flux_hip_linear_part *parts,
                                       int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1) {
-    if (nparts < 1 || nparts > GEMM_MAX_PARTS) return flux_hip_fail("flux_hip_linear_static: nparts=%d (1 to %d)", nparts, GEMM_MAX_PARTS);
-    long long rows = 0;
-    for (int i = 0; i < nparts; i++) rows += parts[i].M > 0 ? parts[i].M : 0;
-    if (N > 0 && rows * (long long)N > (long long)FLUX_HIP_LINEAR_STATIC_MAX_OUTPUTS)
-        return flux_hip_fail("flux_hip_linear_static: %lld rows x %d columns = %lld outputs, beyond the maximum of %lld "
-                             "(two K slices of fp32 partial sums must fit the %zu MiB static workspace)",
-                             rows, N, rows * (long long)N, (long long)FLUX_HIP_LINEAR_STATIC_MAX_OUTPUTS, STATIC_WS_BYTES >> 20);
     float *ws = static_ws_for_current_device();
     if (!ws) return 0;
-    return linear_impl(epilogue, nparts, parts, N, K, lda, ldw, ldc, w_row0, w_row1, nullptr, 0.0f, nullptr, ws, STATIC_WS_BYTES);
+    return linear_impl(epilogue, nparts, parts, N, K, lda, ldw, ldc, w_row0, w_row1, nullptr, 0.0f, nullptr, ws, STATIC_WS_BYTES,
+                       "flux_hip_linear_static");
 }
 
 /* The residual projection, and - when it runs as K slices - the AdaLN of the updated rows in its

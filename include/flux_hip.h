@@ -116,13 +116,17 @@ int flux_hip_linear_qkv_swiglu(const void *A, const void *W, void *qkv_out, void
  * fp32 partial sums in a static device array of FLUX_HIP_LINEAR_STATIC_BYTES instead, which every GPU
  * the library runs on holds until the process ends, and considers only as many slices as fit there.
  * Same arguments, epilogues and results (to fp32 summation order when the number of slices differs)
- * as flux_hip_linear. Fails, before anything is launched, when the row counts of all parts together
- * times N exceed FLUX_HIP_LINEAR_STATIC_MAX_OUTPUTS (two slices must fit). All calls on one GPU share
- * the array: calls that overlap there (two streams, two host threads) race. The array's contents need
- * no clearing between calls.
+ * as flux_hip_linear, at every size: a call whose outputs (row counts of all parts together times N)
+ * exceed FLUX_HIP_LINEAR_STATIC_MAX_OUTPUTS cannot keep even two slices in the array and runs as one
+ * launch without slices, which needs no workspace at all (the large projections of the model never
+ * split anyway). The one thing it refuses, with an error that says so and before anything is
+ * launched, is a number of slices demanded through flux_hip_linear_force_split (flux_hip_debug.h)
+ * whose partial sums exceed the array. It creates no events either: the launch probe of
+ * flux_hip_debug.h does not see these calls. All calls on one GPU share the array: calls that overlap
+ * there (two streams, two host threads) race. The array's contents need no clearing between calls.
  */
 #define FLUX_HIP_LINEAR_STATIC_BYTES (64u << 20)
-#define FLUX_HIP_LINEAR_STATIC_MAX_OUTPUTS (FLUX_HIP_LINEAR_STATIC_BYTES / 8u) /* rows * N */
+#define FLUX_HIP_LINEAR_STATIC_MAX_OUTPUTS (FLUX_HIP_LINEAR_STATIC_BYTES / 8u) /* rows * N up to which K slices are considered */
 int flux_hip_linear_static(int epilogue, int nparts, const flux_hip_linear_part *parts,
                            int N, int K, int lda, int ldw, int ldc, int w_row0, int w_row1);
 

@@ -25,6 +25,11 @@ void flux_hip_linear_force_tile(int tile);
 void flux_hip_linear_tile_mask(unsigned mask);
 /* 0 turns the split-K path off (default 1) */
 void flux_hip_linear_enable_splitk(int on);
+/* slices > 1: projections whose epilogue and K length allow it run as exactly that many K slices (one of 2, 3, 4, 6,
+ * 8, 12, 16, 24, 32; at least four 64-wide K steps per slice), whatever the cost model would choose; 0 (default):
+ * the cost model chooses. With flux_hip_linear_static a demanded number of slices whose partial sums do not fit the
+ * static workspace is refused. */
+void flux_hip_linear_force_split(int slices);
 /* 1 (default): the 4-wave GEMM launches at most one workgroup per compute unit and each walks several
  * tiles; 0: one workgroup per tile */
 void flux_hip_linear_persistent(int on);

@@ -42,6 +42,7 @@ def _default_switches(request):
         L.flux_hip_linear_force_tile(-1)
         L.flux_hip_linear_tile_mask(0)
         L.flux_hip_linear_enable_splitk(1)
+        L.flux_hip_linear_force_split(0)
         L.flux_hip_linear_persistent(1)
         L.flux_hip_linear_ring(1)
         L.flux_hip_attention_force_variant(-1)

@@ -64,7 +64,7 @@ def test_reference_pipeline_runs_on_the_backend(oracle_mod, tmp_path):
 
     ctx = P.flux_load_dir(str(tmp_path).encode())
     assert ctx, P.flux_get_error()
-    width, height, steps, seed, seq = 64, 96, 3, 11, 24
+    width, height, steps, seed, seq = 48, 64, 3, 11, 24      # the reference's CPU VAE decodes it twice: kept small
     lh, lw = height // 16, width // 16
     emb = normal_f32((seq, cfg.text_dim), 40, 1)
     prm = FluxParams(width, height, steps, seed, 0.0, 0, 0, 2.0)
@@ -469,7 +469,8 @@ def _room_for_full_size(path):
     return shutil.disk_usage(path).free >> 30 >= 24 and avail >= 80
 
 
-@pytest.mark.skipif(os.environ.get("FLUX_SKIP_FULLSIZE_E2E") == "1", reason="switched off by FLUX_SKIP_FULLSIZE_E2E=1")
+@pytest.mark.skipif(not os.environ.get("FLUX_SLOW"), reason="the reference's command-line program on a 14 GB model directory: 75 s, "
+                    "and the program is outside the path this backend replaces; set FLUX_SLOW=1")
 @pytest.mark.skipif(not (os.path.exists(CLI) and os.path.exists(REF)), reason="reference-built programs not present")
 def test_full_size_model_through_the_command_line_program(oracle_mod, tmp_path):
     """The model at its real sizes (4B transformer, layers 0-26 of the 4B text encoder, the VAE; random

@@ -1,7 +1,8 @@
 """flux_hip_linear_static, the entry point that allocates nothing (its K slices' partial sums live in a
 static device array), against flux_hip_linear on the same operands, through the C ABI: two calls in a row, the
-second with a smaller input, so that what the first left in the shared array would show; the error for sizes
-beyond the stated maximum; and the device's free memory, which must not move across the calls."""
+second with a smaller input, so that what the first left in the shared array would show; a call too large to keep
+K slices in the array (it runs without slices); the error for a demanded number of slices beyond the array; and the
+device's free memory, which must not move across the calls."""
 import ctypes
 
 import numpy as np
@@ -94,8 +95,33 @@ def test_static_workspace_entry_point(oracle_mod):
     da, dW2, o = hip.DevBuf.from_array(f32_to_bf16(a)), hip.DevBuf.from_array(f32_to_bf16(W2)), hip.DevBuf(M * 256 * 4)
     static_linear(hip, hip.EPI_F32, [(da.ptr, dW2.ptr, o.ptr, None, M)], 256, 256, 256, 256, 256)
     assert rel_l2(o.to_array(np.float32, (M, 256)), oracle_mod.linear(a, W2)) < 2e-6
-    # ... and one beyond the maximum is refused with a reason before anything is launched
+    # ... and so does one whose outputs exceed what two slices of partial sums could keep in the array: as one launch
+    # without slices, bit for bit what flux_hip_linear gives with its K slices switched off, and nothing allocated
     big_rows = MAX_OUTPUTS // N + 1
-    with pytest.raises(hip.FluxHipError) as err:
-        static_linear(hip, hip.EPI_F32, [(da.ptr, dW.ptr, o.ptr, None, big_rows)], N, K, K, K, N)
-    assert "beyond the maximum" in str(err.value)
+    ab = q(normal_f32((big_rows, K), 56, 1))
+    dab = hip.DevBuf.from_array(f32_to_bf16(ab))
+    o1, o2 = hip.DevBuf(big_rows * N * 4), hip.DevBuf(big_rows * N * 4)
+    static_linear(hip, hip.EPI_F32, [(dab.ptr, dW.ptr, o1.ptr, None, big_rows)], N, K, K, K, N)
+    hip.sync()
+    before = free_bytes()
+    static_linear(hip, hip.EPI_F32, [(dab.ptr, dW.ptr, o1.ptr, None, big_rows)], N, K, K, K, N)
+    hip.sync()
+    assert free_bytes() == before
+    L = hip.lib()
+    L.flux_hip_linear_enable_splitk(0)
+    try:
+        hip.linear(hip.EPI_F32, [(dab.ptr, dW.ptr, o2.ptr, None, big_rows)], N, K, K, K, N)
+    finally:
+        L.flux_hip_linear_enable_splitk(1)
+    np.testing.assert_array_equal(o1.to_array(np.float32, (big_rows, N)), o2.to_array(np.float32, (big_rows, N)))
+    # a demanded number of slices beyond the array is the one request it refuses, with a reason, before anything is launched
+    L.flux_hip_linear_force_split(4)
+    try:
+        with pytest.raises(hip.FluxHipError) as err:
+            static_linear(hip, hip.EPI_F32, [(dab.ptr, dW.ptr, o1.ptr, None, big_rows)], N, K, K, K, N)
+        assert "beyond the maximum" in str(err.value)
+        # ... while the same demand on a size that fits is served
+        static_linear(hip, hip.EPI_F32, [(dab.ptr, dW.ptr, o2.ptr, None, 64)], N, K, K, K, N)
+        assert rel_l2(o2.to_array(np.float32, (big_rows, N))[:64], oracle_mod.linear(ab[:64], W)) < 2e-6
+    finally:
+        L.flux_hip_linear_force_split(0)
