@@ -440,8 +440,10 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attention_kernel(bf1
 }
 
 /* The wide kernel's way out for a workgroup whose softmax references did not hold (see first_reference): the same
- * queries once more with moving references, 128 at a time. One copy for all instances of the wide kernel. */
-__device__ __attribute__((noinline)) void attention_redo(char *smem, int h, int q_begin, int q_end, bf16 *out, int ldo, const bf16 *q, int ldq,
+ * queries once more with moving references, 128 at a time. Inlined into every instance of the wide kernel: as an
+ * out-of-line function it gave each of them a call frame in scratch memory (1072 bytes per lane that every launch
+ * had to have backed, though only this path touched it). */
+__device__ __forceinline__ void attention_redo(char *smem, int h, int q_begin, int q_end, bf16 *out, int ldo, const bf16 *q, int ldq,
                                                          const bf16 *k, const bf16 *v, int ldv, int seq_k, int heads) {
     for (int qs = q_begin; qs < q_end; qs += 128) {
         attention_block<4>(smem, h, qs, min(qs + 128, q_end), out, ldo, q, ldq, k, v, ldv, seq_k, heads);

@@ -157,17 +157,47 @@ __device__ __forceinline__ bool decode_tile(const GemmArgs &g, int vb, TileId &t
     return true;
 }
 
-/* Weight row that feeds column v of the tile. For the SwiGLU epilogue 16-column blocks alternate
- * gate, up so that a lane ends up holding matching pairs. */
+/* Which feature of its wave's slice of the output row r of MFMA block blk computes, for the two epilogues that
+ * store bf16. In the accumulator a lane holds four consecutive MFMA rows of a block (rows 4 (lane / 16) .. + 3): with
+ * rows numbered plainly that is four consecutive features, an 8-byte store, and a wave's store instruction writes
+ * 32 bytes to each of 16 output rows. Here two neighbouring blocks interleave instead: block 2p takes features
+ * 32 p + 8 q + 0 .. 3 on its rows 4 q .. 4 q + 3 and block 2p + 1 features 32 p + 8 q + 4 .. 7, so that a lane's
+ * results of the two blocks are eight consecutive features: one 16-byte store, 64 bytes per output row and
+ * instruction, half as many store instructions and write requests. Only the weight rows a block reads change. */
+__device__ __forceinline__ int bf16_pair_feature(int blk, int r) { return 32 * (blk >> 1) + 8 * (r >> 2) + 4 * (blk & 1) + (r & 3); }
+/* SiLU(gate) * up: blocks alternate gate, up, so that a lane holds matching pairs; the (gate, up) pairs interleave
+ * two by two in the same way, and a last odd pair keeps the plain numbering (features 16 k + r). */
+template <int TN>
+__device__ __forceinline__ int swiglu_feature(int blk, int r) {
+    const int k = blk >> 1;
+    return k < 2 * (TN / 4) ? bf16_pair_feature(k, r) : 16 * k + r;
+}
+
+/* Weight row that feeds column v of the tile. */
 template <int BN, int WN, int EPI>
 __device__ __forceinline__ int weight_row(const GemmArgs &g, int tn, int v) {
+    constexpr int TN = WN / 16;
+    const int wv = v / WN, blk = (v % WN) >> 4, r = v & 15;
     if (EPI == FLUX_HIP_EPI_SWIGLU || (EPI == EPI_QKV_SWIGLU && tn >= g.nq_tiles)) {
-        int wv = v / WN, blk = (v % WN) >> 4;
-        int idx = wv * (WN / 2) + (blk >> 1) * 16 + (v & 15);
+        const int idx = wv * (WN / 2) + swiglu_feature<TN>(blk, r);
         if (EPI == EPI_QKV_SWIGLU) return ((blk & 1) ? g.w_row2 : g.w_row1) + (tn - g.nq_tiles) * (BN / 2) + idx;
         return ((blk & 1) ? g.w_row1 : g.w_row0) + tn * (BN / 2) + idx;
     }
+    if (EPI == FLUX_HIP_EPI_BF16 || EPI == EPI_QKV_SWIGLU) return g.w_row0 + tn * BN + wv * WN + bf16_pair_feature(blk, r);
     return g.w_row0 + tn * BN + v;
+}
+
+/* eight bf16 to consecutive addresses: one 16-byte store where the address allows it, else two of 8 bytes */
+__device__ __forceinline__ void store_bf16x8(bf16 *p, bf16x4 lo, bf16x4 hi, bool aligned16) {
+    if (aligned16) {
+        bf16x8 o;
+#pragma unroll
+        for (int e = 0; e < 4; e++) { o[e] = lo[e]; o[4 + e] = hi[e]; }
+        *(bf16x8 *)p = o;
+    } else {
+        *(bf16x4 *)p = lo;
+        *(bf16x4 *)(p + 4) = hi;
+    }
 }
 
 /* Accumulator element e of block (i, j): feature n = 4*(lane/16) + e of the 16-column block,
@@ -177,6 +207,7 @@ __device__ __forceinline__ void store_tile_to(const GemmArgs &g, const TileId &t
                                               int wm, int wn, int l15, int lq, int prow, void *Cp, const int ldc, const int tn) {
     constexpr int TM = WM / 16, TN = WN / 16;
     const int prob = t.prob, n0 = tn * BN, ks = t.ks;
+    const bool aligned16 = (((uintptr_t)Cp | ((uintptr_t)ldc << 1)) & 15) == 0; /* every 8-feature group of the output starts on 16 bytes */
     f32x4 acc_here[HERE ? TN : 1][HERE ? TM : 1];
     auto &acc = [&]() -> auto & { if constexpr (HERE) return acc_here; else return acc_in; }();
     float st_s[TN], st_q[TN]; /* convolutions with statistics: this lane's sums per 16-column block */
@@ -199,24 +230,32 @@ __device__ __forceinline__ void store_tile_to(const GemmArgs &g, const TileId &t
             inside = y >= 1 && y < g.conv_hp - 1 && x >= 1 && x < g.conv_wp - 1;
         }
         if (EPI == FLUX_HIP_EPI_SWIGLU) {
-            bf16 *C = (bf16 *)Cp + (size_t)m * ldc + tn * (BN / 2) + wn * (WN / 2) + lq * 4;
+            /* see swiglu_feature: two (gate, up) pairs give eight consecutive features, a last odd pair four */
+            bf16 *C = (bf16 *)Cp + (size_t)m * ldc + tn * (BN / 2) + wn * (WN / 2);
+            bf16x4 o[TN / 2];
 #pragma unroll
-            for (int i = 0; i < TN; i += 2) {
-                bf16x4 o;
+            for (int k = 0; k < TN / 2; k++)
 #pragma unroll
-                for (int e = 0; e < 4; e++) o[e] = (bf16)(silu_f(acc[i][j][e]) * acc[i + 1][j][e]);
-                *(bf16x4 *)(C + (i >> 1) * 16) = o;
+                for (int e = 0; e < 4; e++) o[k][e] = (bf16)(silu_f(acc[2 * k][j][e]) * acc[2 * k + 1][j][e]);
+#pragma unroll
+            for (int p = 0; p < TN / 4; p++) store_bf16x8(C + 32 * p + 8 * lq, o[2 * p], o[2 * p + 1], aligned16);
+            if (TN / 2 % 2) *(bf16x4 *)(C + 16 * (TN / 2 - 1) + 4 * lq) = o[TN / 2 - 1];
+        } else if (EPI == FLUX_HIP_EPI_BF16) {
+            /* see bf16_pair_feature: blocks 2p and 2p + 1 give eight consecutive features */
+            static_assert(EPI != FLUX_HIP_EPI_BF16 || TN % 2 == 0, "bf16 outputs pair 16-column blocks");
+            bf16 *C = (bf16 *)Cp + (size_t)m * ldc + n0 + wn * WN + 8 * lq;
+#pragma unroll
+            for (int p = 0; p < TN / 2; p++) {
+                bf16x4 lo, hi;
+#pragma unroll
+                for (int e = 0; e < 4; e++) { lo[e] = (bf16)acc[2 * p][j][e]; hi[e] = (bf16)acc[2 * p + 1][j][e]; }
+                store_bf16x8(C + 32 * p, lo, hi, aligned16);
             }
         } else {
 #pragma unroll
             for (int i = 0; i < TN; i++) {
                 const int n = n0 + wn * WN + i * 16 + lq * 4;
-                if (EPI == FLUX_HIP_EPI_BF16) {
-                    bf16x4 o;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) o[e] = (bf16)acc[i][j][e];
-                    *(bf16x4 *)((bf16 *)Cp + (size_t)m * ldc + n) = o;
-                } else if (EPI == EPI_PARTIAL) {
+                if (EPI == EPI_PARTIAL) {
                     *(f32x4 *)(g.ws + ((size_t)ks * g.ws_rows + g.moff[prob] + m) * g.N + n) = acc[i][j];
                 } else if (EPI == FLUX_HIP_EPI_F32) {
                     *(f32x4 *)((float *)Cp + (size_t)m * ldc + n) = acc[i][j];
@@ -276,7 +315,7 @@ __device__ __forceinline__ void store_tile_to(const GemmArgs &g, const TileId &t
 
 /* Cp, ldc, tn: where the tile goes - the part's output, or for the fused [Q|K|V|gate|up] projection the output of the
  * side of the boundary the tile lies on (the tile width divides nq_cols, so a tile is wholly on one side) */
-template <int BN, int WM, int WN, int EPI>
+template <int BN, int WM, int WN, int EPI, bool PINNED = false>
 __device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f32x4 (&acc)[WN / 16][WM / 16], int m0, int M,
                                            int wm, int wn, int l15, int lq, int prow) {
     if constexpr (EPI == EPI_QKV_SWIGLU) {
@@ -287,7 +326,9 @@ __device__ __forceinline__ void store_tile(const GemmArgs &g, const TileId &t, f
         if (t.tn < g.nq_tiles) store_tile_to<BN, WM, WN, FLUX_HIP_EPI_BF16, true>(g, t, acc, m0, M, wm, wn, l15, lq, prow, g.C[0], g.ldc, t.tn);
         else store_tile_to<BN, WM, WN, FLUX_HIP_EPI_SWIGLU, true>(g, t, acc, m0, M, wm, wn, l15, lq, prow, g.C2, g.ldc2, t.tn - g.nq_tiles);
     } else {
-        store_tile_to<BN, WM, WN, EPI>(g, t, acc, m0, M, wm, wn, l15, lq, prow, g.C[t.prob], g.ldc, t.tn);
+        /* PINNED: the kernels whose accumulators live in AGPRs take them out row by row as well (the 16-byte / 8-byte
+         * choice of the bf16 stores is a branch with the same conversions on both sides) */
+        store_tile_to<BN, WM, WN, EPI, PINNED>(g, t, acc, m0, M, wm, wn, l15, lq, prow, g.C[t.prob], g.ldc, t.tn);
     }
 }
 
@@ -582,7 +623,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm4w_kernel(GemmArgs g) {
          * across the K loops, beyond what the register file holds beside the accumulators and fragments. */
         int l15e = l15, lqe = lq;
         asm volatile("" : "+v"(l15e), "+v"(lqe));
-        store_tile<BN, WM, WN, EPI>(g, done, acc, done.tml * BM, g.M[done.prob], wm, wn, l15e, lqe, done.tm * WGM + wm);
+        store_tile<BN, WM, WN, EPI, true>(g, done, acc, done.tml * BM, g.M[done.prob], wm, wn, l15e, lqe, done.tm * WGM + wm);
         if (!again) break;
     }
 }
@@ -611,7 +652,8 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm4w_kernel(GemmArgs g) {
  * requested only then, with the matrix pipes idle: 12 % of a 288 x 192 x 3072 tile's time. */
 template <int EPI, int TM, int TN>
 struct EpilogueOps { /* vector memory instructions a wave issues in the epilogue of a tile whose rows are all valid */
-    static constexpr int value = EPI == FLUX_HIP_EPI_SWIGLU || EPI == EPI_QKV_SWIGLU ? TM * TN / 2 : EPI == FLUX_HIP_EPI_F32_T ? 4 * TM * TN : TM * TN;
+    static constexpr int value = EPI == FLUX_HIP_EPI_SWIGLU || EPI == EPI_QKV_SWIGLU ? TM * (TN / 4 + TN / 2 % 2) /* 16-byte stores + a last 8-byte one */
+                                 : EPI == FLUX_HIP_EPI_BF16 ? TM * TN / 2 : EPI == FLUX_HIP_EPI_F32_T ? 4 * TM * TN : TM * TN;
 };
 
 template <int TM, int TN, int EPI, int NSA, int NSW>
@@ -799,9 +841,9 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
         asm volatile("" : "+v"(l15e), "+v"(lqe));
 #if defined(GEMM_ABL_STORE_SAME)
         { TileId d2 = done; d2.tn = g.nq_tiles && done.tn >= g.nq_tiles ? g.nq_tiles : 0; d2.tm = 0; d2.tml = 0; d2.prob = 0;
-          store_tile<BN, WM, WN, EPI>(g, d2, acc, 0, g.M[0], wm, wn, l15e, lqe, wm); }
+          store_tile<BN, WM, WN, EPI, true>(g, d2, acc, 0, g.M[0], wm, wn, l15e, lqe, wm); }
 #elif !defined(GEMM_ABL_NOSTORE)
-        store_tile<BN, WM, WN, EPI>(g, done, acc, done.tml * BM, g.M[done.prob], wm, wn, l15e, lqe, done.tm * WGM + wm);
+        store_tile<BN, WM, WN, EPI, true>(g, done, acc, done.tml * BM, g.M[done.prob], wm, wn, l15e, lqe, done.tm * WGM + wm);
 #endif
         if (!again) break;
         /* not every row of this wave's part of the stored tile was valid: it issued fewer than EpilogueOps operations */

@@ -64,7 +64,7 @@ def test_reference_pipeline_runs_on_the_backend(oracle_mod, tmp_path):
 
     ctx = P.flux_load_dir(str(tmp_path).encode())
     assert ctx, P.flux_get_error()
-    width, height, steps, seed, seq = 48, 64, 3, 11, 24      # the reference's CPU VAE decodes it twice: kept small
+    width, height, steps, seed, seq = 64, 64, 3, 11, 24      # the reference's CPU VAE decodes it twice: kept small (sides are multiples of 64 there)
     lh, lw = height // 16, width // 16
     emb = normal_f32((seq, cfg.text_dim), 40, 1)
     prm = FluxParams(width, height, steps, seed, 0.0, 0, 0, 2.0)

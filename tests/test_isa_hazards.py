@@ -83,10 +83,11 @@ def kernel_bodies(asm):
             name, body = m.group(1), []
             continue
         if name:
-            body.append(line)
-            if "s_endpgm" in line:
+            if re.match(r"^\.Lfunc_end\d+:", line):     # the end of the function (a kernel may hold several s_endpgm)
                 out[name] = body
                 name = None
+            else:
+                body.append(line)
     return out
 
 
@@ -209,6 +210,16 @@ def test_gemm_kernels_fit_the_register_file(assembly):
         assert u["AGPRs"] == 4 * tm * tn, (name, u)
         if epi not in (6, 7):                    # the transformer's epilogues (the convolution ones sit at 252-256, unspilled)
             assert u["VGPRs"] <= 200, (name, u)  # room to spare: 180 at most when this was written
+
+
+def test_attention_kernels_need_no_scratch_memory(assembly):
+    """The flash kernels keep everything in registers: no scratch frame (a frame would have to be backed for every
+    launch, and an out-of-line way out once gave the wide kernels one that only a rare path touched), nothing spilled
+    to memory."""
+    usage = {k: v for k, v in resource_usage(assembly["attention.hip"][1]).items() if "attention" in k}
+    assert len(usage) >= 5, sorted(usage)
+    for name, u in sorted(usage.items()):
+        assert u["ScratchSize"] == 0 and u["VGPRs Spill"] == 0, (name, u)      # (spilled SGPRs go to lanes of a VGPR, not to memory)
 
 
 def test_the_remark_parser_reads_the_fields_the_test_uses():
