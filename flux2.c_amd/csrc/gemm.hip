@@ -448,6 +448,8 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
  * side effects keep their program order, which is what places the LDS reads and global->LDS
  * loads between the MFMAs. */
 #define MFMA_AGPR(acc, a, b) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b))
+/* the first MFMA of an accumulator block: adds to zero instead of to the register's old contents */
+#define MFMA_AGPR_NEW(acc, a, b) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(acc) : "v"(a), "v"(b))
 
 /* The compiler neither sees those MFMAs' register hazards nor keeps plain register moves in order
  * around them. acc_fence passes every accumulator through an empty asm statement that is ordered
@@ -760,23 +762,16 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
     for (;;) {
         const int KT = k_steps(t); /* at least 4: the host sends shorter K ranges to gemm4w_kernel */
 
-        f32x4 acc[TN][TM];
-#pragma unroll
-        for (int i = 0; i < TN; i++)
-#pragma unroll
-            for (int j = 0; j < TM; j++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) acc[i][j][e] = 0.0f;
-        acc_fence<TM, TN>(acc); /* the zeroes are written, and a few cycles pass, before the first MFMA reads them */
-        asm volatile("s_nop 7" ::: "memory");
+        f32x4 acc[TN][TM]; /* started by the MFMAs of step 0's first half (no pass over 4 TM TN registers to clear them) */
 
         auto serp = [](int b) { return ((b / TN) & 1) ? TN - 1 - b % TN : b % TN; };
         /* TAIL = false: steps kt + 1 .. kt + 3 belong to this tile. TAIL = true: one of the last three steps of a tile;
          * loads for steps beyond its K range request the first steps of the tile in nxt instead (every load is issued,
          * so the wait counts stay exact). WAIT: what may be in flight at the barrier. */
-        auto step = [&](int kt, auto tail_c, auto wait_c) {
+        auto step = [&](int kt, auto tail_c, auto wait_c, auto first_c) {
             constexpr bool TAIL = decltype(tail_c)::value;
             constexpr int WAIT = decltype(wait_c)::value;
+            constexpr bool FIRST = decltype(first_c)::value; /* step 0: its first half starts the accumulators */
             auto &accr = acc;
             const int na = ca == NSA - 1 ? 0 : ca + 1, nw = cw == NSW - 1 ? 0 : cw + 1;
             const unsigned van = a_frag + na * ASZ, vwn = w_frag + nw * WSZ;
@@ -791,14 +786,15 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
             };
 #pragma unroll
             for (int b = 0; b < NM; b++) {
-                MFMA_AGPR(accr[serp(b)][b / TN], f0[serp(b)], f0[TN + b / TN]);
+                if (FIRST) MFMA_AGPR_NEW(accr[serp(b)][b / TN], f0[serp(b)], f0[TN + b / TN]);
+                else MFMA_AGPR(accr[serp(b)][b / TN], f0[serp(b)], f0[TN + b / TN]);
                 if (b % RD == 0 && b / RD < NF) f1[b / RD] = frag(va, vw, coff1, b / RD);
                 /* step kt + 2 of the first operand, into the slot that step kt - 1 left */
                 if (b % SF == 1 && b / SF < LF) load(kt + 2, ca == 0 ? 2 : ca - 1, cw == 0 ? 2 : cw - 1, (FIRST_A ? 0 : LA) + b / SF);
             }
             /* step kt + 1 has landed for this wave and its reads of step kt are complete; past the barrier both hold
              * for all */
-            if (WAIT != AHEAD && strict) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AHEAD) : "memory");
+            if (FIRST && strict) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AHEAD) : "memory");
             asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(WAIT) : "memory");
 #pragma unroll
             for (int b = 0; b < NM; b++) {
@@ -814,12 +810,9 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
         };
         /* step 0: the stored tile's memory operations are older than anything its barrier needs (for the first tile
          * everything has landed already) */
-        step(0, BoolC<false>{}, IntC<AHEAD_STORES>{});
+        step(0, BoolC<false>{}, IntC<AHEAD_STORES>{}, BoolC<true>{});
         int kt = 1;
-#ifdef GEMM_ABL_RELAX
-        for (; kt < KT - 3 && kt < 6; kt++) step(kt, BoolC<false>{}, IntC<40>{});
-#endif
-        for (; kt < KT - 3; kt++) step(kt, BoolC<false>{}, IntC<AHEAD>{});
+        for (; kt < KT - 3; kt++) step(kt, BoolC<false>{}, IntC<AHEAD>{}, BoolC<false>{});
 
         /* the workgroup's next tile: its first steps are requested by this tile's last ones. After the last tile they
          * request this tile's first steps once more, into slots that nobody reads again. */
@@ -828,7 +821,7 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
         const bool again = vb < g.vgrid && decode_tile(g, vb, t);
         if (again) set_sources(nxt, t);
         else nxt = cur;
-        for (; kt < KT; kt++) step(kt, BoolC<true>{}, IntC<AHEAD>{});
+        for (; kt < KT; kt++) step(kt, BoolC<true>{}, IntC<AHEAD>{}, BoolC<false>{});
 
         asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); /* the last MFMA results retire before they are read */
         acc_fence<TM, TN>(acc);
