@@ -1296,7 +1296,7 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
     constexpr int NT = 11;
     static const int bm[NT] = {64, 128, 256, 64, 256, 288, 192, 256, 64, 128, 96}, bn[NT] = {128, 128, 256, 64, 256, 192, 192, 192, 128, 128, 128};
     static const int occ[NT] = {3, 2, 1, 4, 1, 1, 1, 1, 1, 1, 1}, ahead[NT] = {1, 1, 1, 1, 1, 1, 1, 1, 5, 4, 4}; /* stages a workgroup keeps in flight */
-    static const double rate[NT] = {2.0e12, 2.9e12, 5.3e12, 1.5e12, 4.6e12, 5.45e12, 5.1e12, 5.55e12, 1.6e12, 3.0e12, 2.4e12}; /* FLOP/s of one CU running this tile */
+    static const double rate[NT] = {2.0e12, 2.9e12, 6.05e12, 1.5e12, 4.6e12, 6.0e12, 5.7e12, 5.75e12, 1.6e12, 3.0e12, 2.4e12}; /* FLOP/s of one CU running this tile */
     const int kt_total = g.K >> 6;
     int tile = -1, best_split = 1;
     {
