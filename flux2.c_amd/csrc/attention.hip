@@ -31,7 +31,7 @@ __device__ __forceinline__ float wave16_sum(float v) {
 }
 
 /* ---------------------------------------------------------------------------------------
- * Q/K preparation. One workgroup handles 64 tokens of one head, Q and K: RMSNorm over the 128 dims *
+ * Q/K preparation. One workgroup handles 16 tokens of up to QK_HG heads, Q and K: RMSNorm over the 128 dims *
  * weight, then rotation of pairs (d, d+1) by the token's cos/sin row.
  * K is written token-major to k_out. Q is written back in place, already multiplied by
  * 1/sqrt(128) and log2(e), so that the attention kernel's scores are base-2 logits and its Q
@@ -42,11 +42,9 @@ __device__ __forceinline__ float wave16_sum(float v) {
  * --------------------------------------------------------------------------------------- */
 #define Q_FOLD (0.08838834764831845f * 1.44269504088896341f)
 /* norm * weight, RoPE and scale of one 8-dim chunk whose squared sum over the row's 16 lanes is already in ss */
-__device__ __forceinline__ bf16x8 qk_prepare_chunk(const float (&x)[8], float ss, float eps, const float *__restrict__ w, const float (&cv)[8],
+__device__ __forceinline__ bf16x8 qk_prepare_chunk(const float (&x)[8], float ss, float eps, const float (&wv)[8], const float (&cv)[8],
                                                    const float (&sv)[8], float scale) {
     const float inv = 1.0f / sqrtf(ss * (1.0f / HD) + eps);
-    f32x4 wa = *(const f32x4 *)w, wb = *(const f32x4 *)(w + 4);
-    float wv[8] = {wa[0], wa[1], wa[2], wa[3], wb[0], wb[1], wb[2], wb[3]};
     bf16x8 o;
 #pragma unroll
     for (int e = 0; e < 8; e += 2) {
@@ -56,52 +54,64 @@ __device__ __forceinline__ bf16x8 qk_prepare_chunk(const float (&x)[8], float ss
     }
     return o;
 }
+/* A thread owns one 8-dim chunk of one token (16 lanes share the token's row of a head) and walks QK_HG heads with it:
+ * the token's cos/sin chunk and the two norm weights' chunks are read once and serve every head's Q and K (read per head,
+ * as an earlier version did, the tables were 113 MB of L2 traffic per call at 4608 tokens, as much as Q and K
+ * themselves). QK_UN heads are requested before the first of them is used. */
+#define QK_HG 12
+#define QK_UN 6
 __global__ __launch_bounds__(256) void qk_prepare_kernel(bf16 *__restrict__ k_out, bf16 *qkv, int ld, int q_col, int k_col,
                                                          int rows, int heads, int split,
                                                          const float *__restrict__ q_w0, const float *__restrict__ q_w1,
                                                          const float *__restrict__ k_w0, const float *__restrict__ k_w1,
                                                          const float *__restrict__ rope_cos,
                                                          const float *__restrict__ rope_sin, float eps) {
-    const int r0 = blockIdx.x * 64, h = blockIdx.y;
     const int tid = threadIdx.x;
     const int c = tid & 15; /* 16-byte chunk of the 128-dim head row */
-    bf16 *qp = qkv + q_col + h * HD + c * 8;
-    const bf16 *kp = qkv + k_col + h * HD + c * 8;
-    bf16 *ko = k_out + h * HD + c * 8;
+    const int row = blockIdx.x * 16 + (tid >> 4), rowc = min(row, rows - 1);
+    const int h0 = blockIdx.y * QK_HG, h1 = min(h0 + QK_HG, heads);
     const int H = heads * HD;
-    int rowc[4];
-    bf16x8 qv[4], kv[4];
-    /* all rows of a thread are requested before the first is used; a row's cos/sin chunk serves its Q and its K */
+    bf16 *qp = qkv + (size_t)rowc * ld + q_col + c * 8;
+    const bf16 *kp = qkv + (size_t)rowc * ld + k_col + c * 8;
+    bf16 *ko = k_out + (size_t)rowc * H + c * 8;
+    float cv[8], sv[8], wq[8], wk[8];
+    {
+        const float *cs = rope_cos + (size_t)rowc * HD + c * 8, *sn = rope_sin + (size_t)rowc * HD + c * 8;
+        const bool first = rowc < split;
+        const float *a = (first ? q_w0 : q_w1) + c * 8, *b = (first ? k_w0 : k_w1) + c * 8;
+        const f32x4 c0 = *(const f32x4 *)cs, c1 = *(const f32x4 *)(cs + 4), s0 = *(const f32x4 *)sn, s1 = *(const f32x4 *)(sn + 4);
+        const f32x4 a0 = *(const f32x4 *)a, a1 = *(const f32x4 *)(a + 4), b0 = *(const f32x4 *)b, b1 = *(const f32x4 *)(b + 4);
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        rowc[i] = min(r0 + (tid >> 4) + i * 16, rows - 1);
-        qv[i] = *(const bf16x8 *)(qp + (size_t)rowc[i] * ld);
-        kv[i] = *(const bf16x8 *)(kp + (size_t)rowc[i] * ld);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int row = r0 + (tid >> 4) + i * 16;
-        const float *cs = rope_cos + (size_t)rowc[i] * HD + c * 8;
-        const float *sn = rope_sin + (size_t)rowc[i] * HD + c * 8;
-        f32x4 c0 = *(const f32x4 *)cs, c1 = *(const f32x4 *)(cs + 4);
-        f32x4 s0 = *(const f32x4 *)sn, s1 = *(const f32x4 *)(sn + 4);
-        float cv[8] = {c0[0], c0[1], c0[2], c0[3], c1[0], c1[1], c1[2], c1[3]};
-        float sv[8] = {s0[0], s0[1], s0[2], s0[3], s1[0], s1[1], s1[2], s1[3]};
-        float xq[8], xk[8];
-        float sq = 0.0f, sk = 0.0f;
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            xq[e] = (float)qv[i][e]; sq += xq[e] * xq[e];
-            xk[e] = (float)kv[i][e]; sk += xk[e] * xk[e];
+        for (int e = 0; e < 4; e++) {
+            cv[e] = c0[e]; cv[4 + e] = c1[e]; sv[e] = s0[e]; sv[4 + e] = s1[e];
+            wq[e] = a0[e]; wq[4 + e] = a1[e]; wk[e] = b0[e]; wk[4 + e] = b1[e];
         }
-        sq = wave16_sum(sq);
-        sk = wave16_sum(sk);
-        const bool first = rowc[i] < split;
-        const bf16x8 oq = qk_prepare_chunk(xq, sq, eps, (first ? q_w0 : q_w1) + c * 8, cv, sv, Q_FOLD);
-        const bf16x8 ok = qk_prepare_chunk(xk, sk, eps, (first ? k_w0 : k_w1) + c * 8, cv, sv, 1.0f);
-        if (row < rows) {
-            *(bf16x8 *)(qp + (size_t)row * ld) = oq;
-            *(bf16x8 *)(ko + (size_t)row * H) = ok;
+    }
+    for (int hb = h0; hb < h1; hb += QK_UN) {
+        bf16x8 qv[QK_UN], kv[QK_UN];
+#pragma unroll
+        for (int u = 0; u < QK_UN; u++) {
+            const int h = min(hb + u, h1 - 1);
+            qv[u] = *(const bf16x8 *)(qp + h * HD);
+            kv[u] = *(const bf16x8 *)(kp + h * HD);
+        }
+#pragma unroll
+        for (int u = 0; u < QK_UN; u++) {
+            float xq[8], xk[8];
+            float sq = 0.0f, sk = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                xq[e] = (float)qv[u][e]; sq += xq[e] * xq[e];
+                xk[e] = (float)kv[u][e]; sk += xk[e] * xk[e];
+            }
+            sq = wave16_sum(sq);
+            sk = wave16_sum(sk);
+            const bf16x8 oq = qk_prepare_chunk(xq, sq, eps, wq, cv, sv, Q_FOLD);
+            const bf16x8 ok = qk_prepare_chunk(xk, sk, eps, wk, cv, sv, 1.0f);
+            if (row < rows && hb + u < h1) {
+                *(bf16x8 *)(qp + (hb + u) * HD) = oq;
+                *(bf16x8 *)(ko + (hb + u) * HD) = ok;
+            }
         }
     }
 }
@@ -123,7 +133,7 @@ extern "C" int flux_hip_qk_prepare(void *k_out, void *qkv, int ld, int q_col, in
         const uintptr_t a0 = (uintptr_t)qkv, a1 = a0 + (size_t)rows * ld * 2, b0 = (uintptr_t)k_out, b1 = b0 + (size_t)rows * heads * HD * 2;
         if (a0 < b1 && b0 < a1) return flux_hip_fail("flux_hip_qk_prepare: k_out overlaps the qkv buffer");
     }
-    hipLaunchKernelGGL(qk_prepare_kernel, dim3((rows + 63) / 64, heads), dim3(256), 0, flux_hip_stream_handle(),
+    hipLaunchKernelGGL(qk_prepare_kernel, dim3((rows + 15) / 16, (heads + QK_HG - 1) / QK_HG), dim3(256), 0, flux_hip_stream_handle(),
                        (bf16 *)k_out, (bf16 *)qkv, ld, q_col, k_col, rows, heads, split, q_w0, q_w1 ? q_w1 : q_w0, k_w0, k_w1 ? k_w1 : k_w0,
                        rope_cos, rope_sin, eps);
     HIP_OK(hipGetLastError());
