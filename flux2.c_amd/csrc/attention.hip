@@ -31,7 +31,7 @@ __device__ __forceinline__ float wave16_sum(float v) {
 }
 
 /* ---------------------------------------------------------------------------------------
- * Q/K preparation. One workgroup handles 16 tokens of up to QK_HG heads, Q and K: RMSNorm over the 128 dims *
+ * Q/K preparation. One workgroup handles 16 tokens of 1 to 12 heads, Q and K: RMSNorm over the 128 dims *
  * weight, then rotation of pairs (d, d+1) by the token's cos/sin row.
  * K is written token-major to k_out. Q is written back in place, already multiplied by
  * 1/sqrt(128) and log2(e), so that the attention kernel's scores are base-2 logits and its Q
@@ -54,12 +54,12 @@ __device__ __forceinline__ bf16x8 qk_prepare_chunk(const float (&x)[8], float ss
     }
     return o;
 }
-/* A thread owns one 8-dim chunk of one token (16 lanes share the token's row of a head) and walks QK_HG heads with it:
+/* A thread owns one 8-dim chunk of one token (16 lanes share the token's row of a head) and walks HG heads with it:
  * the token's cos/sin chunk and the two norm weights' chunks are read once and serve every head's Q and K (read per head,
  * as an earlier version did, the tables were 113 MB of L2 traffic per call at 4608 tokens, as much as Q and K
- * themselves). QK_UN heads are requested before the first of them is used. */
-#define QK_HG 12
-#define QK_UN 6
+ * themselves). UN heads are requested before the first of them is used. With few tokens fewer heads per thread, so
+ * that the launch still has a few hundred workgroups. */
+template <int HG, int UN>
 __global__ __launch_bounds__(256) void qk_prepare_kernel(bf16 *__restrict__ k_out, bf16 *qkv, int ld, int q_col, int k_col,
                                                          int rows, int heads, int split,
                                                          const float *__restrict__ q_w0, const float *__restrict__ q_w1,
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(bf16 *__restrict__ k_ou
     const int tid = threadIdx.x;
     const int c = tid & 15; /* 16-byte chunk of the 128-dim head row */
     const int row = blockIdx.x * 16 + (tid >> 4), rowc = min(row, rows - 1);
-    const int h0 = blockIdx.y * QK_HG, h1 = min(h0 + QK_HG, heads);
+    const int h0 = blockIdx.y * HG, h1 = min(h0 + HG, heads);
     const int H = heads * HD;
     bf16 *qp = qkv + (size_t)rowc * ld + q_col + c * 8;
     const bf16 *kp = qkv + (size_t)rowc * ld + k_col + c * 8;
@@ -87,16 +87,16 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(bf16 *__restrict__ k_ou
             wq[e] = a0[e]; wq[4 + e] = a1[e]; wk[e] = b0[e]; wk[4 + e] = b1[e];
         }
     }
-    for (int hb = h0; hb < h1; hb += QK_UN) {
-        bf16x8 qv[QK_UN], kv[QK_UN];
+    for (int hb = h0; hb < h1; hb += UN) {
+        bf16x8 qv[UN], kv[UN];
 #pragma unroll
-        for (int u = 0; u < QK_UN; u++) {
+        for (int u = 0; u < UN; u++) {
             const int h = min(hb + u, h1 - 1);
             qv[u] = *(const bf16x8 *)(qp + h * HD);
             kv[u] = *(const bf16x8 *)(kp + h * HD);
         }
 #pragma unroll
-        for (int u = 0; u < QK_UN; u++) {
+        for (int u = 0; u < UN; u++) {
             float xq[8], xk[8];
             float sq = 0.0f, sk = 0.0f;
 #pragma unroll
@@ -133,7 +133,11 @@ extern "C" int flux_hip_qk_prepare(void *k_out, void *qkv, int ld, int q_col, in
         const uintptr_t a0 = (uintptr_t)qkv, a1 = a0 + (size_t)rows * ld * 2, b0 = (uintptr_t)k_out, b1 = b0 + (size_t)rows * heads * HD * 2;
         if (a0 < b1 && b0 < a1) return flux_hip_fail("flux_hip_qk_prepare: k_out overlaps the qkv buffer");
     }
-    hipLaunchKernelGGL(qk_prepare_kernel, dim3((rows + 15) / 16, (heads + QK_HG - 1) / QK_HG), dim3(256), 0, flux_hip_stream_handle(),
+    /* as many heads per thread as leave the launch some five hundred workgroups */
+    const int rb = (rows + 15) / 16;
+    const int hg = rb * ((heads + 11) / 12) >= 512 ? 12 : rb * ((heads + 3) / 4) >= 512 ? 4 : rb * ((heads + 1) / 2) >= 512 ? 2 : 1;
+    auto kern = hg == 12 ? qk_prepare_kernel<12, 6> : hg == 4 ? qk_prepare_kernel<4, 4> : hg == 2 ? qk_prepare_kernel<2, 2> : qk_prepare_kernel<1, 1>;
+    hipLaunchKernelGGL(kern, dim3(rb, (heads + hg - 1) / hg), dim3(256), 0, flux_hip_stream_handle(),
                        (bf16 *)k_out, (bf16 *)qkv, ld, q_col, k_col, rows, heads, split, q_w0, q_w1 ? q_w1 : q_w0, k_w0, k_w1 ? k_w1 : k_w0,
                        rope_cos, rope_sin, eps);
     HIP_OK(hipGetLastError());
