@@ -832,12 +832,7 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
          * across the K loops, beyond what the register file holds beside the accumulators and fragments. */
         int l15e = l15, lqe = lq;
         asm volatile("" : "+v"(l15e), "+v"(lqe));
-#if defined(GEMM_ABL_STORE_SAME)
-        { TileId d2 = done; d2.tn = g.nq_tiles && done.tn >= g.nq_tiles ? g.nq_tiles : 0; d2.tm = 0; d2.tml = 0; d2.prob = 0;
-          store_tile<BN, WM, WN, EPI, true>(g, d2, acc, 0, g.M[0], wm, wn, l15e, lqe, wm); }
-#elif !defined(GEMM_ABL_NOSTORE)
         store_tile<BN, WM, WN, EPI, true>(g, done, acc, done.tml * BM, g.M[done.prob], wm, wn, l15e, lqe, done.tm * WGM + wm);
-#endif
         if (!again) break;
         /* not every row of this wave's part of the stored tile was valid: it issued fewer than EpilogueOps operations */
         strict = done.tml * BM + wm * WM + WM > g.M[done.prob];
