@@ -621,6 +621,10 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
      *            the requests for chunk u's V^T fragments and, in its last eight gaps, four tile loads
      *   phase 2: row sums and O += V^T P(u)^T (9 NQ MFMAs)  with  2^S(u+1) (8 NQ exponentials) and the requests for
      *            chunk u+2's K fragments
+     * (The row sums as an MFMA against a fragment of ones cost a seventeenth of the loop's matrix time. Taken by the lanes
+     * themselves from their own eight probabilities per query, in gaps of phase 1 that carry one other instruction or
+     * none, they cost more: v_dot2c_f32_bf16 against (1, 1), four per query block and chunk, +3 % on the kernel, and even
+     * a plain addition in its place, which is not enough instructions for the sums, only -1.4 %.)
      * Vector instructions sit one or two behind each MFMA; sched_barrier keeps them there. Two score buffers
      * alternate, so one trip of the loop is one tile: an "even" step (second chunk's scores, first chunk's
      * product) and an "odd" step (next tile's first chunk's scores, second chunk's product). One barrier per
@@ -644,55 +648,44 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
      * fragments during the product phase before, its sixteen V^T half fragments during the score phase before),
      * spread over the phase in the order of their use (reads in a run cost the matrix pipe 4-5 cycles each, a read
      * every few MFMAs next to nothing): no MFMA waits for LDS. */
-    /* Per-lane LDS addresses of the fragments in the slots that are read next, kept in registers and moved on by one
-     * slot per tile (recomputed from the slot number they cost a vector add per read): the K fragments of head-dim
+    /* Per-lane LDS addresses of the fragments in slot 0 of each ring, kept in registers: the K fragments of head-dim
      * step kk, key block 0 of chunk 0 (the others lie 4096 (2 cp + i) further), and the V^T fragments of chunk 0 for
      * head-dim block x, as this lane of a transposing read sees them (the swizzle moves a block by the lane's key;
-     * chunk 1 lies 8192 further). */
+     * chunk 1 lies 8192 further). The slot is part of each read's immediate offset: the loop is written out for four
+     * tiles, one per slot (moving these twelve registers on by a slot per tile cost twelve vector additions a tile, and
+     * recomputing them from a slot number one addition per read). Only the last two tiles, whose slots depend on the
+     * number of tiles, move the registers instead (move_slots) and read with the offsets of slot 0 (K: slot 1). */
     const unsigned lds0 = (unsigned)(uintptr_t)LDS_PTR(smem); /* folded into the addresses once, not added at every read */
     unsigned ka[4], va[8];
 #pragma unroll
     for (int kk = 0; kk < 4; kk++) ka[kk] = lds0 + l15 * 256 + (((kk * 4 + lq) ^ l15) << 4);
 #pragma unroll
     for (int x = 0; x < 8; x++) va[x] = lds0 + 4 * 16384 + (8 * lq + (l15 >> 2)) * 256 + ((x ^ (l15 >> 2) ^ ((lq & 1) << 2)) << 5) + (l15 & 3) * 8;
-    auto kfrag1 = [&](int cp, int x) { /* x = 0..7: key block 2cp + x%2 of the tile, head dims 32 (x/2) .. +31 */
+    auto kfrag1 = [&](int slot, int cp, int x) { /* x = 0..7: key block 2cp + x%2 of the tile, head dims 32 (x/2) .. +31 */
         const int kk = x >> 1, i = x & 1;
-        kf[kk][i] = lds_read_bf16x8(ka[kk] + (2 * cp + i) * 4096);
+        kf[kk][i] = lds_read_bf16x8(ka[kk] + slot * 16384 + (2 * cp + i) * 4096);
     };
-    auto vhalf1 = [&](int cp, int y) { /* y = 0..15: head-dim block y / 2, keys 8 lq + 4 (y % 2) .. +3 of 32-key chunk cp */
+    auto vhalf1 = [&](int slot, int cp, int y) { /* y = 0..15: head-dim block y / 2, keys 8 lq + 4 (y % 2) .. +3 of 32-key chunk cp */
         const int x = y >> 1;
-        vh[x][y & 1] = v_half_fragment_at(va[x] + cp * 8192 + (y & 1) * 1024);
+        vh[x][y & 1] = v_half_fragment_at(va[x] + slot * 16384 + cp * 8192 + (y & 1) * 1024);
     };
     /* what a phase of 8 NQ MFMAs requests behind MFMA m: K fragment x behind MFMA x NQ, V^T half fragment y behind
      * MFMA y NQ / 2 */
-    auto k_reads_at = [&](int cp, int m) {
+    auto k_reads_at = [&](int slot, int cp, int m) {
 #pragma unroll
         for (int x = 0; x < 8; x++)
-            if (x * NQ == m) kfrag1(cp, x);
+            if (x * NQ == m) kfrag1(slot, cp, x);
     };
-    auto v_reads_at = [&](int cp, int m) {
+    auto v_reads_at = [&](int slot, int cp, int m) {
 #pragma unroll
         for (int y = 0; y < 16; y++)
-            if (y * NQ / 2 == m) vhalf1(cp, y);
+            if (y * NQ / 2 == m) vhalf1(slot, cp, y);
     };
-    auto move_slots = [&](int dk, int dv) { /* byte distances to the next K slot and the next V slot */
+    auto move_slots = [&](int dk, int dv) { /* byte distances by which the K and the V^T addresses move */
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) ka[kk] += dk;
 #pragma unroll
         for (int x = 0; x < 8; x++) va[x] += dv;
-    };
-    /* The same a few registers at a time behind the row-sum MFMAs (the only MFMAs of the loop that carry no other
-     * vector instruction; next to an exponential an addition costs the matrix pipe some nine cycles): the V addresses
-     * in the odd step, whose score phase was their last user, the K addresses in the even step after it. */
-    auto move_v_slots_at = [&](int dv, int j) {
-#pragma unroll
-        for (int x = 0; x < 8; x++)
-            if (x * NQ / 8 == j) asm volatile("v_add_u32 %0, %1, %0" : "+v"(va[x]) : "s"(dv));
-    };
-    auto move_k_slots_at = [&](int dk, int j) {
-#pragma unroll
-        for (int kk = 0; kk < 4; kk++)
-            if (kk * NQ / 4 == j) asm volatile("v_add_u32 %0, %1, %0" : "+v"(ka[kk]) : "s"(dk));
     };
     /* The vector instructions of the loop are inline assembly as well: an ordinary expression the compiler may
      * sink to its use in the next phase, and then nothing overlaps.
@@ -746,14 +739,14 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
         }
     };
     /* row sums and O^T += V^T P^T for one chunk; vh must already hold (or be receiving) the chunk's fragments.
-     * head(j) runs behind row-sum MFMA j (j = 0 .. NQ - 1), between(m) behind PV MFMA m (m = 0 .. 8 NQ - 1). */
-    auto pv_phase = [&](auto &&head, auto &&between, auto guard_c) {
+     * between(m) runs behind PV MFMA m (m = 0 .. 8 NQ - 1); the row-sum MFMAs carry nothing (starting the exponentials
+     * behind them, so that the last NQ product MFMAs carry none, changed nothing). */
+    auto pv_phase = [&](auto &&between, auto guard_c) {
         constexpr bool GUARD = decltype(guard_c)::value;
         /* the row sums are the first readers of each probability fragment */
 #pragma unroll
         for (int j = 0; j < NQ; j++) {
             MFMA_ACC_A_ONES_GUARDED(l_acc[j], ones, pf[j]);
-            head(j);
             __builtin_amdgcn_sched_barrier(0);
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -816,7 +809,7 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
     /* ---- first chunk, not pipelined: S(0) and its exact maxima ---- */
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(6 * LP) : "memory"); /* K(0) is in LDS, the other six tiles on their way */
 #pragma unroll
-    for (int x = 0; x < 8; x++) kfrag1(0, x);
+    for (int x = 0; x < 8; x++) kfrag1(0, 0, x);
     s_phase(s_a, nothing, AttFlag<true>{});
     fence_scores(s_a);
     mask_chunk(s_a, 0);
@@ -826,8 +819,7 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
 #pragma unroll
     for (int n = 0; n < 8 * NQ; n++) exp1(s_a, n);
 #pragma unroll
-    for (int x = 0; x < 8; x++) kfrag1(1, x);
-    move_slots(16384, 0); /* K fragments now come from tile 1's slot, V^T fragments from tile 0's */
+    for (int x = 0; x < 8; x++) kfrag1(0, 1, x);
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(4 * LP) : "memory"); /* V(0), K(1) are in LDS; V(1), K(2), V(2), K(3) on their way */
 
     /* The tile's eight loads, K(t+4) and V(t+3): the four of K in the last eight gaps of the odd step's score phase, the
@@ -847,66 +839,82 @@ __device__ __forceinline__ void attention_wide_body(char *smem, const int h, con
             if (m == 8 * NQ - 7 + 2 * i) next_v1(i);
         }
     };
-    /* Even step of tile t: scores of its second chunk into s_b, product of its first chunk. The K fragments of the
-     * odd step's chunk (first chunk of tile t + 1) are requested meanwhile. Only the last tile can be ragged:
-     * the check for keys beyond the end (a branch: 30 cycles with nothing to hide it) is compiled into the copies
-     * of the steps that can meet it, not into the loop. */
-    auto even_step = [&](int t, auto loads_c, auto last_c, auto guard_c) {
+    /* Even step of tile t, whose slot is sv: scores of its second chunk into s_b, product of its first chunk. The K
+     * fragments of the odd step's chunk (first chunk of tile t + 1, slot sk) are requested meanwhile, and V(t+2) into
+     * slot sl. Only the last tile can be ragged: the check for keys beyond the end (a branch: 30 cycles with nothing to
+     * hide it) is compiled into the copies of the steps that can meet it, not into the loop. */
+    auto even_step = [&](int t, int sv, int sk, int sl, auto loads_c, auto last_c, auto guard_c) {
         constexpr bool LOADS = decltype(loads_c)::value, LAST = decltype(last_c)::value;
         s_phase(s_b, [&](int m) {
-            v_reads_at(0, m);
+            v_reads_at(sv, 0, m);
             if (m >= CVT0 && m < CVT0 + 4 * NQ) cvt1(s_a, m - CVT0);
-            if (LOADS) v_loads_at((t + 2) & 3, m);
+            if (LOADS) v_loads_at(sl, m);
         }, guard_c);
         if (LAST) mask_chunk(s_b, 2 * t + 1);
-        const int dk = ((t + 1) & 3) ? 16384 : -3 * 16384; /* K fragments from tile t + 1's slot now: one slot on, or three back */
-        pv_phase([&](int j) {
-            if (LOADS) move_k_slots_at(dk, j);
-        }, [&](int m) {
-            if (!LAST) k_reads_at(0, m);
+        pv_phase([&](int m) {
+            if (!LAST) k_reads_at(sk, 0, m);
             if (m >= EXP0) exp1(s_b, m - EXP0);
         }, guard_c);
 #pragma unroll
         for (int n = 8 * NQ - EXP0; n < 8 * NQ; n++) exp1(s_b, n);
     };
-    /* Odd step of tile t: the barrier, scores of tile t+1's first chunk into s_a, product of tile t's second chunk. */
-    auto odd_step = [&](int t, auto ragged_c, auto guard_c) {
-        const int dv = ((t + 1) & 3) ? 16384 : -3 * 16384; /* V^T fragments from tile t + 1's slot after this step */
+    /* Odd step of tile t (slot sv): the barrier, scores of tile t+1's first chunk into s_a, product of tile t's second
+     * chunk; tile t+1's second chunk of K fragments (slot sk) requested meanwhile, and K(t+4) into slot sl (tile t's). */
+    auto odd_step = [&](int t, int sv, int sk, int sl, auto ragged_c, auto guard_c) {
         /* this wave's parts of K(t+2) and V(t+1) are in LDS: everything but the eight loads issued since the last barrier */
         asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * LP) : "memory");
         s_phase(s_a, [&](int m) {
-            v_reads_at(1, m);
+            v_reads_at(sv, 1, m);
             if (m >= CVT0 && m < CVT0 + 4 * NQ) cvt1(s_b, m - CVT0);
-            k_loads_at(t & 3, m);
+            k_loads_at(sl, m);
         }, guard_c);
         if (decltype(ragged_c)::value) mask_chunk(s_a, 2 * t + 2);
-        pv_phase([&](int j) { move_v_slots_at(dv, j); }, [&](int m) {
-            k_reads_at(1, m);
+        pv_phase([&](int m) {
+            k_reads_at(sk, 1, m);
             if (m >= EXP0) exp1(s_a, m - EXP0);
         }, guard_c);
 #pragma unroll
         for (int n = 8 * NQ - EXP0; n < 8 * NQ; n++) exp1(s_a, n);
     };
-    /* the last chunk: nothing left to overlap */
+    /* the last chunk (second chunk of the tile whose V^T fragments va points at): nothing left to overlap */
     auto last_step = [&]() {
 #pragma unroll
-        for (int y = 0; y < 16; y++) vhalf1(1, y);
+        for (int y = 0; y < 16; y++) vhalf1(0, 1, y);
 #pragma unroll
         for (int n = 0; n < 4 * NQ; n++) cvt1(s_b, n);
         __builtin_amdgcn_sched_barrier(0);
-        pv_phase(nothing, nothing, AttFlag<true>{});
+        pv_phase(nothing, AttFlag<true>{});
+    };
+    /* a pair of steps in the loop: tile t (slot S) finishes, tile t + 1 starts */
+    auto pair = [&](int t, auto slot_c) {
+        constexpr int S = decltype(slot_c)::value;
+        odd_step(t, S, (S + 1) & 3, S, AttFlag<false>{}, AttFlag<false>{});
+        even_step(t + 1, (S + 1) & 3, (S + 2) & 3, (S + 3) & 3, AttFlag<true>{}, AttFlag<false>{}, AttFlag<false>{});
     };
     /* (outside the loop every MFMA carries its guard, see s_phase) */
     if (ntiles == 1) {
-        even_step(0, AttFlag<false>{}, AttFlag<true>{}, AttFlag<true>{});
+        even_step(0, 0, 1, 2, AttFlag<false>{}, AttFlag<true>{}, AttFlag<true>{});
     } else {
-        even_step(0, AttFlag<false>{}, AttFlag<false>{}, AttFlag<true>{});
-        for (int t = 0; t < ntiles - 2; t++) {
-            odd_step(t, AttFlag<false>{}, AttFlag<false>{});
-            even_step(t + 1, AttFlag<true>{}, AttFlag<false>{}, AttFlag<false>{});
+        even_step(0, 0, 1, 2, AttFlag<false>{}, AttFlag<false>{}, AttFlag<true>{});
+        int t = 0;
+        for (; t + 4 <= ntiles - 2; t += 4) {
+            pair(t, AttInt<0>{});
+            pair(t + 1, AttInt<1>{});
+            pair(t + 2, AttInt<2>{});
+            pair(t + 3, AttInt<3>{});
         }
-        odd_step(ntiles - 2, AttFlag<true>{}, AttFlag<true>{});
-        even_step(ntiles - 1, AttFlag<false>{}, AttFlag<true>{}, AttFlag<true>{});
+        /* t is a multiple of four; up to three pairs are left before the last one */
+        if (t < ntiles - 2) pair(t, AttInt<0>{});
+        if (t + 1 < ntiles - 2) pair(t + 1, AttInt<1>{});
+        if (t + 2 < ntiles - 2) pair(t + 2, AttInt<2>{});
+        /* The last two tiles: their slots depend on the number of tiles, so the address registers move instead: V^T
+         * fragments of tile ntiles - 2 at slot offset 0, K fragments of tile ntiles - 1 at slot offset 1. The odd step's
+         * loads go where nobody reads any more (beyond the last tile the loaders fetch its last row again). */
+        const int sv = (ntiles - 2) & 3, sk = (ntiles - 1) & 3;
+        move_slots((sk - 1) * 16384, sv * 16384);
+        odd_step(ntiles - 2, 0, 1, sv, AttFlag<true>{}, AttFlag<true>{});
+        move_slots(0, (sk - sv) * 16384);
+        even_step(ntiles - 1, 0, 1, 2, AttFlag<false>{}, AttFlag<true>{}, AttFlag<true>{});
     }
     last_step();
     __builtin_amdgcn_s_waitcnt(0x0F70); /* no load into LDS is left in flight */

@@ -468,7 +468,10 @@ def _attention_case(hip, oracle_mod, n, split, heads, seed, qk_scale=1.0, qkv=No
     return got[:, :H], want
 
 
-@pytest.mark.parametrize("n,split,heads", [(1, 0, 1), (64, 64, 2), (80, 64, 2), (191, 50, 3), (333, 128, 2), (768, 512, 2)])
+# (the key loop is written out for four tiles of 64 keys, with up to three more pairs of steps behind it: 300, 440 and 1100 keys
+# are 5, 7 and 18 tiles, i.e. three, one and no pairs left over; the others leave none or two)
+@pytest.mark.parametrize("n,split,heads", [(1, 0, 1), (64, 64, 2), (80, 64, 2), (191, 50, 3), (300, 100, 2), (333, 128, 2), (440, 128, 2),
+                                           (768, 512, 2), (1100, 512, 2)])
 def test_attention(hip, oracle_mod, n, split, heads):
     got, want = _attention_case(hip, oracle_mod, n, split, heads, 8)
     # q, k, p are rounded to bf16 inside the kernel and the output is bf16
