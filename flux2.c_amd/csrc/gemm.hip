@@ -165,6 +165,13 @@ __device__ __forceinline__ bool decode_tile(const GemmArgs &g, int vb, TileId &t
  * results of the two blocks are eight consecutive features: one 16-byte store, 64 bytes per output row and
  * instruction, half as many store instructions and write requests. Only the weight rows a block reads change. */
 __device__ __forceinline__ int bf16_pair_feature(int blk, int r) { return 32 * (blk >> 1) + 8 * (r >> 2) + 4 * (blk & 1) + (r & 3); }
+/* the same for a wave that owns TN blocks: with TN odd the last block has no neighbour and keeps the plain numbering */
+template <int TN>
+__device__ __forceinline__ int bf16_feature(int blk, int r) { return blk < (TN & ~1) ? bf16_pair_feature(blk, r) : 16 * blk + r; }
+/* Tile widths that divide none of the model's matrix widths (224: 3072 = 13 x 224 + 160, 9216 = 41 x 224 + 32): the
+ * last column tile is cut off. Its missing weight rows are read from the matrix's last row and its missing columns are
+ * not stored (whole 16-column blocks for fp32 outputs, whole pairs of blocks for bf16: N is a multiple of 32). */
+template <int BN> struct CutTile { static constexpr bool value = BN % 64 != 0; };
 /* SiLU(gate) * up: blocks alternate gate, up, so that a lane holds matching pairs; the (gate, up) pairs interleave
  * two by two in the same way, and a last odd pair keeps the plain numbering (features 16 k + r). */
 template <int TN>
@@ -183,8 +190,11 @@ __device__ __forceinline__ int weight_row(const GemmArgs &g, int tn, int v) {
         if (EPI == EPI_QKV_SWIGLU) return ((blk & 1) ? g.w_row2 : g.w_row1) + (tn - g.nq_tiles) * (BN / 2) + idx;
         return ((blk & 1) ? g.w_row1 : g.w_row0) + tn * (BN / 2) + idx;
     }
-    if (EPI == FLUX_HIP_EPI_BF16 || EPI == EPI_QKV_SWIGLU) return g.w_row0 + tn * BN + wv * WN + bf16_pair_feature(blk, r);
-    return g.w_row0 + tn * BN + v;
+    int col;
+    if (EPI == FLUX_HIP_EPI_BF16 || EPI == EPI_QKV_SWIGLU) col = tn * BN + wv * WN + bf16_feature<TN>(blk, r);
+    else col = tn * BN + v;
+    if (CutTile<BN>::value) col = min(col, g.N - 1);
+    return g.w_row0 + col;
 }
 
 /* eight bf16 to consecutive addresses: one 16-byte store where the address allows it, else two of 8 bytes */
@@ -200,6 +210,9 @@ __device__ __forceinline__ void store_bf16x8(bf16 *p, bf16x4 lo, bf16x4 hi, bool
     }
 }
 
+template <bool V> struct BoolC { static constexpr bool value = V; };
+template <int V> struct IntC { static constexpr int value = V; };
+
 /* Accumulator element e of block (i, j): feature n = 4*(lane/16) + e of the 16-column block,
  * token m = lane%16 of the 16-row block. */
 template <int BN, int WM, int WN, int EPI, bool HERE = false>
@@ -210,6 +223,58 @@ __device__ __forceinline__ void store_tile_to(const GemmArgs &g, const TileId &t
     const bool aligned16 = (((uintptr_t)Cp | ((uintptr_t)ldc << 1)) & 15) == 0; /* every 8-feature group of the output starts on 16 bytes */
     f32x4 acc_here[HERE ? TN : 1][HERE ? TM : 1];
     auto &acc = [&]() -> auto & { if constexpr (HERE) return acc_here; else return acc_in; }();
+    if constexpr (EPI == FLUX_HIP_EPI_RESID && HERE) {
+        /* x += gate * acc on the fp32 residual: a read, and a write that depends on it. Row block by row block in
+         * program order that is a chain of round trips to memory (request a row's values, wait, store; the wait
+         * counter also holds the stores of the row before, so every wait is for those as well): nine such chains made
+         * up most of the 57 us that this epilogue cost a 288 x 192 x 12288 tile's launch of 261 us. Here the values of
+         * row block j + 1 are requested before row block j is touched: the wait for block j's values leaves the block
+         * before's stores and the next block's loads in flight. Rows beyond M read the last row (no branch around the
+         * loads) and store nothing; a wave whose rows are all valid runs a copy without that test, i.e. without
+         * branches (behind a skipped store the compiler must assume that the loads in front of it are still under
+         * way, and it waits for them before it reuses their registers: one row block in flight instead of two). */
+        const auto cut = [&](int i) { return CutTile<BN>::value && n0 + wn * WN + i * 16 >= g.N; }; /* the same for the whole wave */
+        /* the unit that is requested ahead: a row block's TN column blocks, or half of them where the accumulators fill the
+         * AGPRs and the fragments most of the VGPRs (256 x 256) */
+        constexpr int UN = TM * TN * 4 > 224 && TN % 2 == 0 ? TN / 2 : TN, UPR = TN / UN, NU = TM * UPR;
+        f32x4 gt[TN], xb[2][UN];
+#pragma unroll
+        for (int i = 0; i < TN; i++)
+            if (!cut(i)) gt[i] = *(const f32x4 *)(g.gate[prob] + n0 + wn * WN + i * 16 + lq * 4);
+        const auto fetch = [&](int u) {
+            const int j = u / UPR, i0 = u % UPR * UN;
+            const float *p = (const float *)Cp + (size_t)min(m0 + wm * WM + j * 16 + l15, M - 1) * ldc + n0 + wn * WN + lq * 4;
+#pragma unroll
+            for (int i = 0; i < UN; i++)
+                if (!cut(i0 + i)) xb[u & 1][i] = *(const f32x4 *)(p + (i0 + i) * 16);
+        };
+        const auto rows = [&](auto full_c) {
+            fetch(0);
+#pragma unroll
+            for (int u = 0; u < NU; u++) {
+                const int j = u / UPR, i0 = u % UPR * UN;
+                if (u + 1 < NU) fetch(u + 1);
+#pragma unroll
+                for (int i = 0; i < UN; i++) {
+                    acc[i0 + i][j] = acc_in[i0 + i][j];
+                    asm volatile("" : "+v"(acc[i0 + i][j]));
+                }
+                const int m = m0 + wm * WM + j * 16 + l15;
+                float *p = (float *)Cp + (size_t)m * ldc + n0 + wn * WN + lq * 4;
+#pragma unroll
+                for (int i = 0; i < UN; i++) {
+                    if (cut(i0 + i)) continue;
+                    f32x4 x = xb[u & 1][i];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) x[e] += gt[i0 + i][e] * acc[i0 + i][j][e];
+                    if (decltype(full_c)::value || m < M) *(f32x4 *)(p + (i0 + i) * 16) = x;
+                }
+            }
+        };
+        if (m0 + wm * WM + WM <= M) rows(BoolC<true>{});
+        else rows(BoolC<false>{});
+        return;
+    }
     float st_s[TN], st_q[TN]; /* convolutions with statistics: this lane's sums per 16-column block */
 #pragma unroll
     for (int i = 0; i < TN; i++) st_s[i] = st_q[i] = 0.0f;
@@ -242,18 +307,25 @@ __device__ __forceinline__ void store_tile_to(const GemmArgs &g, const TileId &t
             if (TN / 2 % 2) *(bf16x4 *)(C + 16 * (TN / 2 - 1) + 4 * lq) = o[TN / 2 - 1];
         } else if (EPI == FLUX_HIP_EPI_BF16) {
             /* see bf16_pair_feature: blocks 2p and 2p + 1 give eight consecutive features */
-            static_assert(EPI != FLUX_HIP_EPI_BF16 || TN % 2 == 0, "bf16 outputs pair 16-column blocks");
             bf16 *C = (bf16 *)Cp + (size_t)m * ldc + n0 + wn * WN + 8 * lq;
 #pragma unroll
             for (int p = 0; p < TN / 2; p++) {
+                if (CutTile<BN>::value && n0 + wn * WN + 32 * p >= g.N) continue; /* the same for the whole wave */
                 bf16x4 lo, hi;
 #pragma unroll
                 for (int e = 0; e < 4; e++) { lo[e] = (bf16)acc[2 * p][j][e]; hi[e] = (bf16)acc[2 * p + 1][j][e]; }
                 store_bf16x8(C + 32 * p, lo, hi, aligned16);
             }
+            if (TN % 2 && !(CutTile<BN>::value && n0 + wn * WN + 16 * (TN - 1) >= g.N)) { /* a last block without a neighbour */
+                bf16x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; e++) o[e] = (bf16)acc[TN - 1][j][e];
+                *(bf16x4 *)((bf16 *)Cp + (size_t)m * ldc + n0 + wn * WN + 16 * (TN - 1) + 4 * lq) = o;
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < TN; i++) {
+                if (CutTile<BN>::value && n0 + wn * WN + i * 16 >= g.N) continue; /* the same for the whole wave */
                 const int n = n0 + wn * WN + i * 16 + lq * 4;
                 if (EPI == EPI_PARTIAL) {
                     *(f32x4 *)(g.ws + ((size_t)ks * g.ws_rows + g.moff[prob] + m) * g.N + n) = acc[i][j];
@@ -457,10 +529,13 @@ __global__ __launch_bounds__(WGM *WGN * 64) void gemm_kernel(GemmArgs g) {
  * Idle cycles for the hazards are placed explicitly next to it. */
 template <int TM, int TN>
 __device__ __forceinline__ void acc_fence(f32x4 (&acc)[TN][TM]) {
-    static_assert(TN == 8 || TN == 6 || TN == 4, "one asm statement per accumulator column");
+    static_assert(TN == 8 || TN == 7 || TN == 6 || TN == 4, "one asm statement per accumulator column");
 #pragma unroll
     for (int j = 0; j < TM; j++) {
-        if constexpr (TN == 8)
+        if constexpr (TN == 7)
+            asm volatile("" : "+a"(acc[0][j]), "+a"(acc[1][j]), "+a"(acc[2][j]), "+a"(acc[3][j]),
+                              "+a"(acc[4][j]), "+a"(acc[5][j]), "+a"(acc[6][j]));
+        else if constexpr (TN == 8)
             asm volatile("" : "+a"(acc[0][j]), "+a"(acc[1][j]), "+a"(acc[2][j]), "+a"(acc[3][j]),
                               "+a"(acc[4][j]), "+a"(acc[5][j]), "+a"(acc[6][j]), "+a"(acc[7][j]));
         else if constexpr (TN == 6)
@@ -471,8 +546,6 @@ __device__ __forceinline__ void acc_fence(f32x4 (&acc)[TN][TM]) {
     }
 }
 
-template <bool V> struct BoolC { static constexpr bool value = V; };
-template <int V> struct IntC { static constexpr int value = V; };
 /* whether a workgroup of gemm4w_kernel goes on to further tiles (the 4-wave form of the transformer's epilogues;
  * with the convolution epilogues the values kept across tiles would spill) */
 template <int EPI, int WAVES> struct Walks4w { static constexpr bool value = !IsConv<EPI>::value && WAVES == 4; };
@@ -655,7 +728,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm4w_kernel(GemmArgs g) {
 template <int EPI, int TM, int TN>
 struct EpilogueOps { /* vector memory instructions a wave issues in the epilogue of a tile whose rows are all valid */
     static constexpr int value = EPI == FLUX_HIP_EPI_SWIGLU || EPI == EPI_QKV_SWIGLU ? TM * (TN / 4 + TN / 2 % 2) /* 16-byte stores + a last 8-byte one */
-                                 : EPI == FLUX_HIP_EPI_BF16 ? TM * TN / 2 : EPI == FLUX_HIP_EPI_F32_T ? 4 * TM * TN : TM * TN;
+                                 : EPI == FLUX_HIP_EPI_BF16 ? TM * (TN / 2 + TN % 2) : EPI == FLUX_HIP_EPI_F32_T ? 4 * TM * TN : TM * TN;
 };
 
 template <int TM, int TN, int EPI, int NSA, int NSW>
@@ -834,8 +907,9 @@ __global__ __launch_bounds__(256) void gemm4d_kernel(GemmArgs g) {
         asm volatile("" : "+v"(l15e), "+v"(lqe));
         store_tile<BN, WM, WN, EPI, true>(g, done, acc, done.tml * BM, g.M[done.prob], wm, wn, l15e, lqe, done.tm * WGM + wm);
         if (!again) break;
-        /* not every row of this wave's part of the stored tile was valid: it issued fewer than EpilogueOps operations */
-        strict = done.tml * BM + wm * WM + WM > g.M[done.prob];
+        /* not every row of this wave's part of the stored tile was valid, or not every column: it issued fewer than
+         * EpilogueOps operations */
+        strict = done.tml * BM + wm * WM + WM > g.M[done.prob] || (CutTile<BN>::value && done.tn == g.ntiles - 1);
         cur = nxt;
     }
     /* the requests made in place of a next tile's land in this workgroup's LDS: not after it has gone */
@@ -925,7 +999,7 @@ static int launch_4d(GemmArgs &g) {
         attr_done = true;
     }
     set_row_tiles(g, BM);
-    g.ntiles = g.N / BN;
+    g.ntiles = (g.N + BN - 1) / BN; /* (a last tile that is cut off: CutTile) */
     g.nq_tiles = g.nq_cols / BN;
     g.total_tiles = g.mtiles * g.ntiles;
     size_t span = ((size_t)max(max(g.w_row0, g.w_row1), g.w_row2) + g.N) * g.ldw * 2;
@@ -952,9 +1026,13 @@ static int launch_epi(GemmArgs &g, int tile) {
             case 5: return launch_4d<9, 6, EPI, 2, 3>(g);
             case 6: return launch_4d<6, 6, EPI, 3, 3>(g);
             case 7: return launch_4d<8, 6, EPI, 2, 3>(g);
+            case 11:
+                if constexpr (EPI == FLUX_HIP_EPI_RESID || EPI == FLUX_HIP_EPI_BF16) return launch_4d<8, 7, EPI, 2, 3>(g);
+                break;
             default: break;
         }
     }
+    if (tile == 11) tile = g.N % 256 == 0 ? 2 : 1; /* (the dispatch offers 256 x 224 only where the ring kernel takes it) */
     switch (tile) {
         case 2: return launch_4w<8, 8, EPI>(g);
         case 5: return launch_4w<9, 6, EPI>(g);
@@ -1210,10 +1288,10 @@ extern "C" void flux_hip_linear_release(void) {
 }
 
 static int g_force_tile = -1;
-static unsigned g_tile_mask = 0x7EF; /* tiles the automatic choice may use: all but the 8-wave form of 256 x 256 */
+static unsigned g_tile_mask = 0xFEF; /* tiles the automatic choice may use: all but the 8-wave form of 256 x 256 */
 static int g_splitk_enabled = 1;
 extern "C" void flux_hip_linear_force_tile(int tile) { g_force_tile = tile; }
-extern "C" void flux_hip_linear_tile_mask(unsigned mask) { g_tile_mask = mask ? mask : 0x7EF; }
+extern "C" void flux_hip_linear_tile_mask(unsigned mask) { g_tile_mask = mask ? mask : 0xFEF; }
 extern "C" void flux_hip_linear_enable_splitk(int on) { g_splitk_enabled = on; }
 static int g_force_split = 0; /* > 1: every projection that can run as K slices runs as this many (comparison runs and tests) */
 extern "C" void flux_hip_linear_force_split(int slices) { g_force_split = slices > 1 ? slices : 0; }
@@ -1287,11 +1365,12 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
     /* tile ids: 0..3 the small tiles and 256 x 256, 4 = the 8-wave form of 256 x 256 (only when
      * forced, for comparison runs), 5 = 288 x 192, 6 = 192 x 192, 7 = 256 x 192, 8, 9 and 10 = 64 x 128, 128 x 128 and
      * 96 x 128 with a ring of 6, 5 and 5 stages instead of 2 (one workgroup per compute unit; for parts of at most that
-     * many rows) */
-    constexpr int NT = 11;
-    static const int bm[NT] = {64, 128, 256, 64, 256, 288, 192, 256, 64, 128, 96}, bn[NT] = {128, 128, 256, 64, 256, 192, 192, 192, 128, 128, 128};
-    static const int occ[NT] = {3, 2, 1, 4, 1, 1, 1, 1, 1, 1, 1}, ahead[NT] = {1, 1, 1, 1, 1, 1, 1, 1, 5, 4, 4}; /* stages a workgroup keeps in flight */
-    static const double rate[NT] = {2.0e12, 2.9e12, 6.05e12, 1.5e12, 4.6e12, 6.0e12, 5.7e12, 5.75e12, 1.6e12, 3.0e12, 2.4e12}; /* FLOP/s of one CU running this tile */
+     * many rows), 11 = 256 x 224 (4096 + 512 rows x 3072 columns are 252 such tiles, one round of workgroups on 256
+     * compute units of which each does 7/8 of a 256 x 256 tile's work; 216 tiles of 256 x 256 are one round as well) */
+    constexpr int NT = 12;
+    static const int bm[NT] = {64, 128, 256, 64, 256, 288, 192, 256, 64, 128, 96, 256}, bn[NT] = {128, 128, 256, 64, 256, 192, 192, 192, 128, 128, 128, 224};
+    static const int occ[NT] = {3, 2, 1, 4, 1, 1, 1, 1, 1, 1, 1, 1}, ahead[NT] = {1, 1, 1, 1, 1, 1, 1, 1, 5, 4, 4, 1}; /* stages a workgroup keeps in flight */
+    static const double rate[NT] = {2.0e12, 2.9e12, 6.05e12, 1.5e12, 4.6e12, 6.0e12, 5.7e12, 5.75e12, 1.6e12, 3.0e12, 2.4e12, 5.9e12}; /* FLOP/s of one CU running this tile */
     const int kt_total = g.K >> 6;
     int tile = -1, best_split = 1;
     {
@@ -1306,7 +1385,13 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
         double rows = 0.0;
         for (int i = 0; i < np; i++) rows += g.M[i];
         for (int t = 0; t < NT; t++) {
-            if (N % bn[t] || g.nq_cols % bn[t]) continue;
+            /* 256 x 224 (tile 11) divides no width and cuts its last column tile off: for the outputs whose stores can do
+             * that, through the ring kernel only, never in K slices */
+            const bool cut = t == 11;
+            if (cut && !((epilogue == FLUX_HIP_EPI_RESID || epilogue == FLUX_HIP_EPI_BF16) && g_ring && g_persistent && kt_total >= 4)) continue;
+            /* bf16 outputs leave in pairs of 16-column blocks: the cut must fall between two pairs of a wave's 112 columns */
+            if (cut && epilogue == FLUX_HIP_EPI_BF16 && (N % 224) % 112 % 32 != 0) continue;
+            if (!cut && (N % bn[t] || g.nq_cols % bn[t])) continue;
             if (!((allowed >> t) & 1)) continue;
             if (ahead[t] > 1) { /* the deep rings stream the weights once: every part in one row tile */
                 bool fits = true;
@@ -1315,10 +1400,10 @@ static int gemm_dispatch(GemmArgs &g, int np, int epilogue, unsigned allowed, in
             }
             long tiles = 0;
             for (int i = 0; i < np; i++) tiles += (g.M[i] + bm[t] - 1) / bm[t];
-            tiles *= N / bn[t];
+            tiles *= (N + bn[t] - 1) / bn[t];
             for (int si = 0; si < 10; si++) {
                 const int sp = splits[si];
-                if (sp > 1 && (!can_split || kt_total / sp < 4)) break;
+                if (sp > 1 && (cut || !can_split || kt_total / sp < 4)) break;
                 if (g_force_split && can_split && sp != g_force_split && kt_total / g_force_split >= 4) continue;
                 if (sp > 1 && fixed_ws && (double)sp * rows * N * sizeof(float) > (double)fixed_ws_bytes) {
                     /* the slices must fit the given workspace: fewer slices then, down to none - unless this number
@@ -1440,7 +1525,7 @@ static int linear_impl(int epilogue, int nparts, const flux_hip_linear_part *par
     g.N = N; g.K = K; g.lda = lda; g.ldw = ldw; g.ldc = ldc; g.w_row0 = w_row0; g.w_row1 = w_row1;
     a.ldo = N;
     a.eps = eps;
-    return gemm_dispatch(g, np, epilogue, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0x7FFu, nullptr, norm ? &a : nullptr, fused,
+    return gemm_dispatch(g, np, epilogue, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0xFFFu, nullptr, norm ? &a : nullptr, fused,
                          fixed_ws, fixed_ws_bytes);
 }
 
@@ -1468,7 +1553,7 @@ extern "C" int flux_hip_linear_qkv_swiglu(const void *A, const void *W, void *qk
     int tile = -1;
     const int saved = g_splitk_enabled;
     g_splitk_enabled = 0;
-    const int ok = gemm_dispatch(g, 1, EPI_QKV_SWIGLU, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0x7FFu, &tile);
+    const int ok = gemm_dispatch(g, 1, EPI_QKV_SWIGLU, (g_force_tile >= 0 ? 1u << g_force_tile : g_tile_mask) & 0xFFFu, &tile);
     g_splitk_enabled = saved;
     return ok;
 }

@@ -95,6 +95,61 @@ def test_linear_swiglu(hip, oracle_mod, tile):
     assert not got[:, :64].any() and not got[:, 64 + mlp:].any()   # nothing written outside
 
 
+@pytest.mark.parametrize("N", [640, 768, 896, 1152])
+@pytest.mark.parametrize("K", [256, 448])
+def test_linear_tile_with_cut_last_column_tile(hip, oracle_mod, N, K):
+    """256 x 224 (tile 11) divides none of these widths: the last column tile ends after 192, 96, 224 and 32 columns (in
+    the second wave's columns, inside the first wave's, nowhere, inside the first pair of blocks). Gated residual
+    epilogue on two row ranges, and the bf16 store where its pairs of 16-column blocks allow the cut (not at 640):
+    against the oracle, and bit for bit against the 128 x 128 tile, which accumulates in the same order."""
+    L = hip.lib()
+    M0, M1 = 300, 70
+    a = q(normal_f32((M0 + M1, K), 41, 1))
+    W0 = q(normal_f32((N, K), 41, 2, 0.0, 0.1))
+    W1 = q(normal_f32((N, K), 41, 3, 0.0, 0.1))
+    res = normal_f32((M0 + M1, N), 41, 4)
+    g0, g1 = normal_f32((N,), 41, 5), normal_f32((N,), 41, 6)
+    want = res.copy()
+    want[:M0] += g0 * oracle_mod.linear(a[:M0], W0)
+    want[M0:] += g1 * oracle_mod.linear(a[M0:], W1)
+    da, dW0, dW1 = dev_bf16(hip, a), dev_bf16(hip, W0), dev_bf16(hip, W1)
+    dg0, dg1 = hip.DevBuf.from_array(g0), hip.DevBuf.from_array(g1)
+    got = {}
+    for tile in (11, 1):
+        L.flux_hip_linear_force_tile(tile)
+        L.flux_hip_linear_probe(hip.EPI_RESID)
+        # (a guard row behind the output: nothing may be written past the last column)
+        dres = hip.DevBuf.from_array(np.concatenate([res, np.full((1, N), 7.0, np.float32)]))
+        hip.linear(hip.EPI_RESID, [(da.ptr, dW0.ptr, dres.ptr, dg0.ptr, M0), (da.at(M0 * K * 2), dW1.ptr, dres.at(M0 * N * 4), dg1.ptr, M1)],
+                   N, K, K, K, N)
+        tiles = np.zeros(4, np.int32)
+        assert L.flux_hip_linear_probe_read_launches(4, tiles.ctypes.data, None) == 1 and tiles[0] == tile
+        full = dres.to_array(np.float32, (M0 + M1 + 1, N))
+        assert (full[-1] == 7.0).all()
+        got[tile] = full[:-1]
+    assert rel_l2(got[11], want) < 2e-6
+    assert np.array_equal(got[11], got[1])
+    # bf16 output with a row stride wider than N: the columns behind N stay as they were
+    ldc = N + 64
+    x = a[:M0]
+    want16 = oracle_mod.linear(x, W0)
+    out = {}
+    for tile in (11, 1):
+        L.flux_hip_linear_force_tile(tile)
+        L.flux_hip_linear_probe(hip.EPI_BF16)
+        dout = hip.DevBuf.from_array(np.full((M0, ldc), 0x4242, np.uint16))
+        hip.linear(hip.EPI_BF16, [(da.ptr, dW0.ptr, dout.ptr, None, M0)], N, K, K, K, ldc, 0, 0)
+        tiles = np.zeros(4, np.int32)
+        assert L.flux_hip_linear_probe_read_launches(4, tiles.ctypes.data, None) == 1
+        assert tiles[0] == (tile if tile == 1 or (N % 224) % 112 % 32 == 0 else 1)   # refused where a pair would be cut in two
+        out[tile] = dout.to_array(np.uint16, (M0, ldc))
+        assert (out[tile][:, N:] == 0x4242).all()
+    assert np.array_equal(out[11], out[1])
+    assert rel_l2(bf16_to_f32(out[11][:, :N]), want16) < 4e-3
+    L.flux_hip_linear_probe(-1)
+    L.flux_hip_linear_force_tile(-1)
+
+
 @pytest.mark.parametrize("tile", [2, 5, 6, 7])
 @pytest.mark.parametrize("K", [64, 128, 192, 256, 448])
 def test_linear_large_tile_k_steps(hip, oracle_mod, K, tile):

@@ -191,12 +191,28 @@ def resource_usage(remarks):
     return out
 
 
+def innermost_loops(body):
+    """(first line, last line) of every loop of the kernel that holds no other loop: label ... backward branch to it."""
+    labels = {}
+    for ln, line in enumerate(body):
+        m = re.match(r"^(\.LBB\d+_\d+):", line)
+        if m:
+            labels[m.group(1)] = ln
+    loops = []
+    for ln, line in enumerate(body):
+        m = re.search(r"\bs_c?branch\w*\s+(\.LBB\d+_\d+)", line)
+        if m and labels.get(m.group(1), len(body)) < ln:
+            loops.append((labels[m.group(1)], ln))
+    return [(a, b) for a, b in loops if not any((c, d) != (a, b) and a <= c and d <= b for c, d in loops)]
+
+
 def test_gemm_kernels_fit_the_register_file(assembly):
     """No GEMM kernel may spill: a spilled register is a scratch store next to the next tile's primed loads (the
     compiler waits for all of them first), and the fused [Q|K|V|gate|up] epilogue went over the ceiling that way
-    before its two store bodies were kept apart. Every kernel of gemm.hip: no scratch frame, no spilled VGPR or SGPR;
-    the 4-wave kernels keep their accumulators in AGPRs and nothing else (AGPRs == 16 TM TN / 4 means that no
-    vector register was parked there either)."""
+    before its two store bodies were kept apart. Every kernel of gemm.hip: no scratch frame, no spilled VGPR or SGPR.
+    The 4-wave kernels keep their accumulators in AGPRs (at least 16 TM TN / 4 of them) and their K loops free of
+    copies between the two register files; outside the loops the residual epilogue, which keeps two row blocks of
+    the residual in flight, may park a few values in spare AGPRs. The other transformer epilogues stay under 200 VGPRs."""
     usage = resource_usage(assembly["gemm.hip"][1])
     big = {k: v for k, v in usage.items() if "gemm4d_kernel" in k or "gemm4w_kernel" in k}
     assert len(big) >= 60 and len(usage) >= 100, (len(big), len(usage))
@@ -205,11 +221,25 @@ def test_gemm_kernels_fit_the_register_file(assembly):
         if u["ScratchSize"] or u["VGPRs Spill"] or u["SGPRs Spill"]:
             bad.append((name, u))
     assert not bad, bad
+    bodies = kernel_bodies(assembly["gemm.hip"][0])
     for name, u in sorted(big.items()):
         tm, tn, epi = map(int, re.search(r"kernelILi(\d+)ELi(\d+)ELi(\d+)E", name).groups())
-        assert u["AGPRs"] == 4 * tm * tn, (name, u)
-        if epi not in (6, 7):                    # the transformer's epilogues (the convolution ones sit at 252-256, unspilled)
+        assert 4 * tm * tn <= u["AGPRs"] <= 4 * tm * tn + (8 if epi == 3 else 0), (name, u)
+        if epi not in (3, 6, 7):                 # (the convolution epilogues sit at 252-256, unspilled; the residual one at up to 256)
             assert u["VGPRs"] <= 200, (name, u)  # room to spare: 180 at most when this was written
+        body = bodies[name]
+        k_loops = [(a, b) for a, b in innermost_loops(body) if sum("v_mfma" in l for l in body[a:b]) >= 2 * tm * tn]
+        assert k_loops, name
+        for a, b in k_loops:
+            copies = [l.strip() for l in body[a:b] if "v_accvgpr" in l or "scratch_" in l]
+            assert not copies, (name, copies[:4])
+
+
+def test_the_loop_finder_sees_a_planted_copy():
+    body = [".LBB0_1:", "\tv_mfma_f32_16x16x32_bf16 a[0:3], v[4:7], v[8:11], a[0:3]", ".LBB0_2:", "\tv_accvgpr_read_b32 v1, a9",
+            "\tv_mfma_f32_16x16x32_bf16 a[0:3], v[4:7], v[8:11], a[0:3]", "\ts_cbranch_scc1 .LBB0_2", "\ts_cbranch_vccnz .LBB0_1", "\ts_endpgm"]
+    assert innermost_loops(body) == [(2, 5)]
+    assert any("v_accvgpr" in l for l in body[2:5])
 
 
 def test_attention_kernels_need_no_scratch_memory(assembly):
