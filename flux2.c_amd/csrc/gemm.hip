@@ -237,7 +237,8 @@ __device__ __forceinline__ void store_tile_to(const GemmArgs &g, const TileId &t
         /* the unit that is requested ahead: a row block's TN column blocks, or half of them where the accumulators fill the
          * AGPRs and the fragments most of the VGPRs (256 x 256) */
         constexpr int UN = TM * TN * 4 > 224 && TN % 2 == 0 ? TN / 2 : TN, UPR = TN / UN, NU = TM * UPR;
-        f32x4 gt[TN], xb[2][UN];
+        constexpr int NB = 2; /* units in flight, the one being stored included (a third one measured no different: what is left is the burst itself) */
+        f32x4 gt[TN], xb[NB][UN];
 #pragma unroll
         for (int i = 0; i < TN; i++)
             if (!cut(i)) gt[i] = *(const f32x4 *)(g.gate[prob] + n0 + wn * WN + i * 16 + lq * 4);
@@ -246,27 +247,25 @@ __device__ __forceinline__ void store_tile_to(const GemmArgs &g, const TileId &t
             const float *p = (const float *)Cp + (size_t)min(m0 + wm * WM + j * 16 + l15, M - 1) * ldc + n0 + wn * WN + lq * 4;
 #pragma unroll
             for (int i = 0; i < UN; i++)
-                if (!cut(i0 + i)) xb[u & 1][i] = *(const f32x4 *)(p + (i0 + i) * 16);
+                if (!cut(i0 + i)) xb[u % NB][i] = *(const f32x4 *)(p + (i0 + i) * 16);
         };
         const auto rows = [&](auto full_c) {
-            fetch(0);
+#pragma unroll
+            for (int u = 0; u < NB - 1 && u < NU; u++) fetch(u);
 #pragma unroll
             for (int u = 0; u < NU; u++) {
                 const int j = u / UPR, i0 = u % UPR * UN;
-                if (u + 1 < NU) fetch(u + 1);
-#pragma unroll
-                for (int i = 0; i < UN; i++) {
-                    acc[i0 + i][j] = acc_in[i0 + i][j];
-                    asm volatile("" : "+v"(acc[i0 + i][j]));
-                }
+                if (u + NB - 1 < NU) fetch(u + NB - 1);
                 const int m = m0 + wm * WM + j * 16 + l15;
                 float *p = (float *)Cp + (size_t)m * ldc + n0 + wn * WN + lq * 4;
 #pragma unroll
                 for (int i = 0; i < UN; i++) {
                     if (cut(i0 + i)) continue;
-                    f32x4 x = xb[u & 1][i];
+                    f32x4 a = acc_in[i0 + i][j]; /* out of its AGPRs here, one block at a time */
+                    asm volatile("" : "+v"(a));
+                    f32x4 x = xb[u % NB][i];
 #pragma unroll
-                    for (int e = 0; e < 4; e++) x[e] += gt[i0 + i][e] * acc[i0 + i][j][e];
+                    for (int e = 0; e < 4; e++) x[e] += gt[i0 + i][e] * a[e];
                     if (decltype(full_c)::value || m < M) *(f32x4 *)(p + (i0 + i) * 16) = x;
                 }
             }

@@ -210,9 +210,10 @@ def test_gemm_kernels_fit_the_register_file(assembly):
     """No GEMM kernel may spill: a spilled register is a scratch store next to the next tile's primed loads (the
     compiler waits for all of them first), and the fused [Q|K|V|gate|up] epilogue went over the ceiling that way
     before its two store bodies were kept apart. Every kernel of gemm.hip: no scratch frame, no spilled VGPR or SGPR.
-    The 4-wave kernels keep their accumulators in AGPRs (at least 16 TM TN / 4 of them) and their K loops free of
-    copies between the two register files; outside the loops the residual epilogue, which keeps two row blocks of
-    the residual in flight, may park a few values in spare AGPRs. The other transformer epilogues stay under 200 VGPRs."""
+    The 4-wave kernels keep their accumulators in AGPRs and nothing else (AGPRs == 16 TM TN / 4 means that no vector
+    register was parked there either), and their K loops free of copies between the two register files. The residual
+    epilogue keeps two row blocks of the residual in flight and may use the whole VGPR file; the other transformer
+    epilogues stay under 200 VGPRs."""
     usage = resource_usage(assembly["gemm.hip"][1])
     big = {k: v for k, v in usage.items() if "gemm4d_kernel" in k or "gemm4w_kernel" in k}
     assert len(big) >= 60 and len(usage) >= 100, (len(big), len(usage))
@@ -224,7 +225,7 @@ def test_gemm_kernels_fit_the_register_file(assembly):
     bodies = kernel_bodies(assembly["gemm.hip"][0])
     for name, u in sorted(big.items()):
         tm, tn, epi = map(int, re.search(r"kernelILi(\d+)ELi(\d+)ELi(\d+)E", name).groups())
-        assert 4 * tm * tn <= u["AGPRs"] <= 4 * tm * tn + (8 if epi == 3 else 0), (name, u)
+        assert u["AGPRs"] == 4 * tm * tn, (name, u)
         if epi not in (3, 6, 7):                 # (the convolution epilogues sit at 252-256, unspilled; the residual one at up to 256)
             assert u["VGPRs"] <= 200, (name, u)  # room to spare: 180 at most when this was written
         body = bodies[name]
