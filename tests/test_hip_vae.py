@@ -317,10 +317,11 @@ def test_vae_attention_in_chunks(hip, vae_pair):
     assert rel_l2(f1, cpu.decode(lat, 6, 5)[0]) <= 2e-2
 
 
-@pytest.mark.parametrize("side", [32, 64])
+@pytest.mark.parametrize("side", [32, pytest.param(64, marks=pytest.mark.skipif(not os.environ.get("FLUX_SLOW"), reason=(
+    "the 1024x1024 decode takes the CPU oracle half a minute; the 512x512 case chooses the same kernels; set FLUX_SLOW=1")))])
 def test_vae_decode_large(vae_pair, side):
     """Full-size decodes (512x512, 1024x1024: the 256x256 convolution tile and the chunked attention are
-    only chosen there) against the oracle (about half a minute of CPU work on 16 cores)."""
+    only chosen there) against the oracle."""
     dev, cpu = vae_pair
     lat = normal_f32((128, side, side), 308, 1)
     f, u = dev.decode(lat, side, side)
