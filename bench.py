@@ -643,7 +643,9 @@ def measure_workload(model, cfg, name, K, Wm, fused, args, headline):
 
     for i in range(Wm):
         sess.step(i)
+    sess.latent()                            # (reading the latent also collects the stage events recorded so far)
     fluxhip.sync()
+    stages_warm = fluxhip.stage_timing()     # the stage counters run from the session's first step on: the timed steps' share is the difference
     L = fluxhip.lib()
     if not args.no_kernel_timing:
         L.flux_hip_linear_probe(EPI_QKV_SWIGLU if fused else fluxhip.EPI_SWIGLU)   # events around the dominant kernel's launches
@@ -672,7 +674,7 @@ def measure_workload(model, cfg, name, K, Wm, fused, args, headline):
     L.flux_hip_linear_probe(-1)
     zf = sess.latent()
     assert np.isfinite(zf).all(), "latent is not finite"
-    stages = fluxhip.stage_timing()
+    stages = [a - b for a, b in zip(fluxhip.stage_timing(), stages_warm)]
     sess.close()
 
     # The drop-in sampler entry point on host buffers (upload of latent and text, modulation for
@@ -712,7 +714,7 @@ def measure_workload(model, cfg, name, K, Wm, fused, args, headline):
         if headline:
             roof["ms_per_launch_back_to_back"] = round(time_dominant_kernel(cfg, seqs * (n_img + nt), fused), 4)
     return {"ms_per_step": ms_per_step, "tflops": tflops, "flops_per_step": flops_step, "forwards": forwards, "roofline": roof,
-            "stages": [x / (K + Wm) for x in stages], "ev_ms": ev_ms, "host_run_ms": host_run_ms, "host_run_steps": n_run, "steps": K,
+            "stages": [x / K for x in stages], "ev_ms": ev_ms, "host_run_ms": host_run_ms, "host_run_steps": n_run, "steps": K,
             "tokens": n_img + nt}
 
 

@@ -1137,6 +1137,20 @@ __global__ __launch_bounds__(256) void splitk_finish_adaln_kernel(GemmArgs g, Ad
     f32x4 v[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) v[i] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    /* What the row needs besides the partial sums is requested ahead of its use - the residual and its gate in front of
+     * the slices, scale and shift in front of the sums over the row - so that the row costs two round trips to memory
+     * rather than four in a row (with 80 to 768 rows the kernel is a few waves per compute unit that wait for memory
+     * most of their time). */
+    float *xr = (float *)g.C[prob] + (size_t)m * g.ldc;
+    f32x4 x0[4], gt0[4], sc0[4], sh0[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int c = (i * 256 + threadIdx.x) * 4;
+        if (c < N) {
+            x0[i] = *(const f32x4 *)(xr + c);
+            gt0[i] = *(const f32x4 *)(g.gate[prob] + c);
+        }
+    }
     /* slices four at a time, so that a row with many short slices keeps enough loads in flight;
      * the additions stay in slice order */
     const size_t slice = (size_t)g.ws_rows * N;
@@ -1173,14 +1187,21 @@ __global__ __launch_bounds__(256) void splitk_finish_adaln_kernel(GemmArgs g, Ad
             }
         }
     }
-    float *xr = (float *)g.C[prob] + (size_t)m * g.ldc;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int c = (i * 256 + threadIdx.x) * 4;
+        if (c < N) {
+            sc0[i] = *(const f32x4 *)(a.scale[prob] + c);
+            if (!RMS) sh0[i] = *(const f32x4 *)(a.shift[prob] + c);
+        }
+    }
     float s1 = 0.0f;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         const int c = (i * 256 + threadIdx.x) * 4;
         if (c < N) {
-            f32x4 x = *(f32x4 *)(xr + c);
-            const f32x4 gt = *(const f32x4 *)(g.gate[prob] + c);
+            f32x4 x = x0[i];
+            const f32x4 gt = gt0[i];
 #pragma unroll
             for (int e = 0; e < 4; e++) x[e] += gt[e] * v[i][e];
             *(f32x4 *)(xr + c) = x;
@@ -1204,13 +1225,13 @@ __global__ __launch_bounds__(256) void splitk_finish_adaln_kernel(GemmArgs g, Ad
     for (int i = 0; i < 4; i++) {
         const int c = (i * 256 + threadIdx.x) * 4;
         if (c < N) {
-            const f32x4 sc = *(const f32x4 *)(a.scale[prob] + c);
+            const f32x4 sc = sc0[i];
             bf16x4 r;
             if (RMS) {
 #pragma unroll
                 for (int e = 0; e < 4; e++) r[e] = (bf16)(v[i][e] * inv * sc[e]);
             } else {
-                const f32x4 sh = *(const f32x4 *)(a.shift[prob] + c);
+                const f32x4 sh = sh0[i];
 #pragma unroll
                 for (int e = 0; e < 4; e++) r[e] = (bf16)((1.0f + sc[e]) * ((v[i][e] - mean) * inv) + sh[e]);
             }
