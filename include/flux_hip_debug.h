@@ -17,11 +17,12 @@ extern "C" {
 
 /* force_tile: 0/1/2/3/5/6/7 pins the GEMM tile of flux_hip_linear (64x128, 128x128, 256x256, 64x64,
  * 288x192, 192x192, 256x192; 4 = 256x256 in its 8-wave form, never chosen automatically; 8 / 9 / 10 = 64x128 / 128x128 / 96x128
- * with a ring of 6 / 5 / 5 LDS stages, only for row ranges of at most 64 / 128 / 96 rows), -1 restores
- * the automatic choice (a tile whose width does not divide N is skipped; if none is left the 128x128
- * tile runs). */
+ * with a ring of 6 / 5 / 5 LDS stages, only for row ranges of at most 64 / 128 / 96 rows; 11 = 256x224, whose last column
+ * tile is cut off at N: for the residual and bf16 epilogues with at least four 64-wide K steps and no K slices), -1
+ * restores the automatic choice (a tile whose width does not divide N is skipped, tile 11 apart; if none is left the
+ * 128x128 tile runs). */
 void flux_hip_linear_force_tile(int tile);
-/* bit t set = the automatic choice may use tile t (default 0x7EF: all but tile 4; 0 restores it) */
+/* bit t set = the automatic choice may use tile t (default 0xFEF: all but tile 4; 0 restores it) */
 void flux_hip_linear_tile_mask(unsigned mask);
 /* 0 turns the split-K path off (default 1) */
 void flux_hip_linear_enable_splitk(int on);
