@@ -150,6 +150,46 @@ def test_linear_tile_with_cut_last_column_tile(hip, oracle_mod, N, K):
     L.flux_hip_linear_force_tile(-1)
 
 
+@pytest.mark.parametrize("epi,N", [("resid", 3072), ("bf16", 9216)])
+def test_linear_cut_tile_at_the_double_stream_shapes(hip, epi, N):
+    """256 x 224 where the model uses it: 4096 image + 512 text rows with weights of their own, K = 3072, the gated residual
+    add at N = 3072 (252 tiles: one per workgroup, the last of every 14 cut off after 160 columns) and the bf16 store at
+    N = 9216 (756 tiles: three per workgroup in one pipeline, a cut tile of 32 columns in the middle of some workgroups'
+    runs, so the first barrier of the tile behind it must not count on stores that were never issued). Bit for bit what
+    the 256 x 256 tile gives, which the whole-model tests hold against the oracle; nothing written behind the outputs."""
+    L = hip.lib()
+    K, M0, M1 = 3072, 4096, 512
+    a = q(normal_f32((M0 + M1, K), 43, 1))
+    W0 = q(normal_f32((N, K), 43, 2, 0.0, 0.02))
+    W1 = q(normal_f32((N, K), 43, 3, 0.0, 0.02))
+    da, dW0, dW1 = dev_bf16(hip, a), dev_bf16(hip, W0), dev_bf16(hip, W1)
+    got = {}
+    for tile in (11, 2):
+        L.flux_hip_linear_force_tile(tile)
+        L.flux_hip_linear_probe(hip.EPI_RESID if epi == "resid" else hip.EPI_BF16)
+        if epi == "resid":
+            res = normal_f32((M0 + M1 + 1, N), 43, 4)
+            g0, g1 = hip.DevBuf.from_array(normal_f32((N,), 43, 5)), hip.DevBuf.from_array(normal_f32((N,), 43, 6))
+            out = hip.DevBuf.from_array(res)
+            hip.linear(hip.EPI_RESID, [(da.ptr, dW0.ptr, out.ptr, g0.ptr, M0), (da.at(M0 * K * 2), dW1.ptr, out.at(M0 * N * 4), g1.ptr, M1)],
+                       N, K, K, K, N)
+            full = out.to_array(np.float32, (M0 + M1 + 1, N))
+            assert np.array_equal(full[-1], res[-1])
+        else:
+            out = hip.DevBuf.from_array(np.full((M0 + M1 + 1, N), 0x4242, np.uint16))
+            hip.linear(hip.EPI_BF16, [(da.ptr, dW0.ptr, out.ptr, None, M0), (da.at(M0 * K * 2), dW1.ptr, out.at(M0 * N * 2), None, M1)],
+                       N, K, K, K, N, 0, 0)
+            full = out.to_array(np.uint16, (M0 + M1 + 1, N))
+            assert (full[-1] == 0x4242).all()
+        tiles = np.zeros(4, np.int32)
+        assert L.flux_hip_linear_probe_read_launches(4, tiles.ctypes.data, None) == 1 and tiles[0] == tile
+        got[tile] = full[:-1]
+    L.flux_hip_linear_probe(-1)
+    L.flux_hip_linear_force_tile(-1)
+    assert np.array_equal(got[11], got[2])
+    assert np.isfinite(got[11].astype(np.float32)).all() if epi == "resid" else True
+
+
 @pytest.mark.parametrize("tile", [2, 5, 6, 7])
 @pytest.mark.parametrize("K", [64, 128, 192, 256, 448])
 def test_linear_large_tile_k_steps(hip, oracle_mod, K, tile):
